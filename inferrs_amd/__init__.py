@@ -1,0 +1,11 @@
+"""inferrs_amd: a small, whole inference engine for one AMD MI355X, in the manner of inferrs.
+
+    config/    typed configuration from config.json, the architecture registry, layer specs
+    weights/   safetensors by tensor name, load checks, random model folders
+    parts/     norm, position encoding, attention, feed-forward, block: built from specs
+    cache/     pages with block tables per request, per-request state slots
+    engine/    model assembly, the step function, the scheduler, generation
+    sampling/  sampling parameters and the device sampler
+    ops/       host checks and C calls into the HIP kernels of csrc/
+"""
+__version__ = "0.1.0"

@@ -1,0 +1,182 @@
+"""Typed configuration of the Qwen3 dense decoder, read from its config.json keys.
+
+Keys and defaults follow the reference's `to_qwen3_config`
+(`inferrs-models/src/config.rs:468-502`): `head_dim` defaults to
+`hidden_size / num_attention_heads`, `rms_norm_eps` to 1e-6, `rope_theta` to
+1e6, `tie_word_embeddings` to true, `max_position_embeddings` to 40960
+(`config.rs:728`).  Unlike the reference, the sizes themselves have no default
+here: a config.json without them is an error that names the key.  As in the
+reference, `sliding_window`, `max_window_layers`, `layer_types`,
+`rope_scaling` and `hidden_act` do not change the model (`qwen3.rs:28-45`
+holds none of them): every layer attends to all earlier positions and the
+activation is SiLU.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass, asdict
+from typing import Any, Dict, Tuple
+
+from .spec import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec,
+                   PositionSpec, SpecError, default_schedule)
+
+
+class ConfigError(ValueError):
+    pass
+
+
+def _require_int(raw: Dict[str, Any], key: str, minimum: int = 1) -> int:
+    if key not in raw or raw[key] is None:
+        raise ConfigError(f"config.json: required key '{key}' is missing")
+    v = raw[key]
+    if isinstance(v, bool) or not isinstance(v, int):
+        raise ConfigError(f"config.json: '{key}' must be an integer, got {v!r}")
+    if v < minimum:
+        raise ConfigError(f"config.json: '{key}' must be >= {minimum}, got {v}")
+    return v
+
+
+def _opt_number(raw: Dict[str, Any], key: str, default: float) -> float:
+    v = raw.get(key)
+    if v is None:
+        return float(default)
+    if isinstance(v, bool) or not isinstance(v, (int, float)):
+        raise ConfigError(f"config.json: '{key}' must be a number, got {v!r}")
+    return float(v)
+
+
+@dataclass(frozen=True)
+class Qwen3Config:
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_hidden_layers: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    rms_norm_eps: float
+    rope_theta: float
+    tie_word_embeddings: bool
+    max_position_embeddings: int
+    eos_token_ids: Tuple[int, ...] = ()
+
+    architecture = "Qwen3ForCausalLM"
+    model_type = "qwen3"
+
+    @classmethod
+    def from_dict(cls, raw: Dict[str, Any]) -> "Qwen3Config":
+        hidden = _require_int(raw, "hidden_size")
+        heads = _require_int(raw, "num_attention_heads")
+        kv_heads = raw.get("num_key_value_heads")
+        if kv_heads is None:
+            kv_heads = heads
+        else:
+            kv_heads = _require_int(raw, "num_key_value_heads")
+        head_dim = raw.get("head_dim")
+        if head_dim is None:
+            if hidden % heads:
+                raise ConfigError(
+                    f"config.json: 'head_dim' is absent and hidden_size {hidden} is not a "
+                    f"multiple of num_attention_heads {heads}")
+            head_dim = hidden // heads
+        else:
+            head_dim = _require_int(raw, "head_dim")
+        tie = raw.get("tie_word_embeddings")
+        if tie is None:
+            tie = True
+        if not isinstance(tie, bool):
+            raise ConfigError(f"config.json: 'tie_word_embeddings' must be a boolean, got {tie!r}")
+        eos = raw.get("eos_token_id")
+        if eos is None:
+            eos_ids: Tuple[int, ...] = ()
+        elif isinstance(eos, int) and not isinstance(eos, bool):
+            eos_ids = (eos,)
+        elif isinstance(eos, list) and all(isinstance(e, int) for e in eos):
+            eos_ids = tuple(eos)
+        else:
+            raise ConfigError(f"config.json: 'eos_token_id' must be an integer or a list, got {eos!r}")
+        maxpos = raw.get("max_position_embeddings")
+        maxpos = 40960 if maxpos is None else _require_int(raw, "max_position_embeddings")
+        cfg = cls(
+            vocab_size=_require_int(raw, "vocab_size"),
+            hidden_size=hidden,
+            intermediate_size=_require_int(raw, "intermediate_size"),
+            num_hidden_layers=_require_int(raw, "num_hidden_layers"),
+            num_attention_heads=heads,
+            num_key_value_heads=kv_heads,
+            head_dim=head_dim,
+            rms_norm_eps=_opt_number(raw, "rms_norm_eps", 1e-6),
+            rope_theta=_opt_number(raw, "rope_theta", 1_000_000.0),
+            tie_word_embeddings=tie,
+            max_position_embeddings=maxpos,
+            eos_token_ids=eos_ids,
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.num_attention_heads % self.num_key_value_heads:
+            raise ConfigError(
+                f"config.json: num_attention_heads {self.num_attention_heads} is not a multiple "
+                f"of num_key_value_heads {self.num_key_value_heads}")
+        if self.head_dim % 2:
+            raise ConfigError(f"config.json: head_dim {self.head_dim} must be even for rotary pairs")
+        if not (self.rms_norm_eps > 0.0):
+            raise ConfigError(f"config.json: rms_norm_eps must be positive, got {self.rms_norm_eps}")
+        if not (self.rope_theta > 0.0):
+            raise ConfigError(f"config.json: rope_theta must be positive, got {self.rope_theta}")
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = asdict(self)
+        eos = d.pop("eos_token_ids")
+        d["architectures"] = [self.architecture]
+        d["model_type"] = self.model_type
+        d["hidden_act"] = "silu"
+        if eos:
+            d["eos_token_id"] = eos[0] if len(eos) == 1 else list(eos)
+        return d
+
+    def to_spec(self) -> ModelSpec:
+        """The layer list of the reference's `Qwen3Model::new` (`qwen3.rs:341-395`)."""
+        position = PositionSpec(kind="rope", head_dim=self.head_dim, rot_dim=self.head_dim,
+                                theta=self.rope_theta, pairing="half")
+        head_norm = NormSpec(size=self.head_dim, eps=self.rms_norm_eps)
+        layer_norm = NormSpec(size=self.hidden_size, eps=self.rms_norm_eps)
+        layers = []
+        for i in range(self.num_hidden_layers):
+            p = f"model.layers.{i}."
+            layers.append(LayerSpec(
+                mixer=AttentionSpec(hidden=self.hidden_size, n_heads=self.num_attention_heads,
+                                    n_kv_heads=self.num_key_value_heads, head_dim=self.head_dim,
+                                    position=position, qk_norm=head_norm, window=None),
+                ffn=GatedMlpSpec(hidden=self.hidden_size, intermediate=self.intermediate_size,
+                                 activation="silu"),
+                norm_mixer=layer_norm, norm_ffn=layer_norm,
+                mixer_prefix=p + "self_attn.", ffn_prefix=p + "mlp.",
+                norm_mixer_name=p + "input_layernorm.weight",
+                norm_ffn_name=p + "post_attention_layernorm.weight",
+            ))
+        spec = ModelSpec(
+            architecture=self.architecture, vocab_size=self.vocab_size, hidden=self.hidden_size,
+            layers=tuple(layers), schedule=default_schedule(self.num_hidden_layers),
+            final_norm=layer_norm, final_norm_name="model.norm.weight",
+            embed_name="model.embed_tokens.weight", head_name="lm_head.weight",
+            head_required=not self.tie_word_embeddings,
+            max_position=self.max_position_embeddings, eos_token_ids=self.eos_token_ids)
+        spec.validate()
+        return spec
+
+
+def read_config_json(model_dir: str) -> Dict[str, Any]:
+    path = os.path.join(model_dir, "config.json")
+    if not os.path.isfile(path):
+        raise ConfigError(f"config.json not found in {model_dir}")
+    try:
+        with open(path, "r", encoding="utf-8") as f:
+            raw = json.load(f)
+    except json.JSONDecodeError as e:
+        raise ConfigError(f"Failed to parse config.json in {model_dir}: {e}") from e
+    if not isinstance(raw, dict):
+        raise ConfigError(f"config.json in {model_dir} must hold a JSON object")
+    return raw

@@ -1,0 +1,136 @@
+"""Architecture-neutral description of a decoder: parts, layers and run order.
+
+A model is data before it is code: a `ModelSpec` lists one `LayerSpec` per
+layer, each naming its mixer, feed-forward and norms by `kind` together with
+every size and constant they need, and a `schedule` that says in which order
+layers run and whose cache each of them uses.  Nothing in here knows a model
+family; an architecture is a function from its config.json to a `ModelSpec`
+(see `inferrs_amd.config.registry`).
+
+The reference wires the same information into Rust structs per model
+(`inferrs-models/src/models/qwen3.rs:28-45`, `:264-290`); here it is explicit
+so that layers of one model may differ and parts can be reused.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Optional, Tuple
+
+
+class SpecError(ValueError):
+    """A specification that the parts or kernels cannot honour."""
+
+
+@dataclass(frozen=True)
+class NormSpec:
+    """Root-mean-square norm over the last dimension."""
+    size: int
+    eps: float
+    add_one: bool = False          # weight is stored as (w - 1) when True
+    kind: str = "rmsnorm"
+
+
+@dataclass(frozen=True)
+class PositionSpec:
+    """How positions enter queries and keys.
+
+    kind "rope": rotate the first `rot_dim` features of each head by
+    angle = position * theta**(-2i/rot_dim); pairing "half" pairs feature i
+    with i + rot_dim/2, "interleaved" pairs 2i with 2i+1.
+    kind "none": nothing is applied.
+    """
+    kind: str = "rope"
+    head_dim: int = 0
+    rot_dim: int = 0
+    theta: float = 10000.0
+    pairing: str = "half"
+
+
+@dataclass(frozen=True)
+class AttentionSpec:
+    """Grouped-query softmax attention over a paged key/value cache."""
+    hidden: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    position: PositionSpec
+    qk_norm: Optional[NormSpec] = None     # per-head norm of q and k before rotation
+    window: Optional[int] = None           # keys kept: the last `window` positions; None = all
+    scale: Optional[float] = None          # None = 1/sqrt(head_dim)
+    kind: str = "attention"
+
+    @property
+    def softmax_scale(self) -> float:
+        return self.scale if self.scale is not None else self.head_dim ** -0.5
+
+
+@dataclass(frozen=True)
+class GatedMlpSpec:
+    """down( act(gate(x)) * up(x) ), no biases."""
+    hidden: int
+    intermediate: int
+    activation: str = "silu"
+    kind: str = "gated_mlp"
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One residual block: which parts, and the tensor-name prefixes they load from."""
+    mixer: Any
+    ffn: Any
+    norm_mixer: NormSpec
+    norm_ffn: NormSpec
+    mixer_prefix: str
+    ffn_prefix: str
+    norm_mixer_name: str
+    norm_ffn_name: str
+    arrangement: str = "pre_norm"
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    """One stop in the run order: run `layer`; its mixer uses the cache of `cache_of`.
+
+    `cache_of == layer` (the default) means the layer owns and writes its cache.
+    Another index means it only reads that layer's cache and writes none.
+    """
+    layer: int
+    cache_of: Optional[int] = None
+
+    @property
+    def cache_owner(self) -> int:
+        return self.layer if self.cache_of is None else self.cache_of
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    architecture: str
+    vocab_size: int
+    hidden: int
+    layers: Tuple[LayerSpec, ...]
+    schedule: Tuple[ScheduleEntry, ...]
+    final_norm: NormSpec
+    final_norm_name: str
+    embed_name: str
+    head_name: Optional[str]            # None: logits use the embedding table
+    max_position: int
+    head_required: bool = True          # False: use `head_name` if the file has it, else the table
+    eos_token_ids: Tuple[int, ...] = field(default_factory=tuple)
+
+    def validate(self) -> None:
+        n = len(self.layers)
+        if n == 0:
+            raise SpecError("a model needs at least one layer")
+        for e in self.schedule:
+            if not (0 <= e.layer < n) or not (0 <= e.cache_owner < n):
+                raise SpecError(f"schedule entry {e} names a layer outside 0..{n - 1}")
+        owners = {e.layer for e in self.schedule if e.cache_of in (None, e.layer)}
+        for e in self.schedule:
+            if e.cache_owner not in owners:
+                raise SpecError(
+                    f"schedule entry {e} reads the cache of layer {e.cache_owner}, "
+                    "which never runs as the owner of its cache")
+
+
+def default_schedule(n_layers: int) -> Tuple[ScheduleEntry, ...]:
+    return tuple(ScheduleEntry(i) for i in range(n_layers))

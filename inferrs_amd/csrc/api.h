@@ -1,0 +1,50 @@
+// C entry points of the kernel library.  Every function takes device pointers and a HIP
+// stream, launches asynchronously on it, returns 0 on success and a non-zero code after
+// leaving a message for ia_last_error().  dtype arguments: 0 = float32, 1 = bfloat16.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#define IA_ABI_VERSION 1
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* ia_last_error(void);
+int ia_abi_version(void);
+
+int ia_embed_gather(void* out, const void* table, const int* ids, int n, int hidden, int vocab,
+                    int dtype, hipStream_t stream);
+int ia_gather_rows(void* out, const void* x, const int* rows, int n, int cols, int dtype,
+                   hipStream_t stream);
+int ia_rmsnorm(void* out, const void* x, const float* w, float eps, int rows, int cols,
+               int add_one, int dtype, hipStream_t stream);
+int ia_add_rmsnorm(void* out, void* x, const void* delta, const float* w, float eps, int rows,
+                   int cols, int add_one, int dtype, hipStream_t stream);
+int ia_add_inplace(void* x, const void* delta, long long n, int dtype, hipStream_t stream);
+int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream);
+int ia_rope_table(float* cos_out, float* sin_out, const int* positions, const float* inv_freq,
+                  int n, int half, hipStream_t stream);
+
+int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const void* qkv,
+                  const float* q_norm_w, const float* k_norm_w, const float* cos_t,
+                  const float* sin_t, const int* slots, int n, int nq, int nkv, int d, int rot,
+                  int interleaved, int page_size, float eps, int add_one, int dtype,
+                  hipStream_t stream);
+
+int ia_attention_generic(void* out, const void* q, const void* k_cache, const void* v_cache,
+                         const int* positions, const int* token_seq, const int* block_table,
+                         int n, int max_pages, int nq, int nkv, int d, int page_size, int window,
+                         float scale, int dtype, hipStream_t stream);
+
+int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
+                  int out_dtype, hipStream_t stream);
+int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, float* partial, int M, int N,
+                        int K, int splits, int out_dtype, hipStream_t stream);
+
+int ia_argmax(int* out, const float* logits, int rows, int vocab, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,212 @@
+// Row-wise and element-wise kernels: embedding gather, RMS norm (plain and fused with the
+// residual add), SiLU-gate product, rotary angle tables, row gather, residual add.
+//
+// Formulas follow the reference's CUDA kernels: rmsnorm keeps the sum of squares and the
+// scale in 32-bit and rounds once (inferrs-kernels/candle-kernels/src/reduce.cu:189-228);
+// silu(z) = z / (1 + exp(-z)) (unary.cu:59-61); rotary angles are position * inv_freq in
+// 32-bit (inferrs-models/src/models/attention_utils.rs:186-216).
+#include "common.h"
+#include "api.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+
+void ia_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char* ia_last_error(void) { return g_error; }
+
+extern "C" int ia_abi_version(void) { return IA_ABI_VERSION; }
+
+// ---- embedding ------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(T* __restrict__ out, const T* __restrict__ table,
+                                    const int* __restrict__ ids, int hidden, int vocab) {
+    const int row = blockIdx.x;
+    const int id = ids[row];
+    const bool ok = id >= 0 && id < vocab;
+    const T* src = table + (size_t)(ok ? id : 0) * hidden;
+    T* dst = out + (size_t)row * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+        if (ok) dst[c] = src[c];
+        else st(dst + c, 0.f);
+    }
+}
+
+extern "C" int ia_embed_gather(void* out, const void* table, const int* ids, int n, int hidden,
+                               int vocab, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes n=%d hidden=%d vocab=%d", n, hidden, vocab);
+    if (n == 0) return 0;
+    const int block = hidden >= 1024 ? 256 : 64;
+    if (dtype == IA_F32)
+        embed_gather_kernel<float><<<n, block, 0, stream>>>((float*)out, (const float*)table, ids, hidden, vocab);
+    else if (dtype == IA_BF16)
+        embed_gather_kernel<bf16_t><<<n, block, 0, stream>>>((bf16_t*)out, (const bf16_t*)table, ids, hidden, vocab);
+    else
+        IA_CHECK(false, "embed_gather: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("embed_gather");
+    return 0;
+}
+
+// ---- row gather -----------------------------------------------------------------------------
+template <typename T>
+__global__ void gather_rows_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                   const int* __restrict__ rows, int cols) {
+    const T* src = x + (size_t)rows[blockIdx.x] * cols;
+    T* dst = out + (size_t)blockIdx.x * cols;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) dst[c] = src[c];
+}
+
+extern "C" int ia_gather_rows(void* out, const void* x, const int* rows, int n, int cols,
+                              int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && cols > 0, "gather_rows: bad sizes n=%d cols=%d", n, cols);
+    if (n == 0) return 0;
+    const int block = cols >= 1024 ? 256 : 64;
+    if (dtype == IA_F32)
+        gather_rows_kernel<float><<<n, block, 0, stream>>>((float*)out, (const float*)x, rows, cols);
+    else if (dtype == IA_BF16)
+        gather_rows_kernel<bf16_t><<<n, block, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, rows, cols);
+    else
+        IA_CHECK(false, "gather_rows: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("gather_rows");
+    return 0;
+}
+
+// ---- RMS norm -------------------------------------------------------------------------------
+// One block per row.  The block size depends on the row length only, so a row's result does
+// not depend on how many rows are normalised together.
+template <typename T, bool ADD>
+__global__ void rmsnorm_kernel(T* __restrict__ out, T* __restrict__ x, const T* __restrict__ delta,
+                               const float* __restrict__ w, float eps, int cols, int add_one) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * cols;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        float v = ld(x + base + c);
+        if (ADD) {
+            v = round_to(x, v + ld(delta + base + c));
+            st(x + base + c, v);
+        }
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)cols + eps);
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        const float v = ld(x + base + c);
+        const float g = add_one ? 1.0f + w[c] : w[c];
+        st(out + base + c, scale * v * g);
+    }
+}
+
+static int norm_block(int cols) { return cols >= 2048 ? 512 : (cols >= 512 ? 256 : 64); }
+
+extern "C" int ia_rmsnorm(void* out, const void* x, const float* w, float eps, int rows, int cols,
+                          int add_one, int dtype, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && cols > 0, "rmsnorm: bad sizes rows=%d cols=%d", rows, cols);
+    if (rows == 0) return 0;
+    const int block = norm_block(cols);
+    if (dtype == IA_F32)
+        rmsnorm_kernel<float, false><<<rows, block, 0, stream>>>((float*)out, (float*)x, nullptr, w, eps, cols, add_one);
+    else if (dtype == IA_BF16)
+        rmsnorm_kernel<bf16_t, false><<<rows, block, 0, stream>>>((bf16_t*)out, (bf16_t*)x, nullptr, w, eps, cols, add_one);
+    else
+        IA_CHECK(false, "rmsnorm: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("rmsnorm");
+    return 0;
+}
+
+// x += delta (sum in 32-bit, stored in the model's precision); out = rmsnorm(x).
+extern "C" int ia_add_rmsnorm(void* out, void* x, const void* delta, const float* w, float eps,
+                              int rows, int cols, int add_one, int dtype, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && cols > 0, "add_rmsnorm: bad sizes rows=%d cols=%d", rows, cols);
+    if (rows == 0) return 0;
+    const int block = norm_block(cols);
+    if (dtype == IA_F32)
+        rmsnorm_kernel<float, true><<<rows, block, 0, stream>>>((float*)out, (float*)x, (const float*)delta, w, eps, cols, add_one);
+    else if (dtype == IA_BF16)
+        rmsnorm_kernel<bf16_t, true><<<rows, block, 0, stream>>>((bf16_t*)out, (bf16_t*)x, (const bf16_t*)delta, w, eps, cols, add_one);
+    else
+        IA_CHECK(false, "add_rmsnorm: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+}
+
+// ---- residual add ---------------------------------------------------------------------------
+template <typename T>
+__global__ void add_kernel(T* __restrict__ x, const T* __restrict__ delta, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        st(x + i, ld(x + i) + ld(delta + i));
+}
+
+extern "C" int ia_add_inplace(void* x, const void* delta, long long n, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0, "add_inplace: bad size %lld", n);
+    if (n == 0) return 0;
+    const int block = 256;
+    const int grid = (int)((n + block - 1) / block < 65535 ? (n + block - 1) / block : 65535);
+    if (dtype == IA_F32)
+        add_kernel<float><<<grid, block, 0, stream>>>((float*)x, (const float*)delta, (size_t)n);
+    else if (dtype == IA_BF16)
+        add_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)x, (const bf16_t*)delta, (size_t)n);
+    else
+        IA_CHECK(false, "add_inplace: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("add_inplace");
+    return 0;
+}
+
+// ---- SiLU(gate) * up ------------------------------------------------------------------------
+// `gu` holds rows of [gate(0..inter) | up(0..inter)]; the product is formed in 32-bit.
+template <typename T>
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t row = i / inter;
+        const int c = (int)(i - row * inter);
+        const float g = ld(gu + row * 2 * inter + c);
+        const float u = ld(gu + row * 2 * inter + inter + c);
+        st(out + i, g / (1.0f + expf(-g)) * u);
+    }
+}
+
+extern "C" int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && inter > 0, "silu_mul: bad sizes rows=%d inter=%d", rows, inter);
+    if (rows == 0) return 0;
+    const size_t total = (size_t)rows * inter;
+    const int block = 256;
+    const size_t want = (total + block - 1) / block;
+    const int grid = (int)(want < 65535 ? want : 65535);
+    if (dtype == IA_F32)
+        silu_mul_kernel<float><<<grid, block, 0, stream>>>((float*)out, (const float*)gu, inter, total);
+    else if (dtype == IA_BF16)
+        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, inter, total);
+    else
+        IA_CHECK(false, "silu_mul: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("silu_mul");
+    return 0;
+}
+
+// ---- rotary angle table for the tokens of one step ----------------------------------------------
+__global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict__ sin_out,
+                                  const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  int half, int total) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int t = i / half, f = i - t * half;
+    const float ang = (float)positions[t] * inv_freq[f];
+    cos_out[i] = cosf(ang);
+    sin_out[i] = sinf(ang);
+}
+
+extern "C" int ia_rope_table(float* cos_out, float* sin_out, const int* positions,
+                             const float* inv_freq, int n, int half, hipStream_t stream) {
+    IA_CHECK(n >= 0 && half > 0, "rope_table: bad sizes n=%d half=%d", n, half);
+    if (n == 0) return 0;
+    const int total = n * half;
+    rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(cos_out, sin_out, positions, inv_freq, half, total);
+    IA_LAUNCH_CHECK("rope_table");
+    return 0;
+}

@@ -1,0 +1,111 @@
+// Per-head RMS norm of queries and keys, rotary position encoding, and the write of the new
+// keys and values into their cache pages, in one pass over the projection output.
+//
+// Order as in the reference: norm per head over head_dim with one shared weight vector
+// (inferrs-models/src/models/qwen3.rs:128-129, attention_utils.rs:52-58), then rotation
+// (qwen3.rs:132-135) with out[i] = x[i]c - x[j]s, out[j] = x[i]s + x[j]c
+// (inferrs-kernels/candle-kernels/src/reduce.cu:292-312 for j = i + rot/2, :275-289 for the
+// interleaved pairing), then the cache append (qwen3.rs:145-161).  Values are copied as they are.
+// Norm, angles and rotation stay in 32-bit registers; one rounding happens at the store.
+#include "common.h"
+#include "api.h"
+
+#define QK_MAX_HEAD_DIM 512
+#define QK_WAVES 4
+
+// One wave per (token, head).  Heads 0..nq are queries, nq..nq+nkv keys, the rest values.
+template <typename T>
+__global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_kernel(
+    T* __restrict__ q_out,              // [n, nq, d]
+    T* __restrict__ k_cache,            // [pages, nkv, page_size, d] or null
+    T* __restrict__ v_cache,
+    const T* __restrict__ qkv,          // [n, (nq + 2 nkv) d]
+    const float* __restrict__ q_norm_w, // [d] or null
+    const float* __restrict__ k_norm_w, // [d] or null
+    const float* __restrict__ cos_t,    // [n, rot/2] or null
+    const float* __restrict__ sin_t,
+    const int* __restrict__ slots,      // [n] page * page_size + offset, or null (no write)
+    int n, int nq, int nkv, int d, int rot, int interleaved, int page_size, float eps, int add_one) {
+    __shared__ float buf[QK_WAVES][QK_MAX_HEAD_DIM];
+    const int lane = threadIdx.x & (IA_WAVE - 1);
+    const int wave = threadIdx.x / IA_WAVE;
+    const int heads = slots ? nq + 2 * nkv : nq;
+    const long long unit = (long long)blockIdx.x * QK_WAVES + wave;
+    const bool active = unit < (long long)n * heads;
+    const int tok = active ? (int)(unit / heads) : 0;
+    const int hh = active ? (int)(unit % heads) : 0;
+    const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);
+    const T* src = qkv + ((size_t)tok * (nq + 2 * nkv) + hh) * d;
+    float* row = buf[wave];
+
+    float ss = 0.f;
+    if (active) {
+        for (int j = lane; j < d; j += IA_WAVE) {
+            const float v = ld(src + j);
+            row[j] = v;
+            ss += v * v;
+        }
+    }
+    const float* nw = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+    if (nw != nullptr) {
+        ss = wave_sum(ss);
+        const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+        if (active)
+            for (int j = lane; j < d; j += IA_WAVE) row[j] = scale * row[j] * (add_one ? 1.0f + nw[j] : nw[j]);
+    }
+    __syncthreads();
+    if (!active) return;
+
+    T* dst;
+    if (kind == 0) {
+        dst = q_out + ((size_t)tok * nq + hh) * d;
+    } else {
+        const int slot = slots[tok];
+        const int page = slot / page_size, off = slot - page * page_size;
+        const int kh = kind == 1 ? hh - nq : hh - nq - nkv;
+        T* cache = kind == 1 ? k_cache : v_cache;
+        dst = cache + (((size_t)page * nkv + kh) * page_size + off) * d;
+    }
+    if (kind == 2 || cos_t == nullptr) {
+        for (int j = lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
+        return;
+    }
+    const int half = rot / 2;
+    for (int i = lane; i < half; i += IA_WAVE) {
+        const float c = cos_t[(size_t)tok * half + i], s = sin_t[(size_t)tok * half + i];
+        const int ia = interleaved ? 2 * i : i;
+        const int ib = interleaved ? 2 * i + 1 : i + half;
+        const float a = row[ia], b = row[ib];
+        st(dst + ia, a * c - b * s);
+        st(dst + ib, a * s + b * c);
+    }
+    for (int j = rot + lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
+}
+
+extern "C" int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const void* qkv,
+                             const float* q_norm_w, const float* k_norm_w, const float* cos_t,
+                             const float* sin_t, const int* slots, int n, int nq, int nkv, int d,
+                             int rot, int interleaved, int page_size, float eps, int add_one,
+                             int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && nq > 0 && nkv > 0, "qk_rope_kv: bad sizes n=%d nq=%d nkv=%d", n, nq, nkv);
+    IA_CHECK(d > 0 && d <= QK_MAX_HEAD_DIM, "qk_rope_kv: head_dim %d is outside 1..%d", d, QK_MAX_HEAD_DIM);
+    IA_CHECK(rot >= 0 && rot <= d && rot % 2 == 0, "qk_rope_kv: rot_dim %d must be even and <= head_dim %d", rot, d);
+    IA_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_rope_kv: cos and sin tables must come together");
+    IA_CHECK(cos_t == nullptr || rot > 0, "qk_rope_kv: a rotary table needs rot_dim > 0");
+    IA_CHECK(slots == nullptr || (k_cache && v_cache && page_size > 0), "qk_rope_kv: slots given without a cache");
+    if (n == 0) return 0;
+    const long long units = (long long)n * (slots ? nq + 2 * nkv : nq);
+    const unsigned grid = (unsigned)((units + QK_WAVES - 1) / QK_WAVES);
+    if (dtype == IA_F32)
+        qk_rope_kv_kernel<float><<<grid, QK_WAVES * IA_WAVE, 0, stream>>>(
+            (float*)q_out, (float*)k_cache, (float*)v_cache, (const float*)qkv, q_norm_w, k_norm_w,
+            cos_t, sin_t, slots, n, nq, nkv, d, rot, interleaved, page_size, eps, add_one);
+    else if (dtype == IA_BF16)
+        qk_rope_kv_kernel<bf16_t><<<grid, QK_WAVES * IA_WAVE, 0, stream>>>(
+            (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)qkv, q_norm_w, k_norm_w,
+            cos_t, sin_t, slots, n, nq, nkv, d, rot, interleaved, page_size, eps, add_one);
+    else
+        IA_CHECK(false, "qk_rope_kv: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("qk_rope_kv");
+    return 0;
+}

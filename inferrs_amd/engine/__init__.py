@@ -1,0 +1,3 @@
+from .batch import GroupStep, StepContext
+from .model import DecoderModel, parse_dtype
+from .engine import Engine, Entry, StepError

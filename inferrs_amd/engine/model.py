@@ -1,0 +1,99 @@
+"""A decoder assembled from a `ModelSpec`: embedding, the blocks in schedule order, final norm
+and logits at the wanted rows (`inferrs-models/src/models/qwen3.rs:398-440`,
+`attention_utils.rs:382-395`).  Nothing here names an architecture."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.spec import ModelSpec
+from ..parts.base import part_class
+from ..parts.block import Block
+from ..parts.linear import Linear, to_compute
+from .batch import StepContext
+
+DTYPES = {"float32": torch.float32, "f32": torch.float32, "fp32": torch.float32,
+          "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"the engine computes in float32 or bfloat16, not {name}")
+        return name
+    try:
+        return DTYPES[str(name).lower()]
+    except KeyError:
+        raise ValueError(f"unknown dtype {name!r}; choose bfloat16 or float32") from None
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
+        """`tensors`: every tensor of `model_tensors(spec)` by name, in its stored precision,
+        on any device.  Entries are dropped from the dict as they are taken over."""
+        spec.validate()
+        self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
+        self.embed = to_compute(tensors[spec.embed_name], dtype, device)
+        head = tensors.pop(spec.head_name, None) if spec.head_name is not None else None
+        if head is not None:
+            self.head = Linear([head], dtype, device)
+        else:
+            self.head = Linear.__new__(Linear)           # logits share the embedding table
+            self.head.weight = self.embed
+            self.head.out_features, self.head.in_features = self.embed.shape
+        del head
+        tensors.pop(spec.embed_name, None)
+        self.blocks = []
+        for layer in spec.layers:
+            names = [n for n in tensors if n.startswith(layer.mixer_prefix) or n.startswith(layer.ffn_prefix)
+                     or n in (layer.norm_mixer_name, layer.norm_ffn_name)]
+            self.blocks.append(Block(layer, {n: tensors[n] for n in names}, dtype, device))
+            for n in names:
+                del tensors[n]
+        self.final_norm = part_class("norm", spec.final_norm)(
+            spec.final_norm, {"weight": tensors.pop(spec.final_norm_name)}, dtype, device)
+
+    def cache_needs(self) -> Dict[int, object]:
+        """Cache-owning layer -> what its mixer keeps per request."""
+        needs: Dict[int, object] = {}
+        for e in self.spec.schedule:
+            if e.cache_owner == e.layer:
+                mixer = self.spec.layers[e.layer].mixer
+                needs[e.layer] = part_class("mixer", mixer).cache_need(mixer)
+        return needs
+
+    def forward(self, ctx: StepContext, storage) -> torch.Tensor:
+        """Runs the step's tokens through every scheduled layer (which appends to the caches)
+        and returns float32 logits `[n_want, vocab]`."""
+        x = ops.embed_gather(self.embed, ctx.token_ids)
+        pending: Optional[torch.Tensor] = None
+        for e in self.spec.schedule:
+            cache = storage.layers.get(e.cache_owner)
+            if cache is not None and e.cache_owner != e.layer:
+                cache = cache.reader()
+            x, pending = self.blocks[e.layer].forward(ctx, x, pending, cache)
+        n_want = ctx.want_rows.numel()
+        if n_want == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
+        xs = ops.gather_rows(x, ctx.want_rows)
+        ps = ops.gather_rows(pending, ctx.want_rows)
+        h = self.final_norm.add_forward(xs, ps)
+        return self.head(h, out_dtype=torch.float32)
+
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+        def add(t):
+            nonlocal total
+            if t is not None and t.data_ptr() not in seen:
+                seen.add(t.data_ptr()); total += t.numel() * t.element_size()
+        add(self.embed); add(self.head.weight); add(self.final_norm.weight)
+        for b in self.blocks:
+            for part in (b.mixer, b.ffn, b.norm_mixer, b.norm_ffn):
+                for v in vars(part).values():
+                    if isinstance(v, torch.Tensor):
+                        add(v)
+                    elif isinstance(v, Linear):
+                        add(v.weight)
+        return total

@@ -1,0 +1,304 @@
+"""Python face of the HIP kernels: shape checks on the host, then one C call per kernel.
+
+There is no other implementation behind these functions: without a GPU, or
+without the compiled library, they raise.  Tensors are torch tensors on the
+GPU; torch serves as the allocator and, for large bfloat16 matrix products,
+as the door to the vendor's GEMM library (the reference uses cuBLAS there,
+`candle-core/src/cuda_backend/mod.rs:2260-2305`).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Tuple
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_LIB = None
+_LIB_PATH: Optional[str] = None
+
+
+def library() -> ctypes.CDLL:
+    """The compiled kernel library; compiled on first use when no built one is found."""
+    global _LIB, _LIB_PATH
+    if _LIB is not None:
+        return _LIB
+    path = _build.library_path()
+    if path is None:
+        path = _build.build(verbose=True)
+    lib = ctypes.CDLL(path)
+    lib.ia_last_error.restype = ctypes.c_char_p
+    if lib.ia_abi_version() != 1:
+        raise KernelError(f"{path}: unexpected ABI version {lib.ia_abi_version()}")
+    _LIB, _LIB_PATH = lib, path
+    return lib
+
+
+def library_file() -> Optional[str]:
+    return _LIB_PATH
+
+
+def require_gpu() -> None:
+    if not torch.cuda.is_available():
+        raise KernelError("inferrs_amd runs on an AMD GPU through its HIP kernels; "
+                          "no GPU is visible and there is no CPU fallback")
+    library()
+
+
+def _check(code: int) -> None:
+    if code:
+        raise KernelError(library().ia_last_error().decode("utf-8", "replace"))
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+
+
+def _dev(*ts: Optional[torch.Tensor]) -> None:
+    for t in ts:
+        if t is not None and (not t.is_cuda or not t.is_contiguous()):
+            raise KernelError("kernel operands must be contiguous GPU tensors "
+                              f"(got device={t.device}, contiguous={t.is_contiguous()}, shape={tuple(t.shape)})")
+
+
+def _i32(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int32:
+        raise KernelError(f"{name} must be int32, got {t.dtype}")
+
+
+def _f32(t: Optional[torch.Tensor], name: str) -> None:
+    if t is not None and t.dtype != torch.float32:
+        raise KernelError(f"{name} must be float32, got {t.dtype}")
+
+
+# ---- embedding, gathers ---------------------------------------------------------------------
+
+def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    _dev(table, ids); _i32(ids, "ids")
+    vocab, hidden = table.shape
+    n = ids.numel()
+    out = torch.empty((n, hidden), dtype=table.dtype, device=table.device)
+    _check(library().ia_embed_gather(_p(out), _p(table), _p(ids), n, hidden, vocab, _dt(table), _stream()))
+    return out
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    _dev(x, rows); _i32(rows, "rows")
+    n, cols = rows.numel(), x.shape[-1]
+    out = torch.empty((n, cols), dtype=x.dtype, device=x.device)
+    _check(library().ia_gather_rows(_p(out), _p(x), _p(rows), n, cols, _dt(x), _stream()))
+    return out
+
+
+# ---- norms ----------------------------------------------------------------------------------
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, add_one: bool = False) -> torch.Tensor:
+    _dev(x, w); _f32(w, "norm weight")
+    cols = x.shape[-1]
+    if w.numel() != cols:
+        raise KernelError(f"rmsnorm: weight has {w.numel()} entries, rows have {cols}")
+    rows = x.numel() // cols
+    out = torch.empty_like(x)
+    _check(library().ia_rmsnorm(_p(out), _p(x), _p(w), ctypes.c_float(eps), rows, cols, int(add_one),
+                                _dt(x), _stream()))
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, delta: torch.Tensor, w: torch.Tensor, eps: float,
+                add_one: bool = False) -> torch.Tensor:
+    """x += delta in place (summed in 32-bit); returns rmsnorm(x)."""
+    _dev(x, delta, w); _f32(w, "norm weight")
+    if x.shape != delta.shape or x.dtype != delta.dtype:
+        raise KernelError(f"add_rmsnorm: x {tuple(x.shape)} {x.dtype} and delta {tuple(delta.shape)} {delta.dtype} differ")
+    cols = x.shape[-1]
+    if w.numel() != cols:
+        raise KernelError(f"add_rmsnorm: weight has {w.numel()} entries, rows have {cols}")
+    rows = x.numel() // cols
+    out = torch.empty_like(x)
+    _check(library().ia_add_rmsnorm(_p(out), _p(x), _p(delta), _p(w), ctypes.c_float(eps), rows, cols,
+                                    int(add_one), _dt(x), _stream()))
+    return out
+
+
+def add_inplace(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _dev(x, delta)
+    if x.shape != delta.shape or x.dtype != delta.dtype:
+        raise KernelError("add_inplace: operands differ in shape or dtype")
+    _check(library().ia_add_inplace(_p(x), _p(delta), ctypes.c_longlong(x.numel()), _dt(x), _stream()))
+    return x
+
+
+def silu_mul(gu: torch.Tensor) -> torch.Tensor:
+    """rows of [gate | up] -> silu(gate) * up."""
+    _dev(gu)
+    if gu.shape[-1] % 2:
+        raise KernelError(f"silu_mul: last dimension {gu.shape[-1]} must be even")
+    inter = gu.shape[-1] // 2
+    rows = gu.numel() // (2 * inter)
+    out = torch.empty((*gu.shape[:-1], inter), dtype=gu.dtype, device=gu.device)
+    _check(library().ia_silu_mul(_p(out), _p(gu), rows, inter, _dt(gu), _stream()))
+    return out
+
+
+# ---- position encoding ----------------------------------------------------------------------
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    _dev(positions, inv_freq); _i32(positions, "positions"); _f32(inv_freq, "inv_freq")
+    n, half = positions.numel(), inv_freq.numel()
+    cos = torch.empty((n, half), dtype=torch.float32, device=positions.device)
+    sin = torch.empty_like(cos)
+    _check(library().ia_rope_table(_p(cos), _p(sin), _p(positions), _p(inv_freq), n, half, _stream()))
+    return cos, sin
+
+
+def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, *,
+               q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor],
+               eps: float, add_one: bool, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+               rot: int, interleaved: bool, k_cache: Optional[torch.Tensor],
+               v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+               page_size: int) -> torch.Tensor:
+    """Norm and rotate q and k, write k and v at `slots` of the cache; returns q [n, nq, d]."""
+    _dev(qkv, q_norm_w, k_norm_w, cos, sin, k_cache, v_cache, slots)
+    _f32(q_norm_w, "q_norm weight"); _f32(k_norm_w, "k_norm weight"); _f32(cos, "cos"); _f32(sin, "sin")
+    n = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.shape[1] != (nq + 2 * nkv) * d:
+        raise KernelError(f"qk_rope_kv: qkv has shape {tuple(qkv.shape)}, expected [n, {(nq + 2 * nkv) * d}]")
+    for w, name in ((q_norm_w, "q_norm"), (k_norm_w, "k_norm")):
+        if w is not None and w.numel() != d:
+            raise KernelError(f"qk_rope_kv: {name} weight has {w.numel()} entries, head_dim is {d}")
+    if cos is not None:
+        if sin is None or cos.shape != (n, rot // 2) or sin.shape != cos.shape:
+            raise KernelError(f"qk_rope_kv: rotary tables must be [{n}, {rot // 2}]")
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None:
+            raise KernelError("qk_rope_kv: slots given without a cache")
+        if slots.numel() != n:
+            raise KernelError(f"qk_rope_kv: {slots.numel()} slots for {n} tokens")
+        for c in (k_cache, v_cache):
+            if c.dtype != qkv.dtype or c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, d):
+                raise KernelError(f"qk_rope_kv: cache has shape {tuple(c.shape)} {c.dtype}, expected "
+                                  f"[pages, {nkv}, {page_size}, {d}] {qkv.dtype}")
+    q_out = torch.empty((n, nq, d), dtype=qkv.dtype, device=qkv.device)
+    _check(library().ia_qk_rope_kv(
+        _p(q_out), _p(k_cache if slots is not None else None), _p(v_cache if slots is not None else None),
+        _p(qkv), _p(q_norm_w), _p(k_norm_w), _p(cos), _p(sin), _p(slots), n, nq, nkv, d, rot,
+        int(interleaved), page_size, ctypes.c_float(eps), int(add_one), _dt(qkv), _stream()))
+    return q_out
+
+
+# ---- attention --------------------------------------------------------------------------------
+
+def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
+                      *, window: Optional[int], scale: float) -> torch.Tensor:
+    """q [n, nq, d] against the paged cache [pages, nkv, page_size, d]; token i sees the keys
+    at positions <= positions[i] (and > positions[i] - window) of row token_seq[i] of the table."""
+    _dev(q, k_cache, v_cache, positions, token_seq, block_table)
+    _i32(positions, "positions"); _i32(token_seq, "token_seq"); _i32(block_table, "block_table")
+    n, nq, d = q.shape
+    _, nkv, page_size, dk = k_cache.shape
+    if dk != d or k_cache.shape != v_cache.shape or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError(f"attention: q {tuple(q.shape)} {q.dtype} does not fit the cache "
+                          f"{tuple(k_cache.shape)} {k_cache.dtype}")
+    if positions.numel() != n or token_seq.numel() != n or block_table.dim() != 2:
+        raise KernelError("attention: positions, token_seq and block_table do not fit the batch")
+    out = torch.empty_like(q)
+    _check(library().ia_attention_generic(
+        _p(out), _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_seq), _p(block_table), n,
+        block_table.shape[1], nq, nkv, d, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
+        _stream()))
+    return out
+
+
+# ---- matrix products --------------------------------------------------------------------------
+
+SKINNY_MAX_ROWS = 64
+
+
+def _skinny_splits(n_out: int, k: int) -> int:
+    """How many blocks share k in the skinny product: a function of the weight's shape only,
+    so that a row's rounding does not depend on the batch it is in."""
+    blocks = (n_out + 15) // 16
+    ksteps = (k + 31) // 32
+    splits = 1
+    while blocks * splits < 1024 and ksteps // (4 * splits * 2) >= 4 and splits < 16:
+        splits *= 2
+    return splits
+
+
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    _dev(x, w)
+    m, k = x.shape
+    n, k2 = w.shape
+    if k != k2 or x.dtype != w.dtype:
+        raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _check(library().ia_gemm_tiled(_p(out), _p(x), _p(w), m, n, k, _dt(x), _DT[out_dtype], _stream()))
+    return out
+
+
+def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                     splits: Optional[int] = None) -> torch.Tensor:
+    _dev(x, w)
+    m, k = x.shape
+    n, k2 = w.shape
+    if k != k2 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"gemm_skinny: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
+    if splits is None:
+        splits = _skinny_splits(n, k)
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device) if splits > 1 else None
+    _check(library().ia_gemm_skinny_bf16(_p(out), _p(x), _p(w), _p(partial), m, n, k, splits,
+                                         _DT[out_dtype], _stream()))
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
+    skinny MFMA kernel for up to 64 rows, the vendor's GEMM beyond that; a 32-bit result of
+    bfloat16 operands with many rows goes through the skinny kernel 64 rows at a time."""
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32:
+        return gemm_tiled(x, w, out_dtype)
+    m, k = x.shape
+    if k % 8 or (x.data_ptr() | w.data_ptr()) % 16:
+        return gemm_tiled(x, w, out_dtype)
+    if m <= SKINNY_MAX_ROWS or out_dtype == torch.float32:
+        return gemm_skinny_bf16(x, w, out_dtype)
+    _dev(x, w)
+    if w.shape[1] != k or w.dtype != x.dtype:
+        raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
+    return torch.nn.functional.linear(x, w)
+
+
+# ---- sampling ---------------------------------------------------------------------------------
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    _dev(logits); _f32(logits, "logits")
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _check(library().ia_argmax(_p(out), _p(logits), rows, vocab, _stream()))
+    return out

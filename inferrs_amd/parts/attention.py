@@ -1,0 +1,79 @@
+"""Grouped-query attention over the paged cache.
+
+Order of operations as in the reference (`inferrs-models/src/models/qwen3.rs:105-195`):
+q, k, v projections without bias; per-head RMS norm of q and k; rotation of q and k by
+position; append of k and v to the cache; scores (q.k)/sqrt(d) against keys at positions
+<= the query's (and inside the window, when one is set); softmax; weighted sum of values;
+output projection.  q head h reads kv head h // (n_heads / n_kv_heads)
+(`attention_utils.rs:38-49`).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.spec import AttentionSpec, SpecError
+from ..weights.loader import TensorSpec
+from .base import Mixer, PagedKV, part_class, register_mixer
+from .linear import Linear
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    @classmethod
+    def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorSpec]:
+        q_out, kv_out = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim
+        t = {
+            "q_proj.weight": TensorSpec((q_out, spec.hidden)),
+            "k_proj.weight": TensorSpec((kv_out, spec.hidden)),
+            "v_proj.weight": TensorSpec((kv_out, spec.hidden)),
+            "o_proj.weight": TensorSpec((spec.hidden, q_out)),
+        }
+        if spec.qk_norm is not None:
+            t["q_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
+            t["k_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
+        return t
+
+    @classmethod
+    def cache_need(cls, spec: AttentionSpec):
+        return PagedKV(spec.n_kv_heads, spec.head_dim, spec.window)
+
+    def __init__(self, spec: AttentionSpec, tensors: Dict[str, torch.Tensor], dtype, device):
+        if spec.n_heads % spec.n_kv_heads:
+            raise SpecError(f"attention: {spec.n_heads} heads are not a multiple of {spec.n_kv_heads} kv heads")
+        if spec.head_dim % 16 or not (16 <= spec.head_dim <= 512):
+            raise SpecError(f"attention: head_dim {spec.head_dim} must be a multiple of 16 in 16..512")
+        if spec.window is not None and spec.window < 1:
+            raise SpecError(f"attention: window {spec.window} must be >= 1")
+        if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
+            raise SpecError("attention: qk_norm must span head_dim")
+        self.spec = spec
+        self.qkv = Linear([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]],
+                          dtype, device)
+        self.o = Linear([tensors["o_proj.weight"]], dtype, device)
+        if spec.qk_norm is not None:
+            self.q_norm_w = tensors["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            self.k_norm_w = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            self.norm_eps, self.norm_add_one = float(spec.qk_norm.eps), bool(spec.qk_norm.add_one)
+        else:
+            self.q_norm_w = self.k_norm_w = None
+            self.norm_eps, self.norm_add_one = 0.0, False
+        self.position = part_class("position", spec.position)(spec.position, {}, dtype, device)
+
+    def forward(self, ctx, h: torch.Tensor, cache) -> torch.Tensor:
+        s = self.spec
+        group = ctx.groups[cache.group]
+        qkv = self.qkv(h)
+        table = ctx.position_table(self.position)
+        cos, sin = table if table is not None else (None, None)
+        q = ops.qk_rope_kv(
+            qkv, s.n_heads, s.n_kv_heads, s.head_dim,
+            q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one,
+            cos=cos, sin=sin, rot=self.position.rot_dim, interleaved=self.position.interleaved,
+            k_cache=cache.k, v_cache=cache.v, slots=group.slots if cache.writable else None,
+            page_size=group.page_size)
+        a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
+                                  window=s.window, scale=s.softmax_scale)
+        return self.o(a.view(a.shape[0], s.n_heads * s.head_dim))

@@ -1,0 +1,34 @@
+"""Gated feed-forward: down( silu(gate(x)) * up(x) ), no biases
+(`inferrs-models/src/models/attention_utils.rs:94-118`).  Gate and up share one product."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.spec import GatedMlpSpec, SpecError
+from ..weights.loader import TensorSpec
+from .base import FeedForward, register_ffn
+from .linear import Linear
+
+
+@register_ffn("gated_mlp")
+class GatedMlp(FeedForward):
+    @classmethod
+    def tensors(cls, spec: GatedMlpSpec) -> Dict[str, TensorSpec]:
+        return {
+            "gate_proj.weight": TensorSpec((spec.intermediate, spec.hidden)),
+            "up_proj.weight": TensorSpec((spec.intermediate, spec.hidden)),
+            "down_proj.weight": TensorSpec((spec.hidden, spec.intermediate)),
+        }
+
+    def __init__(self, spec: GatedMlpSpec, tensors: Dict[str, torch.Tensor], dtype, device):
+        if spec.activation != "silu":
+            raise SpecError(f"gated_mlp: activation {spec.activation!r} has no kernel (only 'silu')")
+        self.spec = spec
+        self.gate_up = Linear([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dtype, device)
+        self.down = Linear([tensors["down_proj.weight"]], dtype, device)
+
+    def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
+        return self.down(ops.silu_mul(self.gate_up(h)))

@@ -1,0 +1,32 @@
+"""RMS norm: x / sqrt(mean(x^2) + eps) * w, statistics in 32-bit
+(`candle-nn/src/ops.rs:443-504`, `inferrs-kernels/candle-kernels/src/reduce.cu:189-228`)."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.spec import NormSpec
+from ..weights.loader import TensorSpec
+from .base import Norm, register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Norm):
+    @classmethod
+    def tensors(cls, spec: NormSpec) -> Dict[str, TensorSpec]:
+        return {"weight": TensorSpec((spec.size,), "norm")}
+
+    def __init__(self, spec: NormSpec, tensors: Dict[str, torch.Tensor], dtype, device):
+        self.spec = spec
+        self.eps = float(spec.eps)
+        self.add_one = bool(spec.add_one)
+        # Norm weights are vectors: kept in 32-bit whatever the activations are stored in.
+        self.weight = tensors["weight"].to(device=device, dtype=torch.float32).contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.rmsnorm(x, self.weight, self.eps, self.add_one)
+
+    def add_forward(self, x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+        return ops.add_rmsnorm(x, delta, self.weight, self.eps, self.add_one)

@@ -1,0 +1,48 @@
+"""Position encodings.  "rope": angle[p, i] = p * theta**(-2i/rot_dim), computed in 32-bit
+(`inferrs-models/src/models/attention_utils.rs:186-216`); "none": nothing."""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..config.spec import PositionSpec, SpecError
+from .base import Position, register_position
+
+
+def inverse_frequencies(theta: float, rot_dim: int) -> np.ndarray:
+    """1 / theta**(2i/rot_dim) for i in 0..rot_dim/2, every step in 32-bit as the reference's
+    `powf` on f32 operands (`attention_utils.rs:198-203`)."""
+    i = np.arange(rot_dim // 2, dtype=np.float32)
+    exponent = (np.float32(2.0) * i) / np.float32(rot_dim)
+    return (np.float32(1.0) / np.power(np.float32(theta), exponent, dtype=np.float32)).astype(np.float32)
+
+
+@register_position("rope")
+class Rotary(Position):
+    def __init__(self, spec: PositionSpec, tensors, dtype, device):
+        if spec.rot_dim <= 0 or spec.rot_dim % 2 or spec.rot_dim > spec.head_dim:
+            raise SpecError(f"rot_dim {spec.rot_dim} must be even and within head_dim {spec.head_dim}")
+        if spec.pairing not in ("half", "interleaved"):
+            raise SpecError(f"unknown rotary pairing {spec.pairing!r}")
+        self.spec = spec
+        self.rot_dim = spec.rot_dim
+        self.interleaved = spec.pairing == "interleaved"
+        self.inv_freq = torch.from_numpy(inverse_frequencies(spec.theta, spec.rot_dim)).to(device)
+
+    def table(self, positions: torch.Tensor) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
+        return ops.rope_table(positions, self.inv_freq)
+
+
+@register_position("none")
+class NoPosition(Position):
+    rot_dim = 0
+    interleaved = False
+
+    def __init__(self, spec, tensors, dtype, device):
+        self.spec = spec
+
+    def table(self, positions):
+        return None

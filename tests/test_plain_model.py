@@ -1,0 +1,189 @@
+"""Pins the plain implementation by what fixes it beside the reference's text: the reference's
+own test vectors, special cases that reduce to a library routine, and invariants, each chosen
+so that a plausible mistake (a sign, a pairing, a norm in the wrong place) fails it."""
+import math
+
+import pytest
+import torch
+
+import plain_model as pm
+from tiny_configs import TINY, random_tokens, write_model
+
+
+def test_rms_norm_reference_vector():
+    # candle-nn/tests/ops.rs:55-66
+    x = torch.tensor([[[3., 1., 4.], [1., 5., 9.]], [[2., 1., 7.], [8., 2., 8.]]])
+    w = torch.tensor([1., 2., 3.])
+    got = pm.rms_norm(x, w, 1e-5)
+    want = torch.tensor([[[1.019, 0.6794, 4.0762], [0.1674, 1.6744, 4.521]],
+                         [[0.4714, 0.4714, 4.9497], [1.206, 0.603, 3.6181]]])
+    assert torch.equal(torch.round(got * 1e4) / 1e4, want)
+
+
+def test_rms_norm_invariants():
+    torch.manual_seed(0)
+    x = torch.randn(5, 70, dtype=torch.float64)
+    ones = torch.ones(70, dtype=torch.float64)
+    y = pm.rms_norm(x, ones, 0.0)
+    assert torch.allclose((y * y).mean(-1), torch.ones(5, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(pm.rms_norm(3.7 * x, ones, 0.0), y, atol=1e-12)       # scale invariance
+    # eps sits inside the root, added to the MEAN of squares (not the sum, not outside)
+    v = torch.tensor([[2.0, 0.0, 0.0, 0.0]], dtype=torch.float64)
+    assert math.isclose(pm.rms_norm(v, torch.ones(4, dtype=torch.float64), 3.0)[0, 0].item(), 2.0 / 2.0)
+
+
+def test_softmax_reference_vectors():
+    # candle-nn/tests/ops.rs:9-53 (last dimension) and :149-156
+    x = torch.tensor([[[3., 1., 4.], [1., 5., 9.]], [[2., 1., 7.], [8., 2., 8.]]])
+    got = pm.softmax_last(torch.log(x))
+    want = torch.tensor([[[0.375, 0.125, 0.5], [0.0667, 0.3333, 0.6]],
+                         [[0.2, 0.1, 0.7], [0.4444, 0.1111, 0.4444]]])
+    assert torch.equal(torch.round(got * 1e4) / 1e4, want)
+    assert pm.softmax_last(torch.tensor([1234., 0.])).tolist() == [1.0, 0.0]
+
+
+def test_linear_reference_example():
+    # candle-nn/src/linear.rs:7-20
+    w = torch.tensor([[1., 2.], [3., 4.], [5., 6.]])
+    assert pm.linear(torch.tensor([[10., 100.]]), w).tolist() == [[210., 430., 650.]]
+
+
+def test_inv_freq():
+    f = pm.inv_freq(1e6, 32)
+    assert f[0].item() == 1.0
+    want = torch.tensor([1e6 ** (-2 * i / 32) for i in range(16)], dtype=torch.float64)
+    assert torch.allclose(f.double(), want, rtol=2e-6)
+    assert f.dtype == torch.float32
+
+
+def test_rope_equals_slow_form_and_is_split_half():
+    # candle-nn/tests/ops.rs:185-210 compares rope with rope_slow on (2,5,10,16)-shaped data
+    torch.manual_seed(299792458)
+    x = torch.rand(5, 10, 16)
+    cos, sin = torch.rand(10, 8), torch.rand(10, 8)
+    assert torch.equal(pm.rope_half(x, cos, sin), pm.rope_slow(x, cos, sin))
+    # pairing is (i, i + d/2): rotating a vector with one non-zero feature moves it there
+    e = torch.zeros(1, 1, 16); e[0, 0, 3] = 1.0
+    c, s = torch.zeros(1, 8), torch.ones(1, 8)
+    out = pm.rope_half(e, c, s)
+    assert out[0, 0, 3 + 8].item() == 1.0 and out.abs().sum().item() == 1.0
+    out_i = pm.rope_interleaved(e, c, s)
+    assert out_i[0, 0, 2].item() == -1.0            # the other pairing puts it elsewhere
+
+
+def test_rope_position_zero_norm_and_relative_property():
+    torch.manual_seed(1)
+    q, k = torch.randn(1, 1, 32, dtype=torch.float64), torch.randn(1, 1, 32, dtype=torch.float64)
+    def rot(x, p):
+        cos, sin = pm.rope_tables(torch.tensor([p]), 10000.0, 32)
+        return pm.rope_half(x, cos.double(), sin.double())
+    assert torch.allclose(rot(q, 0), q)
+    assert torch.allclose(rot(q, 17).norm(), q.norm())
+    a = (rot(q, 40) * rot(k, 33)).sum()
+    b = (rot(q, 107) * rot(k, 100)).sum()
+    assert torch.allclose(a, b, atol=1e-5)           # only the distance counts
+    c = (rot(q, 33) * rot(k, 40)).sum()
+    assert not torch.allclose(a, c, atol=1e-3)       # and its sign
+
+
+def test_attention_reduces_to_library_sdpa():
+    torch.manual_seed(2)
+    q, k, v = torch.randn(4, 9, 16), torch.randn(4, 9, 16), torch.randn(4, 9, 16)
+    want = torch.nn.functional.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+    assert torch.allclose(pm.attention_core(q, k, v), want, atol=1e-5)
+    nomask = torch.nn.functional.scaled_dot_product_attention(q[None], k[None], v[None])[0]
+    assert torch.allclose(pm.attention_core(q, k, v, masked=False), nomask, atol=1e-5)
+    # a portion with offset: rows see keys j <= offset + i
+    off = 5
+    mask = torch.arange(9)[None, :] <= (torch.arange(4)[:, None] + off)
+    want = torch.nn.functional.scaled_dot_product_attention(q[None, :, :4], k[None], v[None], attn_mask=mask)[0]
+    assert torch.allclose(pm.attention_core(q[:, :4], k, v, offset=off), want, atol=1e-5)
+    # first token attends to itself alone
+    assert torch.allclose(pm.attention_core(q, k, v)[:, 0], v[:, 0], atol=1e-6)
+
+
+def test_gqa_head_mapping():
+    # query head h reads kv head h // g: make kv heads distinguishable constants
+    nq, nkv, t, d = 6, 3, 4, 8
+    q = torch.randn(nq, t, d)
+    k = torch.randn(nkv, t, d)
+    v = torch.stack([torch.full((t, d), float(h + 1)) for h in range(nkv)])
+    out = pm.attention_core(q, k, v)
+    for h in range(nq):
+        assert torch.allclose(out[h], torch.full((t, d), float(h // 2 + 1)))
+    r = pm.repeat_kv(v, 2)
+    assert [r[i, 0, 0].item() for i in range(6)] == [1., 1., 2., 2., 3., 3.]
+
+
+def test_silu_and_mlp():
+    assert pm.silu(torch.tensor(0.0)).item() == 0.0
+    assert abs(pm.silu(torch.tensor(30.0)).item() - 30.0) < 1e-5
+    x = torch.randn(3, 8)
+    g, u, d = torch.randn(12, 8), torch.randn(12, 8), torch.randn(8, 12)
+    want = torch.nn.functional.linear(torch.nn.functional.silu(torch.nn.functional.linear(x, g))
+                                      * torch.nn.functional.linear(x, u), d)
+    assert torch.allclose(pm.mlp(x, g, u, d), want, atol=1e-5)
+
+
+def test_rand_f32_matches_integer_transcription():
+    # a second, independent transcription of inferrs/src/sampler.rs:370-397 with numpy uint64
+    import numpy as np
+    def ref(seed, step):
+        with np.errstate(over="ignore"):
+            x = np.uint64(seed) + np.uint64(0x9e3779b97f4a7c15)
+            for rnd in range(2):
+                if rnd == 1:
+                    x = x + (np.uint64(step) + np.uint64(1)) * np.uint64(0x9e3779b97f4a7c15)
+                x = (x ^ (x >> np.uint64(30))) * np.uint64(0xbf58476d1ce4e5b9)
+                x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94d049bb133111eb)
+                x = x ^ (x >> np.uint64(31))
+            x ^= x << np.uint64(13); x ^= x >> np.uint64(7); x ^= x << np.uint64(17)
+            u = (x * np.uint64(0x2545f4914f6cdd1d)) >> np.uint64(32)
+        return float(np.float32(u) / np.float32(4294967296.0))
+    vals = [pm.rand_f32(42, s) for s in range(50)]
+    assert vals == [ref(42, s) for s in range(50)]
+    assert all(0.0 <= v < 1.0 for v in vals) and len(set(vals)) == 50
+
+
+def test_sampler_penalty_window_and_greedy():
+    # inferrs/src/sampler.rs:613-644: the window holds the last repeat_last_n tokens only
+    logits = torch.zeros(8); logits[1] = 10.0; logits[2] = 9.99
+    assert pm.sample(logits, [1] + [5] * 3, temperature=0.0, repetition_penalty=2.0, repeat_last_n=4) == 2
+    assert pm.sample(logits, [1] + [5] * 4, temperature=0.0, repetition_penalty=2.0, repeat_last_n=4) == 1
+    assert pm.sample(logits, [1], temperature=0.0, repetition_penalty=2.0, repeat_last_n=0) == 1
+    tie = torch.tensor([1.0, 3.0, 3.0, 0.0])
+    assert pm.sample(tie, [], temperature=0.0) == 1                  # lowest index among maxima
+    assert pm.sample(torch.tensor([0.0, 50.0, 0.0]), [], temperature=1.0, top_k=1, seed=3) == 1
+
+
+def test_sampler_frequencies_follow_tempered_softmax():
+    logits = torch.tensor([0.0, 1.0, 2.0, -1.0])
+    temp = 0.7
+    want = torch.softmax(logits / temp, 0)
+    counts = torch.zeros(4)
+    n = 4000
+    for step in range(n):
+        prev = [0] * step if step < 64 else [0] * 64
+        # step enters through len(previous): feed a list of that length without penalties
+        t = pm.sample(logits, list(range(step % 97)), temperature=temp, top_k=0, top_p=1.0,
+                      repetition_penalty=1.0, seed=step)
+        counts[t] += 1
+    assert torch.allclose(counts / n, want, atol=0.03)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_model_shift_and_prefix_invariants(tmp_path, name):
+    raw = TINY[name]
+    folder = write_model(str(tmp_path / name), raw, seed=5)
+    cfg, p = pm.read_model(folder, torch.float64)
+    toks = random_tokens(24, raw["vocab_size"], 7)
+    full = pm.forward(cfg, p, toks)
+    assert full.shape == (24, raw["vocab_size"])
+    # causality: logits of a prefix do not depend on what follows
+    assert torch.allclose(pm.forward(cfg, p, toks[:11]), full[:11], atol=1e-9)
+    # the head: tied models use the embedding table
+    if raw["tie_word_embeddings"]:
+        assert "lm_head.weight" not in p
+    else:
+        assert p["lm_head.weight"].shape == (raw["vocab_size"], raw["hidden_size"])
+    assert pm.greedy(cfg, p, toks[:5], 3) == pm.greedy(cfg, p, toks[:5], 3)
