@@ -1,0 +1,260 @@
+"""Each HIP kernel alone against a plain 32-bit torch formula of the same operation, at sizes
+other than the engine's tests use: head sizes in steps of 16, head counts and groups that are no
+power of two, widths and vocabularies that are no multiple of any tile.
+
+bfloat16 bounds: inputs are exact in both; the kernel accumulates in 32-bit and rounds its
+result once, so the error is half a unit in the last place of the result, 2**-9 relative, plus
+the 32-bit summation error; the checks allow 2**-8 of the row's scale."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def tol(dtype, f32=2e-6, bf16=2 ** -8):
+    return f32 if dtype == torch.float32 else bf16
+
+
+def close(got, want, rel, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    scale = max(float(want.abs().max()), 1e-6)
+    err = float((got - want).abs().max()) / scale
+    assert err <= rel, f"{what}: error {err:.3e} of the scale exceeds {rel:.1e}"
+
+
+def randn(*shape, dtype, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_and_gather(dtype):
+    from inferrs_amd import ops
+    table = randn(133, 72, dtype=dtype)
+    ids = torch.tensor([0, 132, 5, 5, 77], dtype=torch.int32)
+    assert torch.equal(ops.embed_gather(dev(table), dev(ids)).cpu(), table[ids.long()])
+    assert torch.equal(ops.gather_rows(dev(table), dev(ids)).cpu(), table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cols", [1, 40, 1000, 4096, 5120])
+@pytest.mark.parametrize("add_one", [False, True])
+def test_rmsnorm(dtype, cols, add_one):
+    from inferrs_amd import ops
+    x = randn(7, cols, dtype=dtype, seed=1, scale=3.0)
+    d = randn(7, cols, dtype=dtype, seed=2)
+    w = randn(cols, dtype=torch.float32, seed=3)
+    eps = 1e-5
+
+    def ref(v):
+        v = v.float()
+        return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * (w + 1.0 if add_one else w)
+    close(ops.rmsnorm(dev(x), dev(w), eps, add_one), ref(x), tol(dtype), "rmsnorm")
+    xs = dev(x.clone())
+    out = ops.add_rmsnorm(xs, dev(d), dev(w), eps, add_one)
+    summed = (x.float() + d.float()).to(dtype)
+    assert torch.equal(xs.cpu(), summed), "add_rmsnorm must leave x + delta in x"
+    close(out, ref(summed), tol(dtype), "add_rmsnorm")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    from inferrs_amd import ops
+    gu = randn(5, 2 * 203, dtype=dtype, seed=4, scale=4.0)
+    g, u = gu[:, :203].float(), gu[:, 203:].float()
+    close(ops.silu_mul(dev(gu)), g / (1 + torch.exp(-g)) * u, tol(dtype), "silu_mul")
+    z = torch.zeros(1, 8, dtype=dtype)
+    assert float(ops.silu_mul(dev(z)).abs().max()) == 0.0
+
+
+def test_rope_table():
+    from inferrs_amd import ops
+    from inferrs_amd.parts.position import inverse_frequencies
+    inv = torch.from_numpy(inverse_frequencies(1e6, 48))
+    pos = torch.tensor([0, 1, 17, 4095, 40000], dtype=torch.int32)
+    cos, sin = ops.rope_table(dev(pos), dev(inv))
+    ang = (pos.float()[:, None] * inv[None, :]).double()          # the product itself is 32-bit
+    assert float((cos.cpu().double() - torch.cos(ang)).abs().max()) < 2e-6
+    assert float((sin.cpu().double() - torch.sin(ang)).abs().max()) < 2e-6
+    assert inv[0].item() == 1.0
+
+
+def ref_qk_rope(qkv, nq, nkv, d, qw, kw, eps, add_one, cos, sin, rot, interleaved):
+    n = qkv.shape[0]
+    x = qkv.float().view(n, nq + 2 * nkv, d)
+    q, k, v = x[:, :nq], x[:, nq:nq + nkv], x[:, nq + nkv:]
+
+    def norm(t, w):
+        if w is None:
+            return t
+        return t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps) * (w + 1.0 if add_one else w)
+
+    def rope(t):
+        if cos is None:
+            return t
+        c, s = cos[:, None, :], sin[:, None, :]
+        out = t.clone()
+        if interleaved:
+            a, b = t[..., 0:rot:2], t[..., 1:rot:2]
+            out[..., 0:rot:2], out[..., 1:rot:2] = a * c - b * s, a * s + b * c
+        else:
+            a, b = t[..., :rot // 2], t[..., rot // 2:rot]
+            out[..., :rot // 2], out[..., rot // 2:rot] = a * c - b * s, a * s + b * c
+        return out
+    return rope(norm(q, qw)), rope(norm(k, kw)), v
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rot,interleaved,normed", [
+    (4, 2, 16, 16, False, True), (5, 1, 48, 48, False, True), (32, 8, 128, 128, False, True),
+    (6, 3, 80, 32, False, False), (3, 3, 256, 64, True, True), (2, 1, 512, 512, False, True),
+    (7, 7, 112, 0, False, True)])
+def test_qk_rope_kv(dtype, nq, nkv, d, rot, interleaved, normed):
+    from inferrs_amd import ops
+    n, page, pages = 13, 4, 9
+    qkv = randn(n, (nq + 2 * nkv) * d, dtype=dtype, seed=5, scale=2.0)
+    qw = randn(d, dtype=torch.float32, seed=6) if normed else None
+    kw = randn(d, dtype=torch.float32, seed=7) if normed else None
+    g = torch.Generator().manual_seed(8)
+    cos = torch.rand(n, rot // 2, generator=g) if rot else None
+    sin = torch.rand(n, rot // 2, generator=g) if rot else None
+    slots = torch.randperm(pages * page, generator=g)[:n].to(torch.int32)
+    kc = torch.full((pages, nkv, page, d), 7.0, dtype=dtype)
+    vc = torch.full((pages, nkv, page, d), 7.0, dtype=dtype)
+    kc_d, vc_d = dev(kc), dev(vc)
+    q = ops.qk_rope_kv(dev(qkv), nq, nkv, d, q_norm_w=None if qw is None else dev(qw),
+                       k_norm_w=None if kw is None else dev(kw), eps=1e-5, add_one=False,
+                       cos=None if cos is None else dev(cos), sin=None if sin is None else dev(sin),
+                       rot=rot, interleaved=interleaved, k_cache=kc_d, v_cache=vc_d, slots=dev(slots),
+                       page_size=page)
+    rq, rk, rv = ref_qk_rope(qkv, nq, nkv, d, qw, kw, 1e-5, False, cos, sin, rot, interleaved)
+    close(q, rq, tol(dtype, 3e-6), "q")
+    want_k, want_v = kc.float().clone(), vc.float().clone()
+    for t in range(n):
+        s = int(slots[t])
+        want_k[s // page, :, s % page] = rk[t]
+        want_v[s // page, :, s % page] = rv[t]
+    close(kc_d, want_k, tol(dtype, 3e-6), "k cache")         # untouched slots keep their 7.0
+    assert torch.equal(vc_d.cpu().float(), want_v.to(dtype).float()), "values are copied as they are"
+
+
+def ref_attention(q, kc, vc, positions, token_seq, table, window, scale):
+    n, nq, d = q.shape
+    nkv, page = kc.shape[1], kc.shape[2]
+    out = torch.zeros(n, nq, d)
+    for t in range(n):
+        pos = int(positions[t])
+        lo = max(0, pos - window + 1) if window else 0
+        keys = list(range(lo, pos + 1))
+        pg = [int(table[int(token_seq[t]), j // page]) for j in keys]
+        for h in range(nq):
+            kvh = h // (nq // nkv)
+            k = torch.stack([kc[p, kvh, j % page] for p, j in zip(pg, keys)]).float()
+            v = torch.stack([vc[p, kvh, j % page] for p, j in zip(pg, keys)]).float()
+            s = (k @ q[t, h].float()) * scale
+            out[t, h] = torch.softmax(s, 0) @ v
+    return out
+
+
+def attention_case(dtype, nq, nkv, d, page, lens, q_lens, seed, needle=False):
+    """Requests with `lens` cached tokens of which the last `q_lens` are this step's queries,
+    pages handed out in a shuffled order."""
+    g = torch.Generator().manual_seed(seed)
+    n_seqs = len(lens)
+    max_pages = max(-(-l // page) for l in lens)
+    total_pages = sum(-(-l // page) for l in lens) + 3
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    table = torch.zeros(n_seqs, max_pages, dtype=torch.int32)
+    for s, l in enumerate(lens):
+        for j in range(-(-l // page)):
+            table[s, j] = perm.pop()
+    kc = randn(total_pages, nkv, page, d, dtype=dtype, seed=seed + 1)
+    vc = randn(total_pages, nkv, page, d, dtype=dtype, seed=seed + 2)
+    positions = torch.tensor([p for l, ql in zip(lens, q_lens) for p in range(l - ql, l)], dtype=torch.int32)
+    token_seq = torch.tensor([s for s, ql in enumerate(q_lens) for _ in range(ql)], dtype=torch.int32)
+    q = randn(len(positions), nq, d, dtype=dtype, seed=seed + 3)
+    if needle:
+        # one far key per request that every query of head 0 points at: its score stands out,
+        # so the output is that key's value unless the key is lost
+        for s, l in enumerate(lens):
+            j = l // 3
+            kc[int(table[s, j // page]), 0, j % page] = (q[token_seq == s][-1, 0].float() * 4).to(dtype)
+    return q, kc, vc, positions, token_seq, table
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,page,window", [
+    (4, 2, 16, 4, None), (5, 1, 48, 16, None), (8, 1, 128, 16, None), (6, 3, 32, 8, 37),
+    (3, 3, 80, 5, None), (2, 2, 256, 16, 100)])
+def test_attention_generic(dtype, nq, nkv, d, page, window):
+    from inferrs_amd import ops
+    lens, q_lens = [1, 70, 129, 200, 64], [1, 70, 2, 1, 17]
+    q, kc, vc, positions, token_seq, table = attention_case(dtype, nq, nkv, d, page, lens, q_lens, 11, needle=True)
+    scale = 1.0 / math.sqrt(d)
+    got = ops.attention_generic(dev(q), dev(kc), dev(vc), dev(positions), dev(token_seq), dev(table),
+                                window=window, scale=scale)
+    want = ref_attention(q, kc, vc, positions, token_seq, table, window, scale)
+    close(got, want, tol(dtype, 5e-6, 2 ** -7), "attention")
+
+
+def test_gemm_reference_products():
+    # candle-core/tests/matmul_tests.rs:18-33 and candle-nn/src/linear.rs:7-20
+    from inferrs_amd import ops
+    a = torch.tensor([[1., 2.], [3., 4.]])
+    b = torch.tensor([[4., 5.], [6., 7.]])
+    assert ops.linear(dev(a), dev(b.t().contiguous())).cpu().tolist() == [[16., 19.], [36., 43.]]
+    w = torch.tensor([[1., 2.], [3., 4.], [5., 6.]])
+    assert ops.linear(dev(torch.tensor([[10., 100.]])), dev(w)).cpu().tolist() == [[210., 430., 650.]]
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 130, 40), (65, 64, 64), (17, 515, 136), (130, 72, 200), (2, 7, 1000)])
+def test_gemm_tiled_float32_is_true_32_bit(m, n, k):
+    from inferrs_amd import ops
+    x, w = randn(m, k, dtype=torch.float32, seed=1), randn(n, k, dtype=torch.float32, seed=2)
+    want = (x.double() @ w.double().t())
+    got = ops.linear(dev(x), dev(w)).cpu().double()
+    # a reduced-precision matrix mode (tf32-like, 10 bits) would be off by about 1e-3
+    assert float((got - want).abs().max()) <= 4e-6 * max(1.0, float(want.abs().max()))
+    # rows do not depend on what else is in the batch
+    assert torch.equal(ops.linear(dev(x[:1]), dev(w)).cpu(), ops.linear(dev(x), dev(w)).cpu()[:1])
+
+
+@pytest.mark.parametrize("m", [1, 2, 8, 16, 17, 33, 64, 65, 200])
+@pytest.mark.parametrize("n,k", [(130, 40), (515, 136), (4096, 4096), (1000, 12288), (16, 8)])
+@pytest.mark.parametrize("out_dtype", DTYPES)
+def test_linear_bfloat16(m, n, k, out_dtype):
+    from inferrs_amd import ops
+    x, w = randn(m, k, dtype=torch.bfloat16, seed=1), randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    want = x.double() @ w.double().t()
+    got = ops.linear(dev(x), dev(w), out_dtype)
+    assert got.dtype == out_dtype
+    close(got, want, tol(out_dtype, 2e-5), f"linear {m}x{n}x{k}")
+
+
+def test_gemm_skinny_splits_agree():
+    from inferrs_amd import ops
+    x, w = randn(5, 4096, dtype=torch.bfloat16, seed=1), randn(77, 4096, dtype=torch.bfloat16, seed=2)
+    want = x.double() @ w.double().t()
+    for splits in (1, 2, 8, 16):
+        close(ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32, splits=splits), want, 2e-5, f"splits {splits}")
+
+
+def test_argmax_lowest_index_among_equal_maxima():
+    from inferrs_amd import ops
+    z = randn(4, 151936, dtype=torch.float32, seed=3)
+    z[1, 150000] = z[1, 77] = 9.0
+    z[2, :] = 0.0
+    z[3, 151935] = 10.0
+    got = ops.argmax(dev(z)).cpu().tolist()
+    assert got == [int(torch.argmax(z[0])), 77, 0, 151935]
+    small = torch.tensor([[1.0, 3.0, 3.0]])
+    assert ops.argmax(dev(small)).cpu().tolist() == [1]

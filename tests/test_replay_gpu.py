@@ -1,0 +1,193 @@
+"""The engine against the plain implementation under every way of cutting the work: each
+request alone and whole; most of it in one step and the last 32 tokens one by one; portions of
+changing size down to two tokens; and up to four live requests mixed, portions of some beside
+decoded tokens of others, in a pool so small that pages are used again.  32-bit and bfloat16.
+
+The plain implementation runs in 64-bit and stands for the exact result.
+
+Tolerances.  32-bit: 1e-5 of the largest logit.  The plain implementation run in 32-bit is
+itself 4e-7 to 7e-6 away from the 64-bit result on these models, the engine 3e-7 to 9e-6.  Between two cuttings the 32-bit engine has the same order of sums for every
+position (per-row norms, keys walked in tiles aligned to absolute position, a fixed k order in
+the products), so they agree to 1e-6 of the scale.  bfloat16: every stored activation is rounded to 8 bits of mantissa, and how far that moves
+a logit depends on the model (sharper attention amplifies it).  The bound is therefore measured
+on the model itself: the plain implementation run in bfloat16 tensor arithmetic (every
+operation rounded, as the reference's CPU path does) against the same in 32-bit, largest
+difference over all positions.  The engine keeps more in 32-bit registers than that, so it has to
+be at least as close to the 32-bit result (measured: 0.4 to 0.7 of the bound).  Sharpened models
+(see `write_model`) make a lost or misplaced key change logits by 10 % and more.  The sharpening
+is 2.0 for 32-bit (scores spread 16 times wider) and 1.5 for bfloat16 (5 times): sharper
+than that, rounding of queries and keys alone moves the scores so far that the comparison
+says little (at 2.5 the plain implementation in 32-bit is 1.5e-5 away from 64-bit)."""
+import io
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+import trace_modes as tm
+from tiny_configs import PAGE_SIZE, TINY, random_tokens, write_model
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LENGTHS = [1, 2, 3, 37, 64, 65, 130, 257, 300]
+TOL_PLAIN_F32 = 1e-5
+TOL_CROSS_F32 = 1e-6
+SHARP = {"float32": 2.0, "bfloat16": 1.5}
+# (configuration, sharpened or not)
+CASES = [("A", False), ("B", False), ("C", False), ("D", False), ("A", True), ("B", True), ("D", True)]
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """(name, sharpen factor) -> folder, raw config, requests, plain logits."""
+    out = {}
+    for name, sharp in CASES:
+        for sharpen in (sorted(set(SHARP.values())) if sharp else [1.0]):
+            raw = TINY[name]
+            folder = write_model(str(tmp_path_factory.mktemp(f"model_{name}")), raw, seed=5, sharpen=sharpen)
+            cfg, params = pm.read_model(folder, torch.float64)
+            reqs = {f"r{i}": random_tokens(n, raw["vocab_size"], 100 + i) for i, n in enumerate(LENGTHS)}
+            ref = {r: pm.forward(cfg, params, t).numpy().astype(np.float32) for r, t in reqs.items()}
+            out[(name, sharpen)] = (folder, raw, reqs, ref)
+    return out
+
+
+_BF16_BOUND = {}
+
+
+def bound(folder, reqs, ref, dtype, cross=False):
+    """Largest allowed difference as a fraction of the largest logit."""
+    if dtype == "float32":
+        return TOL_CROSS_F32 if cross else TOL_PLAIN_F32
+    if folder not in _BF16_BOUND:
+        cfg, params = pm.read_model(folder, torch.bfloat16)
+        rounded = {r: pm.forward(cfg, params, t).float().numpy() for r, t in reqs.items()}
+        _BF16_BOUND[folder] = worst(rounded, ref, reqs)[0]
+    return _BF16_BOUND[folder]
+
+
+def pick(models, name, sharp, dtype):
+    return models[(name, SHARP[dtype] if sharp else 1.0)]
+
+
+def replay(folder, raw, name, dtype, trace, out_dir, page_size=None):
+    from inferrs_amd.engine import Engine, run_trace
+    page = page_size or PAGE_SIZE[name]
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-trace.max_tokens // page),
+                             max_seqs=4)
+    run_trace(eng, trace.lines, out_dir, io.StringIO())
+    eng.cache.check_invariants()
+    assert not eng.cache.sequences and all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups)
+    return trace.read(out_dir, raw["vocab_size"])
+
+
+def worst(got, ref, reqs, scale=None):
+    if scale is None:
+        scale = max(float(np.abs(v).max()) for v in ref.values())
+    err, where = 0.0, None
+    for r, toks in reqs.items():
+        for p in range(len(toks)):
+            e = float(np.abs(got[r][p] - ref[r][p]).max())
+            if not e <= err:            # also catches NaN
+                err, where = e, (r, p)
+    return err / scale, where
+
+
+def traces(reqs):
+    return {
+        "whole": tm.whole(reqs),
+        "tail32": tm.prefix_then_single(reqs, 32),
+        "portions": tm.portions(reqs, [7, 2, 16, 3, 2, 33, 5, 2, 64]),
+        "mixed": tm.mixed(reqs, seed=1),
+        "mixed2": tm.mixed(dict(reversed(list(reqs.items()))), seed=2, max_live=3),
+    }
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c[0] + ("sharp" if c[1] else ""))
+def test_every_cutting_matches_plain(models, tmp_path, case, dtype):
+    folder, raw, reqs, ref = pick(models, case[0], case[1], dtype)
+    first = None
+    for mode, trace in traces(reqs).items():
+        if mode.startswith("mixed"):
+            assert trace.max_live >= 3 and trace.max_tokens < sum(tm.round_up(len(t), 64) for t in reqs.values())
+        got = replay(folder, raw, case[0], dtype, trace, str(tmp_path / mode))
+        err, where = worst(got, ref, reqs)
+        assert err <= bound(folder, reqs, ref, dtype), f"{mode}: {err:.3e} of the scale at {where} against the plain implementation"
+        if first is None:
+            first = got
+        else:
+            err, where = worst(got, first, reqs, scale=max(float(np.abs(v).max()) for v in ref.values()))
+            assert err <= bound(folder, reqs, ref, dtype, cross=True), f"{mode}: {err:.3e} of the scale at {where} against the whole-request run"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(models, tmp_path, dtype):
+    """Three tokens in one step, then three hundred one by one."""
+    folder, raw, reqs, ref = pick(models, "B", True, dtype)
+    one = {"r8": reqs["r8"]}
+    got = replay(folder, raw, "B", dtype, tm.prefix_then_single(one, len(one["r8"]) - 3), str(tmp_path))
+    err, where = worst(got, ref, one)
+    assert err <= bound(folder, reqs, ref, dtype), f"{err:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_page_sizes(models, tmp_path, dtype):
+    """Results do not depend on the page size (1, 3: no power of two, 64: one page a request)."""
+    folder, raw, reqs, ref = pick(models, "A", True, dtype)
+    for page in (1, 3, 64):
+        got = replay(folder, raw, "A", dtype, tm.mixed(reqs, seed=page), str(tmp_path / str(page)), page_size=page)
+        err, where = worst(got, ref, reqs)
+        assert err <= bound(folder, reqs, ref, dtype), f"page size {page}: {err:.3e} at {where}"
+
+
+def test_poisoned_free_pages_change_nothing(models, tmp_path):
+    """Pages that are free or beyond a request's length are never read: NaN in them is harmless."""
+    import torch
+    from inferrs_amd.engine import Engine, run_trace
+    folder, raw, reqs, ref = pick(models, "B", True, "float32")
+    trace = tm.mixed(reqs, seed=3)
+    eng = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=-(-trace.max_tokens // 8), max_seqs=4)
+    for arr in eng.storage.arrays:
+        arr.fill_(float("nan"))
+    run_trace(eng, trace.lines, str(tmp_path), io.StringIO())
+    err, where = worst(trace.read(str(tmp_path), raw["vocab_size"]), ref, reqs)
+    assert err <= TOL_PLAIN_F32, f"{err:.3e} at {where}"
+    del torch
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, tmp_path, dtype):
+    """bin/trace_run as a user starts it: a child process, steps on standard input, `done`
+    lines on standard output, files in --out."""
+    folder, raw, reqs, ref = pick(models, "B", True, dtype)
+    trace = tm.mixed(reqs, seed=7)
+    out_dir = str(tmp_path / "out")
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", out_dir, "--max-tokens", str(trace.max_tokens)],
+        input=trace.text(), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[:-1] == [f"done {i}" for i in range(len(trace.lines))]
+    err, where = worst(trace.read(out_dir, raw["vocab_size"]), ref, reqs)
+    assert err <= bound(folder, reqs, ref, dtype), f"{err:.3e} at {where}"
+
+
+def test_out_of_pages_is_an_error_and_takes_nothing(models):
+    from inferrs_amd.cache import OutOfPages
+    from inferrs_amd.engine import Engine, Entry
+    folder, raw, reqs, _ = pick(models, "A", False, "float32")
+    eng = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=4, max_seqs=2)
+    with pytest.raises(OutOfPages):
+        eng.step([Entry("x", reqs["r3"], [0])])          # 37 tokens into 16 slots
+    eng.cache.check_invariants()
+    assert not eng.has_request("x") and eng.cache.groups[0].pool.num_free == 4
+    eng.step([Entry("y", reqs["r3"][:16], [15])])
+    with pytest.raises(OutOfPages):
+        eng.step([Entry("y", [1], [0])])
+    assert eng.cached_length("y") == 16

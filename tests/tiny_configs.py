@@ -1,5 +1,5 @@
-"""Two tiny configurations of the architecture that differ in every size and option, plus
-helpers that write them as model folders into a temporary directory."""
+"""Tiny configurations of the architecture that differ in every size and option, plus helpers
+that write them as model folders into a temporary directory."""
 from __future__ import annotations
 
 import os
@@ -16,20 +16,43 @@ TINY_B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size
               intermediate_size=160, num_hidden_layers=3, num_attention_heads=6, num_key_value_heads=3,
               head_dim=32, rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
               max_position_embeddings=1024, hidden_act="silu")
-# A third one with a single kv head, one query head per group of 5, head_dim 48 (no power of two).
+# A third one with a single kv head, one group of 5 query heads, head_dim 48 (no power of two).
 TINY_C = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=130, hidden_size=40,
               intermediate_size=72, num_hidden_layers=1, num_attention_heads=5, num_key_value_heads=1,
               head_dim=48, rope_theta=500.0, rms_norm_eps=1e-3, tie_word_embeddings=False,
               max_position_embeddings=512, hidden_act="silu")
+# The serving head size with few of everything else: 8 query heads per kv head, head_dim 128.
+TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=515, hidden_size=136,
+              intermediate_size=200, num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=1,
+              head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+              max_position_embeddings=2048, hidden_act="silu")
 
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
 
 
-def write_model(folder: str, raw: dict, seed: int, dtype=torch.bfloat16) -> str:
+def write_model(folder: str, raw: dict, seed: int, dtype=torch.bfloat16, sharpen: float = 1.0) -> str:
+    """A model folder with random weights.  `sharpen` multiplies the per-head norm weights of
+    queries and keys, so that scores spread by sharpen**4 and each query singles out a few keys
+    somewhere in its context: a key that is lost, misplaced or read from a wrong page then
+    changes the logits by far more than rounding does."""
+    import json
+
     from inferrs_amd.config import Qwen3Config
-    from inferrs_amd.weights import write_random_model
-    return write_random_model(folder, Qwen3Config.from_dict(raw), seed, dtype)
+    from inferrs_amd.parts import model_tensors
+    from inferrs_amd.weights import random_tensors, write_safetensors
+    config = Qwen3Config.from_dict(raw)
+    expected, optional = model_tensors(config.to_spec())
+    tensors = random_tensors({n: s for n, s in expected.items() if n not in optional}, seed, dtype)
+    if sharpen != 1.0:
+        for name in tensors:
+            if name.endswith("q_norm.weight") or name.endswith("k_norm.weight"):
+                tensors[name] = (tensors[name].float() * sharpen).to(dtype)
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(config.to_dict(), f)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    return folder
 
 
 def random_tokens(n: int, vocab: int, seed: int):
