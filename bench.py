@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, Qwen3-8B layer sizes, bfloat16,
+random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+
+A step is one decode step of the whole batch: the step function over one token per request,
+greedy choice of the next token on the device, and feeding it back.  The requests' caches are
+brought to the benchmark's context length by filling their pages with random keys and values
+(decode time does not depend on their content); the prefill figure is measured separately
+on a 2,048-token prompt through the same step function.  One JSON line is printed.
+
+The reference measures the same quantities with `inferrs bench` (`inferrs/src/bench.rs:40-224`,
+`Engine::bench_generate`, `inferrs/src/engine.rs:2557-2641`): synthetic prompt, stop tokens
+ignored, device-synchronised wall time.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+# Qwen3-8B as its config.json gives it (the third configuration of BASELINE.json).
+QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936,
+                hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
+                num_attention_heads=32, num_key_value_heads=8, head_dim=128, rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
+FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+PREFILL_TOKENS = 2048
+PAGE = 16
+
+
+def matmul_params(c) -> int:
+    """Weights of one layer's matrix products."""
+    h, d = c["hidden_size"], c["head_dim"]
+    qkv = (c["num_attention_heads"] + 2 * c["num_key_value_heads"]) * d * h
+    return qkv + c["num_attention_heads"] * d * h + 3 * h * c["intermediate_size"]
+
+
+def prefill_flops(c, t: int, rows_of_logits: int = 1) -> float:
+    linear = 2.0 * t * matmul_params(c) * c["num_hidden_layers"]
+    # causal scores and weighted values: 2 products of t(t+1)/2 x head_dim per query head
+    attn = 4.0 * (t * (t + 1) / 2) * c["head_dim"] * c["num_attention_heads"] * c["num_hidden_layers"]
+    return linear + attn + 2.0 * rows_of_logits * c["vocab_size"] * c["hidden_size"]
+
+
+def decode_bytes(c, batch: int, context: float, esize: int = 2) -> float:
+    """What one decode step has to read: every weight it uses once, and the cache of the live requests."""
+    weights = (matmul_params(c) + 2 * c["hidden_size"] + 2 * c["head_dim"]) * c["num_hidden_layers"]
+    weights += c["vocab_size"] * c["hidden_size"] + c["hidden_size"]          # logits head, final norm
+    kv = 2 * c["num_key_value_heads"] * c["head_dim"] * c["num_hidden_layers"] * context * batch
+    return float(weights * esize + kv * esize + batch * c["hidden_size"] * esize)
+
+
+def fill_context(engine, ids, context: int) -> None:
+    """Gives each request `context` cached tokens without running them: pages are reserved and
+    filled with random keys and values."""
+    import torch
+    for sid in ids:
+        engine.add_request(sid)
+        if not engine.cache.reserve(sid, context):
+            raise RuntimeError("the cache pool is too small for the benchmark's context")
+        engine.cache.commit(sid, context)
+    gen = torch.Generator(device=engine.device).manual_seed(1)
+    for arr in engine.storage.arrays:
+        flat = arr.view(-1)
+        step = 1 << 28
+        for i in range(0, flat.numel(), step):
+            part = flat[i:i + step]
+            part.copy_(torch.randn(part.numel(), generator=gen, device=engine.device, dtype=torch.float32)
+                       .mul_(0.5).to(arr.dtype))
+
+
+def time_decode(engine, batch: int, context: int, steps: int, warmup: int):
+    """(seconds for `steps` steps, mean context length during them)."""
+    import torch
+    from inferrs_amd import ops
+    from inferrs_amd.engine import Entry
+    ids = [f"d{i}" for i in range(batch)]
+    start_len = context - steps - warmup
+    fill_context(engine, ids, start_len)
+    tokens = [1 + i for i in range(batch)]
+    t0 = None
+    for s in range(warmup + steps):
+        if s == warmup:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        logits = engine.step([Entry(sid, [tok], [0]) for sid, tok in zip(ids, tokens)])
+        tokens = ops.argmax(logits).cpu().tolist()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for sid in ids:
+        engine.end_request(sid)
+    return elapsed, start_len + warmup + (steps - 1) / 2.0
+
+
+def time_prefill(engine, n_tokens: int, runs: int, vocab: int):
+    import torch
+    from inferrs_amd.engine import Entry
+    g = torch.Generator().manual_seed(2)
+    prompt = torch.randint(0, vocab, (n_tokens,), generator=g).tolist()
+    best = None
+    for r in range(runs + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([Entry("p", prompt, [n_tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.end_request("p")
+        if r > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS,
+                    help="run fewer layers than the model has (recorded in the config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from inferrs_amd.config import Qwen3Config
+    from inferrs_amd.engine import Engine
+
+    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    config = Qwen3Config.from_dict(raw)
+    dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    esize = 2 if args.dtype == "bfloat16" else 4
+    points_batches = [] if args.no_points else [1, 64]
+    biggest = max([args.batch] + points_batches)
+    num_pages = biggest * (-(-args.context // PAGE) + 1) + 8
+    engine = Engine.from_random(config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=num_pages,
+                                max_seqs=biggest + 1)
+
+    elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = args.batch * args.steps / elapsed
+    nbytes = decode_bytes(raw, args.batch, mean_ctx, esize)
+    achieved = nbytes / (elapsed / args.steps) / 1e9
+
+    record = {
+        "metric": "decode tok/s at batch 8, context 8192 (Qwen3-8B)", "value": round(value, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_key,
+        "data": "synthetic: random-init weights, uniform-random token ids, cache pages of the context "
+                "filled with random keys and values",
+        "config": {
+            "model": "Qwen3-8B shape", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single GPU", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+            "hidden_size": raw["hidden_size"], "intermediate_size": raw["intermediate_size"],
+            "num_attention_heads": raw["num_attention_heads"], "num_key_value_heads": raw["num_key_value_heads"],
+            "head_dim": raw["head_dim"], "vocab_size": raw["vocab_size"], "rope_theta": raw["rope_theta"],
+            "rms_norm_eps": raw["rms_norm_eps"], "tie_word_embeddings": raw["tie_word_embeddings"],
+            "kv_page_size": PAGE, "prefill_tokens": PREFILL_TOKENS,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_points:
+        points = {}
+        for b in points_batches:
+            steps = max(8, args.steps // 2)
+            el, _ = time_decode(engine, b, args.context, steps, min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(b * steps / el, 2)
+        record["points"] = points
+        t = time_prefill(engine, PREFILL_TOKENS, 3, raw["vocab_size"])
+        flops = prefill_flops(raw, PREFILL_TOKENS)
+        record["prefill"] = {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS[dtype_key], 4)}
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

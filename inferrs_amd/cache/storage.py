@@ -1,8 +1,9 @@
 """Device arrays behind the cache manager's bookkeeping.
 
-Paged groups: per layer a key array and a value array `[pages, n_kv_heads, page_size, head_dim]`
-in the model's precision, so one page of one head is `page_size * head_dim` contiguous
-elements.  (The reference keeps `[pages * page_size, n_kv_heads, head_dim]` per layer,
+Paged groups: per layer a key array `[pages, n_kv_heads, page_size, head_dim]` and a value array
+`[pages, n_kv_heads, head_dim, page_size]` (values are kept transposed inside a page: the
+attention kernels multiply probabilities into them along the slots) in the model's precision,
+so one page of one head is `page_size * head_dim` contiguous elements.  (The reference keeps `[pages * page_size, n_kv_heads, head_dim]` per layer,
 `inferrs-models/src/kv_cache.rs:249-270`, and gathers it into a dense copy per pass; here the
 attention kernels read pages through the block table.)  Pages are not cleared on reuse:
 attention never reads beyond a request's length.
@@ -45,7 +46,9 @@ class CacheStorage:
                                manager.page_size, need.head_dim), dtype=dtype, device=device)
             self.arrays.append(arr)
             for i, layer in enumerate(g.layers):
-                self.layers[layer] = LayerCache(layer, g.index, arr[i, 0], arr[i, 1])
+                self.layers[layer] = LayerCache(
+                    layer, g.index, arr[i, 0],
+                    arr[i, 1].view(arr.shape[2], need.n_kv_heads, need.head_dim, manager.page_size))
         for st in manager.states:
             arr = torch.zeros((manager.max_seqs, *st.need.shape), dtype=st.need.dtype, device=device)
             self.arrays.append(arr)

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     T* __restrict__ out,                 // [n, nq, d]
     const T* __restrict__ q,             // [n, nq, d]
     const T* __restrict__ k_cache,       // [pages, nkv, page_size, d]
-    const T* __restrict__ v_cache,
+    const T* __restrict__ v_cache,       // [pages, nkv, d, page_size]  (transposed inside a page)
     const int* __restrict__ positions,   // [n]
     const int* __restrict__ token_seq,   // [n] row of block_table
     const int* __restrict__ block_table, // [seqs, max_pages]
@@ -72,12 +72,12 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
         for (int jj = first; jj <= last; ++jj) {
             const int key = j0 + jj;
             const int page = bt[key / page_size], off = key % page_size;
-            const T* vp = v_cache + (((size_t)page * nkv + kvh) * page_size + off) * d;
+            const T* vp = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
             const float pv = sp[jj];
 #pragma unroll
             for (int t = 0; t < AG_DIMS_PER_LANE; ++t) {
                 const int e = lane + t * IA_WAVE;
-                if (e < d) o[t] = fmaf(pv, ld(vp + e), o[t]);
+                if (e < d) o[t] = fmaf(pv, ld(vp + (size_t)e * page_size), o[t]);
             }
         }
         __syncthreads();

@@ -1,0 +1,339 @@
+// Paged grouped-query attention on the matrix cores, bfloat16, for one head size per build
+// (IA_HEAD_DIM, a multiple of 16 up to 256).  One kernel serves prefill and decode: a wave
+// owns up to 16 * NB columns, a column being one (query token, query head) pair of one
+// request and one key/value head, and walks that request's keys 32 at a time straight from
+// the cache pages into MFMA operands.  Decode batches (one token a request) have few
+// columns and long key ranges, so the keys are split between waves and the partial results
+// are merged by a second kernel.
+//
+// Formula as in the reference: S = (q . k) * scale after the product, keys j <= position
+// (inferrs-models/src/models/attention_utils.rs:61-85), softmax over keys, O = P v
+// (inferrs-models/src/models/qwen3.rs:166-192); query head h reads key/value head
+// h / (nq / nkv) (attention_utils.rs:38-49).  Scores, the running maximum and sum, and the
+// output accumulators are 32-bit; probabilities are rounded to bfloat16 for the second product.
+//
+// Everything is computed transposed so that no operand needs a transpose in flight:
+//   S^T[key][col] = K[key][:] . Q[col][:]      A = 16 keys x 32 dims (rows of the K page),
+//                                              B = 32 dims x 16 columns (rows of Q)
+//   O^T[dim][col] = V^T[dim][:] . P^T[:][col]  A = 16 dims x 32 keys (rows of the V^T page),
+//                                              B = 32 keys x 16 columns (the S^T accumulators)
+// The cache keeps keys as [page][kv head][slot][dim] and values transposed, as
+// [page][kv head][dim][slot], so both A operands are 16-byte pieces of contiguous rows.
+// v_mfma_f32_16x16x32_bf16: lane l supplies row l%16 of A and column l%16 of B with the eight
+// k values 8*(l/16)..+8, and receives D[4*(l/16)+i][l%16], i = 0..3.  The two S^T tiles of a
+// 32-key step assign key k0 + 8G + 4t + i to row 4G+i of tile t, so that lane (col, G) ends
+// up holding the probabilities of keys k0+8G .. k0+8G+7 in order: exactly the B operand of the
+// second product.
+#include "common.h"
+#include "api.h"
+
+#ifndef IA_HEAD_DIM
+#error "compile with -DIA_HEAD_DIM=<multiple of 16 up to 256>"
+#endif
+static_assert(IA_HEAD_DIM % 16 == 0 && IA_HEAD_DIM >= 16 && IA_HEAD_DIM <= 256, "head size");
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define HD IA_HEAD_DIM
+#define DB (HD / 16)            // 16-dim blocks of the output
+#define KS ((HD + 31) / 32)     // 32-dim steps of the first product
+
+struct AttnParams {
+    bf16_t* out;                // [n, nq, d]
+    float* part_o;              // [n, nq, splits, d]   when splits > 1
+    float* part_ml;             // [n, nq, splits, 2]   running maximum (log2 domain) and sum
+    const bf16_t* q;            // [n, nq, d]
+    const bf16_t* k_cache;      // [pages, nkv, page, d]
+    const bf16_t* v_cache;      // [pages, nkv, d, page]
+    const int* block_table;     // [seqs, max_pages]
+    const int* cu_tokens;       // [seqs + 1]  request s owns tokens cu[s]..cu[s+1]
+    const int* positions;       // [n]         absolute position of each token
+    int max_pages, nq, nkv, page, window, splits, chunk;
+    float scale_log2;           // scale * log2(e)
+};
+
+__device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
+
+template <int NB>
+__global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) {
+    const int lane = threadIdx.x;
+    const int r = lane & 15, G = lane >> 4;
+    const int cb = blockIdx.x;
+    const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
+    const int seq = blockIdx.z;
+    const int g = p.nq / p.nkv;
+    const int t0 = p.cu_tokens[seq], q_len = p.cu_tokens[seq + 1] - t0;
+    const int n_cols = q_len * g;
+    const int col0 = cb * 16 * NB;
+    if (col0 >= n_cols) return;
+    const int kv_start = p.positions[t0];
+    const int kv_total = kv_start + q_len;
+    const int* bt = p.block_table + (size_t)seq * p.max_pages;
+
+    // this lane's columns
+    int tq[NB], head[NB], pos[NB];
+    bool cvalid[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int c = col0 + nb * 16 + r;
+        cvalid[nb] = c < n_cols;
+        const int cc = cvalid[nb] ? c : n_cols - 1;
+        tq[nb] = cc / g;
+        head[nb] = kvh * g + (cc - tq[nb] * g);
+        pos[nb] = kv_start + tq[nb];
+    }
+    const int last_col = (col0 + 16 * NB <= n_cols ? col0 + 16 * NB : n_cols) - 1;
+    const int pmin = kv_start + col0 / g, pmax = kv_start + last_col / g;
+
+    // Q^T operands stay in registers for the whole walk.
+    uint4 qreg[NB][KS];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int dim = ks * 32 + G * 8;
+            qreg[nb][ks] = (cvalid[nb] && dim < HD) ? *(const uint4*)(qrow + dim) : zero4();
+        }
+    }
+
+    f32x4 acc[NB][DB];
+    float m[NB], l[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        m[nb] = -INFINITY;
+        l[nb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+
+    int lo = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;
+    int hi = pmax + 1;
+    if (p.splits > 1) {
+        const int c_lo = split * p.chunk, c_hi = c_lo + p.chunk;
+        lo = lo > c_lo ? lo : c_lo;
+        hi = hi < c_hi ? hi : c_hi;
+    }
+    lo &= ~31;
+
+    for (int k0 = lo; k0 < hi; k0 += 32) {
+        // ---- operands of this step: 32 keys = two 16-slot halves, each inside one page -------
+        uint4 kreg[2][KS];      // tile t, dim step ks: row r <-> key k0 + 8*(r/4) + 4t + r%4
+        uint4 vreg[DB];         // dim block db: row r <-> dim 16 db + r, keys k0 + 8G .. +7
+        {
+            // Rows past the request's length are read from its last written slot instead (their
+            // scores are masked below): the pages behind them may not exist.
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                int key = k0 + 8 * (r >> 2) + 4 * t + (r & 3);
+                key = key < kv_total ? key : kv_total - 1;
+                const int kpage = bt[key / p.page];
+                const bf16_t* krow = p.k_cache + (((size_t)kpage * p.nkv + kvh) * p.page + key % p.page) * HD + G * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    kreg[t][ks] = (ks * 32 + G * 8 < HD) ? *(const uint4*)(krow + ks * 32) : zero4();
+            }
+            int vkey = k0 + 8 * G;
+            vkey = vkey < kv_total ? vkey : (kv_total - 1) & ~7;
+            const int vpage = bt[vkey / p.page];
+            const bf16_t* vbase = p.v_cache + (((size_t)vpage * p.nkv + kvh) * HD + r) * p.page + vkey % p.page;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) vreg[db] = *(const uint4*)(vbase + (size_t)db * 16 * p.page);
+        }
+        const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
+        if (k0 + 32 > kv_total) {
+            // slots beyond the request's length hold anything at all: zero those values so that
+            // a probability of zero times their content stays zero
+            const int first_bad = kv_total - (k0 + 8 * G);          // keys >= this index are unwritten
+            if (first_bad < 8) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    uint32_t w[4] = {vreg[db].x, vreg[db].y, vreg[db].z, vreg[db].w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (j >= first_bad) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                    vreg[db] = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+            }
+        }
+
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            // ---- S^T for 32 keys x 16 columns ----------------------------------------------
+            f32x4 s[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                s[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, kreg[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), s[t], 0, 0, 0);
+            }
+            float sc[8];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sc[4 * t + i] = s[t][i] * p.scale_log2;
+            if (edge) {
+                const int kbase_idx = k0 + 8 * G;
+                const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int key = kbase_idx + j;
+                    if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
+                }
+            }
+            float mx = sc[0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j) mx = fmaxf(mx, sc[j]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, IA_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, IA_WAVE));
+            const float m_new = fmaxf(m[nb], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = exp2f(m[nb] - m_use);       // m = -inf gives 0
+            float pr[8], psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                pr[j] = exp2f(sc[j] - m_use);
+                psum += pr[j];
+            }
+            l[nb] = l[nb] * alpha + psum;
+            m[nb] = m_new;
+            uint4 pb;
+            pb.x = (uint32_t)f32_to_bf16_bits(pr[0]) | ((uint32_t)f32_to_bf16_bits(pr[1]) << 16);
+            pb.y = (uint32_t)f32_to_bf16_bits(pr[2]) | ((uint32_t)f32_to_bf16_bits(pr[3]) << 16);
+            pb.z = (uint32_t)f32_to_bf16_bits(pr[4]) | ((uint32_t)f32_to_bf16_bits(pr[5]) << 16);
+            pb.w = (uint32_t)f32_to_bf16_bits(pr[6]) | ((uint32_t)f32_to_bf16_bits(pr[7]) << 16);
+            // ---- O^T += V^T . P^T ----------------------------------------------------------
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    acc[nb][db][0] *= alpha; acc[nb][db][1] *= alpha;
+                    acc[nb][db][2] *= alpha; acc[nb][db][3] *= alpha;
+                }
+            }
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, vreg[db]), __builtin_bit_cast(bf16x8, pb), acc[nb][db], 0, 0, 0);
+        }
+    }
+
+    // ---- results: lane (col, G) holds dims 16 db + 4 G + i of its column ---------------------
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        float lt = l[nb];
+        lt += __shfl_xor(lt, 16, IA_WAVE);
+        lt += __shfl_xor(lt, 32, IA_WAVE);
+        if (!cvalid[nb]) continue;
+        const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
+        if (p.splits == 1) {
+            const float inv = 1.0f / lt;
+            bf16_t* o = p.out + row * HD + 4 * G;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                uint2 w;
+                w.x = (uint32_t)f32_to_bf16_bits(acc[nb][db][0] * inv) | ((uint32_t)f32_to_bf16_bits(acc[nb][db][1] * inv) << 16);
+                w.y = (uint32_t)f32_to_bf16_bits(acc[nb][db][2] * inv) | ((uint32_t)f32_to_bf16_bits(acc[nb][db][3] * inv) << 16);
+                *(uint2*)(o + 16 * db) = w;
+            }
+        } else {
+            float* o = p.part_o + (row * p.splits + split) * HD + 4 * G;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) *(f32x4*)(o + 16 * db) = acc[nb][db];
+            if (G == 0) {
+                float* ml = p.part_ml + (row * p.splits + split) * 2;
+                ml[0] = m[nb];
+                ml[1] = lt;
+            }
+        }
+    }
+}
+
+// Merges the partial results of the key splits of one (token, head): one wave a row.
+__global__ __launch_bounds__(IA_WAVE) void attn_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
+                                                             const float* __restrict__ part_ml, int splits) {
+    const size_t row = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float* ml = part_ml + row * splits * 2;
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml[2 * s]);
+    float total = 0.f;
+    float o[(HD + IA_WAVE - 1) / IA_WAVE];
+#pragma unroll
+    for (int t = 0; t < (HD + IA_WAVE - 1) / IA_WAVE; ++t) o[t] = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float ms = ml[2 * s];
+        if (ms == -INFINITY) continue;                  // a split that held no key of this row
+        const float w = exp2f(ms - mx);
+        total += ml[2 * s + 1] * w;
+        const float* po = part_o + (row * splits + s) * HD;
+#pragma unroll
+        for (int t = 0; t < (HD + IA_WAVE - 1) / IA_WAVE; ++t) {
+            const int e = lane + t * IA_WAVE;
+            if (e < HD) o[t] += po[e] * w;
+        }
+    }
+    const float inv = 1.0f / total;
+#pragma unroll
+    for (int t = 0; t < (HD + IA_WAVE - 1) / IA_WAVE; ++t) {
+        const int e = lane + t * IA_WAVE;
+        if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(o[t] * inv);
+    }
+}
+
+extern "C" int ia_attention_mfma_head_dim(void) { return HD; }
+
+// Floats of workspace that `splits` > 1 needs: partial outputs, then maxima and sums.
+extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
+    return splits > 1 ? (long long)n * nq * splits * (HD + 2) : 0;
+}
+
+// max_q_len: the most tokens any request has in this step; `chunk`: keys per split (a multiple
+// of 32, splits * chunk >= the longest request's length after the step).
+extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
+                                 const void* v_cache, const int* block_table, const int* cu_tokens,
+                                 const int* positions, int n, int n_seqs, int max_q_len, int max_pages,
+                                 int nq, int nkv, int d, int page_size, int window, float scale,
+                                 int splits, int chunk, hipStream_t stream) {
+    IA_CHECK(d == HD, "attention_mfma: built for head_dim %d, called with %d", HD, d);
+    IA_CHECK(n >= 0 && n_seqs >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0,
+             "attention_mfma: bad sizes n=%d seqs=%d nq=%d nkv=%d", n, n_seqs, nq, nkv);
+    IA_CHECK(page_size > 0 && page_size % 16 == 0, "attention_mfma: page size %d must be a multiple of 16", page_size);
+    IA_CHECK(max_pages > 0 && window >= 0 && max_q_len >= 1, "attention_mfma: bad geometry max_pages=%d window=%d max_q_len=%d",
+             max_pages, window, max_q_len);
+    IA_CHECK(splits >= 1 && splits <= 256 && (splits == 1 || (workspace != nullptr && chunk >= 32 && chunk % 32 == 0)),
+             "attention_mfma: bad split of the keys (splits=%d chunk=%d)", splits, chunk);
+    IA_CHECK((long long)nkv * splits <= 65535 && n_seqs <= 65535, "attention_mfma: grid too large (nkv*splits=%d seqs=%d)",
+             nkv * splits, n_seqs);
+    if (n == 0 || n_seqs == 0) return 0;
+    const int g = nq / nkv;
+    AttnParams p;
+    p.out = (bf16_t*)out;
+    p.part_o = workspace;
+    p.part_ml = workspace ? workspace + (size_t)n * nq * splits * HD : nullptr;
+    p.q = (const bf16_t*)q;
+    p.k_cache = (const bf16_t*)k_cache;
+    p.v_cache = (const bf16_t*)v_cache;
+    p.block_table = block_table;
+    p.cu_tokens = cu_tokens;
+    p.positions = positions;
+    p.max_pages = max_pages; p.nq = nq; p.nkv = nkv; p.page = page_size; p.window = window;
+    p.splits = splits; p.chunk = chunk;
+    p.scale_log2 = scale * 1.4426950408889634f;
+    const long long cols = (long long)max_q_len * g;
+    if (cols <= 16) {
+        const dim3 grid(1, nkv * splits, n_seqs);
+        attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
+    } else {
+        const dim3 grid((unsigned)((cols + 31) / 32), nkv * splits, n_seqs);
+        attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
+    }
+    IA_LAUNCH_CHECK("attention_mfma");
+    if (splits > 1) {
+        attn_merge_kernel<<<(unsigned)((long long)n * nq), IA_WAVE, 0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits);
+        IA_LAUNCH_CHECK("attention_merge");
+    }
+    return 0;
+}

@@ -8,22 +8,6 @@
 #include "common.h"
 #include "api.h"
 
-#include <stdarg.h>
-#include <stdio.h>
-
-static thread_local char g_error[512] = "";
-
-void ia_set_error(const char* fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_error, sizeof(g_error), fmt, ap);
-    va_end(ap);
-}
-
-extern "C" const char* ia_last_error(void) { return g_error; }
-
-extern "C" int ia_abi_version(void) { return IA_ABI_VERSION; }
-
 // ---- embedding ------------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_gather_kernel(T* __restrict__ out, const T* __restrict__ table,

@@ -18,7 +18,7 @@ template <typename T>
 __global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_kernel(
     T* __restrict__ q_out,              // [n, nq, d]
     T* __restrict__ k_cache,            // [pages, nkv, page_size, d] or null
-    T* __restrict__ v_cache,
+    T* __restrict__ v_cache,            // [pages, nkv, d, page_size] or null
     const T* __restrict__ qkv,          // [n, (nq + 2 nkv) d]
     const float* __restrict__ q_norm_w, // [d] or null
     const float* __restrict__ k_norm_w, // [d] or null
@@ -62,11 +62,15 @@ __global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_kernel(
     } else {
         const int slot = slots[tok];
         const int page = slot / page_size, off = slot - page * page_size;
-        const int kh = kind == 1 ? hh - nq : hh - nq - nkv;
-        T* cache = kind == 1 ? k_cache : v_cache;
-        dst = cache + (((size_t)page * nkv + kh) * page_size + off) * d;
+        if (kind == 2) {
+            // values are kept transposed inside a page: [dim][slot]
+            T* vt = v_cache + ((size_t)page * nkv + (hh - nq - nkv)) * d * page_size + off;
+            for (int j = lane; j < d; j += IA_WAVE) st(vt + (size_t)j * page_size, row[j]);
+            return;
+        }
+        dst = k_cache + (((size_t)page * nkv + (hh - nq)) * page_size + off) * d;
     }
-    if (kind == 2 || cos_t == nullptr) {
+    if (cos_t == nullptr) {
         for (int j = lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
         return;
     }

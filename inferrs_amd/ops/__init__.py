@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from typing import Optional, Tuple
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -24,28 +24,31 @@ class KernelError(RuntimeError):
     pass
 
 
-_LIB = None
-_LIB_PATH: Optional[str] = None
+_LIBS: Dict[str, ctypes.CDLL] = {}
+_LIB_PATHS: Dict[str, str] = {}
 
 
-def library() -> ctypes.CDLL:
-    """The compiled kernel library; compiled on first use when no built one is found."""
-    global _LIB, _LIB_PATH
-    if _LIB is not None:
-        return _LIB
-    path = _build.library_path()
+def library(target: str = "core") -> ctypes.CDLL:
+    """A compiled kernel library; compiled on first use when no built one is found."""
+    lib = _LIBS.get(target)
+    if lib is not None:
+        return lib
+    path = _build.library_path(target)
     if path is None:
-        path = _build.build(verbose=True)
+        path = _build.build(target, verbose=True)
     lib = ctypes.CDLL(path)
     lib.ia_last_error.restype = ctypes.c_char_p
     if lib.ia_abi_version() != 1:
         raise KernelError(f"{path}: unexpected ABI version {lib.ia_abi_version()}")
-    _LIB, _LIB_PATH = lib, path
+    if target.startswith("attn_d"):
+        lib.ia_attention_mfma_workspace.restype = ctypes.c_longlong
+    _LIBS[target], _LIB_PATHS[target] = lib, path
     return lib
 
 
-def library_file() -> Optional[str]:
-    return _LIB_PATH
+def library_files() -> Dict[str, str]:
+    """The libraries loaded so far: target -> file."""
+    return dict(_LIB_PATHS)
 
 
 def require_gpu() -> None:
@@ -55,9 +58,9 @@ def require_gpu() -> None:
     library()
 
 
-def _check(code: int) -> None:
+def _check(code: int, target: str = "core") -> None:
     if code:
-        raise KernelError(library().ia_last_error().decode("utf-8", "replace"))
+        raise KernelError(library(target).ia_last_error().decode("utf-8", "replace"))
 
 
 def _stream() -> ctypes.c_void_p:
@@ -196,10 +199,7 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, *,
             raise KernelError("qk_rope_kv: slots given without a cache")
         if slots.numel() != n:
             raise KernelError(f"qk_rope_kv: {slots.numel()} slots for {n} tokens")
-        for c in (k_cache, v_cache):
-            if c.dtype != qkv.dtype or c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, d):
-                raise KernelError(f"qk_rope_kv: cache has shape {tuple(c.shape)} {c.dtype}, expected "
-                                  f"[pages, {nkv}, {page_size}, {d}] {qkv.dtype}")
+        _check_cache(k_cache, v_cache, nkv, page_size, d, qkv.dtype, "qk_rope_kv")
     q_out = torch.empty((n, nq, d), dtype=qkv.dtype, device=qkv.device)
     _check(library().ia_qk_rope_kv(
         _p(q_out), _p(k_cache if slots is not None else None), _p(v_cache if slots is not None else None),
@@ -210,18 +210,28 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, *,
 
 # ---- attention --------------------------------------------------------------------------------
 
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, page_size: int, d: int,
+                 dtype: torch.dtype, who: str) -> None:
+    """Keys [pages, nkv, page_size, d]; values transposed inside a page, [pages, nkv, d, page_size]."""
+    if (k_cache.dtype != dtype or v_cache.dtype != dtype or k_cache.dim() != 4 or v_cache.dim() != 4
+            or tuple(k_cache.shape[1:]) != (nkv, page_size, d) or tuple(v_cache.shape[1:]) != (nkv, d, page_size)
+            or k_cache.shape[0] != v_cache.shape[0]):
+        raise KernelError(f"{who}: cache has shapes {tuple(k_cache.shape)} {k_cache.dtype} and "
+                          f"{tuple(v_cache.shape)} {v_cache.dtype}, expected [pages, {nkv}, {page_size}, {d}] "
+                          f"and [pages, {nkv}, {d}, {page_size}] {dtype}")
+
+
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                       *, window: Optional[int], scale: float) -> torch.Tensor:
-    """q [n, nq, d] against the paged cache [pages, nkv, page_size, d]; token i sees the keys
-    at positions <= positions[i] (and > positions[i] - window) of row token_seq[i] of the table."""
+    """q [n, nq, d] against the paged cache; token i sees the keys at positions <= positions[i]
+    (and > positions[i] - window) of row token_seq[i] of the table.  Any head size up to 512, any
+    page size, 32-bit or bfloat16 storage, all arithmetic in 32-bit."""
     _dev(q, k_cache, v_cache, positions, token_seq, block_table)
     _i32(positions, "positions"); _i32(token_seq, "token_seq"); _i32(block_table, "block_table")
     n, nq, d = q.shape
-    _, nkv, page_size, dk = k_cache.shape
-    if dk != d or k_cache.shape != v_cache.shape or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
-        raise KernelError(f"attention: q {tuple(q.shape)} {q.dtype} does not fit the cache "
-                          f"{tuple(k_cache.shape)} {k_cache.dtype}")
+    nkv, page_size = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention")
     if positions.numel() != n or token_seq.numel() != n or block_table.dim() != 2:
         raise KernelError("attention: positions, token_seq and block_table do not fit the batch")
     out = torch.empty_like(q)
@@ -229,6 +239,66 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _p(out), _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_seq), _p(block_table), n,
         block_table.shape[1], nq, nkv, d, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
         _stream()))
+    return out
+
+
+ATTN_TARGET_WAVES = 2048       # waves wanted in flight before the keys stop being split
+ATTN_MIN_CHUNK = 128           # fewest keys a split is worth
+
+
+def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and d in _build.ATTN_HEAD_DIMS and page_size % 16 == 0
+
+
+def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: int) -> Tuple[int, int]:
+    """(splits, keys per split) for the matrix-core kernel: the keys are split between waves
+    when the batch alone has too few (request, kv head, column block) items to fill the chip."""
+    cols = max_q_len * g
+    col_blocks = 1 if cols <= 16 else -(-cols // 32)
+    items = n_seqs * nkv * col_blocks
+    splits = 1
+    while items * splits < ATTN_TARGET_WAVES and max_kv_len >= 2 * splits * ATTN_MIN_CHUNK and splits < 128:
+        splits *= 2
+    chunk = -(-max_kv_len // splits)
+    chunk = -(-chunk // 32) * 32
+    return splits, chunk
+
+
+def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
+                   cu_tokens: torch.Tensor, block_table: torch.Tensor, *, max_q_len: int, max_kv_len: int,
+                   window: Optional[int], scale: float, splits: Optional[int] = None) -> torch.Tensor:
+    """The matrix-core kernel: bfloat16, head sizes in steps of 16 up to 256, page sizes in steps
+    of 16.  Request s owns tokens cu_tokens[s]..cu_tokens[s+1] at consecutive positions;
+    `max_q_len` and `max_kv_len` are the largest token count of a request in this step and the
+    largest length after it."""
+    _dev(q, k_cache, v_cache, positions, cu_tokens, block_table)
+    _i32(positions, "positions"); _i32(cu_tokens, "cu_tokens"); _i32(block_table, "block_table")
+    n, nq, d = q.shape
+    nkv, page_size = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention")
+    if not attention_mfma_fits(q.dtype, d, page_size):
+        raise KernelError(f"attention_mfma: takes bfloat16, head sizes {_build.ATTN_HEAD_DIMS[0]}.."
+                          f"{_build.ATTN_HEAD_DIMS[-1]} in steps of 16 and page sizes in steps of 16; got "
+                          f"{q.dtype}, head size {d}, page size {page_size}")
+    n_seqs = cu_tokens.numel() - 1
+    if positions.numel() != n or block_table.dim() != 2 or block_table.shape[0] < n_seqs or nq % nkv:
+        raise KernelError("attention_mfma: positions, cu_tokens and block_table do not fit the batch")
+    if max_kv_len > block_table.shape[1] * page_size or max_q_len < 1 or max_q_len > n:
+        raise KernelError(f"attention_mfma: max_kv_len {max_kv_len} / max_q_len {max_q_len} do not fit "
+                          f"{block_table.shape[1]} pages of {page_size} and {n} tokens")
+    if splits is None:
+        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len)
+    else:
+        chunk = -(-(-(-max_kv_len // splits)) // 32) * 32
+    target = _build.attn_target(d)
+    lib = library(target)
+    out = torch.empty_like(q)
+    ws_floats = lib.ia_attention_mfma_workspace(n, nq, splits)
+    ws = torch.empty((ws_floats,), dtype=torch.float32, device=q.device) if ws_floats else None
+    _check(lib.ia_attention_mfma(
+        _p(out), _p(ws), _p(q), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions),
+        n, n_seqs, max_q_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
+        ctypes.c_float(scale), splits, chunk, _stream()), target)
     return out
 
 

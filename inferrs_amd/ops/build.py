@@ -1,9 +1,14 @@
-"""Compiles the HIP sources under `inferrs_amd/csrc` for gfx950 into one shared library.
+"""Compiles the HIP sources under `inferrs_amd/csrc` for gfx950 into shared libraries.
 
-The library's file name carries a hash of the sources and flags, so a library
-that is found is never stale.  `build()` always compiles; `library_path()`
-returns a built library or None.  The library lives beside the package when
-that folder can be written, else under the temporary directory.
+Two kinds of library:
+  * "core": every kernel whose code does not depend on a model size;
+  * "attn_d<N>": the matrix-core attention kernel built for head size N (`-DIA_HEAD_DIM=N`),
+    so that a model compiles only the head size it has.
+
+A library's file name carries a hash of its sources and flags, so a library that is found
+is never stale.  `build(target)` always compiles; `library_path(target)` returns a built
+library or None.  Libraries live beside the package when that folder can be written, else
+under the temporary directory.
 """
 from __future__ import annotations
 
@@ -13,45 +18,69 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
-from typing import List, Optional
+from typing import Dict, List, Optional, Sequence, Tuple
 
 ARCH = "gfx950"
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(_PKG, "csrc")
-# -packed-fp32-ops is switched off on purpose: some packed 32-bit forms have given wrong results.
+# Packed 32-bit float instructions are switched off: some of their forms have given wrong
+# results on this hardware.
 FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 
+PER_HEAD_DIM = ("attention_mfma.hip",)
+SHARED = ("error.hip",)
+ATTN_HEAD_DIMS = tuple(range(16, 257, 16))
 
-def _sources() -> List[str]:
-    return sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith(".hip"))
+
+def attn_target(head_dim: int) -> str:
+    return f"attn_d{head_dim}"
 
 
-def _digest() -> str:
+def all_targets() -> List[str]:
+    return ["core"] + [attn_target(d) for d in ATTN_HEAD_DIMS]
+
+
+def _plan(target: str) -> Tuple[List[str], List[str]]:
+    """(sources, extra defines) of a target."""
+    names = sorted(n for n in os.listdir(CSRC) if n.endswith(".hip"))
+    if target == "core":
+        return [os.path.join(CSRC, n) for n in names if n not in PER_HEAD_DIM], []
+    if target.startswith("attn_d"):
+        d = int(target[len("attn_d"):])
+        if d not in ATTN_HEAD_DIMS:
+            raise ValueError(f"no matrix-core attention kernel for head size {d}")
+        return [os.path.join(CSRC, n) for n in PER_HEAD_DIM + SHARED], [f"-DIA_HEAD_DIM={d}"]
+    raise ValueError(f"unknown kernel library {target!r}")
+
+
+def _digest(target: str) -> str:
+    srcs, defines = _plan(target)
     h = hashlib.sha256()
-    for p in sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith((".hip", ".h"))):
+    headers = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith(".h"))
+    for p in srcs + headers:
         h.update(os.path.basename(p).encode())
         with open(p, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + defines).encode())
     return h.hexdigest()[:12]
 
 
-def _lib_name() -> str:
-    return f"libinferrs_amd_{_digest()}.so"
+def _lib_name(target: str) -> str:
+    return f"libinferrs_amd_{target}_{_digest(target)}.so"
 
 
 def _candidate_dirs() -> List[str]:
-    dirs = [os.path.join(_PKG, "_lib")]
-    dirs.append(os.path.join(tempfile.gettempdir(), f"inferrs_amd_lib_{os.getuid()}"))
-    return dirs
+    return [os.path.join(_PKG, "_lib"),
+            os.path.join(tempfile.gettempdir(), f"inferrs_amd_lib_{os.getuid()}")]
 
 
-def library_path() -> Optional[str]:
-    name = _lib_name()
+def library_path(target: str = "core") -> Optional[str]:
+    name = _lib_name(target)
     for d in _candidate_dirs():
         p = os.path.join(d, name)
         if os.path.isfile(p):
@@ -63,14 +92,14 @@ def _writable_dir() -> str:
     for d in _candidate_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".probe_{os.getpid()}")
+            probe = os.path.join(d, f".probe_{os.getpid()}_{threading.get_ident()}")
             with open(probe, "w"):
                 pass
             os.remove(probe)
             return d
         except OSError:
             continue
-    raise RuntimeError("no writable folder for the kernel library: tried " + ", ".join(_candidate_dirs()))
+    raise RuntimeError("no writable folder for the kernel libraries: tried " + ", ".join(_candidate_dirs()))
 
 
 def _hipcc() -> str:
@@ -86,45 +115,59 @@ def _say(msg: str) -> None:
     print(f"[inferrs_amd build] {msg}", file=sys.stderr, flush=True)
 
 
-def build(verbose: bool = True) -> str:
-    """Compile every source and link the library; returns its path."""
+def build(target: str = "core", verbose: bool = True, workers: Optional[int] = None) -> str:
+    """Compile the sources of `target` and link its library; returns the path."""
     hipcc = _hipcc()
     out_dir = _writable_dir()
-    name = _lib_name()
-    obj_dir = os.path.join(out_dir, "_build", name[:-3])
+    name = _lib_name(target)
+    srcs, defines = _plan(target)
+    obj_dir = os.path.join(out_dir, "_build", f"{name[:-3]}_{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
-    srcs = _sources()
     t0 = time.time()
     if verbose:
-        _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
+        _say(f"{target}: compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
-        r = subprocess.run([hipcc, *FLAGS, "-I", CSRC, "-c", src, "-o", obj],
+        r = subprocess.run([hipcc, *FLAGS, *defines, "-I", CSRC, "-c", src, "-o", obj],
                            capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
         if verbose:
-            _say(f"  {os.path.basename(src)} done ({time.time() - t0:.0f} s)")
+            _say(f"  {target}: {os.path.basename(src)} done ({time.time() - t0:.0f} s)")
         return obj
 
-    workers = max(1, min(len(srcs), (os.cpu_count() or 2), 8))
-    with ThreadPoolExecutor(workers) as pool:
+    n = workers or max(1, min(len(srcs), (os.cpu_count() or 2), 8))
+    with ThreadPoolExecutor(n) as pool:
         objs = list(pool.map(compile_one, srcs))
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.tmp")
     r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp, *objs],
                        capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed to link the kernel library:\n{r.stdout}\n{r.stderr}")
+        raise RuntimeError(f"hipcc failed to link {name}:\n{r.stdout}\n{r.stderr}")
     lib = os.path.join(out_dir, name)
     os.replace(tmp, lib)
-    for old in os.listdir(out_dir):          # libraries of older sources
-        if old.startswith("libinferrs_amd_") and old.endswith(".so") and old != name:
+    prefix = f"libinferrs_amd_{target}_"
+    for old in os.listdir(out_dir):          # libraries of older sources of the same target
+        if old.startswith(prefix) and old.endswith(".so") and old != name:
             try:
                 os.remove(os.path.join(out_dir, old))
             except OSError:
                 pass
-    shutil.rmtree(os.path.join(out_dir, "_build"), ignore_errors=True)
+    shutil.rmtree(obj_dir, ignore_errors=True)
+    try:
+        os.rmdir(os.path.join(out_dir, "_build"))
+    except OSError:
+        pass
     if verbose:
-        _say(f"linked {lib} ({time.time() - t0:.0f} s)")
+        _say(f"{target}: linked {lib} ({time.time() - t0:.0f} s)")
     return lib
+
+
+def build_all(verbose: bool = True, targets: Optional[Sequence[str]] = None) -> Dict[str, str]:
+    """Compile every library (or `targets`), a few at a time."""
+    targets = list(targets or all_targets())
+    jobs = max(1, min(len(targets), (os.cpu_count() or 2), 8))
+    with ThreadPoolExecutor(jobs) as pool:
+        paths = list(pool.map(lambda t: build(t, verbose=verbose, workers=2), targets))
+    return dict(zip(targets, paths))

@@ -74,6 +74,11 @@ class Attention(Mixer):
             cos=cos, sin=sin, rot=self.position.rot_dim, interleaved=self.position.interleaved,
             k_cache=cache.k, v_cache=cache.v, slots=group.slots if cache.writable else None,
             page_size=group.page_size)
-        a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
-                                  window=s.window, scale=s.softmax_scale)
+        if ops.attention_mfma_fits(q.dtype, s.head_dim, group.page_size):
+            a = ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                   max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, window=s.window,
+                                   scale=s.softmax_scale)
+        else:
+            a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
+                                      window=s.window, scale=s.softmax_scale)
         return self.o(a.view(a.shape[0], s.n_heads * s.head_dim))

@@ -129,7 +129,7 @@ def test_qk_rope_kv(dtype, nq, nkv, d, rot, interleaved, normed):
     sin = torch.rand(n, rot // 2, generator=g) if rot else None
     slots = torch.randperm(pages * page, generator=g)[:n].to(torch.int32)
     kc = torch.full((pages, nkv, page, d), 7.0, dtype=dtype)
-    vc = torch.full((pages, nkv, page, d), 7.0, dtype=dtype)
+    vc = torch.full((pages, nkv, d, page), 7.0, dtype=dtype)       # values: [dim][slot] inside a page
     kc_d, vc_d = dev(kc), dev(vc)
     q = ops.qk_rope_kv(dev(qkv), nq, nkv, d, q_norm_w=None if qw is None else dev(qw),
                        k_norm_w=None if kw is None else dev(kw), eps=1e-5, add_one=False,
@@ -142,7 +142,7 @@ def test_qk_rope_kv(dtype, nq, nkv, d, rot, interleaved, normed):
     for t in range(n):
         s = int(slots[t])
         want_k[s // page, :, s % page] = rk[t]
-        want_v[s // page, :, s % page] = rv[t]
+        want_v[s // page, :, :, s % page] = rv[t]
     close(kc_d, want_k, tol(dtype, 3e-6), "k cache")         # untouched slots keep their 7.0
     assert torch.equal(vc_d.cpu().float(), want_v.to(dtype).float()), "values are copied as they are"
 
@@ -159,7 +159,7 @@ def ref_attention(q, kc, vc, positions, token_seq, table, window, scale):
         for h in range(nq):
             kvh = h // (nq // nkv)
             k = torch.stack([kc[p, kvh, j % page] for p, j in zip(pg, keys)]).float()
-            v = torch.stack([vc[p, kvh, j % page] for p, j in zip(pg, keys)]).float()
+            v = torch.stack([vc[p, kvh, :, j % page] for p, j in zip(pg, keys)]).float()
             s = (k @ q[t, h].float()) * scale
             out[t, h] = torch.softmax(s, 0) @ v
     return out
@@ -178,7 +178,7 @@ def attention_case(dtype, nq, nkv, d, page, lens, q_lens, seed, needle=False):
         for j in range(-(-l // page)):
             table[s, j] = perm.pop()
     kc = randn(total_pages, nkv, page, d, dtype=dtype, seed=seed + 1)
-    vc = randn(total_pages, nkv, page, d, dtype=dtype, seed=seed + 2)
+    vc = randn(total_pages, nkv, d, page, dtype=dtype, seed=seed + 2)
     positions = torch.tensor([p for l, ql in zip(lens, q_lens) for p in range(l - ql, l)], dtype=torch.int32)
     token_seq = torch.tensor([s for s, ql in enumerate(q_lens) for _ in range(ql)], dtype=torch.int32)
     q = randn(len(positions), nq, d, dtype=dtype, seed=seed + 3)
@@ -204,6 +204,41 @@ def test_attention_generic(dtype, nq, nkv, d, page, window):
                                 window=window, scale=scale)
     want = ref_attention(q, kc, vc, positions, token_seq, table, window, scale)
     close(got, want, tol(dtype, 5e-6, 2 ** -7), "attention")
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,window", [
+    (4, 2, 16, 16, None), (5, 1, 48, 16, None), (8, 1, 128, 16, None), (32, 8, 128, 16, None),
+    (6, 3, 32, 32, 37), (3, 3, 80, 16, None), (2, 2, 256, 64, 100), (40, 2, 64, 16, None), (7, 7, 112, 48, 5)])
+@pytest.mark.parametrize("lens,q_lens", [
+    ([1, 70, 129, 200, 64], [1, 70, 2, 1, 17]),          # mixed: whole prompts, portions, single tokens
+    ([300, 17, 1000, 33], [1, 1, 1, 1]),                  # decode only
+    ([257], [257]), ([16], [16]), ([32, 31, 33], [3, 31, 1])])
+def test_attention_mfma(nq, nkv, d, page, window, lens, q_lens):
+    from inferrs_amd import ops
+    dtype = torch.bfloat16
+    q, kc, vc, positions, token_seq, table = attention_case(dtype, nq, nkv, d, page, lens, q_lens, 13, needle=True)
+    # slots past a request's length hold NaN: they must not reach the result
+    for s, l in enumerate(lens):
+        for j in range(l, -(-l // page) * page):
+            kc[int(table[s, j // page]), :, j % page] = float("nan")
+            vc[int(table[s, j // page]), :, :, j % page] = float("nan")
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    want = ref_attention(q, kc, vc, positions, token_seq, table, window, scale)
+    for splits in (None, 1, 2, 8):
+        got = ops.attention_mfma(dev(q), dev(kc), dev(vc), dev(positions), dev(cu), dev(table),
+                                 max_q_len=max(q_lens), max_kv_len=max(lens), window=window, scale=scale,
+                                 splits=splits)
+        close(got, want, 2 ** -7, f"attention_mfma splits={splits}")
+
+
+def test_attention_mfma_refuses_what_it_cannot_take():
+    from inferrs_amd import ops
+    q, kc, vc, positions, token_seq, table = attention_case(torch.bfloat16, 2, 1, 16, 8, [9], [9], 1)
+    cu = torch.tensor([0, 9], dtype=torch.int32)
+    with pytest.raises(ops.KernelError, match="page sizes in steps of 16"):
+        ops.attention_mfma(dev(q), dev(kc), dev(vc), dev(positions), dev(cu), dev(table), max_q_len=9,
+                           max_kv_len=9, window=None, scale=0.25)
 
 
 def test_gemm_reference_products():
