@@ -129,6 +129,7 @@ def main() -> int:
                     help="run fewer layers than the model has (recorded in the config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -142,12 +143,18 @@ def main() -> int:
     config = Qwen3Config.from_dict(raw)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     esize = 2 if args.dtype == "bfloat16" else 4
-    points_batches = [] if args.no_points else [1, 64]
+    points_batches = [] if args.no_points or args.prefill_only else [1, 64]
     biggest = max([args.batch] + points_batches)
     num_pages = biggest * (-(-args.context // PAGE) + 1) + 8
     engine = Engine.from_random(config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=num_pages,
                                 max_seqs=biggest + 1)
 
+    if args.prefill_only:
+        t = time_prefill(engine, PREFILL_TOKENS, max(1, args.steps), raw["vocab_size"])
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS,
+                                      "ms": round(t * 1e3, 3),
+                                      "frac": round(prefill_flops(raw, PREFILL_TOKENS) / t / PEAK_FLOPS[dtype_key], 4)}}))
+        return 0
     elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
