@@ -6,6 +6,19 @@
     cache/     pages with block tables per request, per-request state slots
     engine/    model assembly, the step function, the scheduler, generation
     sampling/  sampling parameters and the device sampler
+    cli.py     `inferrs-amd run | bench`, in the reference's manner
     ops/       host checks and C calls into the HIP kernels of csrc/
 """
 __version__ = "0.1.0"
+
+
+def __getattr__(name):
+    """`inferrs_amd.Engine`, `inferrs_amd.SamplingParams`, `inferrs_amd.generate`: the Python entry
+    point, loaded on first use (importing the package alone needs no GPU)."""
+    if name in ("Engine", "Entry", "GenerationLoop", "generate"):
+        from . import engine
+        return getattr(engine, name)
+    if name == "SamplingParams":
+        from .sampling import SamplingParams
+        return SamplingParams
+    raise AttributeError(f"module 'inferrs_amd' has no attribute {name!r}")

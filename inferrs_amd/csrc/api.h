@@ -44,6 +44,22 @@ int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, float* partial,
                         int K, int splits, int out_dtype, hipStream_t stream);
 
 int ia_argmax(int* out, const float* logits, int rows, int vocab, hipStream_t stream);
+int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, const float* rep,
+                const float* freq, const float* pres, const int* bias_ids, const float* bias_vals,
+                int nb, hipStream_t stream);
+long long ia_sample_workspace(int rows, int vocab);
+int ia_sample(int* out, const float* logits, void* workspace, int rows, int vocab,
+              const float* temperature, const int* top_k, const float* top_p, const float* min_p,
+              const float* u, hipStream_t stream);
+
+// Built per head size (-DIA_HEAD_DIM) into a library of its own.
+int ia_attention_mfma_head_dim(void);
+long long ia_attention_mfma_workspace(int n, int nq, int splits);
+int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
+                      const void* v_cache, const int* block_table, const int* cu_tokens,
+                      const int* positions, int n, int n_seqs, int max_q_len, int max_pages,
+                      int nq, int nkv, int d, int page_size, int window, float scale,
+                      int splits, int chunk, hipStream_t stream);
 
 #ifdef __cplusplus
 }

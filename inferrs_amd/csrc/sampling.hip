@@ -3,20 +3,32 @@
 // ia_argmax: greedy choice, the lowest index among equal maxima (the reference's CPU argmax
 // keeps the first maximum, candle-core/src/cpu_backend/mod.rs:150-157; its CUDA reduction
 // leaves ties unspecified, inferrs-kernels/candle-kernels/src/reduce.cu:500-520).
+//
+// ia_penalize: logit bias, repetition penalty (z >= 0 ? z / p : z * p, once per distinct token
+// of the window), frequency and presence penalties (z -= f * count + p), in the reference's
+// order (inferrs/src/sampler.rs:186-229), in place on 32-bit logits.
+//
+// ia_sample: the rest of the reference's sampler (sampler.rs:232-335) for a row of logits:
+// divide by the temperature, softmax, order by probability (descending, equal values by
+// index), keep the first top_k, cut where the running sum reaches top_p, drop what is below
+// min_p times the largest probability, renormalise, and walk the kept list until the running
+// sum exceeds the row's random number u.  Every one of these filters keeps a prefix of the
+// ordered list, so no sort is needed: a prefix is named by a threshold key K and a count m of
+// the tokens equal to K (taken by ascending index), and the threshold for "the shortest
+// prefix whose weight reaches a target" is found by bisection over the 32 bits of the key,
+// one block-wide sum per bit.  Sums are tree sums in a fixed order; they differ from the
+// reference's sequential sums by rounding only.
 #include "common.h"
 #include "api.h"
 
-__global__ __launch_bounds__(1024) void argmax_kernel(int* __restrict__ out, const float* __restrict__ logits, int vocab) {
-    __shared__ float sv[16];
-    __shared__ int si[16];
-    const float* row = logits + (size_t)blockIdx.x * vocab;
+// ---- greedy ---------------------------------------------------------------------------------
+__device__ __forceinline__ void argmax_row(const float* __restrict__ row, int vocab, float* sv, int* si, int* out) {
     float best = -INFINITY;
     int idx = 0x7fffffff;
     for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
         const float v = row[c];
         if (v > best || (v == best && c < idx)) { best = v; idx = c; }
     }
-    if (idx == 0x7fffffff && threadIdx.x < vocab) idx = threadIdx.x;   // row of NaN or -inf
 #pragma unroll
     for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, IA_WAVE);
@@ -24,14 +36,21 @@ __global__ __launch_bounds__(1024) void argmax_kernel(int* __restrict__ out, con
         if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
     }
     const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+    __syncthreads();
     if (lane == 0) { sv[wave] = best; si[wave] = idx; }
     __syncthreads();
     if (threadIdx.x == 0) {
         const int nw = (blockDim.x + IA_WAVE - 1) / IA_WAVE;
         for (int w = 1; w < nw; ++w)
             if (sv[w] > best || (sv[w] == best && si[w] < idx)) { best = sv[w]; idx = si[w]; }
-        out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+        *out = idx == 0x7fffffff ? 0 : idx;       // a row of NaN or -inf
     }
+}
+
+__global__ __launch_bounds__(1024) void argmax_kernel(int* __restrict__ out, const float* __restrict__ logits, int vocab) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    argmax_row(logits + (size_t)blockIdx.x * vocab, vocab, sv, si, out + blockIdx.x);
 }
 
 extern "C" int ia_argmax(int* out, const float* logits, int rows, int vocab, hipStream_t stream) {
@@ -39,5 +58,294 @@ extern "C" int ia_argmax(int* out, const float* logits, int rows, int vocab, hip
     if (rows == 0) return 0;
     argmax_kernel<<<rows, 1024, 0, stream>>>(out, logits, vocab);
     IA_LAUNCH_CHECK("argmax");
+    return 0;
+}
+
+// ---- penalties ------------------------------------------------------------------------------
+// window [rows, w]: the last tokens of prompt and output, -1 where a row has fewer.
+// bias_ids / bias_vals [rows, nb]: -1 ends a row's list.
+__global__ void penalize_kernel(float* __restrict__ logits, int vocab, const int* __restrict__ window, int w,
+                                const float* __restrict__ rep, const float* __restrict__ freq,
+                                const float* __restrict__ pres, const int* __restrict__ bias_ids,
+                                const float* __restrict__ bias_vals, int nb) {
+    const int rowi = blockIdx.x;
+    float* row = logits + (size_t)rowi * vocab;
+    for (int j = threadIdx.x; j < nb; j += blockDim.x) {
+        const int id = bias_ids[(size_t)rowi * nb + j];
+        if (id >= 0 && id < vocab) atomicAdd(row + id, bias_vals[(size_t)rowi * nb + j]);
+    }
+    __syncthreads();
+    const int* win = window + (size_t)rowi * w;
+    const float rp = rep[rowi], fp = freq[rowi], pp = pres[rowi];
+    // one thread per distinct token: the one holding its first occurrence
+    for (int j = threadIdx.x; j < w; j += blockDim.x) {
+        const int id = win[j];
+        if (id < 0 || id >= vocab) continue;
+        bool first = true;
+        int count = 0;
+        for (int i = 0; i < w; ++i) {
+            if (win[i] == id) {
+                if (i < j) { first = false; break; }
+                ++count;
+            }
+        }
+        if (!first) continue;
+        float v = row[id];
+        if (rp != 1.0f && rp != 0.0f) v = v >= 0.f ? v / rp : v * rp;
+        if (fp != 0.0f || pp != 0.0f) {
+            v -= fp * (float)count;
+            v -= pp;
+        }
+        row[id] = v;
+    }
+}
+
+extern "C" int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, const float* rep,
+                           const float* freq, const float* pres, const int* bias_ids, const float* bias_vals,
+                           int nb, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && vocab > 0 && w >= 0 && nb >= 0, "penalize: bad sizes rows=%d vocab=%d window=%d bias=%d", rows, vocab, w, nb);
+    IA_CHECK(w == 0 || window != nullptr, "penalize: a window of %d tokens without its array", w);
+    IA_CHECK(nb == 0 || (bias_ids != nullptr && bias_vals != nullptr), "penalize: %d bias entries without their arrays", nb);
+    if (rows == 0 || (w == 0 && nb == 0)) return 0;
+    penalize_kernel<<<rows, 256, 0, stream>>>(logits, vocab, window, w, rep, freq, pres, bias_ids, bias_vals, nb);
+    IA_LAUNCH_CHECK("penalize");
+    return 0;
+}
+
+// ---- sampling -------------------------------------------------------------------------------
+#define SAMPLE_THREADS 512
+
+// Keys order like the values they come from; NaN sorts below everything.
+__device__ __forceinline__ uint32_t order_key(float z) {
+    if (z != z) return 0u;
+    const uint32_t u = __float_as_uint(z);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+struct Sums { float w; float n; };
+
+__device__ __forceinline__ Sums block_sums(float w, float n, float* scratch) {
+    Sums s;
+    s.w = block_sum(w, scratch);
+    s.n = block_sum(n, scratch + 16);
+    return s;
+}
+
+// Weight (probability, or 1 when `by_count`) and number of the tokens with key >= t.
+__device__ __forceinline__ Sums at_least(const uint32_t* __restrict__ keys, const float* __restrict__ probs,
+                                         int vocab, uint32_t t, bool by_count, float* scratch) {
+    float w = 0.f, n = 0.f;
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x)
+        if (keys[c] >= t) { w += by_count ? 1.0f : probs[c]; n += 1.0f; }
+    return block_sums(w, n, scratch);
+}
+
+struct Prefix { uint32_t key; int above; int ties; int take; float w_above; float p_key; };
+
+// The shortest prefix of the ordered list whose weight reaches `target` (strictly exceeds it
+// when `strict`): every token with a key above `key` and the first `take` of the `ties` tokens
+// equal to it.  When even the whole list does not reach the target, the whole list.
+__device__ Prefix shortest_prefix(const uint32_t* __restrict__ keys, const float* __restrict__ probs, int vocab,
+                                  float target, bool by_count, bool strict, float* scratch) {
+    uint32_t k = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t t = k | (1u << bit);
+        const float w = at_least(keys, probs, vocab, t, by_count, scratch).w;
+        if (strict ? w > target : w >= target) k = t;
+    }
+    // k is the largest key whose "at least" weight reaches the target (0 if none does).
+    float wa = 0.f, na = 0.f, ne = 0.f, pk = 0.f;
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const uint32_t key = keys[c];
+        if (key > k) { wa += by_count ? 1.0f : probs[c]; na += 1.0f; }
+        else if (key == k) { ne += 1.0f; pk = by_count ? 1.0f : probs[c]; }
+    }
+    Prefix r;
+    r.key = k;
+    r.w_above = block_sum(wa, scratch);
+    r.above = (int)block_sum(na, scratch + 16);
+    r.ties = (int)block_sum(ne, scratch);
+    // every token with this key has the same probability: take it from any thread that saw one
+    __shared__ float s_pk;
+    if (threadIdx.x == 0) s_pk = 0.f;
+    __syncthreads();
+    if (ne > 0.f) s_pk = pk;
+    __syncthreads();
+    r.p_key = s_pk;
+    int take = r.ties;
+    if (r.ties > 0 && r.p_key > 0.f) {
+        float run = r.w_above;
+        take = 0;
+        while (take < r.ties) {
+            run += r.p_key;
+            ++take;
+            if (strict ? run > target : run >= target) break;
+        }
+    }
+    r.take = take < 1 ? (r.ties > 0 ? 1 : 0) : take;
+    return r;
+}
+
+// Index of the `rank`-th (1-based, ascending index) token whose key equals `key`.
+__device__ int nth_with_key(const uint32_t* __restrict__ keys, int vocab, uint32_t key, int rank, int* s_counts) {
+    const int per = (vocab + blockDim.x - 1) / blockDim.x;
+    const int lo = threadIdx.x * per, hi = lo + per < vocab ? lo + per : vocab;
+    int mine = 0;
+    for (int c = lo; c < hi; ++c) mine += keys[c] == key;
+    __syncthreads();
+    s_counts[threadIdx.x] = mine;
+    __syncthreads();
+    __shared__ int s_found;
+    if (threadIdx.x == 0) {
+        s_found = -1;
+        int before = 0;
+        for (int t = 0; t < (int)blockDim.x; ++t) {
+            if (before + s_counts[t] >= rank) { s_found = t; s_counts[0] = before; break; }
+            before += s_counts[t];
+        }
+    }
+    __syncthreads();
+    __shared__ int s_index;
+    if (threadIdx.x == 0) s_index = -1;
+    __syncthreads();
+    if ((int)threadIdx.x == s_found) {
+        int seen = s_counts[0];
+        for (int c = lo; c < hi; ++c)
+            if (keys[c] == key && ++seen == rank) { s_index = c; break; }
+    }
+    __syncthreads();
+    return s_index;
+}
+
+// workspace: [rows, 2, vocab] words: the keys, then the probabilities.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
+    int* __restrict__ out, const float* __restrict__ logits, uint32_t* __restrict__ workspace, int vocab,
+    const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const float* __restrict__ min_p, const float* __restrict__ u) {
+    __shared__ float scratch[32];
+    __shared__ int s_counts[SAMPLE_THREADS];
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const int rowi = blockIdx.x;
+    const float* row = logits + (size_t)rowi * vocab;
+    float temp = temperature[rowi];
+    if (temp < 1e-5f) {
+        argmax_row(row, vocab, sv, si, out + rowi);
+        return;
+    }
+    uint32_t* keys = workspace + (size_t)rowi * 2 * vocab;
+    float* probs = (float*)(keys + vocab);
+
+    // temperature, softmax (sampler.rs:232-249)
+    float mx = -INFINITY;
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const float z = row[c] / temp;
+        keys[c] = order_key(z);
+        probs[c] = z;
+        mx = fmaxf(mx, z);
+    }
+    mx = wave_max(mx);
+    __syncthreads();
+    if ((threadIdx.x & (IA_WAVE - 1)) == 0) scratch[threadIdx.x / IA_WAVE] = mx;
+    __syncthreads();
+    for (int w = 0; w < SAMPLE_THREADS / IA_WAVE; ++w) mx = fmaxf(mx, scratch[w]);
+    float sum = 0.f;
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const float e = expf(probs[c] - mx);
+        probs[c] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, scratch);
+    if (sum > 0.f)
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) probs[c] /= sum;
+    __syncthreads();
+
+    // how long the kept prefix is (sampler.rs:256-283)
+    int keep = vocab;
+    const int k = top_k[rowi];
+    if (k > 0 && k < keep) keep = k;
+    const float tp = top_p[rowi];
+    if (tp < 1.0f) {
+        const Prefix p = shortest_prefix(keys, probs, vocab, tp, false, false, scratch);
+        const int n = p.above + p.take;
+        if (n < keep) keep = n;
+    }
+    const float mp = min_p[rowi];
+    if (mp > 0.0f) {
+        const float thr = (sum > 0.f ? 1.0f / sum : 1.0f) * mp;       // the largest probability is exp(0) / sum
+        float n = 0.f;
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) n += probs[c] >= thr ? 1.0f : 0.0f;
+        const int cnt = (int)block_sum(n, scratch);
+        if (cnt > 0 && cnt < keep) keep = cnt;
+    }
+
+    // the kept prefix by key and tie count, and its weight (sampler.rs:286-292)
+    Prefix kept;
+    float filtered;
+    if (keep < vocab) {
+        kept = shortest_prefix(keys, probs, vocab, (float)keep, true, false, scratch);
+        float wa = 0.f;
+        float pk = 0.f, seen = 0.f;
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+            if (keys[c] > kept.key) wa += probs[c];
+            else if (keys[c] == kept.key) { pk = probs[c]; seen = 1.f; }
+        }
+        wa = block_sum(wa, scratch);
+        __shared__ float s_pk2;
+        if (threadIdx.x == 0) s_pk2 = 0.f;
+        __syncthreads();
+        if (seen > 0.f) s_pk2 = pk;
+        __syncthreads();
+        filtered = wa + (float)kept.take * s_pk2;
+    } else {
+        kept.key = 0u; kept.above = 0; kept.ties = 0; kept.take = 0;
+        float t = 0.f;
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) t += probs[c];
+        filtered = block_sum(t, scratch);
+    }
+
+    // the walk (sampler.rs:323-335): the first place where the running sum of p / filtered exceeds u
+    int token;
+    if (!(filtered > 0.f)) {
+        argmax_row(row, vocab, sv, si, out + rowi);
+        return;
+    }
+    const Prefix hit = shortest_prefix(keys, probs, vocab, u[rowi] * filtered, false, true, scratch);
+    if (keep < vocab && (hit.ties == 0 || hit.above + hit.take > keep)) {
+        token = nth_with_key(keys, vocab, kept.key, kept.take, s_counts);          // the last kept token
+    } else if (hit.ties == 0) {
+        // u * filtered is not exceeded even by the whole list (rounding): the last of the list,
+        // that is the last token with the smallest key
+        uint32_t lowest = 0xffffffffu;
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) lowest = keys[c] < lowest ? keys[c] : lowest;
+#pragma unroll
+        for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
+            const uint32_t other = (uint32_t)__shfl_xor((int)lowest, o, IA_WAVE);
+            lowest = other < lowest ? other : lowest;
+        }
+        __syncthreads();
+        if ((threadIdx.x & (IA_WAVE - 1)) == 0) si[threadIdx.x / IA_WAVE] = (int)lowest;
+        __syncthreads();
+        for (int w = 0; w < SAMPLE_THREADS / IA_WAVE; ++w) lowest = (uint32_t)si[w] < lowest ? (uint32_t)si[w] : lowest;
+        float n = 0.f;
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) n += keys[c] == lowest ? 1.0f : 0.0f;
+        token = nth_with_key(keys, vocab, lowest, (int)block_sum(n, scratch), s_counts);
+    } else {
+        token = nth_with_key(keys, vocab, hit.key, hit.take, s_counts);
+    }
+    if (threadIdx.x == 0) out[rowi] = token;
+}
+
+extern "C" long long ia_sample_workspace(int rows, int vocab) { return (long long)rows * 2 * vocab; }
+
+extern "C" int ia_sample(int* out, const float* logits, void* workspace, int rows, int vocab,
+                         const float* temperature, const int* top_k, const float* top_p, const float* min_p,
+                         const float* u, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+    IA_CHECK(workspace != nullptr || rows == 0, "sample: needs a workspace of rows * 2 * vocab words");
+    if (rows == 0) return 0;
+    sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, (uint32_t*)workspace, vocab, temperature,
+                                                       top_k, top_p, min_p, u);
+    IA_LAUNCH_CHECK("sample");
     return 0;
 }

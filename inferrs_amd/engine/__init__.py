@@ -2,3 +2,5 @@ from .batch import GroupStep, StepContext
 from .model import DecoderModel, parse_dtype
 from .engine import Engine, Entry, StepError
 from .replay import TraceError, run_trace
+from .scheduler import Plan, PlannedEntry, Request, Scheduler
+from .generate import Generation, GenerationLoop, generate

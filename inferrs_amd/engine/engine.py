@@ -59,6 +59,8 @@ class Engine:
                            for g in probe.groups)
             free, _total = torch.cuda.mem_get_info(self.device)
             num_pages = max(1, int(free * memory_fraction) // max(per_page, 1))
+            # more than every request slot at the longest sequence is never used
+            num_pages = min(num_pages, max_seqs * -(-model.spec.max_position // page_size))
         self.cache = CacheManager(needs, page_size, num_pages, max_seqs)
         self.storage = CacheStorage(self.cache, model.dtype, self.device)
         self._stage_host: Optional[torch.Tensor] = None
@@ -91,6 +93,11 @@ class Engine:
         eng.config = config
         return eng
 
+    def generate(self, prompts, params=None, **loop_options):
+        """Token ids in, token ids out: see `inferrs_amd.engine.generate.generate`."""
+        from .generate import generate
+        return generate(self, prompts, params, **loop_options)
+
     # ---- requests ---------------------------------------------------------------------------
     def add_request(self, seq_id: Hashable) -> None:
         seq = self.cache.add_sequence(seq_id)
@@ -116,9 +123,11 @@ class Engine:
             self._stage_event.synchronize()      # the previous step's copy has left the host buffer
         return self._stage_host, self._stage_dev
 
-    def step(self, entries: Sequence[Entry]) -> torch.Tensor:
+    def step(self, entries: Sequence[Entry], commit: bool = True) -> torch.Tensor:
         """Run one batch; returns float32 logits `[wanted, vocab]` on the device, in the order
-        of the entries and of each entry's `want`."""
+        of the entries and of each entry's `want`.  Pages that the entries need beyond what is
+        reserved for them are reserved here.  With `commit` the requests' cached lengths advance;
+        a caller that passes False (the scheduler) does that itself."""
         if not entries:
             raise StepError("a step needs at least one entry")
         vocab = self.spec.vocab_size
@@ -153,8 +162,9 @@ class Engine:
 
         ctx = self._build_context(entries)
         logits = self.model.forward(ctx, self.storage)
-        for e in entries:
-            self.cache.commit(e.seq_id, len(e.tokens))
+        if commit:
+            for e in entries:
+                self.cache.commit(e.seq_id, len(e.tokens))
         return logits
 
     def _build_context(self, entries: Sequence[Entry]) -> StepContext:

@@ -1,0 +1,101 @@
+"""Generation: requests go through the scheduler, the step function and the sampler until
+they finish.  This is the loop behind `Engine.generate` and the command line; the reference's
+counterpart is `run_engine_loop` (`inferrs/src/engine.rs:1380-1912`)."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, Hashable, List, Optional, Sequence
+
+from ..sampling import Sampler, SamplingParams, fresh_seed
+from .engine import Engine, Entry
+from .scheduler import Plan, Request, Scheduler
+
+
+@dataclass
+class Generation:
+    request_id: Hashable
+    prompt: List[int]
+    tokens: List[int]
+    finish_reason: str
+    error: Optional[str] = None
+    preemptions: int = 0
+
+
+class GenerationLoop:
+    def __init__(self, engine: Engine, *, max_batch_size: int = 32, max_tokens_per_step: int = 2048,
+                 prefill_chunk: Optional[int] = None, max_seq_len: Optional[int] = None,
+                 stop_token_ids: Optional[Sequence[int]] = None):
+        self.engine = engine
+        limit = engine.spec.max_position if not max_seq_len else min(max_seq_len, engine.spec.max_position)
+        self.scheduler = Scheduler(
+            engine.cache, max_batch_size=min(max_batch_size, engine.cache.max_seqs),
+            max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk, max_seq_len=limit,
+            stop_token_ids=engine.spec.eos_token_ids if stop_token_ids is None else stop_token_ids)
+        self.sampler = Sampler(engine.device)
+        self.steps = 0
+        self._next_id = 0
+
+    def add(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+            request_id: Optional[Hashable] = None) -> Request:
+        params = params or SamplingParams()
+        if request_id is None:
+            request_id = f"req-{self._next_id}"
+            self._next_id += 1
+        vocab = self.engine.spec.vocab_size
+        if any((not isinstance(t, int)) or t < 0 or t >= vocab for t in prompt):
+            raise ValueError(f"request {request_id!r}: token ids must be integers in 0..{vocab - 1}")
+        seed = params.seed if params.seed is not None else fresh_seed()
+        req = Request(request_id, list(prompt), params, seed=seed)
+        self.scheduler.add(req)
+        return req
+
+    def step(self) -> List[Request]:
+        """One scheduler step; returns the requests that finished in it (failed ones included)."""
+        plan: Plan = self.scheduler.plan()
+        done = list(plan.failed)
+        if not plan.entries:
+            return done
+        for e in plan.entries:
+            if not self.engine.has_request(e.request.request_id):
+                raise RuntimeError(f"request {e.request.request_id!r} was planned without a cache entry")
+            if e.request.computed == 0:
+                self.engine.storage.clear_state_slot(self.engine.cache.sequences[e.request.request_id].state_slot)
+        entries = [Entry(e.request.request_id, e.tokens, [len(e.tokens) - 1] if e.samples else [])
+                   for e in plan.entries]
+        logits = self.engine.step(entries, commit=False)
+        drawing = [e.request for e in plan.entries if e.samples]
+        tokens = self.sampler.sample(logits, [r.params for r in drawing], [r.tokens for r in drawing],
+                                     [r.seed for r in drawing])
+        sampled: Dict[Hashable, int] = {r.request_id: t for r, t in zip(drawing, tokens)}
+        done += self.scheduler.commit(plan, sampled)
+        self.steps += 1
+        return done
+
+    def run(self, on_token: Optional[Callable[[Request, int], None]] = None) -> List[Request]:
+        """Steps until nothing is waiting or running; returns everything that finished."""
+        finished: List[Request] = []
+        emitted: Dict[Hashable, int] = {}
+        while self.scheduler.has_work():
+            live = list(self.scheduler.running) + list(self.scheduler.waiting)
+            done = self.step()
+            if on_token is not None:
+                for r in live:
+                    for t in r.output[emitted.get(r.request_id, 0):]:
+                        on_token(r, t)
+                    emitted[r.request_id] = len(r.output)
+            finished += done
+        return finished
+
+
+def generate(engine: Engine, prompts: Sequence[Sequence[int]], params=None, **loop_options) -> List[Generation]:
+    """Generates for every prompt (lists of token ids); `params` is one `SamplingParams` for all
+    or one per prompt.  Results come in the order of the prompts."""
+    loop = GenerationLoop(engine, **loop_options)
+    if params is None or isinstance(params, SamplingParams):
+        params = [params] * len(prompts)
+    if len(params) != len(prompts):
+        raise ValueError("one SamplingParams for all prompts, or one per prompt")
+    requests = [loop.add(p, sp, request_id=i) for i, (p, sp) in enumerate(zip(prompts, params))]
+    loop.run()
+    return [Generation(r.request_id, r.prompt, list(r.output), r.finish_reason or "error", r.error, r.preemptions)
+            for r in requests]

@@ -42,6 +42,8 @@ def library(target: str = "core") -> ctypes.CDLL:
         raise KernelError(f"{path}: unexpected ABI version {lib.ia_abi_version()}")
     if target.startswith("attn_d"):
         lib.ia_attention_mfma_workspace.restype = ctypes.c_longlong
+    else:
+        lib.ia_sample_workspace.restype = ctypes.c_longlong
     _LIBS[target], _LIB_PATHS[target] = lib, path
     return lib
 
@@ -371,4 +373,50 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     rows, vocab = logits.shape
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     _check(library().ia_argmax(_p(out), _p(logits), rows, vocab, _stream()))
+    return out
+
+
+def penalize(logits: torch.Tensor, window: Optional[torch.Tensor], repetition: torch.Tensor,
+             frequency: torch.Tensor, presence: torch.Tensor, bias_ids: Optional[torch.Tensor] = None,
+             bias_vals: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """In place on float32 logits [rows, vocab]: logit bias, then repetition, frequency and presence
+    penalties over each row's `window` of earlier tokens (int32 [rows, w], -1 = none)."""
+    _dev(logits, window, repetition, frequency, presence, bias_ids, bias_vals)
+    _f32(logits, "logits"); _f32(repetition, "repetition"); _f32(frequency, "frequency"); _f32(presence, "presence")
+    rows, vocab = logits.shape
+    w = 0 if window is None else window.shape[1]
+    nb = 0 if bias_ids is None else bias_ids.shape[1]
+    if window is not None:
+        _i32(window, "window")
+        if window.shape[0] != rows:
+            raise KernelError("penalize: one window row per row of logits")
+    if (bias_ids is None) != (bias_vals is None):
+        raise KernelError("penalize: bias ids and values come together")
+    if bias_ids is not None:
+        _i32(bias_ids, "bias_ids"); _f32(bias_vals, "bias_vals")
+        if bias_ids.shape != bias_vals.shape or bias_ids.shape[0] != rows:
+            raise KernelError("penalize: bias arrays must be [rows, entries]")
+    for t in (repetition, frequency, presence):
+        if t.numel() != rows:
+            raise KernelError("penalize: one penalty value per row of logits")
+    _check(library().ia_penalize(_p(logits), rows, vocab, _p(window), w, _p(repetition), _p(frequency),
+                                 _p(presence), _p(bias_ids), _p(bias_vals), nb, _stream()))
+    return logits
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    """One token per row of float32 logits: greedy where temperature < 1e-5, else temperature,
+    top-k, top-p, min-p and the walk to the row's random number u in [0, 1)."""
+    _dev(logits, temperature, top_k, top_p, min_p, u)
+    _f32(logits, "logits"); _f32(temperature, "temperature"); _f32(top_p, "top_p"); _f32(min_p, "min_p"); _f32(u, "u")
+    _i32(top_k, "top_k")
+    rows, vocab = logits.shape
+    for t in (temperature, top_k, top_p, min_p, u):
+        if t.numel() != rows:
+            raise KernelError("sample: one parameter value per row of logits")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    ws = torch.empty((library().ia_sample_workspace(rows, vocab),), dtype=torch.int32, device=logits.device)
+    _check(library().ia_sample(_p(out), _p(logits), _p(ws), rows, vocab, _p(temperature), _p(top_k), _p(top_p),
+                               _p(min_p), _p(u), _stream()))
     return out

@@ -1,0 +1,3 @@
+from .params import SAMPLING_EPS, SamplingParams
+from .rng import rand_f32, fresh_seed
+from .sampler import Sampler

@@ -1,0 +1,70 @@
+"""Turns rows of logits into tokens on the device, one row per request, in the reference's
+order of operations (`inferrs/src/sampler.rs:146-335`): logit bias, repetition, frequency and
+presence penalties over the last `repeat_last_n` tokens, temperature, softmax, top-k, top-p,
+min-p, and the walk to a random number that depends on the request's seed and step only."""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from .params import SAMPLING_EPS, SamplingParams
+from .rng import rand_f32
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = torch.device(device)
+
+    def _dev(self, array: np.ndarray) -> torch.Tensor:
+        return torch.from_numpy(array).to(self.device, non_blocking=False)
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], previous: Sequence[Sequence[int]],
+               seeds: Sequence[int]) -> List[int]:
+        """`logits` float32 [rows, vocab] on the device; row i belongs to a request with
+        `params[i]`, whose prompt and output so far are `previous[i]` and whose seed is `seeds[i]`."""
+        rows = logits.shape[0]
+        if not (len(params) == len(previous) == len(seeds) == rows):
+            raise ValueError("one parameter set, token history and seed per row of logits")
+        if rows == 0:
+            return []
+        if all(p.is_plain_greedy for p in params):
+            return ops.argmax(logits).cpu().tolist()
+
+        # penalties and bias, on a copy only if something is changed
+        width = max((min(p.repeat_last_n, len(prev)) if p.has_penalty else 0) for p, prev in zip(params, previous))
+        n_bias = max(len(p.logit_bias) for p in params)
+        if width or n_bias:
+            logits = logits.clone()
+            window = np.full((rows, max(width, 1)), -1, dtype=np.int32)
+            rep = np.ones(rows, dtype=np.float32)
+            freq = np.zeros(rows, dtype=np.float32)
+            pres = np.zeros(rows, dtype=np.float32)
+            for i, (p, prev) in enumerate(zip(params, previous)):
+                if p.has_penalty and prev:
+                    tail = list(prev[-p.repeat_last_n:])
+                    window[i, :len(tail)] = tail
+                    rep[i], freq[i], pres[i] = p.repetition_penalty, p.frequency_penalty, p.presence_penalty
+            bias_ids = bias_vals = None
+            if n_bias:
+                ids = np.full((rows, n_bias), -1, dtype=np.int32)
+                vals = np.zeros((rows, n_bias), dtype=np.float32)
+                for i, p in enumerate(params):
+                    for j, (tid, b) in enumerate(sorted(p.logit_bias.items())):
+                        ids[i, j], vals[i, j] = int(tid), float(b)
+                bias_ids, bias_vals = self._dev(ids), self._dev(vals)
+            ops.penalize(logits, self._dev(window) if width else None, self._dev(rep), self._dev(freq),
+                         self._dev(pres), bias_ids, bias_vals)
+
+        temperature = np.asarray([p.temperature for p in params], dtype=np.float32)
+        top_k = np.asarray([p.top_k for p in params], dtype=np.int32)
+        top_p = np.asarray([p.top_p for p in params], dtype=np.float32)
+        min_p = np.asarray([p.min_p for p in params], dtype=np.float32)
+        # the step of a draw is the number of tokens before it (`sampler.rs:323-325`)
+        u = np.asarray([rand_f32(seed, len(prev)) if p.temperature >= SAMPLING_EPS else 0.0
+                        for p, prev, seed in zip(params, previous, seeds)], dtype=np.float32)
+        out = ops.sample(logits, self._dev(temperature), self._dev(top_k), self._dev(top_p), self._dev(min_p),
+                         self._dev(u))
+        return out.cpu().tolist()

@@ -1,0 +1,137 @@
+"""Generation through the entry points: the Python one (`Engine.generate`), the scheduler under
+a tight pool, and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_model as pm
+from tiny_configs import TINY, random_tokens, write_model
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def tiny(tmp_path_factory):
+    out = {}
+    for name in ("A", "B"):
+        folder = write_model(str(tmp_path_factory.mktemp(f"gen_{name}")), TINY[name], seed=21)
+        out[name] = (folder, *pm.read_model(folder, torch.float64))
+    return out
+
+
+def plain_greedy_with_margins(cfg, params, prompt, n):
+    """Greedy continuation and, per step, the gap between the best and the second logit."""
+    toks, margins = list(prompt), []
+    for _ in range(n):
+        row = pm.forward(cfg, params, toks)[-1]
+        top = torch.topk(row, 2).values
+        margins.append(float(top[0] - top[1]))
+        toks.append(int(torch.argmax(row)))
+    return toks[len(prompt):], margins
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16")])
+def test_greedy_generation_matches_plain(tiny, name, dtype):
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny[name]
+    vocab = TINY[name]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 50 + n) for n in (5, 17, 33, 1)]       # BASELINE's tiny workload, and one token
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=4, num_pages=64, max_seqs=4)
+    outs = eng.generate(prompts, SamplingParams.greedy(max_tokens=16), max_tokens_per_step=24, prefill_chunk=16)
+    for prompt, out in zip(prompts, outs):
+        want, margins = plain_greedy_with_margins(cfg, params, prompt, 16)
+        assert out.finish_reason == "length" and len(out.tokens) == 16
+        if dtype == "float32":
+            assert out.tokens == want
+        else:
+            # bfloat16 may legitimately differ where two logits are closer than its rounding; up to there it agrees
+            for i, (g, w) in enumerate(zip(out.tokens, want)):
+                if g != w:
+                    assert margins[i] < 0.02, f"token {i}: {g} != {w} with a margin of {margins[i]:.3f}"
+                    break
+    eng.cache.check_invariants()
+    assert not eng.cache.sequences
+
+
+def test_seeded_temperature_is_reproducible_and_independent_of_the_batch(tiny):
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 70 + n) for n in (1, 9, 64, 100)]      # BASELINE's second tiny workload
+    sp = [SamplingParams(temperature=0.7, top_p=1.0, top_k=0, repetition_penalty=1.0, max_tokens=12, seed=40 + i)
+          for i in range(4)]
+    eng = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=64, max_seqs=4)
+    together = eng.generate(prompts, sp, prefill_chunk=16)
+    alone = [eng.generate([p], [s])[0] for p, s in zip(prompts, sp)]
+    assert [g.tokens for g in together] == [g.tokens for g in alone]
+    # and each token is what the plain sampler draws from the plain model's logits
+    toks = list(prompts[1])
+    for t in together[1].tokens:
+        row = pm.forward(cfg, params, toks)[-1].float()
+        assert t == pm.sample(row, toks, temperature=0.7, top_p=1.0, top_k=0, repetition_penalty=1.0, seed=41)
+        toks.append(t)
+
+
+def test_tight_pool_preempts_and_still_gives_the_same_tokens(tiny):
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 90 + n) for n in (20, 24, 28, 18)]
+    sp = SamplingParams.greedy(max_tokens=24)
+    roomy = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=256, max_seqs=4)
+    want = roomy.generate(prompts, sp)
+    tight = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=30, max_seqs=4)    # 120 slots for ~186 tokens
+    got = tight.generate(prompts, sp)
+    assert sum(g.preemptions for g in got) > 0 and sum(g.preemptions for g in want) == 0
+    assert [g.tokens for g in got] == [g.tokens for g in want]
+    assert all(g.finish_reason == "length" for g in got)
+    tight.cache.check_invariants()
+    too_small = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=5, max_seqs=4)
+    res = too_small.generate([prompts[0], prompts[0][:6]], SamplingParams.greedy(max_tokens=4))
+    assert res[0].finish_reason == "error" and "out of KV blocks" in res[0].error
+    assert res[1].finish_reason == "length" and len(res[1].tokens) == 4
+
+
+def test_stop_token_ends_generation(tiny):
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["A"]
+    prompt = random_tokens(9, TINY["A"]["vocab_size"], 5)
+    want, _ = plain_greedy_with_margins(cfg, params, prompt, 6)
+    eng = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=64, max_seqs=2)
+    out = eng.generate([prompt], SamplingParams.greedy(max_tokens=6, extra_stop_token_ids=(want[2],)))[0]
+    first = want.index(want[2])
+    assert out.tokens == want[:first + 1] and out.finish_reason == "stop"
+    out = eng.generate([prompt], SamplingParams.greedy(max_tokens=6, extra_stop_token_ids=(want[2],),
+                                                       bypass_stop_tokens=True))[0]
+    assert out.tokens == want and out.finish_reason == "length"
+
+
+def test_command_line_run_and_bench(tiny):
+    folder, cfg, params = tiny["A"]
+    prompt = random_tokens(7, TINY["A"]["vocab_size"], 3)
+    want, _ = plain_greedy_with_margins(cfg, params, prompt, 5)
+    exe = [sys.executable, os.path.join(ROOT, "bin", "inferrs-amd")]
+    proc = subprocess.run(exe + ["run", folder, ",".join(map(str, prompt)), "--dtype", "f32", "--temperature", "0",
+                                 "--repetition-penalty", "1.0", "--max-tokens", "5", "--block-size", "4",
+                                 "--max-blocks", "32", "--max-batch-size", "2"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == want
+    assert "finish: length" in proc.stderr
+    proc = subprocess.run(exe + ["bench", folder, "--dtype", "bf16", "--prompt-len", "32", "--max-tokens", "8",
+                                 "--runs", "2", "--max-blocks", "32", "--max-batch-size", "2"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert rec["prefill_tok_s"] > 0 and rec["decode_tok_s"] > 0
+    proc = subprocess.run(exe + ["serve", folder], capture_output=True, text=True, timeout=60)
+    assert proc.returncode == 2 and "not part of this engine" in proc.stderr

@@ -1,0 +1,106 @@
+"""The device sampler against the plain transcription of the reference's sampler
+(`tests/plain_model.py: sample`, from `inferrs/src/sampler.rs:146-335`), and the per-step random
+number against the same transcription bit for bit."""
+import math
+
+import pytest
+import torch
+
+import plain_model as pm
+
+from inferrs_amd.sampling import SamplingParams, rand_f32
+
+
+def test_rand_f32_is_the_reference_function():
+    for seed, step in [(0, 0), (1, 0), (42, 17), (2**63 + 5, 123456), (2**64 - 1, 2**40)]:
+        assert rand_f32(seed, step) == pm.rand_f32(seed, step)
+        assert 0.0 <= rand_f32(seed, step) <= 1.0
+    draws = [rand_f32(7, s) for s in range(2000)]
+    assert len(set(draws)) > 1990 and abs(sum(draws) / len(draws) - 0.5) < 0.03
+
+
+def _case(vocab, seed, scale=3.0):
+    g = torch.Generator().manual_seed(seed)
+    z = torch.randn(vocab, generator=g) * scale
+    prev = torch.randint(0, vocab, (90,), generator=g).tolist()
+    return z, prev
+
+
+PARAMS = [
+    dict(temperature=0.7, top_p=1.0, top_k=0, repetition_penalty=1.0),                 # plain tempered softmax
+    dict(),                                                                            # the reference's defaults
+    dict(temperature=1.3, top_p=0.5, top_k=0, repetition_penalty=1.0),
+    dict(temperature=1.0, top_p=1.0, top_k=5, repetition_penalty=1.3, repeat_last_n=16),
+    dict(temperature=0.9, top_p=0.95, top_k=40, min_p=0.2, frequency_penalty=0.4, presence_penalty=0.3),
+    dict(temperature=2.0, top_p=1.0, top_k=0, min_p=0.05, repetition_penalty=1.0),
+    dict(temperature=0.0, top_p=1.0, top_k=0, repetition_penalty=1.5),                 # greedy after penalties
+    dict(temperature=0.8, top_k=1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("vocab", [130, 387, 151936])
+@pytest.mark.parametrize("kw", PARAMS, ids=[str(i) for i in range(len(PARAMS))])
+def test_sampler_matches_the_plain_transcription(vocab, kw):
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    rows, params, prevs, seeds, zs = 6, [], [], [], []
+    for i in range(rows):
+        z, prev = _case(vocab, 100 * len(zs) + i + hash(str(kw)) % 1000)
+        zs.append(z)
+        prevs.append(prev[: 3 + 17 * i])
+        seeds.append(1000 + i)
+        params.append(SamplingParams(seed=seeds[-1], **kw))
+    logits = torch.stack(zs).to("cuda")
+    before = logits.clone()
+    got = sampler.sample(logits, params, prevs, seeds)
+    assert torch.equal(logits, before), "the sampler must not change the caller's logits"
+    for i in range(rows):
+        if vocab > 1000 and i > 1:
+            continue                                   # the plain sampler is slow at full vocabulary
+        want = pm.sample(zs[i], prevs[i], seed=seeds[i], **{**dict(temperature=0.7, top_p=0.9, top_k=50, min_p=0.0,
+                         repetition_penalty=1.1, repeat_last_n=64, frequency_penalty=0.0, presence_penalty=0.0), **kw})
+        assert got[i] == want, f"row {i}: device {got[i]}, plain {want}"
+
+
+@pytest.mark.gpu
+def test_mixed_rows_do_not_influence_each_other():
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    z0, p0 = _case(387, 1)
+    z1, p1 = _case(387, 2)
+    a = SamplingParams(temperature=0.9, top_k=20, seed=5)
+    b = SamplingParams.greedy()
+    alone = sampler.sample(z0[None].to("cuda"), [a], [p0], [5])[0]
+    both = sampler.sample(torch.stack([z1, z0]).to("cuda"), [b, a], [p1, p0], [0, 5])
+    assert both == [int(torch.argmax(z1)), alone]
+
+
+@pytest.mark.gpu
+def test_equal_logits_are_taken_in_index_order():
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    z = torch.zeros(1, 64)
+    z[0, 10:20] = 5.0                                   # ten equal favourites, the rest far below
+    for step in range(40):
+        p = SamplingParams(temperature=1.0, top_p=1.0, top_k=4, repetition_penalty=1.0, seed=3)
+        prev = [0] * step
+        got = sampler.sample(z.to("cuda"), [p], [prev], [3])[0]
+        want = pm.sample(z[0], prev, temperature=1.0, top_p=1.0, top_k=4, repetition_penalty=1.0, seed=3)
+        assert got == want and 10 <= got <= 13          # top-4 of ten equals: the first four by index
+
+
+@pytest.mark.gpu
+def test_frequencies_follow_the_tempered_softmax():
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    z = torch.tensor([2.0, 1.0, 0.0, -1.0, 0.5, 1.5, -3.0, 0.2])
+    temp = 0.7
+    probs = torch.softmax(z / temp, 0)
+    n = 4000
+    p = SamplingParams(temperature=temp, top_p=1.0, top_k=0, repetition_penalty=1.0, seed=11)
+    logits = z[None].repeat(n, 1).to("cuda")
+    got = sampler.sample(logits, [p] * n, [[0] * s for s in range(n)], [11] * n)
+    counts = torch.bincount(torch.tensor(got), minlength=8).float()
+    chi2 = float(((counts - n * probs) ** 2 / (n * probs)).sum())
+    assert chi2 < 24.3, f"chi-square {chi2:.1f} with 7 degrees of freedom (0.999 quantile is 24.3)"

@@ -1,0 +1,161 @@
+"""The scheduler's decisions, without a GPU: a stand-in executor commits what the scheduler
+planned and "samples" a function of the request alone."""
+import random
+
+import pytest
+
+from inferrs_amd.cache import CacheManager
+from inferrs_amd.engine.scheduler import OUT_OF_BLOCKS, Request, Scheduler
+from inferrs_amd.parts.base import PagedKV
+from inferrs_amd.sampling import SamplingParams
+
+
+def make(num_pages=64, page_size=4, max_seqs=8, **kw):
+    cache = CacheManager({0: PagedKV(2, 16)}, page_size=page_size, num_pages=num_pages, max_seqs=max_seqs)
+    kw.setdefault("max_batch_size", max_seqs)
+    return cache, Scheduler(cache, **kw)
+
+
+def token_for(r):
+    """What the stand-in model "generates": depends on the request and its length only."""
+    return (hash((r.request_id, r.total)) % 97) + 3
+
+
+def run(sched, cache, max_steps=10000, trace=None):
+    steps = 0
+    while sched.has_work():
+        plan = sched.plan()
+        assert plan.n_tokens <= sched.max_tokens_per_step
+        assert len({id(e.request) for e in plan.entries}) == len(plan.entries)
+        for e in plan.entries:
+            assert e.tokens == e.request.tokens[e.request.computed:e.request.computed + len(e.tokens)]
+            assert cache.sequences[e.request.request_id].reserved >= len(e.tokens)
+            assert e.samples == (e.request.computed + len(e.tokens) == e.request.total)
+        if trace is not None:
+            trace.append(plan)
+        sched.commit(plan, {e.request.request_id: token_for(e.request) for e in plan.entries if e.samples})
+        cache.check_invariants()
+        steps += 1
+        assert steps < max_steps, "the scheduler does not come to an end"
+    return steps
+
+
+def req(i, n_prompt, max_tokens=8, **kw):
+    return Request(i, list(range(1, n_prompt + 1)), SamplingParams.greedy(max_tokens=max_tokens, **kw))
+
+
+def test_decode_first_then_portions_under_the_budget():
+    cache, s = make(max_tokens_per_step=16, prefill_chunk=8)
+    a, b = req("a", 5, 4), req("b", 30, 4)
+    s.add(a); s.add(b)
+    trace = []
+    run(s, cache, trace=trace)
+    first = trace[0]
+    assert [(e.request.request_id, len(e.tokens), e.samples) for e in first.entries] == [("a", 5, True), ("b", 8, False)]
+    second = trace[1]       # a decodes first (1 token), b's next portion takes up to the chunk
+    assert [(e.request.request_id, len(e.tokens)) for e in second.entries] == [("a", 1), ("b", 8)]
+    assert a.finish_reason == b.finish_reason == "length" and len(a.output) == len(b.output) == 4
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
+def test_stop_tokens_length_and_context_limit():
+    cache, s = make(stop_token_ids=[50], max_seq_len=12)
+    a = req("a", 4, 100)
+    s.add(a)
+    plan = s.plan()
+    s.commit(plan, {"a": 50})
+    assert a.finish_reason == "stop" and a.output == [50]
+    b = req("b", 4, 100, bypass_stop_tokens=True)       # like the reference's bench: stop tokens bypassed
+    s.add(b)
+    while s.has_work():
+        plan = s.plan()
+        s.commit(plan, {"b": 50})
+    assert b.finish_reason == "length" and b.total == 12           # the context limit
+    c = Request("c", [1, 2], SamplingParams.greedy(max_tokens=9, extra_stop_token_ids=(7,)))
+    s.add(c)
+    s.commit(s.plan(), {"c": 7})
+    assert c.finish_reason == "stop"
+    with pytest.raises(ValueError, match="limit"):
+        s.add(req("d", 12))
+    with pytest.raises(ValueError, match="empty"):
+        s.add(Request("e", [], SamplingParams()))
+
+
+def test_admission_stops_at_max_batch_size_and_keeps_arrival_order():
+    cache, s = make(max_batch_size=2)
+    for i in range(4):
+        s.add(req(i, 3, 2))
+    plan = s.plan()
+    assert [e.request.request_id for e in plan.entries] == [0, 1] and len(s.waiting) == 2
+    s.commit(plan, {0: 5, 1: 5})
+    plan = s.plan()
+    assert [e.request.request_id for e in plan.entries] == [0, 1]
+    s.commit(plan, {0: 5, 1: 5})                    # both reach max_tokens and leave
+    assert [e.request.request_id for e in s.plan().entries] == [2, 3]
+
+
+def test_pages_run_out_the_latest_request_is_preempted_and_recomputed():
+    # 6 pages of 4 tokens.  a (8 tokens) and b (8 tokens) fill 4; both decode; when b needs the
+    # 7th page there is none: b, the latest, goes back to the head of the line.
+    cache, s = make(num_pages=6, page_size=4, max_tokens_per_step=64)
+    a, b = req("a", 8, 12), req("b", 8, 12)
+    s.add(a); s.add(b)
+    trace = []
+    run(s, cache, trace=trace)
+    preempted = [r.request_id for p in trace for r in p.preempted]
+    assert preempted and set(preempted) == {"b"} and b.preemptions >= 1 and a.preemptions == 0
+    assert a.finish_reason == b.finish_reason == "length" and len(a.output) == len(b.output) == 12
+    # recomputation feeds prompt and output so far again, and the result is what an undisturbed run gives
+    cache2, s2 = make(num_pages=64, page_size=4)
+    b2 = req("b", 8, 12)
+    s2.add(b2)
+    run(s2, cache2)
+    assert b2.output == b.output and b2.preemptions == 0
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
+def test_a_request_that_can_never_fit_fails_with_the_reference_error():
+    cache, s = make(num_pages=3, page_size=4)
+    big, small = req("big", 12, 4), req("small", 3, 2)
+    s.add(big); s.add(small)
+    run(s, cache)
+    assert big.finish_reason == "error" and OUT_OF_BLOCKS in big.error
+    assert small.finish_reason == "length"
+    # one that fits at first and outgrows the whole pool fails when it does
+    cache, s = make(num_pages=3, page_size=4)
+    grow = req("grow", 10, 10)
+    s.add(grow)
+    run(s, cache)
+    assert grow.finish_reason == "error" and OUT_OF_BLOCKS in grow.error and len(grow.output) == 3
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_every_request_finishes_whatever_the_order_and_the_pool(seed):
+    rng = random.Random(seed)
+    page = rng.choice([1, 4, 16])
+    cache, s = make(num_pages=rng.randint(40, 120) // page + 8, page_size=page, max_seqs=6,
+                    max_batch_size=rng.randint(1, 6), max_tokens_per_step=rng.choice([4, 16, 64]),
+                    prefill_chunk=rng.choice([None, 3, 16]))
+    reqs = [req(i, rng.randint(1, 30), rng.randint(1, 12)) for i in range(25)]
+    pending = list(reqs)
+    steps = 0
+    while pending or s.has_work():
+        for _ in range(rng.randint(0, 3)):
+            if pending:
+                s.add(pending.pop(0))
+        if s.has_work():
+            plan = s.plan()
+            assert plan.n_tokens <= s.max_tokens_per_step and len(s.running) <= s.max_batch_size
+            s.commit(plan, {e.request.request_id: token_for(e.request) for e in plan.entries if e.samples})
+            cache.check_invariants()
+        steps += 1
+        assert steps < 20000
+    for r in reqs:
+        assert r.finish_reason == "length" and len(r.output) == r.params.max_tokens, (r.request_id, r.finish_reason, r.error)
+        # outputs do not depend on interleaving or preemption: each token is a function of the request alone
+        alone = Request(r.request_id, list(r.prompt), r.params)
+        while len(alone.output) < r.params.max_tokens:
+            alone.output.append(token_for(alone))
+        assert alone.output == r.output
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups) and cache.slots.num_free == 6
