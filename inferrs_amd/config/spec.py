@@ -89,17 +89,15 @@ class LayerSpec:
 
 @dataclass(frozen=True)
 class ScheduleEntry:
-    """One stop in the run order: run `layer`; its mixer uses the cache of `cache_of`.
+    """One stop in the run order: run `layer` (its weights); its mixer uses a cache.
 
-    `cache_of == layer` (the default) means the layer owns and writes its cache.
-    Another index means it only reads that layer's cache and writes none.
+    By default a stop owns a cache of its own and writes it, so a layer that is named at two
+    stops keeps two caches and a request's results do not depend on how its tokens were cut
+    into steps.  `cache_of = j` (an earlier stop's index in the schedule) makes this stop
+    read stop j's cache and write none.
     """
     layer: int
     cache_of: Optional[int] = None
-
-    @property
-    def cache_owner(self) -> int:
-        return self.layer if self.cache_of is None else self.cache_of
 
 
 @dataclass(frozen=True)
@@ -121,15 +119,21 @@ class ModelSpec:
         n = len(self.layers)
         if n == 0:
             raise SpecError("a model needs at least one layer")
-        for e in self.schedule:
-            if not (0 <= e.layer < n) or not (0 <= e.cache_owner < n):
-                raise SpecError(f"schedule entry {e} names a layer outside 0..{n - 1}")
-        owners = {e.layer for e in self.schedule if e.cache_of in (None, e.layer)}
-        for e in self.schedule:
-            if e.cache_owner not in owners:
-                raise SpecError(
-                    f"schedule entry {e} reads the cache of layer {e.cache_owner}, "
-                    "which never runs as the owner of its cache")
+        if not self.schedule:
+            raise SpecError("the schedule is empty")
+        for i, e in enumerate(self.schedule):
+            if not (0 <= e.layer < n):
+                raise SpecError(f"schedule stop {i} names layer {e.layer}, outside 0..{n - 1}")
+            if e.cache_of is not None:
+                if not (0 <= e.cache_of < i):
+                    raise SpecError(f"schedule stop {i} reads the cache of stop {e.cache_of}, which is not an earlier stop")
+                if self.schedule[e.cache_of].cache_of is not None:
+                    raise SpecError(f"schedule stop {i} reads the cache of stop {e.cache_of}, which owns none")
+
+    def cache_stop(self, stop: int) -> int:
+        """The schedule stop whose cache stop `stop` uses (itself unless it reads another's)."""
+        e = self.schedule[stop]
+        return stop if e.cache_of is None else e.cache_of
 
 
 def default_schedule(n_layers: int) -> Tuple[ScheduleEntry, ...]:

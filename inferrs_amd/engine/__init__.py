@@ -1,4 +1,4 @@
-from .batch import GroupStep, StepContext
+from .batch import GroupStep, StepBuilder, StepContext
 from .model import DecoderModel, parse_dtype
 from .engine import Engine, Entry, StepError
 from .replay import TraceError, run_trace

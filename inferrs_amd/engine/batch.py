@@ -9,9 +9,12 @@ its cached length, and no mask is built: kernels derive causality from `position
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
+
+from ..cache.manager import RELEASED, CacheManager
 
 
 @dataclass
@@ -52,3 +55,85 @@ class StepContext:
         if key not in self._tables:
             self._tables[key] = position_part.table(self.positions)
         return self._tables[key]
+
+
+class StepError(ValueError):
+    pass
+
+
+class StepBuilder:
+    """Turns (request, its next tokens, wanted places) into a `StepContext`: everything the
+    kernels need goes to the device in one copy from a pinned staging buffer."""
+
+    def __init__(self, cache: CacheManager, device):
+        self.cache = cache
+        self.device = torch.device(device)
+        self._host: Optional[torch.Tensor] = None
+        self._dev: Optional[torch.Tensor] = None
+        self._event: Optional[torch.cuda.Event] = None
+
+    def _staging(self, n: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        if self._host is None or self._host.numel() < n:
+            size = 1 << max(12, (n - 1).bit_length())
+            self._host = torch.empty(size, dtype=torch.int32, pin_memory=True)
+            self._dev = torch.empty(size, dtype=torch.int32, device=self.device)
+            self._event = None
+        if self._event is not None:
+            self._event.synchronize()      # the previous step's copy has left the host buffer
+        return self._host, self._dev
+
+    def build(self, entries: Sequence[Tuple[Hashable, Sequence[int], Sequence[int]]]) -> StepContext:
+        """`entries`: (request, tokens, want).  The requests are live and hold pages for the
+        positions `length .. length + len(tokens)`."""
+        ps = self.cache.page_size
+        seqs = [self.cache.sequences[e[0]] for e in entries]
+        q_lens = [len(e[1]) for e in entries]
+        starts = [s.length for s in seqs]
+        n, s_count = sum(q_lens), len(entries)
+        n_groups = len(self.cache.groups)
+        max_pages = max(1, max(-(-(st + q) // ps) for st, q in zip(starts, q_lens)))
+        cu = np.zeros(s_count + 1, dtype=np.int64)
+        np.cumsum(q_lens, out=cu[1:])
+        token_ids = np.concatenate([np.asarray(e[1], dtype=np.int32) for e in entries])
+        positions = np.concatenate([np.arange(st, st + q, dtype=np.int32) for st, q in zip(starts, q_lens)])
+        token_seq = np.repeat(np.arange(s_count, dtype=np.int32), q_lens)
+        want = np.asarray([cu[i] + w for i, e in enumerate(entries) for w in e[2]], dtype=np.int32)
+        state_slots = np.asarray([s.state_slot for s in seqs], dtype=np.int32)
+        tables, slots = [], []
+        for g in range(n_groups):
+            bt = np.zeros((s_count, max_pages), dtype=np.int32)
+            for i, s in enumerate(seqs):
+                row = s.tables[g][:max_pages]
+                if len(row) * ps < starts[i] + q_lens[i]:
+                    raise StepError(f"request {s.seq_id!r} holds {len(row)} pages, too few for "
+                                    f"{starts[i] + q_lens[i]} tokens")
+                bt[i, :len(row)] = row
+            pages_of_token = bt[token_seq, positions // ps]
+            if n and (pages_of_token == RELEASED).any():
+                raise StepError("a new token falls into a page that was already released")
+            slots.append((pages_of_token * ps + positions % ps).astype(np.int32))
+            np.maximum(bt, 0, out=bt)                 # released pages are never read
+            tables.append(bt)
+
+        parts = [token_ids, positions, token_seq, cu.astype(np.int32), state_slots, want]
+        for g in range(n_groups):
+            parts += [slots[g], tables[g].reshape(-1)]
+        sizes = [p.size for p in parts]
+        total = sum(sizes)
+        host, dev = self._staging(max(total, 1))
+        flat = host.numpy()
+        off, views = 0, []
+        for p, sz in zip(parts, sizes):
+            flat[off:off + sz] = p
+            views.append(dev[off:off + sz])
+            off += sz
+        dev[:total].copy_(host[:total], non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record()
+        groups = [GroupStep(ps, views[6 + 2 * g], views[7 + 2 * g].view(s_count, max_pages))
+                  for g in range(n_groups)]
+        return StepContext(
+            n_tokens=n, n_seqs=s_count, token_ids=views[0], positions=views[1], token_seq=views[2],
+            cu_tokens=views[3], state_slots=views[4], want_rows=views[5], groups=groups,
+            q_lens=q_lens, kv_starts=starts, state_slots_host=[int(x) for x in state_slots],
+            max_q_len=max(q_lens), max_kv_len=max(st + q for st, q in zip(starts, q_lens)))

@@ -12,21 +12,16 @@ from __future__ import annotations
 
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
-import numpy as np
 import torch
 
 from .. import ops
-from ..cache import RELEASED, CacheManager, CacheStorage, OutOfPages
+from ..cache import CacheManager, CacheStorage, OutOfPages
 from ..config.registry import load_config
 from ..parts.assemble import model_tensors
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
-from .batch import GroupStep, StepContext
+from .batch import StepBuilder, StepError
 from .model import DecoderModel, parse_dtype
-
-
-class StepError(ValueError):
-    pass
 
 
 class Entry:
@@ -63,9 +58,7 @@ class Engine:
             num_pages = min(num_pages, max_seqs * -(-model.spec.max_position // page_size))
         self.cache = CacheManager(needs, page_size, num_pages, max_seqs)
         self.storage = CacheStorage(self.cache, model.dtype, self.device)
-        self._stage_host: Optional[torch.Tensor] = None
-        self._stage_dev: Optional[torch.Tensor] = None
-        self._stage_event: Optional[torch.cuda.Event] = None
+        self.builder = StepBuilder(self.cache, self.device)
 
     # ---- construction -----------------------------------------------------------------------
     @classmethod
@@ -113,16 +106,6 @@ class Engine:
         return self.cache.sequences[seq_id].length
 
     # ---- the step ---------------------------------------------------------------------------
-    def _staging(self, n: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        if self._stage_host is None or self._stage_host.numel() < n:
-            size = 1 << max(12, (n - 1).bit_length())
-            self._stage_host = torch.empty(size, dtype=torch.int32, pin_memory=True)
-            self._stage_dev = torch.empty(size, dtype=torch.int32, device=self.device)
-            self._stage_event = None
-        if self._stage_event is not None:
-            self._stage_event.synchronize()      # the previous step's copy has left the host buffer
-        return self._stage_host, self._stage_dev
-
     def step(self, entries: Sequence[Entry], commit: bool = True) -> torch.Tensor:
         """Run one batch; returns float32 logits `[wanted, vocab]` on the device, in the order
         of the entries and of each entry's `want`.  Pages that the entries need beyond what is
@@ -160,60 +143,9 @@ class Engine:
                     self.cache.free_sequence(sid)
             raise
 
-        ctx = self._build_context(entries)
+        ctx = self.builder.build([(e.seq_id, e.tokens, e.want) for e in entries])
         logits = self.model.forward(ctx, self.storage)
         if commit:
             for e in entries:
                 self.cache.commit(e.seq_id, len(e.tokens))
         return logits
-
-    def _build_context(self, entries: Sequence[Entry]) -> StepContext:
-        ps = self.page_size
-        seqs = [self.cache.sequences[e.seq_id] for e in entries]
-        q_lens = [len(e.tokens) for e in entries]
-        starts = [s.length for s in seqs]
-        n, s_count = sum(q_lens), len(entries)
-        n_groups = len(self.cache.groups)
-        max_pages = max(1, max(-(-(st + q) // ps) for st, q in zip(starts, q_lens)))
-        cu = np.zeros(s_count + 1, dtype=np.int64)
-        np.cumsum(q_lens, out=cu[1:])
-        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
-        positions = np.concatenate([np.arange(st, st + q, dtype=np.int32) for st, q in zip(starts, q_lens)])
-        token_seq = np.repeat(np.arange(s_count, dtype=np.int32), q_lens)
-        want = np.asarray([cu[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
-        state_slots = np.asarray([s.state_slot for s in seqs], dtype=np.int32)
-        tables, slots = [], []
-        for g in range(n_groups):
-            bt = np.zeros((s_count, max_pages), dtype=np.int32)
-            for i, s in enumerate(seqs):
-                row = s.tables[g][:max_pages]
-                bt[i, :len(row)] = row
-            pages_of_token = bt[token_seq, positions // ps]
-            if n and (pages_of_token == RELEASED).any():
-                raise StepError("a new token falls into a page that was already released")
-            slots.append((pages_of_token * ps + positions % ps).astype(np.int32))
-            np.maximum(bt, 0, out=bt)                 # released pages are never read
-            tables.append(bt)
-
-        parts = [token_ids, positions, token_seq, cu.astype(np.int32), state_slots, want]
-        for g in range(n_groups):
-            parts += [slots[g], tables[g].reshape(-1)]
-        sizes = [p.size for p in parts]
-        total = sum(sizes)
-        host, dev = self._staging(max(total, 1))
-        flat = host.numpy()
-        off, views = 0, []
-        for p, sz in zip(parts, sizes):
-            flat[off:off + sz] = p
-            views.append(dev[off:off + sz])
-            off += sz
-        dev[:total].copy_(host[:total], non_blocking=True)
-        self._stage_event = torch.cuda.Event()
-        self._stage_event.record()
-        groups = [GroupStep(ps, views[6 + 2 * g], views[7 + 2 * g].view(s_count, max_pages))
-                  for g in range(n_groups)]
-        return StepContext(
-            n_tokens=n, n_seqs=s_count, token_ids=views[0], positions=views[1], token_seq=views[2],
-            cu_tokens=views[3], state_slots=views[4], want_rows=views[5], groups=groups,
-            q_lens=q_lens, kv_starts=starts, state_slots_host=[int(x) for x in state_slots],
-            max_q_len=max(q_lens), max_kv_len=max(st + q for st, q in zip(starts, q_lens)))

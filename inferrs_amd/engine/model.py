@@ -56,22 +56,22 @@ class DecoderModel:
             spec.final_norm, {"weight": tensors.pop(spec.final_norm_name)}, dtype, device)
 
     def cache_needs(self) -> Dict[int, object]:
-        """Cache-owning layer -> what its mixer keeps per request."""
+        """Schedule stop that owns a cache -> what its mixer keeps per request."""
         needs: Dict[int, object] = {}
-        for e in self.spec.schedule:
-            if e.cache_owner == e.layer:
+        for stop, e in enumerate(self.spec.schedule):
+            if e.cache_of is None:
                 mixer = self.spec.layers[e.layer].mixer
-                needs[e.layer] = part_class("mixer", mixer).cache_need(mixer)
+                needs[stop] = part_class("mixer", mixer).cache_need(mixer)
         return needs
 
     def forward(self, ctx: StepContext, storage) -> torch.Tensor:
-        """Runs the step's tokens through every scheduled layer (which appends to the caches)
-        and returns float32 logits `[n_want, vocab]`."""
+        """Runs the step's tokens through every stop of the schedule (which appends to the
+        caches) and returns float32 logits `[n_want, vocab]`."""
         x = ops.embed_gather(self.embed, ctx.token_ids)
         pending: Optional[torch.Tensor] = None
-        for e in self.spec.schedule:
-            cache = storage.layers.get(e.cache_owner)
-            if cache is not None and e.cache_owner != e.layer:
+        for stop, e in enumerate(self.spec.schedule):
+            cache = storage.layers.get(self.spec.cache_stop(stop))
+            if cache is not None and e.cache_of is not None:
                 cache = cache.reader()
             x, pending = self.blocks[e.layer].forward(ctx, x, pending, cache)
         n_want = ctx.want_rows.numel()

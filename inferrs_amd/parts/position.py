@@ -13,11 +13,14 @@ from .base import Position, register_position
 
 
 def inverse_frequencies(theta: float, rot_dim: int) -> np.ndarray:
-    """1 / theta**(2i/rot_dim) for i in 0..rot_dim/2, every step in 32-bit as the reference's
-    `powf` on f32 operands (`attention_utils.rs:198-203`)."""
+    """1 / theta**(2i/rot_dim) for i in 0..rot_dim/2 as the reference computes it
+    (`attention_utils.rs:198-203`): the exponent, the power and the quotient are 32-bit
+    operations.  The power is taken in 64-bit and rounded once, which is what a correctly
+    rounded `powf` returns."""
     i = np.arange(rot_dim // 2, dtype=np.float32)
     exponent = (np.float32(2.0) * i) / np.float32(rot_dim)
-    return (np.float32(1.0) / np.power(np.float32(theta), exponent, dtype=np.float32)).astype(np.float32)
+    power = np.power(np.float64(np.float32(theta)), exponent.astype(np.float64)).astype(np.float32)
+    return (np.float32(1.0) / power).astype(np.float32)
 
 
 @register_position("rope")

@@ -25,12 +25,14 @@ def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def inv_freq(theta: float, rot_dim: int) -> torch.Tensor:
-    """1 / theta^(2i/rot_dim), i in [0, rot_dim/2), in float32 powf.
+    """1 / theta^(2i/rot_dim), i in [0, rot_dim/2), every operation on float32 values with a
+    correctly rounded powf (the power is taken in float64 and rounded once).
     inferrs-models/src/models/attention_utils.rs:198-203."""
     out = []
+    base = torch.tensor(theta, dtype=torch.float32).double()
     for i in range(rot_dim // 2):
         exp = torch.tensor(2.0 * i, dtype=torch.float32) / torch.tensor(float(rot_dim), dtype=torch.float32)
-        out.append(1.0 / torch.pow(torch.tensor(theta, dtype=torch.float32), exp))
+        out.append(torch.tensor(1.0, dtype=torch.float32) / torch.pow(base, exp.double()).float())
     return torch.stack(out)
 
 

@@ -1,0 +1,336 @@
+"""Each part of a layer alone against its plain formula, and the generality of the assembly:
+a toy mixer with state of its own, a layer that reads another layer's cache, and a layer that
+runs twice, registered and built from a test without a change to the framework's files."""
+import io
+import os
+from dataclasses import dataclass
+from typing import Any, Dict, Tuple
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+import trace_modes as tm
+from tiny_configs import TINY_B, random_tokens
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
+
+
+def rel_err(got, want):
+    got, want = got.detach().float().cpu().double(), want.double()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-9))
+
+
+TOL = {torch.float32: 2e-6, torch.bfloat16: 2 ** -7}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from inferrs_amd.config import NormSpec
+    from inferrs_amd.parts import part_class
+    spec = NormSpec(size=96, eps=1e-5)
+    w = rnd(96, seed=1) * 0.1 + 1
+    norm = part_class("norm", spec)(spec, {"weight": w.to(torch.bfloat16)}, dtype, DEV)
+    x, d = rnd(9, 96, seed=2, dtype=dtype), rnd(9, 96, seed=3, dtype=dtype)
+    wq = w.to(torch.bfloat16).double()
+    assert rel_err(norm.forward(x.to(DEV)), pm.rms_norm(x.double(), wq, 1e-5)) < TOL[dtype]
+    xs = x.to(DEV)
+    out = norm.add_forward(xs, d.to(DEV))
+    summed = (x.float() + d.float()).to(dtype)
+    assert torch.equal(xs.cpu(), summed)
+    assert rel_err(out, pm.rms_norm(summed.double(), wq, 1e-5)) < TOL[dtype]
+    # the other convention of storing the weight (w - 1) is a parameter of the part, not another part
+    plus = part_class("norm", spec)(NormSpec(size=96, eps=1e-5, add_one=True), {"weight": w - 1}, dtype, DEV)
+    assert rel_err(plus.forward(x.to(DEV)), pm.rms_norm(x.double(), w.double(), 1e-5)) < 2 * TOL[dtype]
+
+
+def test_position_part():
+    from inferrs_amd.config import PositionSpec
+    from inferrs_amd.parts import part_class
+    spec = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e6)
+    rope = part_class("position", spec)(spec, {}, torch.float32, DEV)
+    assert torch.equal(rope.inv_freq.cpu(), pm.inv_freq(1e6, 32))
+    pos = torch.tensor([0, 3, 999, 12345], dtype=torch.int32)
+    cos, sin = rope.table(pos.to(DEV))
+    want_cos, want_sin = pm.rope_tables(pos, 1e6, 32)
+    assert float((cos.cpu() - want_cos).abs().max()) < 2e-6 and float((sin.cpu() - want_sin).abs().max()) < 2e-6
+    none = part_class("position", PositionSpec(kind="none"))(PositionSpec(kind="none"), {}, torch.float32, DEV)
+    assert none.table(pos.to(DEV)) is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from inferrs_amd.config import GatedMlpSpec
+    from inferrs_amd.parts import part_class
+    spec = GatedMlpSpec(hidden=72, intermediate=200)
+    t = {"gate_proj.weight": rnd(200, 72, seed=1, scale=0.1, dtype=torch.bfloat16),
+         "up_proj.weight": rnd(200, 72, seed=2, scale=0.1, dtype=torch.bfloat16),
+         "down_proj.weight": rnd(72, 200, seed=3, scale=0.1, dtype=torch.bfloat16)}
+    ffn = part_class("ffn", spec)(spec, dict(t), dtype, DEV)
+    x = rnd(11, 72, seed=4, dtype=dtype)
+    want = pm.mlp(x.double(), t["gate_proj.weight"].double(), t["up_proj.weight"].double(), t["down_proj.weight"].double())
+    assert rel_err(ffn.forward(None, x.to(DEV)), want) < 2 * TOL[dtype]
+
+
+def attention_setup(dtype, page_size, spec, tensors, requests):
+    """A cache of its own for one attention part, and the step contexts to run `requests`
+    (name -> (tokens' hidden rows, cut points)) through it."""
+    from inferrs_amd.cache import CacheManager, CacheStorage
+    from inferrs_amd.engine import StepBuilder
+    from inferrs_amd.parts import part_class
+    cls = part_class("mixer", spec)
+    manager = CacheManager({0: cls.cache_need(spec)}, page_size, 64, 4)
+    storage = CacheStorage(manager, dtype, DEV)
+    return cls(spec, dict(tensors), dtype, DEV), manager, storage, StepBuilder(manager, DEV)
+
+
+@pytest.mark.parametrize("dtype,page", [(torch.float32, 4), (torch.bfloat16, 16), (torch.bfloat16, 8)])
+def test_attention_part(dtype, page):
+    """The mixer alone, over its own cache, in two steps (a portion, then the rest beside a
+    second request), against the plain attention layer on the whole sequences."""
+    from inferrs_amd.config import AttentionSpec, NormSpec, PositionSpec
+    cfg = dict(num_attention_heads=6, num_key_value_heads=3, head_dim=32, rms_norm_eps=1e-5)
+    hidden = 96
+    spec = AttentionSpec(hidden=hidden, n_heads=6, n_kv_heads=3, head_dim=32,
+                         position=PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4),
+                         qk_norm=NormSpec(size=32, eps=1e-5))
+    t = {"q_proj.weight": rnd(192, hidden, seed=1, scale=0.1, dtype=torch.bfloat16),
+         "k_proj.weight": rnd(96, hidden, seed=2, scale=0.1, dtype=torch.bfloat16),
+         "v_proj.weight": rnd(96, hidden, seed=3, scale=0.1, dtype=torch.bfloat16),
+         "o_proj.weight": rnd(hidden, 192, seed=4, scale=0.1, dtype=torch.bfloat16),
+         "q_norm.weight": (rnd(32, seed=5) * 0.1 + 1).to(torch.bfloat16),
+         "k_norm.weight": (rnd(32, seed=6) * 0.1 + 1).to(torch.bfloat16)}
+    attn, manager, storage, builder = attention_setup(dtype, page, spec, t, None)
+    ha, hb = rnd(37, hidden, seed=7, dtype=dtype), rnd(5, hidden, seed=8, dtype=dtype)
+    outs = {"a": [], "b": []}
+    for step in ([("a", ha[:20])], [("a", ha[20:]), ("b", hb)]):
+        for name, rows in step:
+            if name not in manager.sequences:
+                manager.add_sequence(name)
+            assert manager.reserve(name, rows.shape[0])
+        ctx = builder.build([(name, [0] * rows.shape[0], []) for name, rows in step])
+        y = attn.forward(ctx, torch.cat([rows for _, rows in step]).to(DEV), storage.layers[0])
+        off = 0
+        for name, rows in step:
+            outs[name].append(y[off:off + rows.shape[0]].cpu())
+            off += rows.shape[0]
+            manager.commit(name, rows.shape[0])
+    p = {"x." + k: v.double() for k, v in t.items()}
+    for name, h in (("a", ha), ("b", hb)):
+        cos, sin = pm.rope_tables(torch.arange(h.shape[0]), 1e4, 32)
+        want = pm.attention_layer(h.double(), p, "x.", cfg, cos.double(), sin.double())
+        assert rel_err(torch.cat(outs[name]), want) < 4 * TOL[dtype], name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_part_without_norm_or_rotation_is_plain_attention(dtype):
+    """With no per-head norm and no position encoding the mixer reduces to a library routine."""
+    from inferrs_amd.config import AttentionSpec, PositionSpec
+    hidden, nq, nkv, d = 64, 4, 4, 16
+    spec = AttentionSpec(hidden=hidden, n_heads=nq, n_kv_heads=nkv, head_dim=d, position=PositionSpec(kind="none"))
+    eye = torch.eye(hidden, dtype=torch.bfloat16)
+    t = {"q_proj.weight": eye, "k_proj.weight": eye, "v_proj.weight": eye, "o_proj.weight": eye}
+    attn, manager, storage, builder = attention_setup(dtype, 16, spec, t, None)
+    h = rnd(50, hidden, seed=9, dtype=dtype)
+    manager.add_sequence("a")
+    manager.reserve("a", 50)
+    y = attn.forward(builder.build([("a", [0] * 50, [])]), h.to(DEV), storage.layers[0])
+    q = h.double().view(50, nq, d).transpose(0, 1)
+    want = torch.nn.functional.scaled_dot_product_attention(q, q, q, is_causal=True).transpose(0, 1).reshape(50, hidden)
+    assert rel_err(y, want) < 4 * TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_alone(dtype, tmp_path):
+    """One block built from a layer spec equals the plain decoder layer."""
+    from inferrs_amd.cache import CacheManager, CacheStorage
+    from inferrs_amd.config import Qwen3Config
+    from inferrs_amd.engine import StepBuilder
+    from inferrs_amd.parts import Block, layer_tensors, part_class
+    from inferrs_amd.weights import random_tensors
+    cfg = Qwen3Config.from_dict(TINY_B)
+    layer = cfg.to_spec().layers[1]
+    tensors = random_tensors(layer_tensors(layer), 3, torch.bfloat16)
+    block = Block(layer, dict(tensors), dtype, DEV)
+    manager = CacheManager({0: part_class("mixer", layer.mixer).cache_need(layer.mixer)}, 16, 8, 2)
+    storage = CacheStorage(manager, dtype, DEV)
+    x = rnd(23, cfg.hidden_size, seed=5, dtype=dtype)
+    manager.add_sequence("a")
+    manager.reserve("a", 23)
+    ctx = StepBuilder(manager, DEV).build([("a", [0] * 23, [])])
+    stream, pending = block.forward(ctx, x.to(DEV).clone(), None, storage.layers[0])
+    cos, sin = pm.rope_tables(torch.arange(23), cfg.rope_theta, cfg.head_dim)
+    want = pm.decoder_layer(x.double(), {k: v.double() for k, v in tensors.items()}, 1, TINY_B, cos.double(), sin.double())
+    assert rel_err(stream.float() + pending.float(), want) < 4 * TOL[dtype]
+
+
+# ---- a toy architecture, defined here ---------------------------------------------------------
+
+@dataclass(frozen=True)
+class CumMeanSpec:
+    """A mixer with state of its own: out[t] = W . mean(h[0..t]).  It keeps the running sum and
+    the count per request, not keys and values."""
+    hidden: int
+    kind: str = "toy_cummean"
+
+
+def register_toy():
+    from inferrs_amd import ops
+    from inferrs_amd.config import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec,
+                                    ScheduleEntry)
+    from inferrs_amd.config.registry import register_architecture
+    from inferrs_amd.parts import FixedState, Mixer, register_mixer
+    from inferrs_amd.weights import TensorSpec
+
+    @register_mixer("toy_cummean")
+    class CumMean(Mixer):
+        @classmethod
+        def tensors(cls, spec):
+            return {"mix.weight": TensorSpec((spec.hidden, spec.hidden))}
+
+        @classmethod
+        def cache_need(cls, spec):
+            return FixedState((spec.hidden + 1,), torch.float32)
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.spec = spec
+            self.w = tensors["mix.weight"].to(device=device, dtype=dtype).contiguous()
+
+        def forward(self, ctx, h, cache):
+            out = torch.empty_like(h)
+            off = 0
+            for n, slot in zip(ctx.q_lens, ctx.state_slots_host):      # a toy: one request at a time
+                state = cache.state[slot]
+                sums = state[:-1] + torch.cumsum(h[off:off + n].float(), 0)
+                counts = state[-1] + torch.arange(1, n + 1, device=h.device, dtype=torch.float32)
+                out[off:off + n] = (sums / counts[:, None]).to(h.dtype)
+                state[:-1] = sums[-1]
+                state[-1] = counts[-1]
+                off += n
+            return ops.linear(out, self.w)
+
+    class ToyConfig:
+        architecture = "ToyForCausalLM"
+        model_type = "toy"
+
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def to_dict(self):
+            return dict(self.raw, architectures=[self.architecture], model_type=self.model_type)
+
+        def to_spec(self):
+            r = self.raw
+            h = r["hidden_size"]
+            norm = NormSpec(size=h, eps=r["eps"])
+            attn = AttentionSpec(hidden=h, n_heads=r["heads"], n_kv_heads=r["kv_heads"], head_dim=r["head_dim"],
+                                 position=PositionSpec(kind="rope", head_dim=r["head_dim"], rot_dim=r["head_dim"] // 2,
+                                                       theta=100.0),
+                                 qk_norm=None, window=r["window"])
+            ffn = GatedMlpSpec(hidden=h, intermediate=r["intermediate"])
+
+            def layer(i, mixer):
+                p = f"blocks.{i}."
+                return LayerSpec(mixer=mixer, ffn=ffn, norm_mixer=norm, norm_ffn=norm, mixer_prefix=p + "mixer.",
+                                 ffn_prefix=p + "ffn.", norm_mixer_name=p + "norm1.weight", norm_ffn_name=p + "norm2.weight")
+            layers = (layer(0, attn), layer(1, CumMeanSpec(h)), layer(2, attn))
+            # layer 0 runs twice (two caches), layer 2 reads the cache that stop 0 wrote
+            schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(0))
+            return ModelSpec(architecture=self.architecture, vocab_size=r["vocab"], hidden=h, layers=layers,
+                             schedule=schedule, final_norm=norm, final_norm_name="norm.weight",
+                             embed_name="embed.weight", head_name=None, max_position=512)
+
+    register_architecture(ToyConfig)
+    return ToyConfig
+
+
+def toy_plain(p, raw, ids):
+    """The toy model on a whole sequence, in plain tensor arithmetic (64-bit)."""
+    t = len(ids)
+    x = p["embed.weight"][torch.as_tensor(ids)]
+    d, nq, nkv = raw["head_dim"], raw["heads"], raw["kv_heads"]
+    cos, sin = pm.rope_tables(torch.arange(t), 100.0, d // 2)
+    cos, sin = cos.double(), sin.double()
+
+    def rot(v):          # only the first half of each head is rotated
+        return torch.cat([pm.rope_half(v[..., :d // 2], cos, sin), v[..., d // 2:]], -1)
+
+    def qkv(i, h):
+        pre = f"blocks.{i}.mixer."
+        q = pm.linear(h, p[pre + "q_proj.weight"]).reshape(t, nq, d).transpose(0, 1)
+        k = pm.linear(h, p[pre + "k_proj.weight"]).reshape(t, nkv, d).transpose(0, 1)
+        v = pm.linear(h, p[pre + "v_proj.weight"]).reshape(t, nkv, d).transpose(0, 1)
+        return rot(q), rot(k), v
+
+    def attend(i, q, k, v):
+        g = nq // nkv
+        k, v = pm.repeat_kv(k, g), pm.repeat_kv(v, g)
+        s = torch.matmul(q, k.transpose(1, 2)) / d ** 0.5
+        i_ = torch.arange(t)[:, None]
+        j_ = torch.arange(t)[None, :]
+        s = s.masked_fill((j_ > i_) | (j_ <= i_ - raw["window"]), float("-inf"))
+        o = torch.matmul(pm.softmax_last(s), v).transpose(0, 1).reshape(t, nq * d)
+        return pm.linear(o, p[f"blocks.{i}.mixer.o_proj.weight"])
+
+    def ffn(i, h):
+        pre = f"blocks.{i}.ffn."
+        return pm.mlp(h, p[pre + "gate_proj.weight"], p[pre + "up_proj.weight"], p[pre + "down_proj.weight"])
+
+    def norm(name, h):
+        return pm.rms_norm(h, p[name], raw["eps"])
+
+    kept = None
+    for stop, (layer, reads) in enumerate([(0, None), (1, None), (2, 0), (0, None)]):
+        h = norm(f"blocks.{layer}.norm1.weight", x)
+        if layer == 1:
+            mean = torch.cumsum(h, 0) / torch.arange(1, t + 1, dtype=h.dtype)[:, None]
+            a = pm.linear(mean, p["blocks.1.mixer.mix.weight"])
+        else:
+            q, k, v = qkv(layer, h)
+            if stop == 0:
+                kept = (k, v)
+            if reads is not None:
+                k, v = kept
+            a = attend(layer, q, k, v)
+        x = x + a
+        x = x + ffn(layer, norm(f"blocks.{layer}.norm2.weight", x))
+    return pm.linear(norm("norm.weight", x), p["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype,page", [("float32", 4), ("bfloat16", 16)])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype, page):
+    from inferrs_amd.engine import Engine, run_trace
+    from inferrs_amd.weights import write_random_model
+    ToyConfig = register_toy()
+    raw = dict(hidden_size=48, heads=4, kv_heads=2, head_dim=16, intermediate=80, vocab=101, eps=1e-5, window=23)
+    folder = write_random_model(str(tmp_path / "toy"), ToyConfig(raw), seed=4)
+    from safetensors.torch import load_file
+    p = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    reqs = {f"r{i}": random_tokens(n, 101, 30 + i) for i, n in enumerate([1, 40, 77, 130])}
+    ref = {r: toy_plain(p, raw, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    first = None
+    for mode, trace in (("whole", tm.whole(reqs)), ("portions", tm.portions(reqs, [5, 2, 31, 3])),
+                        ("mixed", tm.mixed(reqs, seed=4, max_live=3, decode_tail=10))):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-trace.max_tokens // page) + 2, max_seqs=4)
+        assert len(eng.cache.groups) == 1 and len(eng.cache.states) == 1      # two attention caches share a group
+        run_trace(eng, trace.lines, str(tmp_path / mode), io.StringIO())
+        got = trace.read(str(tmp_path / mode), 101)
+        err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
+        assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
+        eng.cache.check_invariants()
+        if first is None:
+            first = got
+        elif dtype == "float32":
+            cross = max(float(np.abs(got[r][i] - first[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
+            assert cross < 2e-6, f"{mode} against whole: {cross:.3e}"
