@@ -40,8 +40,8 @@ int ia_attention_generic(void* out, const void* q, const void* k_cache, const vo
 
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
                   int out_dtype, hipStream_t stream);
-int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, float* partial, int M, int N,
-                        int K, int splits, int out_dtype, hipStream_t stream);
+int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
+                        int out_dtype, int dual, hipStream_t stream);
 
 int ia_argmax(int* out, const float* logits, int rows, int vocab, hipStream_t stream);
 int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, const float* rep,

@@ -8,8 +8,8 @@
 //   * ia_gemm_skinny_bf16: few rows (decode batches, logits of a few positions) against a
 //     large weight matrix.  The product is bound by reading the weights once, so each wave
 //     streams 16 weight rows in 16-byte pieces straight into MFMA 16x16x32 operands and
-//     the waves of a block (and, for short outputs, several blocks) split k between them;
-//     partial tiles are summed in a fixed order.
+//     the waves of a block split k between them; partial tiles are summed in a fixed order.
+//     A variant takes [gate; up] and writes silu(gate) * up.
 #include "common.h"
 #include "api.h"
 
@@ -90,119 +90,228 @@ extern "C" int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define SK_WAVES 4
-#define SK_ROWS 16      // weight rows (output features) per block
 #define SK_KSTEP 32     // k per MFMA
+#define SK_MAX_WAVES 16
 
 // Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16) of A and column
 // (l % 16) of B, each with the eight k values (l / 16) * 8 .. + 8; lane l receives
-// D[4 * (l / 16) + i][l % 16], i = 0..3.  A is the weight tile (rows = output features),
+// D[4 * (l / 16) + i][l % 16], i = 0..3.  A is a tile of 16 weight rows (output features),
 // B the activations (columns = batch rows).
-template <int MT>
-__global__ __launch_bounds__(SK_WAVES * IA_WAVE) void gemm_skinny_kernel(
-    float* __restrict__ partial,        // [splits, M, N] when gridDim.y > 1, else unused
-    void* __restrict__ out, int out_f32,
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K, int m_base) {
-    __shared__ f32x4 red[SK_WAVES][MT][IA_WAVE];
+//
+// A block owns 16 * RT output features; its waves split k between them in contiguous ranges
+// (a wave streams RT * 16 rows of `kper` * 64 bytes each) and add their tiles up through
+// shared memory in wave order.  How k is split depends on the weight's shape alone, so a
+// row's rounding does not depend on the batch it is in.  MT tiles of 16 batch rows share
+// every weight load.  DUAL: the weight holds two matrices stacked along the output ([gate;
+// up], N features each) and the result is silu(gate . x) * (up . x).
+template <int MT, int RT, bool DUAL>
+__global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
+    void* __restrict__ out, int out_f32, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+    int M, int N, int K, int kper, int m_base, int rot_mul) {
+    constexpr int NA = DUAL ? 2 : 1;
+    extern __shared__ f32x4 red[];      // [waves][NA][RT][MT][64]
     const int lane = threadIdx.x & (IA_WAVE - 1);
     const int wave = threadIdx.x / IA_WAVE;
-    const int n0 = blockIdx.x * SK_ROWS;
+    const int waves = blockDim.x / IA_WAVE;
+    const int n0 = blockIdx.x * 16 * RT;
     const int r = lane & 15, g = lane >> 4;
-    const int n_read = n0 + r < N ? n0 + r : N - 1;
-    const bf16_t* wrow = w + (size_t)n_read * K + g * 8;
     const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
-    const int stride = SK_WAVES * gridDim.y;
+    const int ks0 = wave * kper, ks1 = ks0 + kper < ksteps ? ks0 + kper : ksteps;
 
-    f32x4 acc[MT];
+    const bf16_t* wrow[NA][RT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            const int n = n0 + t * 16 + r;
+            wrow[a][t] = w + ((size_t)a * N + (n < N ? n : N - 1)) * K + g * 8;
+        }
+    // Batch rows beyond M are read from row 0: their columns of the result are never stored.
     const bf16_t* xrow[MT];
-    bool xok[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = m_base + t * 16 + r;
-        xok[t] = m < M;
-        xrow[t] = x + (size_t)(xok[t] ? m : 0) * K + g * 8;
+        xrow[t] = x + (size_t)(m < M ? m : 0) * K + g * 8;
     }
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-#pragma unroll 4
-    for (int ks = blockIdx.y * SK_WAVES + wave; ks < ksteps; ks += stride) {
-        const int k0 = ks * SK_KSTEP;
-        const bool kin = k0 + g * 8 < K;          // K is a multiple of 8: a piece is in or out
-        const uint4 a = kin ? *(const uint4*)(wrow + k0) : zero;
+    f32x4 acc[NA][RT][MT];
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const uint4 b = (kin && xok[t]) ? *(const uint4*)(xrow[t] + k0) : zero;
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
-                                                             __builtin_bit_cast(bf16x8, b), acc[t], 0, 0, 0);
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int u = 0; u < MT; ++u) acc[a][t][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // Blocks start at different places of their k range and wrap around: rows are a power of
+    // two apart in memory, and blocks that walk them in step would all ask the same few memory
+    // channels at any moment.  The order of the sum depends on the block (the output feature)
+    // only, never on the batch.  Whole steps run without a condition; a last step that K does
+    // not fill is done apart, with zeros beyond K.
+    constexpr int UNROLL = (NA * RT >= 4) ? 2 : (NA * RT == 2 ? 4 : 8);
+    const int whole = K / SK_KSTEP;                         // steps that lie inside K entirely
+    const int ke = ks1 < whole ? ks1 : whole;
+    const int len = ke - ks0;
+    const int rot = len > 0 ? (int)((blockIdx.x * (unsigned)rot_mul) % (unsigned)len) / UNROLL * UNROLL : 0;
+    for (int part = 0; part < 2; ++part) {
+        const int pa = part == 0 ? ks0 + rot : ks0, pb = part == 0 ? ke : ks0 + rot;
+#pragma unroll UNROLL
+        for (int ks = pa; ks < pb; ++ks) {
+            const int k0 = ks * SK_KSTEP;
+            uint4 a[NA][RT];
+#pragma unroll
+            for (int q = 0; q < NA; ++q)
+#pragma unroll
+                for (int t = 0; t < RT; ++t) a[q][t] = *(const uint4*)(wrow[q][t] + k0);
+#pragma unroll
+            for (int u = 0; u < MT; ++u) {
+                const uint4 b = *(const uint4*)(xrow[u] + k0);
+#pragma unroll
+                for (int q = 0; q < NA; ++q)
+#pragma unroll
+                    for (int t = 0; t < RT; ++t)
+                        acc[q][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, a[q][t]), __builtin_bit_cast(bf16x8, b), acc[q][t][u], 0, 0, 0);
+            }
         }
     }
+    if (ks1 > whole && ks0 <= whole) {                      // the step that K leaves unfilled
+        const int k0 = whole * SK_KSTEP;
+        const bool kin = k0 + g * 8 < K;                    // K is a multiple of 8: a piece is in or out
+        const uint4 zero = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
-    __syncthreads();
-    if (wave != 0) return;
+        for (int u = 0; u < MT; ++u) {
+            const uint4 b = kin ? *(const uint4*)(xrow[u] + k0) : zero;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        f32x4 s = red[0][t][lane];
+            for (int q = 0; q < NA; ++q)
 #pragma unroll
-        for (int wv = 1; wv < SK_WAVES; ++wv) {
-            const f32x4 o = red[wv][t][lane];
-            s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
-        }
-        const int m = m_base + t * 16 + r;
-        if (m >= M) continue;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = n0 + 4 * g + i;
-            if (n >= N) continue;
-            if (gridDim.y > 1)
-                partial[((size_t)blockIdx.y * M + m) * N + n] = s[i];
-            else if (out_f32)
-                ((float*)out)[(size_t)m * N + n] = s[i];
-            else
-                ((bf16_t*)out)[(size_t)m * N + n].bits = f32_to_bf16_bits(s[i]);
+                for (int t = 0; t < RT; ++t) {
+                    const uint4 a = kin ? *(const uint4*)(wrow[q][t] + k0) : zero;
+                    acc[q][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc[q][t][u], 0, 0, 0);
+                }
         }
     }
+    if (waves > 1) {
+#pragma unroll
+        for (int q = 0; q < NA; ++q)
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int u = 0; u < MT; ++u)
+                    red[(((wave * NA + q) * RT + t) * MT + u) * IA_WAVE + lane] = acc[q][t][u];
+        __syncthreads();
+    }
+    // the tiles are shared out between the waves for the sum and the store
+    int tile = 0;
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int u = 0; u < MT; ++u, ++tile) {
+            if (tile % waves != wave) continue;
+            f32x4 s[NA];
+#pragma unroll
+            for (int q = 0; q < NA; ++q) {
+                if (waves > 1) {
+                    s[q] = red[((q * RT + t) * MT + u) * IA_WAVE + lane];
+                    for (int wv = 1; wv < waves; ++wv) {
+                        const f32x4 o = red[(((wv * NA + q) * RT + t) * MT + u) * IA_WAVE + lane];
+                        s[q][0] += o[0]; s[q][1] += o[1]; s[q][2] += o[2]; s[q][3] += o[3];
+                    }
+                } else {
+                    s[q] = acc[q][t][u];
+                }
+            }
+            const int m = m_base + u * 16 + r;
+            if (m >= M) continue;
+            const int nb = n0 + t * 16 + 4 * g;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (DUAL) {
+                    // the first product is rounded to the storage precision before the
+                    // activation, as the two-kernel path rounds it
+                    const float gate = bf16_bits_to_f32(f32_to_bf16_bits(s[0][i]));
+                    const float up = bf16_bits_to_f32(f32_to_bf16_bits(s[NA - 1][i]));
+                    v[i] = gate / (1.0f + expf(-gate)) * up;
+                } else {
+                    v[i] = s[0][i];
+                }
+            }
+            if (nb + 3 < N && (N & 3) == 0) {
+                if (out_f32) {
+                    *(f32x4*)((float*)out + (size_t)m * N + nb) = (f32x4){v[0], v[1], v[2], v[3]};
+                } else {
+                    uint2 pk;
+                    pk.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+                    pk.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+                    *(uint2*)((bf16_t*)out + (size_t)m * N + nb) = pk;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (nb + i >= N) continue;
+                    if (out_f32) ((float*)out)[(size_t)m * N + nb + i] = v[i];
+                    else ((bf16_t*)out)[(size_t)m * N + nb + i].bits = f32_to_bf16_bits(v[i]);
+                }
+            }
+        }
 }
 
-__global__ void gemm_split_reduce_kernel(void* __restrict__ out, int out_f32, const float* __restrict__ partial,
-                                         int splits, size_t total) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        float s = partial[i];
-        for (int p = 1; p < splits; ++p) s += partial[(size_t)p * total + i];
-        if (out_f32) ((float*)out)[i] = s;
-        else ((bf16_t*)out)[i].bits = f32_to_bf16_bits(s);
-    }
+// Tuning knobs (ia_gemm_skinny_tune): waves wanted on the chip before k stops being split,
+// fewest k steps worth a wave, and the stagger of the blocks' starting points.
+static int g_target_waves = 2048, g_min_ksteps = 8, g_rot_mul = 5, g_min_waves = 8;
+
+extern "C" void ia_gemm_skinny_tune(int target_waves, int min_ksteps, int rot_mul, int min_waves) {
+    g_target_waves = target_waves; g_min_ksteps = min_ksteps; g_rot_mul = rot_mul; g_min_waves = min_waves;
 }
 
-// `splits` > 1 needs `partial` with room for splits * M * N floats.
-extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, float* partial,
-                                   int M, int N, int K, int splits, int out_dtype, hipStream_t stream) {
+// How many waves share k: a function of the weight's shape and of the row tiling only.
+static int skinny_waves(int N, int K, int rt, int tiles_per_wave) {
+    const int groups = (N + 16 * rt - 1) / (16 * rt);
+    const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
+    // the waves' tiles meet in shared memory: at most 64 KiB of it
+    const int most = 65536 / (tiles_per_wave * IA_WAVE * (int)sizeof(f32x4));
+    int waves = 1;
+    while (waves * 2 <= SK_MAX_WAVES && waves * 2 <= most && ksteps / (waves * 2) >= g_min_ksteps &&
+           (groups * waves < g_target_waves || waves < g_min_waves))
+        waves *= 2;
+    return waves;
+}
+
+template <int MT, int RT, bool DUAL>
+static void launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* w, int M, int N, int K,
+                          int m_base, hipStream_t stream) {
+    const int waves = skinny_waves(N, K, RT, (DUAL ? 2 : 1) * RT * MT);
+    const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
+    const int kper = (ksteps + waves - 1) / waves;
+    const size_t lds = waves > 1 ? (size_t)waves * (DUAL ? 2 : 1) * RT * MT * IA_WAVE * sizeof(f32x4) : 0;
+    const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
+    gemm_skinny_kernel<MT, RT, DUAL><<<grid, waves * IA_WAVE, lds, stream>>>(out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
+}
+
+// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` out[M, N] = silu(x . w[0:N]^T) * (x . w[N:2N]^T).
+extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
+                                   int out_dtype, int dual, hipStream_t stream) {
     IA_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     IA_CHECK(K % 8 == 0, "gemm_skinny: K=%d must be a multiple of 8 (use the tiled product)", K);
     IA_CHECK(out_dtype == IA_F32 || out_dtype == IA_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
-    IA_CHECK(splits >= 1 && splits <= 64, "gemm_skinny: splits=%d is outside 1..64", splits);
-    IA_CHECK(splits == 1 || partial != nullptr, "gemm_skinny: splits=%d without a partial buffer", splits);
     IA_CHECK((((uintptr_t)x | (uintptr_t)w) & 15) == 0, "gemm_skinny: x and w must be 16-byte aligned");
+    IA_CHECK((((uintptr_t)out) & 15) == 0, "gemm_skinny: out must be 16-byte aligned");
     if (M == 0) return 0;
     const int out_f32 = out_dtype == IA_F32;
-    const dim3 grid((N + SK_ROWS - 1) / SK_ROWS, splits);
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)w;
     for (int m_base = 0; m_base < M; m_base += 64) {
         const int rows = M - m_base;
-        // Rows beyond the first 64 are written by later launches: offset by m_base inside.
-        if (rows <= 16)
-            gemm_skinny_kernel<1><<<grid, SK_WAVES * IA_WAVE, 0, stream>>>(partial, out, out_f32, (const bf16_t*)x, (const bf16_t*)w, M, N, K, m_base);
-        else if (rows <= 32)
-            gemm_skinny_kernel<2><<<grid, SK_WAVES * IA_WAVE, 0, stream>>>(partial, out, out_f32, (const bf16_t*)x, (const bf16_t*)w, M, N, K, m_base);
-        else
-            gemm_skinny_kernel<4><<<grid, SK_WAVES * IA_WAVE, 0, stream>>>(partial, out, out_f32, (const bf16_t*)x, (const bf16_t*)w, M, N, K, m_base);
+        if (dual) {
+            if (rows <= 16) launch_skinny<1, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            else if (rows <= 32) launch_skinny<2, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            else launch_skinny<4, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+        } else {
+            if (rows <= 16) launch_skinny<1, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            else if (rows <= 32) launch_skinny<2, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            else launch_skinny<4, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+        }
         IA_LAUNCH_CHECK("gemm_skinny");
-    }
-    if (splits > 1) {
-        const size_t total = (size_t)M * N;
-        const size_t want = (total + 255) / 256;
-        gemm_split_reduce_kernel<<<(unsigned)(want < 65535 ? want : 65535), 256, 0, stream>>>(out, out_f32, partial, splits, total);
-        IA_LAUNCH_CHECK("gemm_split_reduce");
     }
     return 0;
 }

@@ -71,6 +71,8 @@ class StepBuilder:
         self._host: Optional[torch.Tensor] = None
         self._dev: Optional[torch.Tensor] = None
         self._event: Optional[torch.cuda.Event] = None
+        self._rows: Dict[Any, list] = {}
+        self.generation = 0                # grows when the device staging buffer moves
 
     def _staging(self, n: int) -> Tuple[torch.Tensor, torch.Tensor]:
         if self._host is None or self._host.numel() < n:
@@ -78,13 +80,39 @@ class StepBuilder:
             self._host = torch.empty(size, dtype=torch.int32, pin_memory=True)
             self._dev = torch.empty(size, dtype=torch.int32, device=self.device)
             self._event = None
+            self.generation += 1
         if self._event is not None:
             self._event.synchronize()      # the previous step's copy has left the host buffer
         return self._host, self._dev
 
-    def build(self, entries: Sequence[Tuple[Hashable, Sequence[int], Sequence[int]]]) -> StepContext:
+    def _table_row(self, group: int, seq, need: int) -> np.ndarray:
+        """The request's pages of one group as an int32 array, kept between steps and extended
+        by the pages that were added since (tables only grow, except where a window releases)."""
+        table = seq.tables[group]
+        if self.cache.groups[group].need.window is not None:
+            return np.asarray(table, dtype=np.int32)
+        key = (group, seq.seq_id)
+        hit = self._rows.get(key)
+        if hit is None or hit[0] is not seq or hit[1].size < len(table):
+            arr = np.zeros(max(64, 2 * len(table), need), dtype=np.int32)
+            arr[:len(table)] = table
+            if len(self._rows) > 4 * max(len(self.cache.sequences), 16):
+                live = self.cache.sequences
+                self._rows = {k: v for k, v in self._rows.items() if live.get(k[1]) is v[0]}
+            self._rows[key] = [seq, arr, len(table)]
+            return arr[:len(table)]
+        _, arr, filled = hit
+        if len(table) > filled:
+            arr[filled:len(table)] = table[filled:]
+            hit[2] = len(table)
+        return arr[:len(table)]
+
+    def build(self, entries: Sequence[Tuple[Hashable, Sequence[int], Sequence[int]]],
+              pad_pages: Optional[int] = None) -> StepContext:
         """`entries`: (request, tokens, want).  The requests are live and hold pages for the
-        positions `length .. length + len(tokens)`."""
+        positions `length .. length + len(tokens)`.  `pad_pages`: width of the block tables (at
+        least what the longest request needs); with it the place of every array in the staging
+        buffer depends on the counts of tokens, requests and wanted rows only."""
         ps = self.cache.page_size
         seqs = [self.cache.sequences[e[0]] for e in entries]
         q_lens = [len(e[1]) for e in entries]
@@ -92,22 +120,32 @@ class StepBuilder:
         n, s_count = sum(q_lens), len(entries)
         n_groups = len(self.cache.groups)
         max_pages = max(1, max(-(-(st + q) // ps) for st, q in zip(starts, q_lens)))
+        if pad_pages is not None:
+            if pad_pages < max_pages:
+                raise StepError(f"block tables of {pad_pages} pages are too narrow for {max_pages}")
+            max_pages = pad_pages
         cu = np.zeros(s_count + 1, dtype=np.int64)
         np.cumsum(q_lens, out=cu[1:])
-        token_ids = np.concatenate([np.asarray(e[1], dtype=np.int32) for e in entries])
-        positions = np.concatenate([np.arange(st, st + q, dtype=np.int32) for st, q in zip(starts, q_lens)])
-        token_seq = np.repeat(np.arange(s_count, dtype=np.int32), q_lens)
+        if n == s_count:                                   # one token a request
+            token_ids = np.fromiter((e[1][0] for e in entries), dtype=np.int32, count=n)
+            positions = np.asarray(starts, dtype=np.int32)
+            token_seq = np.arange(s_count, dtype=np.int32)
+        else:
+            token_ids = np.concatenate([np.asarray(e[1], dtype=np.int32) for e in entries])
+            positions = np.concatenate([np.arange(st, st + q, dtype=np.int32) for st, q in zip(starts, q_lens)])
+            token_seq = np.repeat(np.arange(s_count, dtype=np.int32), q_lens)
         want = np.asarray([cu[i] + w for i, e in enumerate(entries) for w in e[2]], dtype=np.int32)
         state_slots = np.asarray([s.state_slot for s in seqs], dtype=np.int32)
         tables, slots = [], []
         for g in range(n_groups):
             bt = np.zeros((s_count, max_pages), dtype=np.int32)
             for i, s in enumerate(seqs):
-                row = s.tables[g][:max_pages]
-                if len(row) * ps < starts[i] + q_lens[i]:
-                    raise StepError(f"request {s.seq_id!r} holds {len(row)} pages, too few for "
+                need = -(-(starts[i] + q_lens[i]) // ps)
+                row = self._table_row(g, s, need)
+                if row.size < need:
+                    raise StepError(f"request {s.seq_id!r} holds {row.size} pages, too few for "
                                     f"{starts[i] + q_lens[i]} tokens")
-                bt[i, :len(row)] = row
+                bt[i, :min(row.size, max_pages)] = row[:max_pages]
             pages_of_token = bt[token_seq, positions // ps]
             if n and (pages_of_token == RELEASED).any():
                 raise StepError("a new token falls into a page that was already released")
@@ -132,8 +170,9 @@ class StepBuilder:
         self._event.record()
         groups = [GroupStep(ps, views[6 + 2 * g], views[7 + 2 * g].view(s_count, max_pages))
                   for g in range(n_groups)]
+        max_kv = max(st + q for st, q in zip(starts, q_lens))
         return StepContext(
             n_tokens=n, n_seqs=s_count, token_ids=views[0], positions=views[1], token_seq=views[2],
             cu_tokens=views[3], state_slots=views[4], want_rows=views[5], groups=groups,
             q_lens=q_lens, kv_starts=starts, state_slots_host=[int(x) for x in state_slots],
-            max_q_len=max(q_lens), max_kv_len=max(st + q for st, q in zip(starts, q_lens)))
+            max_q_len=max(q_lens), max_kv_len=max_kv if pad_pages is None else max(max_kv, pad_pages * ps))

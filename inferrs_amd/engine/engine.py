@@ -34,8 +34,12 @@ class Entry:
 
 
 class Engine:
+    GRAPH_BUCKET_TOKENS = 1024      # a captured decode step serves context lengths up to a multiple of this
+    MAX_GRAPHS = 24
+
     def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: Optional[int] = None,
-                 max_seqs: int = 32, cache_tokens: Optional[int] = None, memory_fraction: float = 0.9):
+                 max_seqs: int = 32, cache_tokens: Optional[int] = None, memory_fraction: float = 0.9,
+                 use_graphs: bool = True):
         """`num_pages` pages per cache group, or enough for `cache_tokens` tokens, or, when
         neither is given, `memory_fraction` of the GPU memory that is free now (the reference
         sizes by a fraction of total memory, `inferrs-models/src/kv_cache.rs:44-65`)."""
@@ -59,6 +63,11 @@ class Engine:
         self.cache = CacheManager(needs, page_size, num_pages, max_seqs)
         self.storage = CacheStorage(self.cache, model.dtype, self.device)
         self.builder = StepBuilder(self.cache, self.device)
+        # Decode steps (one token a request) are launch-bound: each distinct shape is captured
+        # into a HIP graph the second time it is seen and replayed from then on.
+        self.use_graphs = use_graphs and model.graph_safe
+        self._graphs: Dict[Tuple[int, int, int], object] = {}
+        self.graph_replays = 0
 
     # ---- construction -----------------------------------------------------------------------
     @classmethod
@@ -143,9 +152,43 @@ class Engine:
                     self.cache.free_sequence(sid)
             raise
 
-        ctx = self.builder.build([(e.seq_id, e.tokens, e.want) for e in entries])
-        logits = self.model.forward(ctx, self.storage)
+        triples = [(e.seq_id, e.tokens, e.want) for e in entries]
+        if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
+            logits = self._decode_step(triples)
+        else:
+            logits = self.model.forward(self.builder.build(triples), self.storage)
         if commit:
             for e in entries:
                 self.cache.commit(e.seq_id, len(e.tokens))
         return logits
+
+    def _decode_step(self, triples) -> torch.Tensor:
+        """One token a request, through a captured graph when this shape has been seen before.
+        The block tables are padded to the bucket's width, so that every kernel argument is the
+        same for all context lengths of the bucket; lengths and pages are read from device memory.
+        The logits that are returned are the graph's own buffer: they hold until the next step."""
+        ps = self.page_size
+        longest = max(self.cache.sequences[t[0]].length for t in triples) + 1
+        bucket_pages = max(1, self.GRAPH_BUCKET_TOKENS // ps)
+        pad_pages = -(-(-(-longest // ps)) // bucket_pages) * bucket_pages
+        n_want = sum(len(t[2]) for t in triples)
+        generation = self.builder.generation
+        ctx = self.builder.build(triples, pad_pages=pad_pages)
+        if self.builder.generation != generation:
+            self._graphs.clear()                        # the staging buffer moved: captured addresses are stale
+        key = (len(triples), n_want, pad_pages)
+        entry = self._graphs.get(key)
+        if entry is None:
+            if len(self._graphs) >= self.MAX_GRAPHS:
+                self._graphs.pop(next(iter(self._graphs)))
+            self._graphs[key] = "seen"
+            return self.model.forward(ctx, self.storage)
+        if entry == "seen":
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = self.model.forward(ctx, self.storage)
+            entry = self._graphs[key] = (graph, out)
+        graph, out = entry
+        graph.replay()
+        self.graph_replays += 1
+        return out

@@ -55,6 +55,14 @@ class DecoderModel:
         self.final_norm = part_class("norm", spec.final_norm)(
             spec.final_norm, {"weight": tensors.pop(spec.final_norm_name)}, dtype, device)
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether every part allows a decode step to be captured and replayed."""
+        parts = [self.final_norm]
+        for b in self.blocks:
+            parts += [b.mixer, b.ffn, b.norm_mixer, b.norm_ffn, getattr(b.mixer, "position", None)]
+        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+
     def cache_needs(self) -> Dict[int, object]:
         """Schedule stop that owns a cache -> what its mixer keeps per request."""
         needs: Dict[int, object] = {}

@@ -306,18 +306,8 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 # ---- matrix products --------------------------------------------------------------------------
 
-SKINNY_MAX_ROWS = 64
-
-
-def _skinny_splits(n_out: int, k: int) -> int:
-    """How many blocks share k in the skinny product: a function of the weight's shape only,
-    so that a row's rounding does not depend on the batch it is in."""
-    blocks = (n_out + 15) // 16
-    ksteps = (k + 31) // 32
-    splits = 1
-    while blocks * splits < 1024 and ksteps // (4 * splits * 2) >= 4 and splits < 16:
-        splits *= 2
-    return splits
+SKINNY_MAX_ROWS = 16          # beyond this the vendor's GEMM reads the weights faster
+SKINNY_MAX_ROWS_F32_OUT = 64  # 32-bit results (logits) have no library route
 
 
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -333,30 +323,37 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
 
 
 def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                     splits: Optional[int] = None) -> torch.Tensor:
+                     dual: bool = False) -> torch.Tensor:
+    """x [m, k] . w[n, k]^T on the matrix cores, made for few rows.  `dual`: w is [gate; up]
+    stacked along its rows and the result is silu(x . gate^T) * (x . up^T)."""
     _dev(x, w)
     m, k = x.shape
     n, k2 = w.shape
     if k != k2 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_skinny: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
-    if splits is None:
-        splits = _skinny_splits(n, k)
+    if dual:
+        if n % 2:
+            raise KernelError(f"gemm_skinny: a stacked [gate; up] weight needs an even row count, got {n}")
+        n //= 2
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device) if splits > 1 else None
-    _check(library().ia_gemm_skinny_bf16(_p(out), _p(x), _p(w), _p(partial), m, n, k, splits,
-                                         _DT[out_dtype], _stream()))
+    _check(library().ia_gemm_skinny_bf16(_p(out), _p(x), _p(w), m, n, k, _DT[out_dtype], int(dual), _stream()))
     return out
+
+
+def skinny_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and (x.data_ptr() | w.data_ptr()) % 16 == 0)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
-    skinny MFMA kernel for up to 64 rows, the vendor's GEMM beyond that; a 32-bit result of
-    bfloat16 operands with many rows goes through the skinny kernel 64 rows at a time."""
+    skinny MFMA kernel for up to 16 rows, the vendor's GEMM beyond that (the reference uses
+    cuBLAS for all of them); a 32-bit result of bfloat16 operands (logits) comes from the skinny
+    kernel, 64 rows at a time."""
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return gemm_tiled(x, w, out_dtype)
     m, k = x.shape
-    if k % 8 or (x.data_ptr() | w.data_ptr()) % 16:
+    if not skinny_fits(x, w):
         return gemm_tiled(x, w, out_dtype)
     if m <= SKINNY_MAX_ROWS or out_dtype == torch.float32:
         return gemm_skinny_bf16(x, w, out_dtype)
@@ -420,3 +417,11 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _check(library().ia_sample(_p(out), _p(logits), _p(ws), rows, vocab, _p(temperature), _p(top_k), _p(top_p),
                                _p(min_p), _p(u), _stream()))
     return out
+
+
+def gated_silu_linear(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x . gate^T) * (x . up^T) for w_gate_up = [gate; up]: one fused kernel for few bfloat16
+    rows, else the product followed by the element-wise kernel."""
+    if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
+        return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True)
+    return silu_mul(linear(x, w_gate_up))

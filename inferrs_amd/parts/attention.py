@@ -22,6 +22,8 @@ from .linear import Linear
 
 @register_mixer("attention")
 class Attention(Mixer):
+    graph_safe = True
+
     @classmethod
     def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorSpec]:
         q_out, kv_out = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim

@@ -82,6 +82,11 @@ def part_class(table: str, spec: Any) -> type:
 
 class Part:
     kind = "?"
+    # True when `forward` launches the same kernels with the same arguments for every step of
+    # one shape, reading everything that changes (positions, pages, slots) from device memory:
+    # only then may a decode step that contains the part be captured into a graph and replayed.
+    # A part that looks at the host-side lists of the step context must leave this False.
+    graph_safe = False
 
     @classmethod
     def tensors(cls, spec) -> Dict[str, TensorSpec]:

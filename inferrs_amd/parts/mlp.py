@@ -15,6 +15,8 @@ from .linear import Linear
 
 @register_ffn("gated_mlp")
 class GatedMlp(FeedForward):
+    graph_safe = True
+
     @classmethod
     def tensors(cls, spec: GatedMlpSpec) -> Dict[str, TensorSpec]:
         return {
@@ -31,4 +33,4 @@ class GatedMlp(FeedForward):
         self.down = Linear([tensors["down_proj.weight"]], dtype, device)
 
     def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
-        return self.down(ops.silu_mul(self.gate_up(h)))
+        return self.down(ops.gated_silu_linear(h, self.gate_up.weight))

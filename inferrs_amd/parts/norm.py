@@ -14,6 +14,8 @@ from .base import Norm, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     @classmethod
     def tensors(cls, spec: NormSpec) -> Dict[str, TensorSpec]:
         return {"weight": TensorSpec((spec.size,), "norm")}

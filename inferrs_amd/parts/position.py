@@ -25,6 +25,8 @@ def inverse_frequencies(theta: float, rot_dim: int) -> np.ndarray:
 
 @register_position("rope")
 class Rotary(Position):
+    graph_safe = True
+
     def __init__(self, spec: PositionSpec, tensors, dtype, device):
         if spec.rot_dim <= 0 or spec.rot_dim % 2 or spec.rot_dim > spec.head_dim:
             raise SpecError(f"rot_dim {spec.rot_dim} must be even and within head_dim {spec.head_dim}")
@@ -41,6 +43,8 @@ class Rotary(Position):
 
 @register_position("none")
 class NoPosition(Position):
+    graph_safe = True
+
     rot_dim = 0
     interleaved = False
 

@@ -275,12 +275,25 @@ def test_linear_bfloat16(m, n, k, out_dtype):
     close(got, want, tol(out_dtype, 2e-5), f"linear {m}x{n}x{k}")
 
 
-def test_gemm_skinny_splits_agree():
+@pytest.mark.parametrize("m", [1, 8, 17, 40, 64])
+@pytest.mark.parametrize("n,k", [(130, 40), (12288, 4096), (200, 136)])
+def test_gated_silu_linear(m, n, k):
     from inferrs_amd import ops
-    x, w = randn(5, 4096, dtype=torch.bfloat16, seed=1), randn(77, 4096, dtype=torch.bfloat16, seed=2)
-    want = x.double() @ w.double().t()
-    for splits in (1, 2, 8, 16):
-        close(ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32, splits=splits), want, 2e-5, f"splits {splits}")
+    x = randn(m, k, dtype=torch.bfloat16, seed=1)
+    w = randn(2 * n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    gate = (x.double() @ w[:n].double().t()).to(torch.bfloat16).double()     # the products are stored, then activated
+    up = (x.double() @ w[n:].double().t()).to(torch.bfloat16).double()
+    want = gate / (1 + torch.exp(-gate)) * up
+    close(ops.gated_silu_linear(dev(x), dev(w)), want, 2 ** -7, "fused")
+    close(ops.silu_mul(ops.linear(dev(x), dev(w))), want, 2 ** -7, "two kernels")
+
+
+def test_skinny_rows_do_not_depend_on_the_batch():
+    from inferrs_amd import ops
+    x, w = randn(16, 4096, dtype=torch.bfloat16, seed=1), randn(77, 4096, dtype=torch.bfloat16, seed=2)
+    full = ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32).cpu()
+    assert torch.equal(ops.gemm_skinny_bf16(dev(x[:1]), dev(w), torch.float32).cpu(), full[:1])
+    assert torch.equal(ops.gemm_skinny_bf16(dev(x[3:9].contiguous()), dev(w), torch.float32).cpu(), full[3:9])
 
 
 def test_argmax_lowest_index_among_equal_maxima():

@@ -191,3 +191,27 @@ def test_out_of_pages_is_an_error_and_takes_nothing(models):
     with pytest.raises(OutOfPages):
         eng.step([Entry("y", [1], [0])])
     assert eng.cached_length("y") == 16
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_eager_ones(models, tmp_path, dtype):
+    """Decode steps are replayed from a captured graph from the third step of a shape on.  Every
+    replay is checked against the same trace run without graphs, with eager steps (portions of
+    prompts, other batch sizes) in between the replays."""
+    from inferrs_amd.engine import Engine, run_trace
+    folder, raw, reqs, ref = pick(models, "D", True, dtype)
+    some = {k: reqs[k] for k in ("r3", "r5", "r6", "r7")}
+    trace = tm.mixed(some, seed=11, max_live=3, decode_tail=40)
+    outs = {}
+    for graphs in (False, True):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-trace.max_tokens // 16), max_seqs=4,
+                                 use_graphs=graphs)
+        run_trace(eng, trace.lines, str(tmp_path / str(graphs)), io.StringIO())
+        outs[graphs] = trace.read(str(tmp_path / str(graphs)), raw["vocab_size"])
+        assert (eng.graph_replays > 20) == graphs
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    err, where = worst(outs[True], outs[False], some, scale=scale)
+    # the same kernels with the same arguments, except that the keys may be split differently
+    assert err <= (1e-6 if dtype == "float32" else bound(folder, reqs, ref, dtype)), f"{err:.3e} at {where}"
+    err, where = worst(outs[True], ref, some, scale=scale)
+    assert err <= bound(folder, reqs, ref, dtype), f"{err:.3e} at {where}"
