@@ -251,33 +251,44 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
     }
 }
 
-// Merges the partial results of the key splits of one (token, head): one wave a row.
+// Merges the partial results of the key splits of one (token, head): one wave a row.  Lane s
+// weighs split s (splits beyond 64 in further rounds), then every lane sums its dims over the
+// splits, in split order.
 __global__ __launch_bounds__(IA_WAVE) void attn_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                                              const float* __restrict__ part_ml, int splits) {
+    __shared__ float weight[256];
     const size_t row = blockIdx.x;
     const int lane = threadIdx.x;
     const float* ml = part_ml + row * splits * 2;
     float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml[2 * s]);
+    for (int s = lane; s < splits; s += IA_WAVE) mx = fmaxf(mx, ml[2 * s]);
+    mx = wave_max(mx);
     float total = 0.f;
-    float o[(HD + IA_WAVE - 1) / IA_WAVE];
-#pragma unroll
-    for (int t = 0; t < (HD + IA_WAVE - 1) / IA_WAVE; ++t) o[t] = 0.f;
-    for (int s = 0; s < splits; ++s) {
+    for (int s = lane; s < splits; s += IA_WAVE) {
         const float ms = ml[2 * s];
-        if (ms == -INFINITY) continue;                  // a split that held no key of this row
-        const float w = exp2f(ms - mx);
+        const float w = ms == -INFINITY ? 0.f : exp2f(ms - mx);      // a split that held no key of this row
+        weight[s] = w;
         total += ml[2 * s + 1] * w;
-        const float* po = part_o + (row * splits + s) * HD;
+    }
+    total = wave_sum(total);
+    __syncthreads();
+    constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
+    float o[PER];
 #pragma unroll
-        for (int t = 0; t < (HD + IA_WAVE - 1) / IA_WAVE; ++t) {
+    for (int t = 0; t < PER; ++t) o[t] = 0.f;
+    const float* po = part_o + row * splits * HD;
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s) {
+        const float w = weight[s];
+#pragma unroll
+        for (int t = 0; t < PER; ++t) {
             const int e = lane + t * IA_WAVE;
-            if (e < HD) o[t] += po[e] * w;
+            if (e < HD) o[t] = fmaf(po[(size_t)s * HD + e], w, o[t]);
         }
     }
     const float inv = 1.0f / total;
 #pragma unroll
-    for (int t = 0; t < (HD + IA_WAVE - 1) / IA_WAVE; ++t) {
+    for (int t = 0; t < PER; ++t) {
         const int e = lane + t * IA_WAVE;
         if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(o[t] * inv);
     }

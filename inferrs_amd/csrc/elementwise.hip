@@ -88,15 +88,91 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, T* __restrict__ x, const T* 
     }
 }
 
+// bfloat16 rows whose length is a multiple of 8 and at most 8 * 1024 * NORM_VECS: every thread
+// keeps its pieces of the row in registers, so the row is read once.  The block size depends
+// on the row length only.
+#define NORM_VECS 2
+template <bool ADD>
+__global__ __launch_bounds__(1024) void rmsnorm_bf16_vec_kernel(bf16_t* __restrict__ out, bf16_t* __restrict__ x,
+                                                                const bf16_t* __restrict__ delta,
+                                                                const float* __restrict__ w, float eps, int cols,
+                                                                int add_one) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * cols;
+    const int nvec = cols / 8;
+    float v[NORM_VECS][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_VECS; ++i) {
+        const int vi = threadIdx.x + i * blockDim.x;
+        if (vi < nvec) {
+            const uint4 raw = *(const uint4*)(x + base + (size_t)vi * 8);
+            const uint32_t wd[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[i][2 * j] = __uint_as_float(wd[j] << 16);
+                v[i][2 * j + 1] = __uint_as_float(wd[j] & 0xffff0000u);
+            }
+            if (ADD) {
+                const uint4 rd = *(const uint4*)(delta + base + (size_t)vi * 8);
+                const uint32_t dd[4] = {rd.x, rd.y, rd.z, rd.w};
+                uint32_t packed[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint16_t lo = f32_to_bf16_bits(v[i][2 * j] + __uint_as_float(dd[j] << 16));
+                    const uint16_t hi = f32_to_bf16_bits(v[i][2 * j + 1] + __uint_as_float(dd[j] & 0xffff0000u));
+                    v[i][2 * j] = bf16_bits_to_f32(lo);
+                    v[i][2 * j + 1] = bf16_bits_to_f32(hi);
+                    packed[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+                }
+                *(uint4*)(x + base + (size_t)vi * 8) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += v[i][j] * v[i][j];
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)cols + eps);
+#pragma unroll
+    for (int i = 0; i < NORM_VECS; ++i) {
+        const int vi = threadIdx.x + i * blockDim.x;
+        if (vi < nvec) {
+            const float4 w0 = *(const float4*)(w + (size_t)vi * 8), w1 = *(const float4*)(w + (size_t)vi * 8 + 4);
+            const float g[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+            uint32_t packed[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float a = scale * v[i][2 * j] * (add_one ? 1.0f + g[2 * j] : g[2 * j]);
+                const float b = scale * v[i][2 * j + 1] * (add_one ? 1.0f + g[2 * j + 1] : g[2 * j + 1]);
+                packed[j] = (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+            }
+            *(uint4*)(out + base + (size_t)vi * 8) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+        }
+    }
+}
+
 static int norm_block(int cols) { return cols >= 2048 ? 512 : (cols >= 512 ? 256 : 64); }
+
+// Threads for the register-resident kernel, or 0 when the row does not fit it.
+static int norm_vec_block(int cols, const void* a, const void* b, const void* c, const void* w) {
+    if (cols % 8 || cols > 8 * 1024 * NORM_VECS) return 0;
+    if ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)w) & 15) != 0) return 0;
+    const int nvec = cols / 8;
+    int block = 64;
+    while (block * NORM_VECS < nvec) block *= 2;       // 64 .. 1024
+    return block;
+}
 
 extern "C" int ia_rmsnorm(void* out, const void* x, const float* w, float eps, int rows, int cols,
                           int add_one, int dtype, hipStream_t stream) {
     IA_CHECK(rows >= 0 && cols > 0, "rmsnorm: bad sizes rows=%d cols=%d", rows, cols);
     if (rows == 0) return 0;
     const int block = norm_block(cols);
+    const int vblock = dtype == IA_BF16 ? norm_vec_block(cols, out, x, nullptr, w) : 0;
     if (dtype == IA_F32)
         rmsnorm_kernel<float, false><<<rows, block, 0, stream>>>((float*)out, (float*)x, nullptr, w, eps, cols, add_one);
+    else if (dtype == IA_BF16 && vblock)
+        rmsnorm_bf16_vec_kernel<false><<<rows, vblock, 0, stream>>>((bf16_t*)out, (bf16_t*)x, nullptr, w, eps, cols, add_one);
     else if (dtype == IA_BF16)
         rmsnorm_kernel<bf16_t, false><<<rows, block, 0, stream>>>((bf16_t*)out, (bf16_t*)x, nullptr, w, eps, cols, add_one);
     else
@@ -111,8 +187,11 @@ extern "C" int ia_add_rmsnorm(void* out, void* x, const void* delta, const float
     IA_CHECK(rows >= 0 && cols > 0, "add_rmsnorm: bad sizes rows=%d cols=%d", rows, cols);
     if (rows == 0) return 0;
     const int block = norm_block(cols);
+    const int vblock = dtype == IA_BF16 ? norm_vec_block(cols, out, x, delta, w) : 0;
     if (dtype == IA_F32)
         rmsnorm_kernel<float, true><<<rows, block, 0, stream>>>((float*)out, (float*)x, (const float*)delta, w, eps, cols, add_one);
+    else if (dtype == IA_BF16 && vblock)
+        rmsnorm_bf16_vec_kernel<true><<<rows, vblock, 0, stream>>>((bf16_t*)out, (bf16_t*)x, (const bf16_t*)delta, w, eps, cols, add_one);
     else if (dtype == IA_BF16)
         rmsnorm_kernel<bf16_t, true><<<rows, block, 0, stream>>>((bf16_t*)out, (bf16_t*)x, (const bf16_t*)delta, w, eps, cols, add_one);
     else

@@ -245,7 +245,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 
 
 ATTN_TARGET_WAVES = 2048       # waves wanted in flight before the keys stop being split
-ATTN_MIN_CHUNK = 128           # fewest keys a split is worth
+ATTN_MIN_CHUNK = 64            # fewest keys a split is worth
 
 
 def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int) -> bool:
