@@ -251,46 +251,71 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
     }
 }
 
-// Merges the partial results of the key splits of one (token, head): one wave a row.  Lane s
-// weighs split s (splits beyond 64 in further rounds), then every lane sums its dims over the
-// splits, in split order.
-__global__ __launch_bounds__(IA_WAVE) void attn_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
-                                                             const float* __restrict__ part_ml, int splits) {
-    __shared__ float weight[256];
-    const size_t row = blockIdx.x;
-    const int lane = threadIdx.x;
-    const float* ml = part_ml + row * splits * 2;
-    float mx = -INFINITY;
-    for (int s = lane; s < splits; s += IA_WAVE) mx = fmaxf(mx, ml[2 * s]);
-    mx = wave_max(mx);
-    float total = 0.f;
-    for (int s = lane; s < splits; s += IA_WAVE) {
-        const float ms = ml[2 * s];
-        const float w = ms == -INFINITY ? 0.f : exp2f(ms - mx);      // a split that held no key of this row
-        weight[s] = w;
-        total += ml[2 * s + 1] * w;
-    }
-    total = wave_sum(total);
-    __syncthreads();
+// Merges the partial results of the key splits of one (token, head): one block a row.  The
+// partial results were written by other compute units, so every read is a long way off: the
+// block's waves share the splits between them (wave w takes splits w, w + waves, ...) and
+// every lane has all its loads in flight at once; the waves' sums meet in shared memory and
+// are added in wave order.
+#define MERGE_WAVES 16
+__global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
+    bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits) {
     constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
-    float o[PER];
-#pragma unroll
-    for (int t = 0; t < PER; ++t) o[t] = 0.f;
+    __shared__ float weight[256];
+    __shared__ float red[MERGE_WAVES][PER * IA_WAVE];
+    __shared__ float s_total;
+    const size_t row = blockIdx.x;
+    const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+    const float* ml = part_ml + row * splits * 2;
     const float* po = part_o + row * splits * HD;
-#pragma unroll 8
-    for (int s = 0; s < splits; ++s) {
-        const float w = weight[s];
+    // this wave's partial outputs, asked for before anything is waited for
+    float v[256 / MERGE_WAVES][PER];
+#pragma unroll
+    for (int i = 0; i < 256 / MERGE_WAVES; ++i) {
+        const int s = wave + i * MERGE_WAVES;
 #pragma unroll
         for (int t = 0; t < PER; ++t) {
             const int e = lane + t * IA_WAVE;
-            if (e < HD) o[t] = fmaf(po[(size_t)s * HD + e], w, o[t]);
+            v[i][t] = (s < splits && e < HD) ? po[(size_t)s * HD + e] : 0.f;
         }
     }
-    const float inv = 1.0f / total;
+    if (wave == 0) {
+        float mx = -INFINITY;
+        for (int s = lane; s < splits; s += IA_WAVE) mx = fmaxf(mx, ml[2 * s]);
+        mx = wave_max(mx);
+        float total = 0.f;
+        for (int s = lane; s < splits; s += IA_WAVE) {
+            const float ms = ml[2 * s];
+            const float w = ms == -INFINITY ? 0.f : exp2f(ms - mx);      // a split that held no key of this row
+            weight[s] = w;
+            total += ml[2 * s + 1] * w;
+        }
+        total = wave_sum(total);
+        if (lane == 0) s_total = total;
+    }
+    __syncthreads();
+    float o[PER];
+#pragma unroll
+    for (int t = 0; t < PER; ++t) o[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 256 / MERGE_WAVES; ++i) {
+        const int s = wave + i * MERGE_WAVES;
+        if (s < splits) {
+            const float w = weight[s];
+#pragma unroll
+            for (int t = 0; t < PER; ++t) o[t] = fmaf(v[i][t], w, o[t]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < PER; ++t) red[wave][lane + t * IA_WAVE] = o[t];
+    __syncthreads();
+    if (wave != 0) return;
+    const float inv = 1.0f / s_total;
 #pragma unroll
     for (int t = 0; t < PER; ++t) {
         const int e = lane + t * IA_WAVE;
-        if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(o[t] * inv);
+        float sum = red[0][e];
+        for (int w = 1; w < MERGE_WAVES; ++w) sum += red[w][e];
+        if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(sum * inv);
     }
 }
 
@@ -343,7 +368,7 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
     }
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
-        attn_merge_kernel<<<(unsigned)((long long)n * nq), IA_WAVE, 0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits);
+        attn_merge_kernel<<<(unsigned)((long long)n * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits);
         IA_LAUNCH_CHECK("attention_merge");
     }
     return 0;

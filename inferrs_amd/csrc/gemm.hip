@@ -307,7 +307,10 @@ extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int 
             else if (rows <= 32) launch_skinny<2, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
             else launch_skinny<4, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
         } else {
-            if (rows <= 16) launch_skinny<1, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            // very tall weights (a logits head) have blocks to spare: two row tiles a wave halve the
+            // loads of the activations
+            if (rows <= 16 && N >= 65536) launch_skinny<1, 2, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            else if (rows <= 16) launch_skinny<1, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
             else if (rows <= 32) launch_skinny<2, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
             else launch_skinny<4, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
         }
