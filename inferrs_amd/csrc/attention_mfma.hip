@@ -49,19 +49,17 @@ struct AttnParams {
     const int* block_table;     // [seqs, max_pages]
     const int* cu_tokens;       // [seqs + 1]  request s owns tokens cu[s]..cu[s+1]
     const int* positions;       // [n]         absolute position of each token
-    int max_pages, nq, nkv, page, window, splits, chunk;
+    int max_pages, nq, nkv, page, window, splits, chunk, pair;
     float scale_log2;           // scale * log2(e)
 };
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
-template <int NB>
-__global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) {
+// One column block (16 * NB columns) of one request and key/value head, over one split of the keys.
+template <int NB, bool PREFETCH>
+__device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, int kvh, int split, int seq) {
     const int lane = threadIdx.x;
     const int r = lane & 15, G = lane >> 4;
-    const int cb = blockIdx.x;
-    const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
-    const int seq = blockIdx.z;
     const int g = p.nq / p.nkv;
     const int t0 = p.cu_tokens[seq], q_len = p.cu_tokens[seq + 1] - t0;
     const int n_cols = q_len * g;
@@ -117,30 +115,38 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
     }
     lo &= ~31;
 
-    for (int k0 = lo; k0 < hi; k0 += 32) {
-        // ---- operands of this step: 32 keys = two 16-slot halves, each inside one page -------
-        uint4 kreg[2][KS];      // tile t, dim step ks: row r <-> key k0 + 8*(r/4) + 4t + r%4
-        uint4 vreg[DB];         // dim block db: row r <-> dim 16 db + r, keys k0 + 8G .. +7
-        {
-            // Rows past the request's length are read from its last written slot instead (their
-            // scores are masked below): the pages behind them may not exist.
+    // ---- operands of a step: 32 keys = two 16-slot halves, each inside one page --------------
+    struct Operands {
+        uint4 k[2][KS];         // tile t, dim step ks: row r <-> key k0 + 8*(r/4) + 4t + r%4
+        uint4 v[DB];            // dim block db: row r <-> dim 16 db + r, keys k0 + 8G .. +7
+    };
+    auto load_step = [&](Operands& op, int k0) {
+        // Rows past the request's length are read from its last written slot instead (their
+        // scores are masked in the step): the pages behind them may not exist.  The two halves
+        // of a step lie in at most two pages, whose numbers are the same for every lane: they
+        // come through the scalar cache, and no load of a key waits for a load of its address.
+        const int last_idx = (kv_total - 1) / p.page;
+        const int idx_a = k0 / p.page;
+        const int idx_b = (k0 + 16) / p.page < last_idx ? (k0 + 16) / p.page : last_idx;
+        const int page_a = bt[idx_a], page_b = bt[idx_b];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                int key = k0 + 8 * (r >> 2) + 4 * t + (r & 3);
-                key = key < kv_total ? key : kv_total - 1;
-                const int kpage = bt[key / p.page];
-                const bf16_t* krow = p.k_cache + (((size_t)kpage * p.nkv + kvh) * p.page + key % p.page) * HD + G * 8;
+        for (int t = 0; t < 2; ++t) {
+            int key = k0 + 8 * (r >> 2) + 4 * t + (r & 3);
+            key = key < kv_total ? key : kv_total - 1;
+            const int kpage = key / p.page == idx_a ? page_a : page_b;
+            const bf16_t* krow = p.k_cache + (((size_t)kpage * p.nkv + kvh) * p.page + key % p.page) * HD + G * 8;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    kreg[t][ks] = (ks * 32 + G * 8 < HD) ? *(const uint4*)(krow + ks * 32) : zero4();
-            }
-            int vkey = k0 + 8 * G;
-            vkey = vkey < kv_total ? vkey : (kv_total - 1) & ~7;
-            const int vpage = bt[vkey / p.page];
-            const bf16_t* vbase = p.v_cache + (((size_t)vpage * p.nkv + kvh) * HD + r) * p.page + vkey % p.page;
-#pragma unroll
-            for (int db = 0; db < DB; ++db) vreg[db] = *(const uint4*)(vbase + (size_t)db * 16 * p.page);
+            for (int ks = 0; ks < KS; ++ks)
+                op.k[t][ks] = (ks * 32 + G * 8 < HD) ? *(const uint4*)(krow + ks * 32) : zero4();
         }
+        int vkey = k0 + 8 * G;
+        vkey = vkey < kv_total ? vkey : (kv_total - 1) & ~7;
+        const int vpage = vkey / p.page == idx_a ? page_a : page_b;
+        const bf16_t* vbase = p.v_cache + (((size_t)vpage * p.nkv + kvh) * HD + r) * p.page + vkey % p.page;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) op.v[db] = *(const uint4*)(vbase + (size_t)db * 16 * p.page);
+    };
+    auto compute_step = [&](Operands& op, int k0) {
         const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
         if (k0 + 32 > kv_total) {
             // slots beyond the request's length hold anything at all: zero those values so that
@@ -149,15 +155,14 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
             if (first_bad < 8) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    uint32_t w[4] = {vreg[db].x, vreg[db].y, vreg[db].z, vreg[db].w};
+                    uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
                         if (j >= first_bad) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
-                    vreg[db] = make_uint4(w[0], w[1], w[2], w[3]);
+                    op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
                 }
             }
         }
-
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             // ---- S^T for 32 keys x 16 columns ----------------------------------------------
@@ -168,13 +173,14 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks)
                     s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8, kreg[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), s[t], 0, 0, 0);
+                        __builtin_bit_cast(bf16x8, op.k[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), s[t], 0, 0, 0);
             }
+            // raw scores; the scale (> 0) and the change to base 2 are folded into the exponent below
             float sc[8];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sc[4 * t + i] = s[t][i] * p.scale_log2;
+                for (int i = 0; i < 4; ++i) sc[4 * t + i] = s[t][i];
             if (edge) {
                 const int kbase_idx = k0 + 8 * G;
                 const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
@@ -184,27 +190,25 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
                     if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
                 }
             }
-            float mx = sc[0];
-#pragma unroll
-            for (int j = 1; j < 8; ++j) mx = fmaxf(mx, sc[j]);
+            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
             mx = fmaxf(mx, __shfl_xor(mx, 16, IA_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, IA_WAVE));
-            const float m_new = fmaxf(m[nb], mx);
+            const float m_new = fmaxf(m[nb], mx * p.scale_log2);        // running maximum of scale * log2(e) * score
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = exp2f(m[nb] - m_use);       // m = -inf gives 0
+            const float alpha = __builtin_amdgcn_exp2f(m[nb] - m_use);  // m = -inf gives 0
             float pr[8], psum = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                pr[j] = exp2f(sc[j] - m_use);
+                pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], p.scale_log2, -m_use));
                 psum += pr[j];
             }
             l[nb] = l[nb] * alpha + psum;
             m[nb] = m_new;
             uint4 pb;
-            pb.x = (uint32_t)f32_to_bf16_bits(pr[0]) | ((uint32_t)f32_to_bf16_bits(pr[1]) << 16);
-            pb.y = (uint32_t)f32_to_bf16_bits(pr[2]) | ((uint32_t)f32_to_bf16_bits(pr[3]) << 16);
-            pb.z = (uint32_t)f32_to_bf16_bits(pr[4]) | ((uint32_t)f32_to_bf16_bits(pr[5]) << 16);
-            pb.w = (uint32_t)f32_to_bf16_bits(pr[6]) | ((uint32_t)f32_to_bf16_bits(pr[7]) << 16);
+            pb.x = pack_bf16x2(pr[0], pr[1]);
+            pb.y = pack_bf16x2(pr[2], pr[3]);
+            pb.z = pack_bf16x2(pr[4], pr[5]);
+            pb.w = pack_bf16x2(pr[6], pr[7]);
             // ---- O^T += V^T . P^T ----------------------------------------------------------
             if (__any(alpha != 1.0f)) {
 #pragma unroll
@@ -216,7 +220,27 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
 #pragma unroll
             for (int db = 0; db < DB; ++db)
                 acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8, vreg[db]), __builtin_bit_cast(bf16x8, pb), acc[nb][db], 0, 0, 0);
+                    __builtin_bit_cast(bf16x8, op.v[db]), __builtin_bit_cast(bf16x8, pb), acc[nb][db], 0, 0, 0);
+        }
+    };
+
+    if (PREFETCH) {
+        // Two sets of operands: the next step's keys and values are on their way while this
+        // step's are multiplied.
+        Operands opa, opb;
+        if (lo < hi) load_step(opa, lo);
+        for (int k0 = lo; k0 < hi; k0 += 64) {
+            if (k0 + 32 < hi) load_step(opb, k0 + 32);
+            compute_step(opa, k0);
+            if (k0 + 32 >= hi) break;
+            if (k0 + 64 < hi) load_step(opa, k0 + 64);
+            compute_step(opb, k0 + 32);
+        }
+    } else {
+        for (int k0 = lo; k0 < hi; k0 += 32) {
+            Operands op;
+            load_step(op, k0);
+            compute_step(op, k0);
         }
     }
 
@@ -234,8 +258,8 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 uint2 w;
-                w.x = (uint32_t)f32_to_bf16_bits(acc[nb][db][0] * inv) | ((uint32_t)f32_to_bf16_bits(acc[nb][db][1] * inv) << 16);
-                w.y = (uint32_t)f32_to_bf16_bits(acc[nb][db][2] * inv) | ((uint32_t)f32_to_bf16_bits(acc[nb][db][3] * inv) << 16);
+                w.x = pack_bf16x2(acc[nb][db][0] * inv, acc[nb][db][1] * inv);
+                w.y = pack_bf16x2(acc[nb][db][2] * inv, acc[nb][db][3] * inv);
                 *(uint2*)(o + 16 * db) = w;
             }
         } else {
@@ -249,6 +273,27 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
             }
         }
     }
+}
+
+// With `pair` a wave takes column block i from the end of its request and then block i from the
+// start: under a causal mask the late blocks walk many keys and the early ones few, and every
+// pair walks about the same number, so all waves end together.  It pays when the step's queries
+// span most of the context; a short portion late in a long context has equal blocks already.
+template <int NB, bool PREFETCH>
+__global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) {
+    const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
+    const int seq = blockIdx.z;
+    const int n_cols = (p.cu_tokens[seq + 1] - p.cu_tokens[seq]) * (p.nq / p.nkv);
+    const int n_blocks = (n_cols + 16 * NB - 1) / (16 * NB);
+    if (!p.pair) {
+        // heavy column blocks first
+        if ((int)blockIdx.x < n_blocks) attn_column_block<NB, PREFETCH>(p, n_blocks - 1 - (int)blockIdx.x, kvh, split, seq);
+        return;
+    }
+    const int late = n_blocks - 1 - (int)blockIdx.x, early = (int)blockIdx.x;
+    if (late < early) return;
+    attn_column_block<NB, PREFETCH>(p, late, kvh, split, seq);
+    if (early != late) attn_column_block<NB, PREFETCH>(p, early, kvh, split, seq);
 }
 
 // Merges the partial results of the key splits of one (token, head): one block a row.  The
@@ -321,6 +366,13 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 
 extern "C" int ia_attention_mfma_head_dim(void) { return HD; }
 
+// Tuning: columns a wave for long portions (2 or 4 tiles of 16), and whether the next step's
+// operands are loaded ahead, for decode and for portions.
+static int g_nb_prefill = 4, g_pf_decode = 0, g_pf_prefill = 0;
+extern "C" void ia_attention_mfma_tune(int nb_prefill, int pf_decode, int pf_prefill) {
+    g_nb_prefill = nb_prefill; g_pf_decode = pf_decode; g_pf_prefill = pf_prefill;
+}
+
 // Floats of workspace that `splits` > 1 needs: partial outputs, then maxima and sums.
 extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
     return splits > 1 ? (long long)n * nq * splits * (HD + 2) : 0;
@@ -330,7 +382,7 @@ extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
 // of 32, splits * chunk >= the longest request's length after the step).
 extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
                                  const void* v_cache, const int* block_table, const int* cu_tokens,
-                                 const int* positions, int n, int n_seqs, int max_q_len, int max_pages,
+                                 const int* positions, int n, int n_seqs, int max_q_len, int max_kv_len, int max_pages,
                                  int nq, int nkv, int d, int page_size, int window, float scale,
                                  int splits, int chunk, hipStream_t stream) {
     IA_CHECK(d == HD, "attention_mfma: built for head_dim %d, called with %d", HD, d);
@@ -359,13 +411,25 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
     p.splits = splits; p.chunk = chunk;
     p.scale_log2 = scale * 1.4426950408889634f;
     const long long cols = (long long)max_q_len * g;
-    if (cols <= 16) {
-        const dim3 grid(1, nkv * splits, n_seqs);
-        attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
-    } else {
-        const dim3 grid((unsigned)((cols + 31) / 32), nkv * splits, n_seqs);
-        attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
+    // Columns a wave: 16 for decode; 32 or 64 for portions of prompts (64 keeps every loaded key
+    // and value in use for twice as many products, but leaves half as many waves).
+    p.pair = (splits == 1 && cols > 16 && 2LL * max_q_len > max_kv_len) ? 1 : 0;
+    int nb = 1;
+    if (cols > 16) {
+        const long long waves4 = ((cols + 63) / 64 + p.pair) / (1 + p.pair) * nkv * splits * n_seqs;
+        nb = (HD <= 128 && g_nb_prefill == 4 && waves4 >= 1024) ? 4 : 2;
     }
+    const bool pf = HD <= 128 && (nb == 1 ? g_pf_decode : g_pf_prefill) != 0;
+    const long long col_blocks = (cols + 16 * nb - 1) / (16 * nb);
+    const dim3 grid((unsigned)(p.pair ? (col_blocks + 1) / 2 : col_blocks), nkv * splits, n_seqs);
+    if (nb == 1 && pf) attn_mfma_kernel<1, true><<<grid, IA_WAVE, 0, stream>>>(p);
+    else if (nb == 1) attn_mfma_kernel<1, false><<<grid, IA_WAVE, 0, stream>>>(p);
+    else if (nb == 2 && pf) attn_mfma_kernel<2, true><<<grid, IA_WAVE, 0, stream>>>(p);
+    else if (nb == 2) attn_mfma_kernel<2, false><<<grid, IA_WAVE, 0, stream>>>(p);
+#if IA_HEAD_DIM <= 128
+    else if (pf) attn_mfma_kernel<4, true><<<grid, IA_WAVE, 0, stream>>>(p);
+    else attn_mfma_kernel<4, false><<<grid, IA_WAVE, 0, stream>>>(p);
+#endif
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
         attn_merge_kernel<<<(unsigned)((long long)n * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits);

@@ -24,6 +24,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// Two 32-bit values to two bfloat16 in one word (low half first), rounded to nearest even by
+// the hardware conversion.
+typedef __bf16 ia_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float ia_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const ia_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ia_bf16x2));
+}
+
 __device__ __forceinline__ float ld(const float* p) { return *p; }
 __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_bits_to_f32(p->bits); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }

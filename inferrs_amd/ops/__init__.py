@@ -256,7 +256,7 @@ def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: i
     """(splits, keys per split) for the matrix-core kernel: the keys are split between waves
     when the batch alone has too few (request, kv head, column block) items to fill the chip."""
     cols = max_q_len * g
-    col_blocks = 1 if cols <= 16 else -(-cols // 32)
+    col_blocks = 1 if cols <= 16 else -(-cols // 32)      # (64 columns a wave beyond 256: then nothing is split anyway)
     items = n_seqs * nkv * col_blocks
     splits = 1
     while items * splits < ATTN_TARGET_WAVES and max_kv_len >= 2 * splits * ATTN_MIN_CHUNK and splits < 128:
@@ -299,7 +299,7 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     ws = torch.empty((ws_floats,), dtype=torch.float32, device=q.device) if ws_floats else None
     _check(lib.ia_attention_mfma(
         _p(out), _p(ws), _p(q), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions),
-        n, n_seqs, max_q_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
+        n, n_seqs, max_q_len, max_kv_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
         ctypes.c_float(scale), splits, chunk, _stream()), target)
     return out
 
