@@ -146,30 +146,53 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     // channels at any moment.  The order of the sum depends on the block (the output feature)
     // only, never on the batch.  Whole steps run without a condition; a last step that K does
     // not fill is done apart, with zeros beyond K.
-    constexpr int UNROLL = (NA * RT >= 4) ? 2 : (NA * RT == 2 ? 4 : 8);
+    // A chunk of k steps has all its loads under way before its first product: a wave is one of
+    // few on its SIMD when the weight is small, and what it has in flight is what hides the memory's
+    // latency.
+    constexpr int UNROLL = (NA * RT * MT >= 8) ? 2 : (NA * RT * MT >= 4 ? 4 : (NA * RT * MT == 2 ? 8 : 16));
     const int whole = K / SK_KSTEP;                         // steps that lie inside K entirely
     const int ke = ks1 < whole ? ks1 : whole;
     const int len = ke - ks0;
     const int rot = len > 0 ? (int)((blockIdx.x * (unsigned)rot_mul) % (unsigned)len) / UNROLL * UNROLL : 0;
     for (int part = 0; part < 2; ++part) {
         const int pa = part == 0 ? ks0 + rot : ks0, pb = part == 0 ? ke : ks0 + rot;
-#pragma unroll UNROLL
-        for (int ks = pa; ks < pb; ++ks) {
+        int ks = pa;
+        for (; ks + UNROLL <= pb; ks += UNROLL) {
+            uint4 a[UNROLL][NA][RT], b[UNROLL][MT];
+#pragma unroll
+            for (int i = 0; i < UNROLL; ++i)
+#pragma unroll
+                for (int q = 0; q < NA; ++q)
+#pragma unroll
+                    for (int t = 0; t < RT; ++t) a[i][q][t] = *(const uint4*)(wrow[q][t] + (ks + i) * SK_KSTEP);
+#pragma unroll
+            for (int i = 0; i < UNROLL; ++i)
+#pragma unroll
+                for (int u = 0; u < MT; ++u) b[i][u] = *(const uint4*)(xrow[u] + (ks + i) * SK_KSTEP);
+#pragma unroll
+            for (int i = 0; i < UNROLL; ++i)
+#pragma unroll
+                for (int u = 0; u < MT; ++u)
+#pragma unroll
+                    for (int q = 0; q < NA; ++q)
+#pragma unroll
+                        for (int t = 0; t < RT; ++t)
+                            acc[q][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                __builtin_bit_cast(bf16x8, a[i][q][t]), __builtin_bit_cast(bf16x8, b[i][u]), acc[q][t][u], 0, 0, 0);
+        }
+        for (; ks < pb; ++ks) {
             const int k0 = ks * SK_KSTEP;
-            uint4 a[NA][RT];
-#pragma unroll
-            for (int q = 0; q < NA; ++q)
-#pragma unroll
-                for (int t = 0; t < RT; ++t) a[q][t] = *(const uint4*)(wrow[q][t] + k0);
 #pragma unroll
             for (int u = 0; u < MT; ++u) {
                 const uint4 b = *(const uint4*)(xrow[u] + k0);
 #pragma unroll
                 for (int q = 0; q < NA; ++q)
 #pragma unroll
-                    for (int t = 0; t < RT; ++t)
+                    for (int t = 0; t < RT; ++t) {
+                        const uint4 a = *(const uint4*)(wrow[q][t] + k0);
                         acc[q][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8, a[q][t]), __builtin_bit_cast(bf16x8, b), acc[q][t][u], 0, 0, 0);
+                            __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc[q][t][u], 0, 0, 0);
+                    }
             }
         }
     }

@@ -86,6 +86,98 @@ __global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_kernel(
     for (int j = rot + lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
 }
 
+// The same work with 16-byte accesses, for bfloat16 and head sizes that are a multiple of 8:
+// a thread owns eight neighbouring features of one (token, head); the threads of a head meet in
+// shared memory for the sum of squares and for their rotation partners.
+#define QKV_THREADS 256
+__global__ __launch_bounds__(QKV_THREADS) void qk_rope_kv_bf16_vec_kernel(
+    bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+    const bf16_t* __restrict__ qkv, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ slots,
+    int n, int nq, int nkv, int d, int rot, int interleaved, int page_size, float eps, int add_one) {
+    __shared__ float rows[QKV_THREADS * 8];          // normalised features, unit after unit
+    __shared__ float partial[QKV_THREADS];
+    const int tpu = d / 8;                            // threads a (token, head) unit
+    const int units_per_block = QKV_THREADS / tpu;
+    const int u = threadIdx.x / tpu, t = threadIdx.x - u * tpu;
+    const int heads = slots ? nq + 2 * nkv : nq;
+    const long long unit = (long long)blockIdx.x * units_per_block + u;
+    const bool active = u < units_per_block && unit < (long long)n * heads;
+    const int tok = active ? (int)(unit / heads) : 0;
+    const int hh = active ? (int)(unit % heads) : 0;
+    const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);
+    float v[8];
+    float ss = 0.f;
+    if (active) {
+        const uint4 raw = *(const uint4*)(qkv + ((size_t)tok * (nq + 2 * nkv) + hh) * d + t * 8);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __uint_as_float(w[j] << 16);
+            v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+    }
+    partial[threadIdx.x] = ss;
+    __syncthreads();
+    const float* nw = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+    if (active && nw != nullptr) {
+        float total = 0.f;
+        for (int i = 0; i < tpu; ++i) total += partial[u * tpu + i];      // the same order in every thread
+        const float scale = 1.0f / sqrtf(total / (float)d + eps);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float g = nw[t * 8 + j];
+            v[j] = scale * v[j] * (add_one ? 1.0f + g : g);
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rows[threadIdx.x * 8 + j] = v[j];
+    }
+    __syncthreads();
+    if (!active) return;
+    if (kind == 2) {
+        // values are kept transposed inside a page: [dim][slot]
+        const int slot = slots[tok];
+        const int page = slot / page_size, off = slot - page * page_size;
+        bf16_t* vt = v_cache + ((size_t)page * nkv + (hh - nq - nkv)) * d * page_size + off;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) st(vt + (size_t)(t * 8 + j) * page_size, v[j]);
+        return;
+    }
+    if (cos_t != nullptr) {
+        const int half = rot / 2;
+        const float* row = rows + (size_t)u * tpu * 8;
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int e = t * 8 + j;
+            o[j] = v[j];
+            if (e < rot) {
+                const int i = interleaved ? e >> 1 : (e < half ? e : e - half);
+                const bool first = interleaved ? (e & 1) == 0 : e < half;
+                const int partner = interleaved ? e ^ 1 : (first ? e + half : e - half);
+                const float c = cos_t[(size_t)tok * half + i], s = sin_t[(size_t)tok * half + i];
+                o[j] = first ? v[j] * c - row[partner] * s : row[partner] * s + v[j] * c;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = o[j];
+    }
+    bf16_t* dst;
+    if (kind == 0) {
+        dst = q_out + ((size_t)tok * nq + hh) * d;
+    } else {
+        const int slot = slots[tok];
+        const int page = slot / page_size, off = slot - page * page_size;
+        dst = k_cache + (((size_t)page * nkv + (hh - nq)) * page_size + off) * d;
+    }
+    *(uint4*)(dst + t * 8) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
+                                        pack_bf16x2(v[6], v[7]));
+}
+
 extern "C" int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const void* qkv,
                              const float* q_norm_w, const float* k_norm_w, const float* cos_t,
                              const float* sin_t, const int* slots, int n, int nq, int nkv, int d,
@@ -100,6 +192,16 @@ extern "C" int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const vo
     if (n == 0) return 0;
     const long long units = (long long)n * (slots ? nq + 2 * nkv : nq);
     const unsigned grid = (unsigned)((units + QK_WAVES - 1) / QK_WAVES);
+    const uintptr_t ptrs = (uintptr_t)q_out | (uintptr_t)qkv | (uintptr_t)(slots ? k_cache : nullptr);
+    if (dtype == IA_BF16 && d % 8 == 0 && d / 8 <= QKV_THREADS && (ptrs & 15) == 0) {
+        const int units_per_block = QKV_THREADS / (d / 8);
+        const unsigned vgrid = (unsigned)((units + units_per_block - 1) / units_per_block);
+        qk_rope_kv_bf16_vec_kernel<<<vgrid, QKV_THREADS, 0, stream>>>(
+            (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)qkv, q_norm_w, k_norm_w,
+            cos_t, sin_t, slots, n, nq, nkv, d, rot, interleaved, page_size, eps, add_one);
+        IA_LAUNCH_CHECK("qk_rope_kv");
+        return 0;
+    }
     if (dtype == IA_F32)
         qk_rope_kv_kernel<float><<<grid, QK_WAVES * IA_WAVE, 0, stream>>>(
             (float*)q_out, (float*)k_cache, (float*)v_cache, (const float*)qkv, q_norm_w, k_norm_w,
