@@ -57,7 +57,8 @@ int ia_attention_mfma_head_dim(void);
 long long ia_attention_mfma_workspace(int n, int nq, int splits);
 int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
                       const void* v_cache, const int* block_table, const int* cu_tokens,
-                      const int* positions, int n, int n_seqs, int max_q_len, int max_kv_len, int max_pages,
+                      const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
+                      int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                       int nq, int nkv, int d, int page_size, int window, float scale,
                       int splits, int chunk, hipStream_t stream);
 

@@ -49,14 +49,14 @@ struct AttnParams {
     const int* block_table;     // [seqs, max_pages]
     const int* cu_tokens;       // [seqs + 1]  request s owns tokens cu[s]..cu[s+1]
     const int* positions;       // [n]         absolute position of each token
-    int max_pages, nq, nkv, page, window, splits, chunk, pair;
+    int max_pages, nq, nkv, page, window, splits, chunk, pair, seq_begin;
     float scale_log2;           // scale * log2(e)
 };
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
 // One column block (16 * NB columns) of one request and key/value head, over one split of the keys.
-template <int NB, bool PREFETCH>
+template <int NB>
 __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, int kvh, int split, int seq) {
     const int lane = threadIdx.x;
     const int r = lane & 15, G = lane >> 4;
@@ -224,24 +224,12 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         }
     };
 
-    if (PREFETCH) {
-        // Two sets of operands: the next step's keys and values are on their way while this
-        // step's are multiplied.
-        Operands opa, opb;
-        if (lo < hi) load_step(opa, lo);
-        for (int k0 = lo; k0 < hi; k0 += 64) {
-            if (k0 + 32 < hi) load_step(opb, k0 + 32);
-            compute_step(opa, k0);
-            if (k0 + 32 >= hi) break;
-            if (k0 + 64 < hi) load_step(opa, k0 + 64);
-            compute_step(opb, k0 + 32);
-        }
-    } else {
-        for (int k0 = lo; k0 < hi; k0 += 32) {
-            Operands op;
-            load_step(op, k0);
-            compute_step(op, k0);
-        }
+    // (Loading the next step's operands ahead of this step's products was tried and lost: it
+    // doubles the operand registers, which costs a wave per SIMD, and that wave hid more latency.)
+    for (int k0 = lo; k0 < hi; k0 += 32) {
+        Operands op;
+        load_step(op, k0);
+        compute_step(op, k0);
     }
 
     // ---- results: lane (col, G) holds dims 16 db + 4 G + i of its column ---------------------
@@ -279,21 +267,21 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
 // start: under a causal mask the late blocks walk many keys and the early ones few, and every
 // pair walks about the same number, so all waves end together.  It pays when the step's queries
 // span most of the context; a short portion late in a long context has equal blocks already.
-template <int NB, bool PREFETCH>
+template <int NB>
 __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) {
     const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
-    const int seq = blockIdx.z;
+    const int seq = p.seq_begin + blockIdx.z;
     const int n_cols = (p.cu_tokens[seq + 1] - p.cu_tokens[seq]) * (p.nq / p.nkv);
     const int n_blocks = (n_cols + 16 * NB - 1) / (16 * NB);
     if (!p.pair) {
         // heavy column blocks first
-        if ((int)blockIdx.x < n_blocks) attn_column_block<NB, PREFETCH>(p, n_blocks - 1 - (int)blockIdx.x, kvh, split, seq);
+        if ((int)blockIdx.x < n_blocks) attn_column_block<NB>(p, n_blocks - 1 - (int)blockIdx.x, kvh, split, seq);
         return;
     }
     const int late = n_blocks - 1 - (int)blockIdx.x, early = (int)blockIdx.x;
     if (late < early) return;
-    attn_column_block<NB, PREFETCH>(p, late, kvh, split, seq);
-    if (early != late) attn_column_block<NB, PREFETCH>(p, early, kvh, split, seq);
+    attn_column_block<NB>(p, late, kvh, split, seq);
+    if (early != late) attn_column_block<NB>(p, early, kvh, split, seq);
 }
 
 // Merges the partial results of the key splits of one (token, head): one block a row.  The
@@ -303,12 +291,13 @@ __global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) 
 // are added in wave order.
 #define MERGE_WAVES 16
 __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
-    bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits) {
+    bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
+    size_t first_row) {
     constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
     __shared__ float weight[256];
     __shared__ float red[MERGE_WAVES][PER * IA_WAVE];
     __shared__ float s_total;
-    const size_t row = blockIdx.x;
+    const size_t row = first_row + blockIdx.x;
     const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
     const float* ml = part_ml + row * splits * 2;
     const float* po = part_o + row * splits * HD;
@@ -366,28 +355,30 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 
 extern "C" int ia_attention_mfma_head_dim(void) { return HD; }
 
-// Tuning: columns a wave for long portions (2 or 4 tiles of 16), and whether the next step's
-// operands are loaded ahead, for decode and for portions.
-static int g_nb_prefill = 4, g_pf_decode = 0, g_pf_prefill = 0;
-extern "C" void ia_attention_mfma_tune(int nb_prefill, int pf_decode, int pf_prefill) {
-    g_nb_prefill = nb_prefill; g_pf_decode = pf_decode; g_pf_prefill = pf_prefill;
-}
+// Tuning: columns a wave for long portions (2 or 4 tiles of 16).
+static int g_nb_prefill = 4;
+extern "C" void ia_attention_mfma_tune(int nb_prefill) { g_nb_prefill = nb_prefill; }
 
 // Floats of workspace that `splits` > 1 needs: partial outputs, then maxima and sums.
 extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
     return splits > 1 ? (long long)n * nq * splits * (HD + 2) : 0;
 }
 
-// max_q_len: the most tokens any request has in this step; `chunk`: keys per split (a multiple
-// of 32, splits * chunk >= the longest request's length after the step).
+// The requests seq_begin .. seq_begin + n_seqs of the step, whose tokens are token_begin ..
+// token_begin + n_tokens of its n.  max_q_len: the most tokens any of them has in this step;
+// max_kv_len: their greatest length after it; `chunk`: keys per split (a multiple of 32,
+// splits * chunk >= max_kv_len).  The workspace is sized for all n tokens.
 extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
                                  const void* v_cache, const int* block_table, const int* cu_tokens,
-                                 const int* positions, int n, int n_seqs, int max_q_len, int max_kv_len, int max_pages,
+                                 const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
+                                 int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                                  int nq, int nkv, int d, int page_size, int window, float scale,
                                  int splits, int chunk, hipStream_t stream) {
     IA_CHECK(d == HD, "attention_mfma: built for head_dim %d, called with %d", HD, d);
     IA_CHECK(n >= 0 && n_seqs >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0,
              "attention_mfma: bad sizes n=%d seqs=%d nq=%d nkv=%d", n, n_seqs, nq, nkv);
+    IA_CHECK(seq_begin >= 0 && token_begin >= 0 && n_tokens >= 0 && token_begin + n_tokens <= n,
+             "attention_mfma: bad ranges seq_begin=%d tokens %d..+%d of %d", seq_begin, token_begin, n_tokens, n);
     IA_CHECK(page_size > 0 && page_size % 16 == 0, "attention_mfma: page size %d must be a multiple of 16", page_size);
     IA_CHECK(max_pages > 0 && window >= 0 && max_q_len >= 1, "attention_mfma: bad geometry max_pages=%d window=%d max_q_len=%d",
              max_pages, window, max_q_len);
@@ -395,7 +386,7 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
              "attention_mfma: bad split of the keys (splits=%d chunk=%d)", splits, chunk);
     IA_CHECK((long long)nkv * splits <= 65535 && n_seqs <= 65535, "attention_mfma: grid too large (nkv*splits=%d seqs=%d)",
              nkv * splits, n_seqs);
-    if (n == 0 || n_seqs == 0) return 0;
+    if (n_tokens == 0 || n_seqs == 0) return 0;
     const int g = nq / nkv;
     AttnParams p;
     p.out = (bf16_t*)out;
@@ -408,7 +399,7 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
     p.cu_tokens = cu_tokens;
     p.positions = positions;
     p.max_pages = max_pages; p.nq = nq; p.nkv = nkv; p.page = page_size; p.window = window;
-    p.splits = splits; p.chunk = chunk;
+    p.splits = splits; p.chunk = chunk; p.seq_begin = seq_begin;
     p.scale_log2 = scale * 1.4426950408889634f;
     const long long cols = (long long)max_q_len * g;
     // Columns a wave: 16 for decode; 32 or 64 for portions of prompts (64 keeps every loaded key
@@ -419,20 +410,17 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
         const long long waves4 = ((cols + 63) / 64 + p.pair) / (1 + p.pair) * nkv * splits * n_seqs;
         nb = (HD <= 128 && g_nb_prefill == 4 && waves4 >= 1024) ? 4 : 2;
     }
-    const bool pf = HD <= 128 && (nb == 1 ? g_pf_decode : g_pf_prefill) != 0;
     const long long col_blocks = (cols + 16 * nb - 1) / (16 * nb);
     const dim3 grid((unsigned)(p.pair ? (col_blocks + 1) / 2 : col_blocks), nkv * splits, n_seqs);
-    if (nb == 1 && pf) attn_mfma_kernel<1, true><<<grid, IA_WAVE, 0, stream>>>(p);
-    else if (nb == 1) attn_mfma_kernel<1, false><<<grid, IA_WAVE, 0, stream>>>(p);
-    else if (nb == 2 && pf) attn_mfma_kernel<2, true><<<grid, IA_WAVE, 0, stream>>>(p);
-    else if (nb == 2) attn_mfma_kernel<2, false><<<grid, IA_WAVE, 0, stream>>>(p);
+    if (nb == 1) attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
+    else if (nb == 2) attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
 #if IA_HEAD_DIM <= 128
-    else if (pf) attn_mfma_kernel<4, true><<<grid, IA_WAVE, 0, stream>>>(p);
-    else attn_mfma_kernel<4, false><<<grid, IA_WAVE, 0, stream>>>(p);
+    else attn_mfma_kernel<4><<<grid, IA_WAVE, 0, stream>>>(p);
 #endif
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
-        attn_merge_kernel<<<(unsigned)((long long)n * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits);
+        attn_merge_kernel<<<(unsigned)((long long)n_tokens * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>(
+            (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq);
         IA_LAUNCH_CHECK("attention_merge");
     }
     return 0;

@@ -43,6 +43,9 @@ class StepContext:
     state_slots_host: List[int] = field(default_factory=list)
     max_q_len: int = 0
     max_kv_len: int = 0
+    n_single: int = 0            # the first n_single requests bring one token each (they come first)
+    max_kv_single: int = 0       # the greatest length among those, after the step
+    max_kv_multi: int = 0        # and among the others
     _tables: Dict[Any, Any] = field(default_factory=dict)
 
     @property
@@ -114,6 +117,12 @@ class StepBuilder:
         least what the longest request needs); with it the place of every array in the staging
         buffer depends on the counts of tokens, requests and wanted rows only."""
         ps = self.cache.page_size
+        # Requests with a single token go first (in their order), the others after them: mixers
+        # can then treat the two runs apart.  Wanted rows keep the callers' order.
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i][1]) != 1)
+        rank = {orig: new for new, orig in enumerate(order)}
+        given = entries
+        entries = [given[i] for i in order]
         seqs = [self.cache.sequences[e[0]] for e in entries]
         q_lens = [len(e[1]) for e in entries]
         starts = [s.length for s in seqs]
@@ -134,7 +143,7 @@ class StepBuilder:
             token_ids = np.concatenate([np.asarray(e[1], dtype=np.int32) for e in entries])
             positions = np.concatenate([np.arange(st, st + q, dtype=np.int32) for st, q in zip(starts, q_lens)])
             token_seq = np.repeat(np.arange(s_count, dtype=np.int32), q_lens)
-        want = np.asarray([cu[i] + w for i, e in enumerate(entries) for w in e[2]], dtype=np.int32)
+        want = np.asarray([cu[rank[i]] + w for i, e in enumerate(given) for w in e[2]], dtype=np.int32)
         state_slots = np.asarray([s.state_slot for s in seqs], dtype=np.int32)
         tables, slots = [], []
         for g in range(n_groups):
@@ -171,8 +180,14 @@ class StepBuilder:
         groups = [GroupStep(ps, views[6 + 2 * g], views[7 + 2 * g].view(s_count, max_pages))
                   for g in range(n_groups)]
         max_kv = max(st + q for st, q in zip(starts, q_lens))
+        n_single = sum(1 for q in q_lens if q == 1)
+        kv_single = max([st + 1 for st, q in zip(starts, q_lens) if q == 1], default=0)
+        kv_multi = max([st + q for st, q in zip(starts, q_lens) if q != 1], default=0)
+        if pad_pages is not None:
+            kv_single = max(kv_single, pad_pages * ps) if n_single else 0
         return StepContext(
             n_tokens=n, n_seqs=s_count, token_ids=views[0], positions=views[1], token_seq=views[2],
             cu_tokens=views[3], state_slots=views[4], want_rows=views[5], groups=groups,
             q_lens=q_lens, kv_starts=starts, state_slots_host=[int(x) for x in state_slots],
-            max_q_len=max(q_lens), max_kv_len=max_kv if pad_pages is None else max(max_kv, pad_pages * ps))
+            max_q_len=max(q_lens), max_kv_len=max_kv if pad_pages is None else max(max_kv, pad_pages * ps),
+            n_single=n_single, max_kv_single=kv_single, max_kv_multi=kv_multi)

@@ -268,12 +268,16 @@ def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: i
 
 def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
                    cu_tokens: torch.Tensor, block_table: torch.Tensor, *, max_q_len: int, max_kv_len: int,
-                   window: Optional[int], scale: float, splits: Optional[int] = None) -> torch.Tensor:
+                   window: Optional[int], scale: float, splits: Optional[int] = None,
+                   seqs: Optional[Tuple[int, int]] = None, tokens: Optional[Tuple[int, int]] = None,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The matrix-core kernel: bfloat16, head sizes in steps of 16 up to 256, page sizes in steps
-    of 16.  Request s owns tokens cu_tokens[s]..cu_tokens[s+1] at consecutive positions;
-    `max_q_len` and `max_kv_len` are the largest token count of a request in this step and the
-    largest length after it."""
-    _dev(q, k_cache, v_cache, positions, cu_tokens, block_table)
+    of 16.  Request s owns tokens cu_tokens[s]..cu_tokens[s+1] at consecutive positions.  `seqs` =
+    (first, count) and `tokens` = (first, count) restrict the call to a run of requests and their
+    tokens (the whole step by default); `max_q_len` and `max_kv_len` are the largest token count of
+    one of these requests in this step and their largest length after it.  `out` receives the result
+    (rows outside `tokens` are left alone)."""
+    _dev(q, k_cache, v_cache, positions, cu_tokens, block_table, out)
     _i32(positions, "positions"); _i32(cu_tokens, "cu_tokens"); _i32(block_table, "block_table")
     n, nq, d = q.shape
     nkv, page_size = k_cache.shape[1], k_cache.shape[2]
@@ -282,25 +286,31 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise KernelError(f"attention_mfma: takes bfloat16, head sizes {_build.ATTN_HEAD_DIMS[0]}.."
                           f"{_build.ATTN_HEAD_DIMS[-1]} in steps of 16 and page sizes in steps of 16; got "
                           f"{q.dtype}, head size {d}, page size {page_size}")
-    n_seqs = cu_tokens.numel() - 1
-    if positions.numel() != n or block_table.dim() != 2 or block_table.shape[0] < n_seqs or nq % nkv:
-        raise KernelError("attention_mfma: positions, cu_tokens and block_table do not fit the batch")
-    if max_kv_len > block_table.shape[1] * page_size or max_q_len < 1 or max_q_len > n:
+    all_seqs = cu_tokens.numel() - 1
+    seq_begin, n_seqs = seqs if seqs is not None else (0, all_seqs)
+    token_begin, n_tokens = tokens if tokens is not None else (0, n)
+    if (positions.numel() != n or block_table.dim() != 2 or block_table.shape[0] < all_seqs or nq % nkv
+            or seq_begin < 0 or seq_begin + n_seqs > all_seqs or token_begin < 0 or token_begin + n_tokens > n):
+        raise KernelError("attention_mfma: positions, cu_tokens, block_table and the ranges do not fit the batch")
+    if max_kv_len > block_table.shape[1] * page_size or max_q_len < 1 or max_q_len > max(n_tokens, 1):
         raise KernelError(f"attention_mfma: max_kv_len {max_kv_len} / max_q_len {max_q_len} do not fit "
-                          f"{block_table.shape[1]} pages of {page_size} and {n} tokens")
+                          f"{block_table.shape[1]} pages of {page_size} and {n_tokens} tokens")
+    if out is None:
+        out = torch.empty_like(q)
+    elif out.shape != q.shape or out.dtype != q.dtype:
+        raise KernelError("attention_mfma: `out` must have the shape and dtype of q")
     if splits is None:
         splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len)
     else:
         chunk = -(-(-(-max_kv_len // splits)) // 32) * 32
     target = _build.attn_target(d)
     lib = library(target)
-    out = torch.empty_like(q)
     ws_floats = lib.ia_attention_mfma_workspace(n, nq, splits)
     ws = torch.empty((ws_floats,), dtype=torch.float32, device=q.device) if ws_floats else None
     _check(lib.ia_attention_mfma(
         _p(out), _p(ws), _p(q), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions),
-        n, n_seqs, max_q_len, max_kv_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
-        ctypes.c_float(scale), splits, chunk, _stream()), target)
+        n, seq_begin, n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, block_table.shape[1], nq, nkv, d,
+        page_size, int(window or 0), ctypes.c_float(scale), splits, chunk, _stream()), target)
     return out
 
 

@@ -77,9 +77,20 @@ class Attention(Mixer):
             k_cache=cache.k, v_cache=cache.v, slots=group.slots if cache.writable else None,
             page_size=group.page_size)
         if ops.attention_mfma_fits(q.dtype, s.head_dim, group.page_size):
-            a = ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
-                                   max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, window=s.window,
-                                   scale=s.softmax_scale)
+            common = dict(window=s.window, scale=s.softmax_scale)
+            if 0 < ctx.n_single < ctx.n_seqs:
+                # single tokens (decode) and portions of prompts want different launches: the first
+                # split their long key ranges between waves, the second have columns enough
+                a = ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                       max_q_len=1, max_kv_len=ctx.max_kv_single, seqs=(0, ctx.n_single),
+                                       tokens=(0, ctx.n_single), **common)
+                ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                   max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_multi,
+                                   seqs=(ctx.n_single, ctx.n_seqs - ctx.n_single),
+                                   tokens=(ctx.n_single, ctx.n_tokens - ctx.n_single), out=a, **common)
+            else:
+                a = ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                       max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, **common)
         else:
             a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
                                       window=s.window, scale=s.softmax_scale)

@@ -27,8 +27,15 @@ TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size
               head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
               max_position_embeddings=2048, hidden_act="silu")
 
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
+# Sizes that fit no vector width or tile: hidden 100 and intermediate 150 are no multiple of 8, the
+# vocabulary is a prime, three query heads share one kv head.
+TINY_E = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=131, hidden_size=100,
+              intermediate_size=150, num_hidden_layers=2, num_attention_heads=3, num_key_value_heads=1,
+              head_dim=16, rope_theta=777.0, rms_norm_eps=1e-4, tie_word_embeddings=True,
+              max_position_embeddings=512, hidden_act="silu")
+
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16, "E": 16}
 
 
 def write_model(folder: str, raw: dict, seed: int, dtype=torch.bfloat16, sharpen: float = 1.0) -> str:
