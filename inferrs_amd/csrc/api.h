@@ -23,6 +23,7 @@ int ia_rmsnorm(void* out, const void* x, const float* w, float eps, int rows, in
 int ia_add_rmsnorm(void* out, void* x, const void* delta, const float* w, float eps, int rows,
                    int cols, int add_one, int dtype, hipStream_t stream);
 int ia_add_inplace(void* x, const void* delta, long long n, int dtype, hipStream_t stream);
+int ia_widen_bf16(float* out, const void* x, long long n, hipStream_t stream);
 int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream);
 int ia_rope_table(float* cos_out, float* sin_out, const int* positions, const float* inv_freq,
                   int n, int half, hipStream_t stream);
@@ -43,7 +44,8 @@ int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, 
 int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
                         int out_dtype, int dual, hipStream_t stream);
 
-int ia_argmax(int* out, const float* logits, int rows, int vocab, hipStream_t stream);
+long long ia_argmax_workspace(int rows, int vocab);
+int ia_argmax(int* out, const float* logits, void* workspace, int rows, int vocab, hipStream_t stream);
 int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, const float* rep,
                 const float* freq, const float* pres, const int* bias_ids, const float* bias_vals,
                 int nb, hipStream_t stream);

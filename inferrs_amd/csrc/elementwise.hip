@@ -280,6 +280,21 @@ extern "C" int ia_silu_mul(void* out, const void* gu, int rows, int inter, int d
     return 0;
 }
 
+// ---- widening copy ---------------------------------------------------------------------------
+__global__ void widen_kernel(float* __restrict__ out, const bf16_t* __restrict__ x, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = bf16_bits_to_f32(x[i].bits);
+}
+
+extern "C" int ia_widen_bf16(float* out, const void* x, long long n, hipStream_t stream) {
+    IA_CHECK(n >= 0, "widen: bad size %lld", n);
+    if (n == 0) return 0;
+    const size_t want = ((size_t)n + 255) / 256;
+    widen_kernel<<<(unsigned)(want < 65535 * 4 ? want : 65535 * 4), 256, 0, stream>>>(out, (const bf16_t*)x, (size_t)n);
+    IA_LAUNCH_CHECK("widen");
+    return 0;
+}
+
 // ---- rotary angle table for the tokens of one step ----------------------------------------------
 __global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict__ sin_out,
                                   const int* __restrict__ positions, const float* __restrict__ inv_freq,

@@ -53,9 +53,63 @@ __global__ __launch_bounds__(1024) void argmax_kernel(int* __restrict__ out, con
     argmax_row(logits + (size_t)blockIdx.x * vocab, vocab, sv, si, out + blockIdx.x);
 }
 
-extern "C" int ia_argmax(int* out, const float* logits, int rows, int vocab, hipStream_t stream) {
+// Long rows in two steps: blocks of a row take a stretch each, then one block a row picks among
+// their candidates (lowest index among equal maxima in both steps).
+#define ARGMAX_STRETCH 8192
+__global__ __launch_bounds__(256) void argmax_stretch_kernel(float* __restrict__ cand_v, int* __restrict__ cand_i,
+                                                             const float* __restrict__ logits, int vocab) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const int row = blockIdx.y, stretch = blockIdx.x;
+    const int lo = stretch * ARGMAX_STRETCH;
+    const int len = vocab - lo < ARGMAX_STRETCH ? vocab - lo : ARGMAX_STRETCH;
+    int idx;
+    argmax_row(logits + (size_t)row * vocab + lo, len, sv, si, &idx);
+    if (threadIdx.x == 0) {
+        cand_i[(size_t)row * gridDim.x + stretch] = lo + idx;
+        cand_v[(size_t)row * gridDim.x + stretch] = logits[(size_t)row * vocab + lo + idx];
+    }
+}
+
+__global__ __launch_bounds__(IA_WAVE) void argmax_pick_kernel(int* __restrict__ out, const float* __restrict__ cand_v,
+                                                              const int* __restrict__ cand_i, int stretches) {
+    const int row = blockIdx.x;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int c = threadIdx.x; c < stretches; c += IA_WAVE) {
+        float v = cand_v[(size_t)row * stretches + c];
+        v = v != v ? -INFINITY : v;                      // a stretch of NaN never wins over a number
+        const int i = cand_i[(size_t)row * stretches + c];
+        if (v > best || (v == best && i < idx) || idx == 0x7fffffff) { best = v; idx = i; }
+    }
+#pragma unroll
+    for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, IA_WAVE);
+        const int oi = __shfl_xor(idx, o, IA_WAVE);
+        if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) { best = ov; idx = oi; }
+    }
+    if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+}
+
+extern "C" long long ia_argmax_workspace(int rows, int vocab) {
+    return vocab > 2 * ARGMAX_STRETCH ? 2LL * rows * ((vocab + ARGMAX_STRETCH - 1) / ARGMAX_STRETCH) : 0;
+}
+
+// `workspace`: ia_argmax_workspace(rows, vocab) words, or null for the one-block-a-row kernel.
+extern "C" int ia_argmax(int* out, const float* logits, void* workspace, int rows, int vocab, hipStream_t stream) {
     IA_CHECK(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
     if (rows == 0) return 0;
+    if (workspace != nullptr && vocab > 2 * ARGMAX_STRETCH) {
+        const int stretches = (vocab + ARGMAX_STRETCH - 1) / ARGMAX_STRETCH;
+        IA_CHECK(rows <= 65535, "argmax: %d rows exceed the grid", rows);
+        float* cand_v = (float*)workspace;
+        int* cand_i = (int*)workspace + (size_t)rows * stretches;
+        argmax_stretch_kernel<<<dim3(stretches, rows), 256, 0, stream>>>(cand_v, cand_i, logits, vocab);
+        IA_LAUNCH_CHECK("argmax");
+        argmax_pick_kernel<<<rows, IA_WAVE, 0, stream>>>(out, cand_v, cand_i, stretches);
+        IA_LAUNCH_CHECK("argmax");
+        return 0;
+    }
     argmax_kernel<<<rows, 1024, 0, stream>>>(out, logits, vocab);
     IA_LAUNCH_CHECK("argmax");
     return 0;

@@ -44,6 +44,7 @@ def library(target: str = "core") -> ctypes.CDLL:
         lib.ia_attention_mfma_workspace.restype = ctypes.c_longlong
     else:
         lib.ia_sample_workspace.restype = ctypes.c_longlong
+        lib.ia_argmax_workspace.restype = ctypes.c_longlong
     _LIBS[target], _LIB_PATHS[target] = lib, path
     return lib
 
@@ -317,7 +318,6 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 # ---- matrix products --------------------------------------------------------------------------
 
 SKINNY_MAX_ROWS = 16          # beyond this the vendor's GEMM reads the weights faster
-SKINNY_MAX_ROWS_F32_OUT = 64  # 32-bit results (logits) have no library route
 
 
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -354,23 +354,36 @@ def skinny_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and (x.data_ptr() | w.data_ptr()) % 16 == 0)
 
 
+def widen(x: torch.Tensor) -> torch.Tensor:
+    """bfloat16 -> float32, exactly."""
+    _dev(x)
+    if x.dtype != torch.bfloat16:
+        raise KernelError(f"widen: takes bfloat16, got {x.dtype}")
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _check(library().ia_widen_bf16(_p(out), _p(x), ctypes.c_longlong(x.numel()), _stream()))
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
     skinny MFMA kernel for up to 16 rows, the vendor's GEMM beyond that (the reference uses
-    cuBLAS for all of them); a 32-bit result of bfloat16 operands (logits) comes from the skinny
-    kernel, 64 rows at a time."""
+    cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
+    the skinny kernel's accumulators for up to 16 rows; beyond that it is the vendor's bfloat16
+    result widened, which is what the reference does for every row (its logits are computed in
+    the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`)."""
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return gemm_tiled(x, w, out_dtype)
     m, k = x.shape
     if not skinny_fits(x, w):
         return gemm_tiled(x, w, out_dtype)
-    if m <= SKINNY_MAX_ROWS or out_dtype == torch.float32:
+    if m <= SKINNY_MAX_ROWS:
         return gemm_skinny_bf16(x, w, out_dtype)
     _dev(x, w)
     if w.shape[1] != k or w.dtype != x.dtype:
         raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
-    return torch.nn.functional.linear(x, w)
+    y = torch.nn.functional.linear(x, w)
+    return widen(y) if out_dtype == torch.float32 else y
 
 
 # ---- sampling ---------------------------------------------------------------------------------
@@ -379,7 +392,9 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _dev(logits); _f32(logits, "logits")
     rows, vocab = logits.shape
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    _check(library().ia_argmax(_p(out), _p(logits), rows, vocab, _stream()))
+    words = library().ia_argmax_workspace(rows, vocab)
+    ws = torch.empty((words,), dtype=torch.int32, device=logits.device) if words else None
+    _check(library().ia_argmax(_p(out), _p(logits), _p(ws), rows, vocab, _stream()))
     return out
 
 
