@@ -23,6 +23,8 @@ int ia_rmsnorm(void* out, const void* x, const float* w, float eps, int rows, in
 int ia_add_rmsnorm(void* out, void* x, const void* delta, const float* w, float eps, int rows,
                    int cols, int add_one, int dtype, hipStream_t stream);
 int ia_add_inplace(void* x, const void* delta, long long n, int dtype, hipStream_t stream);
+int ia_fill_normal(void* out, long long n, unsigned long long seed, double mean, double std,
+                   int dtype, hipStream_t stream);
 int ia_widen_bf16(float* out, const void* x, long long n, hipStream_t stream);
 int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream);
 int ia_rope_table(float* cos_out, float* sin_out, const int* positions, const float* inv_freq,

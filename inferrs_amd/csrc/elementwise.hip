@@ -280,6 +280,47 @@ extern "C" int ia_silu_mul(void* out, const void* gu, int rows, int inter, int d
     return 0;
 }
 
+// ---- random fill ---------------------------------------------------------------------------------
+// Element i of a tensor is a function of (seed, i) alone: two outputs of the splitmix64 sequence
+// started at seed + 2 i steps give two uniforms, Box and Muller turn them into a standard normal
+// value in 64-bit arithmetic, and mean + std * z is rounded to 32-bit and then to the storage
+// type.  The host fill (inferrs_amd/weights/random_init.py) is the same formula in NumPy.
+__device__ __forceinline__ uint64_t splitmix_out(uint64_t state) {
+    uint64_t z = state;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+template <typename T>
+__global__ void fill_normal_kernel(T* __restrict__ out, size_t n, uint64_t seed, double mean, double std) {
+    const uint64_t golden = 0x9e3779b97f4a7c15ull;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const uint64_t h1 = splitmix_out(seed + (2 * (uint64_t)i + 1) * golden);
+        const uint64_t h2 = splitmix_out(seed + (2 * (uint64_t)i + 2) * golden);
+        const double u1 = (double)((h1 >> 11) + 1) * (1.0 / 9007199254740992.0);      // (0, 1]
+        const double u2 = (double)(h2 >> 11) * (1.0 / 9007199254740992.0);            // [0, 1)
+        const double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586 * u2);
+        st(out + i, (float)(mean + std * z));
+    }
+}
+
+extern "C" int ia_fill_normal(void* out, long long n, unsigned long long seed, double mean, double std,
+                              int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0, "fill_normal: bad size %lld", n);
+    if (n == 0) return 0;
+    const size_t want = ((size_t)n + 255) / 256;
+    const unsigned grid = (unsigned)(want < 65535 * 16 ? want : 65535 * 16);
+    if (dtype == IA_F32)
+        fill_normal_kernel<float><<<grid, 256, 0, stream>>>((float*)out, (size_t)n, seed, mean, std);
+    else if (dtype == IA_BF16)
+        fill_normal_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (size_t)n, seed, mean, std);
+    else
+        IA_CHECK(false, "fill_normal: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("fill_normal");
+    return 0;
+}
+
 // ---- widening copy ---------------------------------------------------------------------------
 __global__ void widen_kernel(float* __restrict__ out, const bf16_t* __restrict__ x, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)

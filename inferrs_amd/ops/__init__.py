@@ -354,6 +354,16 @@ def skinny_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and (x.data_ptr() | w.data_ptr()) % 16 == 0)
 
 
+def fill_normal(shape, seed: int, mean: float, std: float, dtype: torch.dtype, device) -> torch.Tensor:
+    """A tensor of mean + std * N(0, 1), element i a function of (seed, i) alone; the same values
+    as the host fill of `inferrs_amd.weights.random_init`."""
+    require_gpu()
+    out = torch.empty(tuple(shape), dtype=dtype, device=device)
+    _check(library().ia_fill_normal(_p(out), ctypes.c_longlong(out.numel()), ctypes.c_ulonglong(seed & (2**64 - 1)),
+                                    ctypes.c_double(mean), ctypes.c_double(std), _dt(out), _stream()))
+    return out
+
+
 def widen(x: torch.Tensor) -> torch.Tensor:
     """bfloat16 -> float32, exactly."""
     _dev(x)

@@ -307,3 +307,18 @@ def test_argmax_lowest_index_among_equal_maxima():
     assert got == [int(torch.argmax(z[0])), 77, 0, 151935]
     small = torch.tensor([[1.0, 3.0, 3.0]])
     assert ops.argmax(dev(small)).cpu().tolist() == [1]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fill_normal_equals_the_host_fill(dtype):
+    from inferrs_amd import ops
+    from inferrs_amd.weights.random_init import normal_values
+    n, seed = 300_001, 0x1234_5678_9ABC_DEF0
+    host = torch.from_numpy(normal_values(n, seed, 1.0, 0.1)).to(dtype)
+    got = ops.fill_normal((n,), seed, 1.0, 0.1, dtype, "cuda").cpu()
+    # the two differ only where the device's and NumPy's 64-bit log or cosine differ in their last
+    # bit AND that falls on a rounding boundary of the narrower type: (almost) never
+    assert int((got != host).sum()) <= (3 if dtype == torch.float32 else 0)
+    z = (ops.fill_normal((n,), 7, 0.0, 1.0, torch.float32, "cuda").cpu()).double()
+    assert abs(float(z.mean())) < 0.01 and abs(float(z.std()) - 1.0) < 0.01
+    assert abs(float((z ** 4).mean()) - 3.0) < 0.1                      # the fourth moment of a normal

@@ -104,3 +104,38 @@ def test_frequencies_follow_the_tempered_softmax():
     counts = torch.bincount(torch.tensor(got), minlength=8).float()
     chi2 = float(((counts - n * probs) ** 2 / (n * probs)).sum())
     assert chi2 < 24.3, f"chi-square {chi2:.1f} with 7 degrees of freedom (0.999 quantile is 24.3)"
+
+
+# The reference's own penalty-window cases (inferrs/src/sampler.rs:606-704): logits, history, parameters, winner.
+REFERENCE_CASES = [
+    ([10.0, 8.0, 0.0, 0.0], [0, 1, 2, 3], dict(repetition_penalty=1.5, repeat_last_n=2), 0),    # 0 outside the window
+    ([10.0, 8.0, 0.0, 0.0], [1, 2, 3, 0], dict(repetition_penalty=1.5, repeat_last_n=2), 1),    # 0 inside: 6.67 < 8
+    ([10.0, 0.0, 0.0, 0.0], [0], dict(repetition_penalty=2.0, repeat_last_n=0), 0),             # window 0 disables
+    ([10.0, 5.0], [0], dict(repetition_penalty=1.5, repeat_last_n=64), 0),                      # window beyond the history
+    ([10.0, 5.0], [0], dict(repetition_penalty=10.0, repeat_last_n=64), 1),
+    ([10.0, 5.0], [0], dict(repetition_penalty=0.0, repeat_last_n=64), 0),                      # 0.0 acts as disabled
+]
+
+
+@pytest.mark.parametrize("logits,history,kw,winner", REFERENCE_CASES)
+def test_plain_sampler_on_the_reference_cases(logits, history, kw, winner):
+    assert pm.sample(torch.tensor(logits), history, temperature=0.0, **kw) == winner
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("logits,history,kw,winner", REFERENCE_CASES)
+def test_device_sampler_on_the_reference_cases(logits, history, kw, winner):
+    from inferrs_amd.sampling import Sampler
+    got = Sampler("cuda:0").sample(torch.tensor([logits]).to("cuda"), [SamplingParams(temperature=0.0, seed=1, **kw)],
+                                   [history], [1])
+    assert got == [winner]
+
+
+def test_sampling_params_defaults_are_the_reference_defaults():
+    # inferrs/src/sampler.rs:90-112 and its test at :586-603
+    p = SamplingParams()
+    assert (p.temperature, p.top_p, p.top_k, p.min_p) == (0.7, 0.9, 50, 0.0)
+    assert (p.repetition_penalty, p.repeat_last_n, p.frequency_penalty, p.presence_penalty) == (1.1, 64, 0.0, 0.0)
+    assert p.max_tokens == 2048 and p.seed is None and not p.bypass_stop_tokens
+    with pytest.raises(ValueError):
+        SamplingParams(top_p=0.0)
