@@ -17,7 +17,7 @@ import torch
 from .. import ops
 from ..cache import CacheManager, CacheStorage, OutOfPages
 from ..config.registry import load_config
-from ..parts.assemble import model_tensors
+from ..parts.assemble import generated_tensors, model_tensors
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
 from .batch import StepBuilder, StepError
@@ -85,8 +85,7 @@ class Engine:
     def from_random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
         """Random weights drawn on the device, without a folder in between."""
         spec = config.to_spec()
-        expected, optional = model_tensors(spec)
-        wanted = {n: s for n, s in expected.items() if n not in optional}
+        wanted = generated_tensors(spec)
         dt = parse_dtype(dtype)
         tensors = random_tensors(wanted, seed, torch.bfloat16 if dt == torch.bfloat16 else torch.float32,
                                  device=device)

@@ -22,7 +22,11 @@ def layer_tensors(layer) -> Dict[str, TensorSpec]:
 
 
 def model_tensors(spec: ModelSpec) -> Tuple[Dict[str, TensorSpec], Set[str]]:
-    """(every tensor name the model may read -> its spec, the names that may be absent)."""
+    """(every tensor name the model may read -> its spec, the names that may be absent).
+
+    A separate logits head may always be absent: the embedding table then serves, as in the
+    reference, which decides by the tensor's presence alone
+    (`inferrs-models/src/models/qwen3.rs:369-372`)."""
     expected: Dict[str, TensorSpec] = {
         spec.embed_name: TensorSpec((spec.vocab_size, spec.hidden), "matrix")}
     for layer in spec.layers:
@@ -32,6 +36,14 @@ def model_tensors(spec: ModelSpec) -> Tuple[Dict[str, TensorSpec], Set[str]]:
     optional: Set[str] = set()
     if spec.head_name is not None:
         expected[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden), "matrix")
-        if not spec.head_required:
-            optional.add(spec.head_name)
+        optional.add(spec.head_name)
     return expected, optional
+
+
+def generated_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
+    """What a random model of this spec is made of: everything, the separate logits head only
+    when the configuration unties it."""
+    expected, _ = model_tensors(spec)
+    if spec.head_name is not None and not spec.head_required:
+        del expected[spec.head_name]
+    return expected

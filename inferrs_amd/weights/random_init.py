@@ -87,10 +87,9 @@ def write_random_model(model_dir: str, config, seed: int,
                        dtype: torch.dtype = torch.bfloat16) -> str:
     """Write `config.json` and `model.safetensors` for `config` (a registered
     architecture's configuration object) and return the folder."""
-    from ..parts.assemble import model_tensors
+    from ..parts.assemble import generated_tensors
     spec = config.to_spec()
-    expected, optional = model_tensors(spec)
-    wanted = {n: s for n, s in expected.items() if n not in optional}
+    wanted = generated_tensors(spec)
     os.makedirs(model_dir, exist_ok=True)
     with open(os.path.join(model_dir, "config.json"), "w", encoding="utf-8") as f:
         json.dump(config.to_dict(), f, indent=2)

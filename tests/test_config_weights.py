@@ -11,7 +11,7 @@ from tiny_configs import TINY_A, TINY_B, write_model
 
 from inferrs_amd.config import ConfigError, Qwen3Config, load_config, registered_architectures
 from inferrs_amd.config.registry import resolve_architecture
-from inferrs_amd.parts import model_tensors
+from inferrs_amd.parts import generated_tensors, model_tensors
 from inferrs_amd.weights import (SafetensorsError, WeightError, load_weights, random_tensors,
                                  write_random_model, write_safetensors)
 
@@ -32,13 +32,16 @@ def test_head_dim_is_decoupled_from_hidden_size():
     assert expected["model.layers.0.self_attn.q_proj.weight"].shape == (192, 96)
     assert expected["model.layers.2.self_attn.o_proj.weight"].shape == (96, 192)
     assert expected["model.layers.0.self_attn.k_norm.weight"].shape == (32,)
-    assert "lm_head.weight" in expected and not optional
+    assert "lm_head.weight" in expected and optional == {"lm_head.weight"}
+    assert "lm_head.weight" in generated_tensors(spec)
 
 
-def test_tied_head_is_optional_by_presence():
-    # qwen3.rs:369-372: lm_head.weight is used when the file has it, else the embedding table
-    expected, optional = model_tensors(Qwen3Config.from_dict(TINY_A).to_spec())
-    assert optional == {"lm_head.weight"}
+def test_the_head_is_optional_by_presence():
+    # qwen3.rs:369-372: lm_head.weight is used when the file has it, else the embedding table,
+    # whatever tie_word_embeddings says; a random model has the head only when the config unties it
+    spec = Qwen3Config.from_dict(TINY_A).to_spec()
+    expected, optional = model_tensors(spec)
+    assert optional == {"lm_head.weight"} and "lm_head.weight" not in generated_tensors(spec)
 
 
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers",
@@ -108,7 +111,7 @@ def test_random_folder_round_trip(tmp_path):
 
 def test_stored_precision_is_kept(tmp_path):
     expected, optional = model_tensors(Qwen3Config.from_dict(TINY_A).to_spec())
-    tensors = random_tensors({n: s for n, s in expected.items() if n not in optional}, 1, torch.bfloat16)
+    tensors = random_tensors(generated_tensors(Qwen3Config.from_dict(TINY_A).to_spec()), 1, torch.bfloat16)
     tensors["model.norm.weight"] = tensors["model.norm.weight"].float() + 1e-4        # stored in 32-bit
     tensors["model.layers.0.mlp.up_proj.weight"] = tensors["model.layers.0.mlp.up_proj.weight"].to(torch.float16)
     os.makedirs(tmp_path / "m")
@@ -148,7 +151,7 @@ def test_truncated_and_malformed_files(tmp_path):
     with pytest.raises(SafetensorsError, match="No safetensors files"):
         load_weights(str(folder), expected, optional)
     good = tmp_path / "good.safetensors"
-    write_safetensors(str(good), random_tensors({n: s for n, s in expected.items() if n not in optional}, 1))
+    write_safetensors(str(good), random_tensors(generated_tensors(Qwen3Config.from_dict(TINY_A).to_spec()), 1))
     blob = good.read_bytes()
     (folder / "model.safetensors").write_bytes(blob[: len(blob) // 2])
     with pytest.raises(SafetensorsError, match="truncated"):
@@ -163,7 +166,7 @@ def test_truncated_and_malformed_files(tmp_path):
 
 def test_sharded_folders_and_last_file_wins(tmp_path):
     expected, optional = model_tensors(Qwen3Config.from_dict(TINY_A).to_spec())
-    tensors = random_tensors({n: s for n, s in expected.items() if n not in optional}, 1)
+    tensors = random_tensors(generated_tensors(Qwen3Config.from_dict(TINY_A).to_spec()), 1)
     names = sorted(tensors)
     folder = tmp_path / "m"
     os.makedirs(folder)

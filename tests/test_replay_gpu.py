@@ -215,3 +215,27 @@ def test_captured_decode_steps_equal_eager_ones(models, tmp_path, dtype):
     assert err <= (1e-6 if dtype == "float32" else bound(folder, reqs, ref, dtype)), f"{err:.3e} at {where}"
     err, where = worst(outs[True], ref, some, scale=scale)
     assert err <= bound(folder, reqs, ref, dtype), f"{err:.3e} at {where}"
+
+
+@pytest.mark.parametrize("name,drop", [("B", True), ("A", False)])
+def test_logits_head_follows_the_tensor_present(tmp_path, name, drop):
+    """`lm_head.weight` is used when the file has it and the embedding table when it has not,
+    whatever `tie_word_embeddings` says (inferrs-models/src/models/qwen3.rs:369-372)."""
+    from safetensors.torch import load_file, save_file
+    from inferrs_amd.engine import Engine, Entry
+    folder = write_model(str(tmp_path / "m"), TINY[name], seed=8)
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    if drop:
+        assert not TINY[name]["tie_word_embeddings"]
+        del tensors["lm_head.weight"]                    # untied by its config, but the head is absent
+    else:
+        assert TINY[name]["tie_word_embeddings"]
+        tensors["lm_head.weight"] = torch.randn_like(tensors["model.embed_tokens.weight"].float()).mul(0.02).bfloat16()
+    save_file(tensors, path)
+    cfg, params = pm.read_model(folder, torch.float64)
+    toks = random_tokens(21, TINY[name]["vocab_size"], 4)
+    want = pm.forward(cfg, params, toks).numpy()
+    eng = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=4, max_seqs=1)
+    got = eng.step([Entry("a", toks, list(range(21)))]).cpu().numpy()
+    assert float(np.abs(got - want).max()) <= 1e-5 * float(np.abs(want).max())

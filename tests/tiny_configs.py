@@ -46,11 +46,10 @@ def write_model(folder: str, raw: dict, seed: int, dtype=torch.bfloat16, sharpen
     import json
 
     from inferrs_amd.config import Qwen3Config
-    from inferrs_amd.parts import model_tensors
+    from inferrs_amd.parts import generated_tensors
     from inferrs_amd.weights import random_tensors, write_safetensors
     config = Qwen3Config.from_dict(raw)
-    expected, optional = model_tensors(config.to_spec())
-    tensors = random_tensors({n: s for n, s in expected.items() if n not in optional}, seed, dtype)
+    tensors = random_tensors(generated_tensors(config.to_spec()), seed, dtype)
     if sharpen != 1.0:
         for name in tensors:
             if name.endswith("q_norm.weight") or name.endswith("k_norm.weight"):
