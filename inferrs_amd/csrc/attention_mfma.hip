@@ -224,8 +224,12 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         }
     };
 
-    // (Loading the next step's operands ahead of this step's products was tried and lost: it
-    // doubles the operand registers, which costs a wave per SIMD, and that wave hid more latency.)
+    // Two variants were tried and lost.  Loading the next step's operands ahead of this step's
+    // products doubles the operand registers, which costs a wave per SIMD, and that wave hid more
+    // latency.  Blocks of four waves that bring each step's keys and values into shared memory
+    // once (double-buffered, conflict-free layouts, one barrier a step) ran at half the speed of
+    // independent waves that read the same pages through the L2: the barrier keeps the four waves
+    // in step, and their matrix and vector work no longer overlap.
     for (int k0 = lo; k0 < hi; k0 += 32) {
         Operands op;
         load_step(op, k0);
