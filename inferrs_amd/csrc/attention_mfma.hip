@@ -272,7 +272,8 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
 // pair walks about the same number, so all waves end together.  It pays when the step's queries
 // span most of the context; a short portion late in a long context has equal blocks already.
 template <int NB>
-__global__ __launch_bounds__(IA_WAVE) void attn_mfma_kernel(const AttnParams p) {
+__global__ __launch_bounds__(IA_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1, HD > 64 ? 2 : 8)))
+void attn_mfma_kernel(const AttnParams p) {
     const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
     const int seq = p.seq_begin + blockIdx.z;
     const int n_cols = (p.cu_tokens[seq + 1] - p.cu_tokens[seq]) * (p.nq / p.nkv);
@@ -359,10 +360,6 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 
 extern "C" int ia_attention_mfma_head_dim(void) { return HD; }
 
-// Tuning: columns a wave for long portions (2 or 4 tiles of 16).
-static int g_nb_prefill = 4;
-extern "C" void ia_attention_mfma_tune(int nb_prefill) { g_nb_prefill = nb_prefill; }
-
 // Floats of workspace that `splits` > 1 needs: partial outputs, then maxima and sums.
 extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
     return splits > 1 ? (long long)n * nq * splits * (HD + 2) : 0;
@@ -406,21 +403,15 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
     p.splits = splits; p.chunk = chunk; p.seq_begin = seq_begin;
     p.scale_log2 = scale * 1.4426950408889634f;
     const long long cols = (long long)max_q_len * g;
-    // Columns a wave: 16 for decode; 32 or 64 for portions of prompts (64 keeps every loaded key
-    // and value in use for twice as many products, but leaves half as many waves).
+    // Columns a wave: 16 for decode, 32 for portions of prompts.  (64 keep every loaded key and
+    // value in use for twice as many products but need the registers of a whole SIMD; with 32
+    // two waves share a SIMD and one's matrix work overlaps the other's softmax, which is faster.)
     p.pair = (splits == 1 && cols > 16 && 2LL * max_q_len > max_kv_len) ? 1 : 0;
-    int nb = 1;
-    if (cols > 16) {
-        const long long waves4 = ((cols + 63) / 64 + p.pair) / (1 + p.pair) * nkv * splits * n_seqs;
-        nb = (HD <= 128 && g_nb_prefill == 4 && waves4 >= 1024) ? 4 : 2;
-    }
+    const int nb = cols > 16 ? 2 : 1;
     const long long col_blocks = (cols + 16 * nb - 1) / (16 * nb);
     const dim3 grid((unsigned)(p.pair ? (col_blocks + 1) / 2 : col_blocks), nkv * splits, n_seqs);
     if (nb == 1) attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
-    else if (nb == 2) attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
-#if IA_HEAD_DIM <= 128
-    else attn_mfma_kernel<4><<<grid, IA_WAVE, 0, stream>>>(p);
-#endif
+    else attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
         attn_merge_kernel<<<(unsigned)((long long)n_tokens * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>(

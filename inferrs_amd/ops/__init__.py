@@ -257,7 +257,7 @@ def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: i
     """(splits, keys per split) for the matrix-core kernel: the keys are split between waves
     when the batch alone has too few (request, kv head, column block) items to fill the chip."""
     cols = max_q_len * g
-    col_blocks = 1 if cols <= 16 else -(-cols // 32)      # (64 columns a wave beyond 256: then nothing is split anyway)
+    col_blocks = 1 if cols <= 16 else -(-cols // 32)
     items = n_seqs * nkv * col_blocks
     splits = 1
     while items * splits < ATTN_TARGET_WAVES and max_kv_len >= 2 * splits * ATTN_MIN_CHUNK and splits < 128:
