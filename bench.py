@@ -77,26 +77,40 @@ def fill_context(engine, ids, context: int) -> None:
                        .mul_(0.5).to(arr.dtype))
 
 
-def time_decode(engine, batch: int, context: int, steps: int, warmup: int):
-    """(seconds for `steps` steps, mean context length during them)."""
+def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decode_run: int = 8):
+    """(seconds for `steps` steps, mean context length during them).  The steps go through the
+    serving loop: scheduler, step function, greedy choice on the device."""
     import torch
-    from inferrs_amd import ops
-    from inferrs_amd.engine import Entry
-    ids = [f"d{i}" for i in range(batch)]
+    from inferrs_amd.engine import GenerationLoop
+    from inferrs_amd.engine.scheduler import RUNNING
+    from inferrs_amd.sampling import SamplingParams
     start_len = context - steps - warmup
+    loop = GenerationLoop(engine, max_batch_size=batch, max_tokens_per_step=max(batch, 16), decode_run=decode_run)
+    params = SamplingParams.greedy(max_tokens=steps + warmup + 8, bypass_stop_tokens=True)
+    reqs = [loop.add([1 + i], params, request_id=f"d{i}") for i in range(batch)]
+    ids = [r.request_id for r in reqs]
+    # the requests enter as if their contexts had been run: random keys and values, and one generated token
     fill_context(engine, ids, start_len)
-    tokens = [1 + i for i in range(batch)]
-    t0 = None
-    for s in range(warmup + steps):
-        if s == warmup:
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-        logits = engine.step([Entry(sid, [tok], [0]) for sid, tok in zip(ids, tokens)])
-        tokens = ops.argmax(logits).cpu().tolist()
+    for r in reqs:
+        loop.scheduler.waiting.remove(r)
+        r.prompt = [1] * start_len
+        r.output = [1 + len(loop.scheduler.running)]
+        r.computed = start_len
+        r.status = RUNNING
+        loop.scheduler.running.append(r)
+    done_steps = 0
+    while done_steps < warmup:
+        loop.step(max_steps=warmup - done_steps)
+        done_steps = loop.steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while loop.steps < warmup + steps:
+        loop.step(max_steps=warmup + steps - loop.steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     for sid in ids:
-        engine.end_request(sid)
+        if engine.has_request(sid):
+            engine.end_request(sid)
     return elapsed, start_len + warmup + (steps - 1) / 2.0
 
 
@@ -130,6 +144,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
+    ap.add_argument("--decode-run", type=int, default=8,
+                    help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -155,7 +171,7 @@ def main() -> int:
                                       "ms": round(t * 1e3, 3),
                                       "frac": round(prefill_flops(raw, PREFILL_TOKENS) / t / PEAK_FLOPS[dtype_key], 4)}}))
         return 0
-    elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup)
+    elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
     nbytes = decode_bytes(raw, args.batch, mean_ctx, esize)
@@ -183,7 +199,7 @@ def main() -> int:
         points = {}
         for b in points_batches:
             steps = max(8, args.steps // 2)
-            el, _ = time_decode(engine, b, args.context, steps, min(args.warmup, 4))
+            el, _ = time_decode(engine, b, args.context, steps, min(args.warmup, 4), args.decode_run)
             points[f"decode_b{b}"] = round(b * steps / el, 2)
         record["points"] = points
         t = time_prefill(engine, PREFILL_TOKENS, 3, raw["vocab_size"])

@@ -71,22 +71,30 @@ class StepBuilder:
     def __init__(self, cache: CacheManager, device):
         self.cache = cache
         self.device = torch.device(device)
-        self._host: Optional[torch.Tensor] = None
+        # One device buffer (its address is what captured graphs hold) and a ring of pinned host
+        # buffers, so that the copies of several steps can be under way at once.
+        self._ring: List[torch.Tensor] = []
+        self._events: List[Optional[torch.cuda.Event]] = []
+        self._next = 0
         self._dev: Optional[torch.Tensor] = None
-        self._event: Optional[torch.cuda.Event] = None
         self._rows: Dict[Any, list] = {}
         self.generation = 0                # grows when the device staging buffer moves
 
-    def _staging(self, n: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        if self._host is None or self._host.numel() < n:
+    RING = 16
+
+    def _staging(self, n: int) -> Tuple[torch.Tensor, torch.Tensor, int]:
+        if self._dev is None or self._dev.numel() < n:
             size = 1 << max(12, (n - 1).bit_length())
-            self._host = torch.empty(size, dtype=torch.int32, pin_memory=True)
+            torch.cuda.synchronize(self.device)
+            self._ring = [torch.empty(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+            self._events = [None] * self.RING
             self._dev = torch.empty(size, dtype=torch.int32, device=self.device)
-            self._event = None
             self.generation += 1
-        if self._event is not None:
-            self._event.synchronize()      # the previous step's copy has left the host buffer
-        return self._host, self._dev
+        slot = self._next
+        self._next = (slot + 1) % self.RING
+        if self._events[slot] is not None:
+            self._events[slot].synchronize()      # that copy has left the host buffer
+        return self._ring[slot], self._dev, slot
 
     def _table_row(self, group: int, seq, need: int) -> np.ndarray:
         """The request's pages of one group as an int32 array, kept between steps and extended
@@ -111,11 +119,14 @@ class StepBuilder:
         return arr[:len(table)]
 
     def build(self, entries: Sequence[Tuple[Hashable, Sequence[int], Sequence[int]]],
-              pad_pages: Optional[int] = None) -> StepContext:
+              pad_pages: Optional[int] = None, advance: int = 0, skip_tokens: bool = False) -> StepContext:
         """`entries`: (request, tokens, want).  The requests are live and hold pages for the
         positions `length .. length + len(tokens)`.  `pad_pages`: width of the block tables (at
         least what the longest request needs); with it the place of every array in the staging
-        buffer depends on the counts of tokens, requests and wanted rows only."""
+        buffer depends on the counts of tokens, requests and wanted rows only.  `advance`: the
+        requests are taken to be that many tokens longer than the cache manager says (steps that
+        are queued before the steps ahead of them are committed).  `skip_tokens`: the token ids
+        are not copied to the device (they are written there by the step before)."""
         ps = self.cache.page_size
         # Requests with a single token go first (in their order), the others after them: mixers
         # can then treat the two runs apart.  Wanted rows keep the callers' order.
@@ -125,7 +136,7 @@ class StepBuilder:
         entries = [given[i] for i in order]
         seqs = [self.cache.sequences[e[0]] for e in entries]
         q_lens = [len(e[1]) for e in entries]
-        starts = [s.length for s in seqs]
+        starts = [s.length + advance for s in seqs]
         n, s_count = sum(q_lens), len(entries)
         n_groups = len(self.cache.groups)
         max_pages = max(1, max(-(-(st + q) // ps) for st, q in zip(starts, q_lens)))
@@ -167,16 +178,17 @@ class StepBuilder:
             parts += [slots[g], tables[g].reshape(-1)]
         sizes = [p.size for p in parts]
         total = sum(sizes)
-        host, dev = self._staging(max(total, 1))
+        host, dev, slot = self._staging(max(total, 1))
         flat = host.numpy()
         off, views = 0, []
         for p, sz in zip(parts, sizes):
             flat[off:off + sz] = p
             views.append(dev[off:off + sz])
             off += sz
-        dev[:total].copy_(host[:total], non_blocking=True)
-        self._event = torch.cuda.Event()
-        self._event.record()
+        first = n if skip_tokens else 0                 # the token ids come first
+        dev[first:total].copy_(host[first:total], non_blocking=True)
+        self._events[slot] = torch.cuda.Event()
+        self._events[slot].record()
         groups = [GroupStep(ps, views[6 + 2 * g], views[7 + 2 * g].view(s_count, max_pages))
                   for g in range(n_groups)]
         max_kv = max(st + q for st, q in zip(starts, q_lens))

@@ -161,15 +161,50 @@ class Engine:
                 self.cache.commit(e.seq_id, len(e.tokens))
         return logits
 
+    def _bucket_pages(self, longest: int) -> int:
+        bucket_pages = max(1, self.GRAPH_BUCKET_TOKENS // self.page_size)
+        return -(-(-(-longest // self.page_size)) // bucket_pages) * bucket_pages
+
+    def chain_ready(self, seq_ids: Sequence[Hashable], steps: int) -> bool:
+        """Whether `decode_chain` can run these requests for `steps` steps: their shape has a
+        captured graph whose context bucket holds them to the end."""
+        if not self.use_graphs or steps < 1 or not seq_ids:
+            return False
+        pad_pages = self._bucket_pages(max(self.cache.sequences[s].length for s in seq_ids) + steps)
+        entry = self._graphs.get((len(seq_ids), len(seq_ids), pad_pages))
+        return entry is not None and entry != "seen"
+
+    def decode_chain(self, seq_ids: Sequence[Hashable], tokens: Sequence[int], steps: int) -> Optional[List[List[int]]]:
+        """`steps` greedy decode steps of the same requests, queued back to back: every step's
+        arg max is written on the device where the next step reads its token ids, so the host
+        prepares and queues step i+1 while step i runs and waits once at the end.  The requests
+        hold reserved pages for `steps` more tokens; nothing is committed here.  Returns the chosen
+        tokens `[steps][requests]`, or None when this shape has no captured graph yet (the caller
+        then takes single steps)."""
+        if not self.chain_ready(seq_ids, steps):
+            return None
+        pad_pages = self._bucket_pages(max(self.cache.sequences[s].length for s in seq_ids) + steps)
+        graph, logits = self._graphs[(len(seq_ids), len(seq_ids), pad_pages)]
+        generation = self.builder.generation
+        chosen = torch.empty((steps, len(seq_ids)), dtype=torch.int32, device=self.device)
+        for i in range(steps):
+            triples = [(sid, [tok if i == 0 else 0], [0]) for sid, tok in zip(seq_ids, tokens)]
+            ctx = self.builder.build(triples, pad_pages=pad_pages, advance=i, skip_tokens=i > 0)
+            if self.builder.generation != generation:
+                raise RuntimeError("the staging buffer moved under a captured graph")
+            graph.replay()
+            ops.argmax(logits, out=chosen[i])
+            ctx.token_ids.copy_(chosen[i])            # the next step's token ids, on the device
+            self.graph_replays += 1
+        return chosen.cpu().tolist()
+
     def _decode_step(self, triples) -> torch.Tensor:
         """One token a request, through a captured graph when this shape has been seen before.
         The block tables are padded to the bucket's width, so that every kernel argument is the
         same for all context lengths of the bucket; lengths and pages are read from device memory.
         The logits that are returned are the graph's own buffer: they hold until the next step."""
-        ps = self.page_size
         longest = max(self.cache.sequences[t[0]].length for t in triples) + 1
-        bucket_pages = max(1, self.GRAPH_BUCKET_TOKENS // ps)
-        pad_pages = -(-(-(-longest // ps)) // bucket_pages) * bucket_pages
+        pad_pages = self._bucket_pages(longest)
         n_want = sum(len(t[2]) for t in triples)
         generation = self.builder.generation
         ctx = self.builder.build(triples, pad_pages=pad_pages)

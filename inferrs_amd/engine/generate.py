@@ -8,7 +8,7 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence
 
 from ..sampling import Sampler, SamplingParams, fresh_seed
 from .engine import Engine, Entry
-from .scheduler import Plan, Request, Scheduler
+from .scheduler import Plan, PlannedEntry, Request, Scheduler
 
 
 @dataclass
@@ -24,8 +24,11 @@ class Generation:
 class GenerationLoop:
     def __init__(self, engine: Engine, *, max_batch_size: int = 32, max_tokens_per_step: int = 2048,
                  prefill_chunk: Optional[int] = None, max_seq_len: Optional[int] = None,
-                 stop_token_ids: Optional[Sequence[int]] = None):
+                 stop_token_ids: Optional[Sequence[int]] = None, decode_run: int = 8):
+        """`decode_run`: when every running request decodes greedily and nobody waits, up to this
+        many decode steps are queued on the GPU at once (`Engine.decode_chain`); 1 switches it off."""
         self.engine = engine
+        self.decode_run = max(1, decode_run)
         limit = engine.spec.max_position if not max_seq_len else min(max_seq_len, engine.spec.max_position)
         self.scheduler = Scheduler(
             engine.cache, max_batch_size=min(max_batch_size, engine.cache.max_seqs),
@@ -49,8 +52,35 @@ class GenerationLoop:
         self.scheduler.add(req)
         return req
 
-    def step(self) -> List[Request]:
-        """One scheduler step; returns the requests that finished in it (failed ones included)."""
+    def _try_decode_run(self, max_steps: int) -> Optional[List[Request]]:
+        """Several decode steps at once, when nothing else could happen in them anyway."""
+        sched = self.scheduler
+        running = list(sched.running)
+        if max_steps < 2 or not running or sched.waiting or len(running) > sched.max_tokens_per_step:
+            return None
+        if any(r.total - r.computed != 1 or not r.output or not r.params.is_plain_greedy for r in running):
+            return None
+        k = min(max_steps, min(min(r.params.max_tokens - len(r.output), sched.max_seq_len - r.total) for r in running))
+        ids = [r.request_id for r in running]
+        if k < 2 or not self.engine.chain_ready(ids, k) or not self.engine.cache.can_reserve([(i, k) for i in ids]):
+            return None
+        for i in ids:
+            self.engine.cache.reserve(i, k)
+        tokens = self.engine.decode_chain(ids, [r.tokens[-1] for r in running], k)
+        done: List[Request] = []
+        for i in range(k):
+            alive = [(j, r) for j, r in enumerate(running) if r.status == "running"]
+            plan = Plan(entries=[PlannedEntry(r, [r.tokens[-1]], True) for _, r in alive])
+            done += sched.commit(plan, {r.request_id: tokens[i][j] for j, r in alive})
+            self.steps += 1
+        return done
+
+    def step(self, max_steps: Optional[int] = None) -> List[Request]:
+        """One scheduler step, or a run of up to `decode_run` decode steps (at most `max_steps`);
+        returns the requests that finished (failed ones included)."""
+        run = self._try_decode_run(min(self.decode_run, max_steps if max_steps is not None else self.decode_run))
+        if run is not None:
+            return run
         plan: Plan = self.scheduler.plan()
         done = list(plan.failed)
         if not plan.entries:

@@ -398,10 +398,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
 
 # ---- sampling ---------------------------------------------------------------------------------
 
-def argmax(logits: torch.Tensor) -> torch.Tensor:
-    _dev(logits); _f32(logits, "logits")
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The lowest index among each row's maxima, int32 [rows] (into `out` when given)."""
+    _dev(logits, out); _f32(logits, "logits")
     rows, vocab = logits.shape
-    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    elif out.dtype != torch.int32 or out.numel() != rows:
+        raise KernelError(f"argmax: `out` must be int32 [{rows}]")
     words = library().ia_argmax_workspace(rows, vocab)
     ws = torch.empty((words,), dtype=torch.int32, device=logits.device) if words else None
     _check(library().ia_argmax(_p(out), _p(logits), _p(ws), rows, vocab, _stream()))

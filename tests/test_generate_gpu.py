@@ -146,3 +146,34 @@ def test_command_line_run_and_bench(tiny):
     assert [int(t) for t in out[4].split()] == want
     proc = subprocess.run(exe + ["serve", folder], capture_output=True, text=True, timeout=60)
     assert proc.returncode == 2 and "not part of this engine" in proc.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_runs_of_decode_steps_give_the_same_tokens_as_single_steps(tiny, dtype):
+    """Greedy requests decode several steps at a time once their shape is captured; the tokens,
+    the stop at a stop token in the middle of a run and the end at max_tokens are those of
+    single steps."""
+    from inferrs_amd.engine import Engine, GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 300 + n) for n in (7, 30, 12)]
+    results = {}
+    for run in (1, 8):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=64, max_seqs=4)
+        loop = GenerationLoop(eng, decode_run=run)
+        stop = None if run == 1 else results[1][0][20]           # a token that request 0 emits on its way
+        sp = [SamplingParams.greedy(max_tokens=40, extra_stop_token_ids=() if i or stop is None else (stop,))
+              for i in range(3)]
+        sp[2] = SamplingParams.greedy(max_tokens=23)
+        reqs = [loop.add(p, s) for p, s in zip(prompts, sp)]
+        loop.run()
+        results[run] = [list(r.output) for r in reqs]
+        if run == 8:
+            assert eng.graph_replays > 10
+            assert reqs[0].finish_reason == "stop" and reqs[1].finish_reason == reqs[2].finish_reason == "length"
+        eng.cache.check_invariants()
+        assert not eng.cache.sequences
+    first = results[1][0].index(results[1][0][20])
+    assert results[8][0] == results[1][0][:first + 1]
+    assert results[8][1] == results[1][1] and results[8][2] == results[1][2] and len(results[8][2]) == 23
