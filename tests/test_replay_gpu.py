@@ -239,3 +239,47 @@ def test_logits_head_follows_the_tensor_present(tmp_path, name, drop):
     eng = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=4, max_seqs=1)
     got = eng.step([Entry("a", toks, list(range(21)))]).cpu().numpy()
     assert float(np.abs(got - want).max()) <= 1e-5 * float(np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_in_every_cutting(tmp_path, dtype):
+    """A 2,500-token request with the serving head size: whole; in portions of 512 beside a
+    second request; and its last 40 tokens decoded one by one (through the split-key kernel and,
+    from the third step on, a captured graph).  Sharpened attention makes every query depend on a
+    few keys that may lie thousands of positions back."""
+    from inferrs_amd.engine import Engine, run_trace
+    raw = dict(TINY["D"], max_position_embeddings=4096)
+    folder = write_model(str(tmp_path / "m"), raw, seed=9, sharpen=SHARP[dtype])
+    cfg, params = pm.read_model(folder, torch.float64)
+    long_req = random_tokens(2500, raw["vocab_size"], 77)
+    other = random_tokens(300, raw["vocab_size"], 78)
+    ref = pm.forward(cfg, params, long_req).numpy().astype(np.float32)
+    watch = list(range(0, 2500, 97)) + list(range(2440, 2500))
+    scale = float(np.abs(ref).max())
+    if dtype == "float32":
+        limit = TOL_PLAIN_F32
+    else:
+        cfg_b, params_b = pm.read_model(folder, torch.bfloat16)
+        rounded = pm.forward(cfg_b, params_b, long_req).float().numpy()
+        limit = float(np.abs(rounded[watch] - ref[watch]).max()) / scale
+
+    def run(trace, name):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-trace.max_tokens // 16), max_seqs=2)
+        run_trace(eng, trace.lines, str(tmp_path / name), io.StringIO())
+        return trace.read(str(tmp_path / name), raw["vocab_size"])["long"]
+
+    whole = tm.Trace()
+    whole.step([("long", long_req, watch)], end=["long"])
+    cut = tm.Trace()
+    for i in range(0, 2460, 512):
+        part = long_req[i:min(i + 512, 2460)]
+        entries = [("long", part, [w - i for w in watch if i <= w < i + len(part)])]
+        if i == 512:
+            entries.append(("other", other, []))
+        cut.step(entries, end=["other"] if i == 1024 else [])
+    for i in range(2460, 2500):
+        cut.step([("long", long_req[i:i + 1], [0])], end=["long"] if i == 2499 else [])
+    for name, trace in (("whole", whole), ("cut", cut)):
+        got = run(trace, name)
+        err = max(float(np.abs(got[w] - ref[w]).max()) for w in watch) / scale
+        assert err <= limit, f"{name}: {err:.3e} of the scale, the bound is {limit:.3e}"
