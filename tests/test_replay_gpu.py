@@ -283,3 +283,34 @@ def test_long_context_in_every_cutting(tmp_path, dtype):
         got = run(trace, name)
         err = max(float(np.abs(got[w] - ref[w]).max()) for w in watch) / scale
         assert err <= limit, f"{name}: {err:.3e} of the scale, the bound is {limit:.3e}"
+
+
+def test_captured_steps_with_the_vendor_gemm_equal_eager_ones(models, tmp_path):
+    """More than 16 requests decode through the vendor's GEMM; those calls are captured into
+    the graph too.  Every replay must equal the eager step, with eager steps and
+    synchronisations in between."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, raw, reqs, ref = pick(models, "D", False, "bfloat16")
+    n_req, n_steps = 24, 14
+    prompts = [random_tokens(5 + 3 * i, raw["vocab_size"], 500 + i) for i in range(n_req)]
+    feeds = [random_tokens(n_steps, raw["vocab_size"], 600 + i) for i in range(n_req)]
+    outs = {}
+    for graphs in (False, True):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=n_req * 8 + 4, max_seqs=n_req + 1,
+                                 use_graphs=graphs)
+        for i, p in enumerate(prompts):
+            eng.step([Entry(i, p, [])])
+        rows = []
+        for s in range(n_steps):
+            logits = eng.step([Entry(i, [feeds[i][s]], [0]) for i in range(n_req)])
+            rows.append(logits.cpu().numpy().copy())
+            if s % 4 == 1:                       # an eager step of another shape between the replays
+                eng.step([Entry("extra", random_tokens(9, raw["vocab_size"], s), [8])])
+                eng.end_request("extra")
+        outs[graphs] = rows
+        assert (eng.graph_replays >= n_steps - 2) == graphs
+    # the captured step pads its block tables to the bucket, which may split the keys differently:
+    # the two runs agree to bfloat16 rounding, and every replay alike (a replay gone wrong is far off)
+    scale = max(float(np.abs(o).max()) for o in outs[False])
+    errs = [float(np.abs(outs[True][s] - outs[False][s]).max()) / scale for s in range(n_steps)]
+    assert max(errs) <= 2 ** -6, f"replays differ from eager steps: {errs}"
