@@ -41,7 +41,7 @@ def test_greedy_generation_matches_plain(tiny, name, dtype):
     from inferrs_amd.sampling import SamplingParams
     folder, cfg, params = tiny[name]
     vocab = TINY[name]["vocab_size"]
-    prompts = [random_tokens(n, vocab, 50 + n) for n in (5, 17, 33, 1)]       # BASELINE's tiny workload, and one token
+    prompts = [random_tokens(n, vocab, 50 + n) for n in (5, 17, 33, 1)]       # prompts of 5, 17 and 33 tokens with 16 greedy tokens each, and a prompt of one token
     eng = Engine.from_folder(folder, dtype=dtype, page_size=4, num_pages=64, max_seqs=4)
     outs = eng.generate(prompts, SamplingParams.greedy(max_tokens=16), max_tokens_per_step=24, prefill_chunk=16)
     for prompt, out in zip(prompts, outs):
@@ -64,7 +64,7 @@ def test_seeded_temperature_is_reproducible_and_independent_of_the_batch(tiny):
     from inferrs_amd.sampling import SamplingParams
     folder, cfg, params = tiny["B"]
     vocab = TINY["B"]["vocab_size"]
-    prompts = [random_tokens(n, vocab, 70 + n) for n in (1, 9, 64, 100)]      # BASELINE's second tiny workload
+    prompts = [random_tokens(n, vocab, 70 + n) for n in (1, 9, 64, 100)]      # prompts of 1, 9, 64 and 100 tokens at temperature 0.7 under fixed seeds, portions of 16
     sp = [SamplingParams(temperature=0.7, top_p=1.0, top_k=0, repetition_penalty=1.0, max_tokens=12, seed=40 + i)
           for i in range(4)]
     eng = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=64, max_seqs=4)
