@@ -8,13 +8,15 @@ its cached length, and no mask is built: kernels derive causality from `position
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass, field
 from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from ..cache.manager import RELEASED, CacheManager
+from .. import native
+from ..cache.manager import CacheManager
 
 
 @dataclass
@@ -65,28 +67,32 @@ class StepError(ValueError):
 
 
 class StepBuilder:
-    """Turns (request, its next tokens, wanted places) into a `StepContext`: everything the
-    kernels need goes to the device in one copy from a pinned staging buffer."""
+    """Turns (request, its next tokens, wanted places) into a `StepContext`.  The native runtime
+    writes every array of the step into a pinned staging buffer (`iar_build_step` in
+    `csrc/runtime.cpp`), and one copy takes it to the device."""
+
+    RING = 16
 
     def __init__(self, cache: CacheManager, device):
         self.cache = cache
         self.device = torch.device(device)
+        self._lib = native.runtime()
         # One device buffer (its address is what captured graphs hold) and a ring of pinned host
         # buffers, so that the copies of several steps can be under way at once.
         self._ring: List[torch.Tensor] = []
+        self._flat: List[np.ndarray] = []
         self._events: List[Optional[torch.cuda.Event]] = []
         self._next = 0
         self._dev: Optional[torch.Tensor] = None
-        self._rows: Dict[Any, list] = {}
+        self._meta = (ctypes.c_int * 16)()
         self.generation = 0                # grows when the device staging buffer moves
-
-    RING = 16
 
     def _staging(self, n: int) -> Tuple[torch.Tensor, torch.Tensor, int]:
         if self._dev is None or self._dev.numel() < n:
             size = 1 << max(12, (n - 1).bit_length())
             torch.cuda.synchronize(self.device)
             self._ring = [torch.empty(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+            self._flat = [t.numpy() for t in self._ring]
             self._events = [None] * self.RING
             self._dev = torch.empty(size, dtype=torch.int32, device=self.device)
             self.generation += 1
@@ -96,110 +102,71 @@ class StepBuilder:
             self._events[slot].synchronize()      # that copy has left the host buffer
         return self._ring[slot], self._dev, slot
 
-    def _table_row(self, group: int, seq, need: int) -> np.ndarray:
-        """The request's pages of one group as an int32 array, kept between steps and extended
-        by the pages that were added since (tables only grow, except where a window releases)."""
-        table = seq.tables[group]
-        if self.cache.groups[group].need.window is not None:
-            return np.asarray(table, dtype=np.int32)
-        key = (group, seq.seq_id)
-        hit = self._rows.get(key)
-        if hit is None or hit[0] is not seq or hit[1].size < len(table):
-            arr = np.zeros(max(64, 2 * len(table), need), dtype=np.int32)
-            arr[:len(table)] = table
-            if len(self._rows) > 4 * max(len(self.cache.sequences), 16):
-                live = self.cache.sequences
-                self._rows = {k: v for k, v in self._rows.items() if live.get(k[1]) is v[0]}
-            self._rows[key] = [seq, arr, len(table)]
-            return arr[:len(table)]
-        _, arr, filled = hit
-        if len(table) > filled:
-            arr[filled:len(table)] = table[filled:]
-            hit[2] = len(table)
-        return arr[:len(table)]
-
     def build(self, entries: Sequence[Tuple[Hashable, Sequence[int], Sequence[int]]],
               pad_pages: Optional[int] = None, advance: int = 0, skip_tokens: bool = False) -> StepContext:
         """`entries`: (request, tokens, want).  The requests are live and hold pages for the
-        positions `length .. length + len(tokens)`.  `pad_pages`: width of the block tables (at
-        least what the longest request needs); with it the place of every array in the staging
-        buffer depends on the counts of tokens, requests and wanted rows only.  `advance`: the
-        requests are taken to be that many tokens longer than the cache manager says (steps that
-        are queued before the steps ahead of them are committed).  `skip_tokens`: the token ids
-        are not copied to the device (they are written there by the step before)."""
-        ps = self.cache.page_size
-        # Requests with a single token go first (in their order), the others after them: mixers
-        # can then treat the two runs apart.  Wanted rows keep the callers' order.
-        order = sorted(range(len(entries)), key=lambda i: len(entries[i][1]) != 1)
-        rank = {orig: new for new, orig in enumerate(order)}
-        given = entries
-        entries = [given[i] for i in order]
-        seqs = [self.cache.sequences[e[0]] for e in entries]
-        q_lens = [len(e[1]) for e in entries]
-        starts = [s.length + advance for s in seqs]
-        n, s_count = sum(q_lens), len(entries)
-        n_groups = len(self.cache.groups)
-        max_pages = max(1, max(-(-(st + q) // ps) for st, q in zip(starts, q_lens)))
-        if pad_pages is not None:
-            if pad_pages < max_pages:
-                raise StepError(f"block tables of {pad_pages} pages are too narrow for {max_pages}")
-            max_pages = pad_pages
-        cu = np.zeros(s_count + 1, dtype=np.int64)
-        np.cumsum(q_lens, out=cu[1:])
-        if n == s_count:                                   # one token a request
-            token_ids = np.fromiter((e[1][0] for e in entries), dtype=np.int32, count=n)
-            positions = np.asarray(starts, dtype=np.int32)
-            token_seq = np.arange(s_count, dtype=np.int32)
+        positions `length .. length + len(tokens)`.  Requests with a single token are put first (in
+        their order), the others after them: mixers can then treat the two runs apart; wanted rows
+        keep the callers' order.  `pad_pages`: width of the block tables (at least what the longest
+        request needs); with it the place of every array in the staging buffer depends on the
+        counts of tokens, requests and wanted rows only.  `advance`: the requests are taken to be
+        that many tokens longer than the cache manager says (steps that are queued before the
+        steps ahead of them are committed).  `skip_tokens`: the token ids are not copied to the
+        device (they are written there by the step before)."""
+        s_count = len(entries)
+        names = self.cache.names
+        key_list = []
+        for e in entries:
+            k = names.find(e[0])
+            if k is None:
+                raise StepError(f"request {e[0]!r} is not live")
+            key_list.append(k)
+        q_given = [len(e[1]) for e in entries]
+        n = sum(q_given)
+        want_counts = [len(e[2]) for e in entries]
+        n_want = sum(want_counts)
+        if n == s_count:
+            tokens = native.ints([e[1][0] for e in entries])
+        elif n <= 256:
+            tokens = native.ints([t for e in entries for t in e[1]])
         else:
-            token_ids = np.concatenate([np.asarray(e[1], dtype=np.int32) for e in entries])
-            positions = np.concatenate([np.arange(st, st + q, dtype=np.int32) for st, q in zip(starts, q_lens)])
-            token_seq = np.repeat(np.arange(s_count, dtype=np.int32), q_lens)
-        want = np.asarray([cu[rank[i]] + w for i, e in enumerate(given) for w in e[2]], dtype=np.int32)
-        state_slots = np.asarray([s.state_slot for s in seqs], dtype=np.int32)
-        tables, slots = [], []
-        for g in range(n_groups):
-            bt = np.zeros((s_count, max_pages), dtype=np.int32)
-            for i, s in enumerate(seqs):
-                need = -(-(starts[i] + q_lens[i]) // ps)
-                row = self._table_row(g, s, need)
-                if row.size < need:
-                    raise StepError(f"request {s.seq_id!r} holds {row.size} pages, too few for "
-                                    f"{starts[i] + q_lens[i]} tokens")
-                bt[i, :min(row.size, max_pages)] = row[:max_pages]
-            pages_of_token = bt[token_seq, positions // ps]
-            if n and (pages_of_token == RELEASED).any():
-                raise StepError("a new token falls into a page that was already released")
-            slots.append((pages_of_token * ps + positions % ps).astype(np.int32))
-            np.maximum(bt, 0, out=bt)                 # released pages are never read
-            tables.append(bt)
-
-        parts = [token_ids, positions, token_seq, cu.astype(np.int32), state_slots, want]
-        for g in range(n_groups):
-            parts += [slots[g], tables[g].reshape(-1)]
-        sizes = [p.size for p in parts]
-        total = sum(sizes)
-        host, dev, slot = self._staging(max(total, 1))
-        flat = host.numpy()
-        off, views = 0, []
-        for p, sz in zip(parts, sizes):
-            flat[off:off + sz] = p
-            views.append(dev[off:off + sz])
-            off += sz
+            tokens = np.concatenate([np.asarray(e[1], dtype=np.int32) for e in entries])
+        want = native.ints([w for e in entries for w in e[2]])
+        c_keys, c_q, c_wc = native.keys(key_list), native.ints(q_given), native.ints(want_counts)
+        pad = pad_pages if pad_pages is not None else 0
+        lib, handle = self._lib, self.cache.handle
+        total = lib.iar_step_words(handle, s_count, c_keys, c_q, n_want, pad, advance)
+        if total < 0:
+            raise StepError(native.last_error())
+        host, dev, slot = self._staging(max(int(total), 1))
+        flat = self._flat[slot]
+        order = (ctypes.c_int * max(s_count, 1))()
+        meta = self._meta
+        token_ptr = tokens.ctypes.data if isinstance(tokens, np.ndarray) else ctypes.addressof(tokens)
+        if lib.iar_build_step(handle, s_count, c_keys, c_q, token_ptr, c_wc, want, pad, advance,
+                              host.data_ptr(), host.numel(), meta, order):
+            raise StepError(native.last_error())
+        total, max_pages, n_groups = meta[0], meta[4], meta[10]
         first = n if skip_tokens else 0                 # the token ids come first
         dev[first:total].copy_(host[first:total], non_blocking=True)
         self._events[slot] = torch.cuda.Event()
         self._events[slot].record()
-        groups = [GroupStep(ps, views[6 + 2 * g], views[7 + 2 * g].view(s_count, max_pages))
-                  for g in range(n_groups)]
-        max_kv = max(st + q for st, q in zip(starts, q_lens))
-        n_single = sum(1 for q in q_lens if q == 1)
-        kv_single = max([st + 1 for st, q in zip(starts, q_lens) if q == 1], default=0)
-        kv_multi = max([st + q for st, q in zip(starts, q_lens) if q != 1], default=0)
-        if pad_pages is not None:
-            kv_single = max(kv_single, pad_pages * ps) if n_single else 0
+        off = 0
+        views = []
+        for sz in (n, n, n, s_count + 1, s_count, n_want):
+            views.append(dev[off:off + sz])
+            off += sz
+        cu_off, slot_off = 3 * n, 3 * n + s_count + 1
+        groups = []
+        for _ in range(n_groups):
+            slots = dev[off:off + n]
+            off += n
+            groups.append(GroupStep(self.cache.page_size, slots, dev[off:off + s_count * max_pages].view(s_count, max_pages)))
+            off += s_count * max_pages
+        cu = flat[cu_off:cu_off + s_count]
         return StepContext(
             n_tokens=n, n_seqs=s_count, token_ids=views[0], positions=views[1], token_seq=views[2],
             cu_tokens=views[3], state_slots=views[4], want_rows=views[5], groups=groups,
-            q_lens=q_lens, kv_starts=starts, state_slots_host=[int(x) for x in state_slots],
-            max_q_len=max(q_lens), max_kv_len=max_kv if pad_pages is None else max(max_kv, pad_pages * ps),
-            n_single=n_single, max_kv_single=kv_single, max_kv_multi=kv_multi)
+            q_lens=[q_given[order[j]] for j in range(s_count)], kv_starts=flat[n + cu].tolist(),
+            state_slots_host=flat[slot_off:slot_off + s_count].tolist(),
+            max_q_len=meta[5], max_kv_len=meta[6], n_single=meta[7], max_kv_single=meta[8], max_kv_multi=meta[9])

@@ -111,7 +111,7 @@ class Engine:
         self.cache.free_sequence(seq_id)
 
     def cached_length(self, seq_id: Hashable) -> int:
-        return self.cache.sequences[seq_id].length
+        return self.cache.length(seq_id)
 
     # ---- the step ---------------------------------------------------------------------------
     def step(self, entries: Sequence[Entry], commit: bool = True) -> torch.Tensor:
@@ -133,18 +133,14 @@ class Engine:
                 raise StepError(f"request {e.seq_id!r}: token ids must lie in 0..{vocab - 1}")
             if any(not (0 <= w < len(e.tokens)) for w in e.want):
                 raise StepError(f"request {e.seq_id!r}: 'want' {e.want} outside its {len(e.tokens)} tokens")
-        fresh = [e.seq_id for e in entries if e.seq_id not in self.cache.sequences]
+        ids = [e.seq_id for e in entries]
+        fresh = [] if self.cache.all_live(ids) else [s for s in ids if s not in self.cache.sequences]
         try:
             for sid in fresh:
                 self.add_request(sid)
-            asks = [(e.seq_id, max(0, len(e.tokens) - self.cache.sequences[e.seq_id].reserved))
-                    for e in entries]
-            if not self.cache.can_reserve(asks):
+            if not self.cache.ensure_reserved([(e.seq_id, len(e.tokens)) for e in entries]):
                 raise OutOfPages("paged attention: out of KV blocks for this step "
                                  f"({[g.pool.num_free for g in self.cache.groups]} pages free)")
-            for sid, n in asks:
-                if n and not self.cache.reserve(sid, n):
-                    raise OutOfPages("paged attention: out of KV blocks")
         except Exception:
             for sid in fresh:
                 if sid in self.cache.sequences:
@@ -157,8 +153,7 @@ class Engine:
         else:
             logits = self.model.forward(self.builder.build(triples), self.storage)
         if commit:
-            for e in entries:
-                self.cache.commit(e.seq_id, len(e.tokens))
+            self.cache.commit_many([(e.seq_id, len(e.tokens)) for e in entries])
         return logits
 
     def _bucket_pages(self, longest: int) -> int:
@@ -170,7 +165,7 @@ class Engine:
         captured graph whose context bucket holds them to the end."""
         if not self.use_graphs or steps < 1 or not seq_ids:
             return False
-        pad_pages = self._bucket_pages(max(self.cache.sequences[s].length for s in seq_ids) + steps)
+        pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
         entry = self._graphs.get((len(seq_ids), len(seq_ids), pad_pages))
         return entry is not None and entry != "seen"
 
@@ -183,7 +178,7 @@ class Engine:
         then takes single steps)."""
         if not self.chain_ready(seq_ids, steps):
             return None
-        pad_pages = self._bucket_pages(max(self.cache.sequences[s].length for s in seq_ids) + steps)
+        pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
         graph, logits = self._graphs[(len(seq_ids), len(seq_ids), pad_pages)]
         generation = self.builder.generation
         chosen = torch.empty((steps, len(seq_ids)), dtype=torch.int32, device=self.device)
@@ -203,7 +198,7 @@ class Engine:
         The block tables are padded to the bucket's width, so that every kernel argument is the
         same for all context lengths of the bucket; lengths and pages are read from device memory.
         The logits that are returned are the graph's own buffer: they hold until the next step."""
-        longest = max(self.cache.sequences[t[0]].length for t in triples) + 1
+        longest = self.cache.max_length([t[0] for t in triples]) + 1
         pad_pages = self._bucket_pages(longest)
         n_want = sum(len(t[2]) for t in triples)
         generation = self.builder.generation

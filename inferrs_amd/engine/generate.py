@@ -8,7 +8,7 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence
 
 from ..sampling import Sampler, SamplingParams, fresh_seed
 from .engine import Engine, Entry
-from .scheduler import Plan, PlannedEntry, Request, Scheduler
+from .scheduler import Plan, Request, Scheduler
 
 
 @dataclass
@@ -69,9 +69,7 @@ class GenerationLoop:
         tokens = self.engine.decode_chain(ids, [r.tokens[-1] for r in running], k)
         done: List[Request] = []
         for i in range(k):
-            alive = [(j, r) for j, r in enumerate(running) if r.status == "running"]
-            plan = Plan(entries=[PlannedEntry(r, [r.tokens[-1]], True) for _, r in alive])
-            done += sched.commit(plan, {r.request_id: tokens[i][j] for j, r in alive})
+            done += sched.commit_decode(running, tokens[i])
             self.steps += 1
         return done
 
@@ -86,8 +84,6 @@ class GenerationLoop:
         if not plan.entries:
             return done
         for e in plan.entries:
-            if not self.engine.has_request(e.request.request_id):
-                raise RuntimeError(f"request {e.request.request_id!r} was planned without a cache entry")
             if e.request.computed == 0:
                 self.engine.storage.clear_state_slot(self.engine.cache.sequences[e.request.request_id].state_slot)
         entries = [Entry(e.request.request_id, e.tokens, [len(e.tokens) - 1] if e.samples else [])

@@ -1,6 +1,6 @@
 """The scheduler: admits requests, cuts prompts into portions under a token budget, decodes,
-finishes and frees.  Host-only bookkeeping over a `CacheManager`; it never touches the GPU, so
-its decisions can be tested without one.
+finishes and frees.  Host-only bookkeeping over a `CacheManager`, done by the native runtime; it
+never touches the GPU, so its decisions can be tested without one.
 
 The reference's loop (`inferrs/src/engine.rs:1380-1912`) admits from a FIFO channel while
 fewer than `max_batch_size` requests are active, runs each request's whole prompt in one pass
@@ -24,10 +24,11 @@ request that could not fit even alone fails with the reference's error.
 """
 from __future__ import annotations
 
-from collections import deque
+import ctypes
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, Hashable, List, Optional, Sequence
 
+from .. import native
 from ..cache.manager import CacheManager
 from ..sampling.params import SamplingParams
 
@@ -77,6 +78,10 @@ class Plan:
 
 
 class Scheduler:
+    """The decisions are taken by the native scheduler (`csrc/runtime.cpp`), which works on the
+    cache manager's native object directly; this class names the requests, keeps their Python
+    records (`Request`: sampling parameters, seed, output) in step with it and hands out plans."""
+
     def __init__(self, cache: CacheManager, *, max_batch_size: int = 32, max_tokens_per_step: int = 2048,
                  prefill_chunk: Optional[int] = None, max_seq_len: int = 40960,
                  stop_token_ids: Sequence[int] = ()):
@@ -84,10 +89,6 @@ class Scheduler:
         `inferrs/src/main.rs:137-138`); `max_tokens_per_step`: token budget of one step (default
         2048, `main.rs:141-142`); `prefill_chunk`: longest portion of one prompt in a step (None: the
         budget); `max_seq_len`: prompt plus output never exceed it (`inferrs/src/server.rs:3680-3695`)."""
-        if max_batch_size < 1 or max_tokens_per_step < 1:
-            raise ValueError("max_batch_size and max_tokens_per_step must be >= 1")
-        if max_batch_size > cache.max_seqs:
-            raise ValueError(f"max_batch_size {max_batch_size} exceeds the cache's {cache.max_seqs} request slots")
         if prefill_chunk is not None and prefill_chunk < 1:
             raise ValueError("prefill_chunk must be >= 1")
         self.cache = cache
@@ -96,166 +97,133 @@ class Scheduler:
         self.prefill_chunk = prefill_chunk or max_tokens_per_step
         self.max_seq_len = max_seq_len
         self.stop_token_ids = frozenset(int(t) for t in stop_token_ids)
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []            # in order of admission
+        self._lib = native.runtime()
+        stops = sorted(self.stop_token_ids)
+        self._ptr = self._lib.iar_sched_create(cache.handle, max_batch_size, max_tokens_per_step, self.prefill_chunk,
+                                               max_seq_len, native.ints(stops), len(stops))
+        if not self._ptr:
+            raise ValueError(native.last_error())
+        self._requests: Dict[int, Request] = {}      # key -> record of every request not yet finished
         self.finished: Dict[Hashable, Request] = {}
         self._arrivals = 0
+        self._room = 0
+        self._grow(max(64, max_batch_size))
+
+    def __del__(self):
+        if getattr(self, "_ptr", None):
+            self._lib.iar_sched_destroy(self._ptr)
+            self._ptr = None
+
+    def _grow(self, n: int) -> None:
+        """Buffers that the native side fills with up to n requests."""
+        if n <= self._room:
+            return
+        self._room = n
+        self._keys = (ctypes.c_int64 * n)()
+        self._a, self._b, self._c = (ctypes.c_int * n)(), (ctypes.c_int * n)(), (ctypes.c_int * n)()
 
     # ---- requests ---------------------------------------------------------------------------
     def add(self, request: Request) -> None:
-        if not request.prompt:
-            raise ValueError(f"request {request.request_id!r}: the prompt is empty")
-        if len(request.prompt) >= self.max_seq_len:
-            raise ValueError(f"request {request.request_id!r}: the prompt has {len(request.prompt)} tokens, "
-                             f"the limit is {self.max_seq_len - 1}")
+        key = self.cache.names.pin(request.request_id)
+        p = request.params
+        extra = [int(t) for t in p.extra_stop_token_ids]
+        if self._lib.iar_sched_add(self._ptr, key, native.ints(request.prompt), len(request.prompt), int(p.max_tokens),
+                                   int(bool(p.bypass_stop_tokens)), native.ints(extra), len(extra)):
+            self.cache.names.unpin(request.request_id, live=request.request_id in self.cache.sequences)
+            raise ValueError(f"request {request.request_id!r}: {native.last_error()}")
         request.arrival = self._arrivals
         self._arrivals += 1
         request.status = WAITING
-        self.waiting.append(request)
+        self._requests[key] = request
+        self._grow(len(self._requests))
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._lib.iar_sched_num_waiting(self._ptr) or self._lib.iar_sched_num_running(self._ptr))
 
-    def _pages_total(self) -> int:
-        return min(g.pool.num_pages for g in self.cache.groups) if self.cache.groups else 1 << 60
+    @property
+    def waiting(self) -> List[Request]:
+        """The line of requests that wait, first in line first."""
+        n = self._lib.iar_sched_waiting(self._ptr, self._keys, self._room)
+        return [self._requests[k] for k in self._keys[:n]]
 
-    def _fits_alone(self, n_tokens: int) -> bool:
-        return -(-n_tokens // self.cache.page_size) <= self._pages_total()
+    @property
+    def running(self) -> List[Request]:
+        """The running requests in order of admission."""
+        n = self._lib.iar_sched_running(self._ptr, self._keys, self._room)
+        return [self._requests[k] for k in self._keys[:n]]
+
+    def _finish(self, key: int, r: Request, reason: str, error: Optional[str] = None) -> None:
+        r.status, r.finish_reason, r.error = FINISHED, reason, error
+        self.finished[r.request_id] = r
+        del self._requests[key]
+        self._lib.iar_sched_forget(self._ptr, key)
+        self.cache.names.unpin(r.request_id, live=False)
 
     # ---- planning ---------------------------------------------------------------------------
     def plan(self) -> Plan:
         """Decide the next step and reserve its pages.  May preempt or fail requests."""
+        lib, ptr = self._lib, self._ptr
         plan = Plan()
-        budget = self.max_tokens_per_step
-
-        # 1. decodes: running requests with exactly one token left to feed
-        decoding = [r for r in self.running if r.total - r.computed == 1 and r.output]
-        for r in decoding:
-            if r not in self.running:               # preempted while serving an earlier one
-                continue
-            if budget < 1:
-                break
-            while not self.cache.reserve(r.request_id, 1):
-                victim = self._preempt_latest(exclude=r)
-                if victim is None:
-                    # it holds every page there is and needs one more: it cannot go on
-                    self._fail(r, f"{OUT_OF_BLOCKS} at position {r.computed}")
-                    plan.failed.append(r)
-                    break
-                plan.preempted.append(victim)
-                budget += sum(len(e.tokens) for e in plan.entries if e.request is victim)
-                plan.entries = [e for e in plan.entries if e.request is not victim]
-            else:
-                plan.entries.append(PlannedEntry(r, [r.tokens[-1]], True))
-                budget -= 1
-
-        # 2. portions of prompts of running requests, oldest first
-        planned = {id(e.request) for e in plan.entries}
-        for r in list(self.running):
-            if budget < 1:
-                break
-            if id(r) in planned or r.total - r.computed < 1:
-                continue
-            if r.total - r.computed == 1 and r.output:
-                continue                                  # a decode that found no budget
-            n = min(r.total - r.computed, self.prefill_chunk, budget)
-            if not self.cache.reserve(r.request_id, n):
-                continue                                  # waits for pages; decodes above free them as they finish
-            plan.entries.append(PlannedEntry(r, r.tokens[r.computed:r.computed + n], r.computed + n == r.total))
-            budget -= n
-
-        # 3. admissions, in arrival order
-        while self.waiting and budget >= 1 and len(self.running) < self.max_batch_size:
-            r = self.waiting[0]
-            if not self._fits_alone(r.total + 1):
-                self.waiting.popleft()
-                self._fail(r, f"{OUT_OF_BLOCKS}: the request needs {-(-(r.total + 1) // self.cache.page_size)} "
-                              f"pages, the pool has {self._pages_total()}", live=False)
-                plan.failed.append(r)
-                continue
-            n = min(r.total - r.computed, self.prefill_chunk, budget)
-            self.cache.add_sequence(r.request_id)
-            # admitted only when all it has so far, and one token more, would fit now: a request
-            # that is let in on its first portion alone tends to be preempted later
-            if not self.cache.can_reserve([(r.request_id, r.total + 1)]) or not self.cache.reserve(r.request_id, n):
-                self.cache.free_sequence(r.request_id)
-                break                                     # no pages now: it stays first in line
-            self.waiting.popleft()
-            r.status = RUNNING
-            self.running.append(r)
-            plan.entries.append(PlannedEntry(r, r.tokens[r.computed:r.computed + n], r.computed + n == r.total))
-            budget -= n
-
-        if not plan.entries and self.running and not plan.failed and not plan.preempted:
-            # Every running request waits for pages that nobody will free: preempt the latest so
-            # that the oldest can go on.
-            victim = self._preempt_latest(exclude=self.running[0])
-            if victim is not None:
-                plan.preempted.append(victim)
-                return self._merge(plan, self.plan())
-            r = self.running[0]
-            self._fail(r, f"{OUT_OF_BLOCKS} at position {r.computed}")
+        n = lib.iar_sched_plan(ptr)
+        for k in self._keys[:lib.iar_sched_plan_preempted(ptr, self._keys, self._room)]:
+            r = self._requests[k]
+            r.computed, r.status = 0, WAITING
+            r.preemptions += 1
+            plan.preempted.append(r)
+        for k in list(self._keys[:lib.iar_sched_plan_failed(ptr, self._keys, self._room)]):
+            r = self._requests[k]
+            self._finish(k, r, "error", lib.iar_sched_failure(ptr, k).decode("utf-8", "replace"))
             plan.failed.append(r)
+        lib.iar_sched_plan_entries(ptr, self._keys, self._a, self._b, self._c)
+        for i in range(n):
+            r = self._requests[self._keys[i]]
+            r.status = RUNNING
+            start, count = self._a[i], self._b[i]
+            if count == 1 and start >= len(r.prompt):
+                tokens = [r.output[start - len(r.prompt)]]
+            else:
+                tokens = r.tokens[start:start + count]
+            plan.entries.append(PlannedEntry(r, tokens, bool(self._c[i])))
         return plan
 
-    @staticmethod
-    def _merge(first: Plan, second: Plan) -> Plan:
-        second.preempted = first.preempted + second.preempted
-        second.failed = first.failed + second.failed
-        return second
-
-    def _preempt_latest(self, exclude: Request) -> Optional[Request]:
-        for victim in reversed(self.running):
-            if victim is exclude:
-                continue
-            self.running.remove(victim)
-            self.cache.free_sequence(victim.request_id)
-            victim.computed = 0
-            victim.status = WAITING
-            victim.preemptions += 1
-            self.waiting.appendleft(victim)
-            return victim
-        return None
-
-    def _fail(self, r: Request, message: str, live: bool = True) -> None:
-        if live:
-            if r in self.running:
-                self.running.remove(r)
-            if r.request_id in self.cache.sequences:
-                self.cache.free_sequence(r.request_id)
-        r.status, r.finish_reason, r.error = FINISHED, "error", message
-        self.finished[r.request_id] = r
-
     # ---- after the step ---------------------------------------------------------------------
-    def commit(self, plan: Plan, sampled: Dict[Hashable, int]) -> List[Request]:
-        """The step ran: `sampled[request_id]` is the token drawn for every entry that
-        `samples`.  Returns the requests that finished."""
-        done: List[Request] = []
-        for e in plan.entries:
-            r = e.request
-            self.cache.commit(r.request_id, len(e.tokens))
-            r.computed += len(e.tokens)
-            if not e.samples:
-                continue
-            token = int(sampled[r.request_id])
-            r.output.append(token)
-            reason = self._stop_reason(r, token)
-            if reason is not None:
-                r.status, r.finish_reason = FINISHED, reason
-                self.running.remove(r)
-                self.cache.free_sequence(r.request_id)
-                self.finished[r.request_id] = r
-                done.append(r)
+    def _advance(self, finished: int) -> List[Request]:
+        done = []
+        for k, reason in zip(list(self._keys[:finished]), list(self._a[:finished])):
+            r = self._requests[k]
+            self._finish(k, r, "stop" if reason == 0 else "length")
+            done.append(r)
         return done
 
-    def _stop_reason(self, r: Request, token: int) -> Optional[str]:
-        """`check_stop` of the reference (`inferrs/src/engine.rs:866-887`): a stop token ends with
-        "stop" unless stop tokens are bypassed; reaching max_tokens or the context limit with "length"."""
-        p = r.params
-        if not p.bypass_stop_tokens and (token in self.stop_token_ids or token in p.extra_stop_token_ids):
-            return "stop"
-        if len(r.output) >= p.max_tokens:
-            return "length"
-        if r.total >= self.max_seq_len:
-            return "length"
-        return None
+    def commit(self, plan: Plan, sampled: Dict[Hashable, int]) -> List[Request]:
+        """The step of the latest plan ran: `sampled[request_id]` is the token drawn for every entry
+        that `samples`.  Returns the requests that finished."""
+        drawn = []
+        for e in plan.entries:
+            r = e.request
+            r.computed += len(e.tokens)
+            if e.samples:
+                token = int(sampled[r.request_id])
+                r.output.append(token)
+                drawn.append(token)
+        n = self._lib.iar_sched_commit(self._ptr, native.ints(drawn), len(drawn), self._keys, self._a, self._room)
+        if n < 0:
+            raise RuntimeError(native.last_error())
+        return self._advance(n)
+
+    def commit_decode(self, requests: Sequence[Request], tokens: Sequence[int]) -> List[Request]:
+        """One decode step of a run that was queued at once: one token for each of `requests` that
+        still runs (those that finished earlier in the run are passed over)."""
+        keys, toks = [], []
+        for r, t in zip(requests, tokens):
+            if r.status != RUNNING:
+                continue
+            r.computed += 1
+            r.output.append(int(t))
+            keys.append(self.cache.names.find(r.request_id))
+            toks.append(int(t))
+        n = self._lib.iar_sched_commit_decode(self._ptr, len(keys), native.keys(keys), native.ints(toks),
+                                              self._keys, self._a, self._room)
+        if n < 0:
+            raise RuntimeError(native.last_error())
+        return self._advance(n)

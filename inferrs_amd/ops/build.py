@@ -1,9 +1,11 @@
-"""Compiles the HIP sources under `inferrs_amd/csrc` for gfx950 into shared libraries.
+"""Compiles the sources under `inferrs_amd/csrc` into shared libraries.
 
-Two kinds of library:
-  * "core": every kernel whose code does not depend on a model size;
+Three kinds of library:
+  * "core": every HIP kernel (gfx950) whose code does not depend on a model size;
   * "attn_d<N>": the matrix-core attention kernel built for head size N (`-DIA_HEAD_DIM=N`),
-    so that a model compiles only the head size it has.
+    so that a model compiles only the head size it has;
+  * "runtime": the host runtime (cache manager, step assembly, scheduler), plain C++ that
+    touches no GPU and is compiled with the host compiler.
 
 A library's file name carries a hash of its sources and flags, so a library that is found
 is never stale.  `build(target)` always compiles; `library_path(target)` returns a built
@@ -32,8 +34,12 @@ FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 
+HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-Wall"]
+
 PER_HEAD_DIM = ("attention_mfma.hip",)
 SHARED = ("error.hip",)
+RUNTIME_SOURCES = ("runtime.cpp",)
+RUNTIME_HEADERS = ("runtime.h",)
 ATTN_HEAD_DIMS = tuple(range(16, 257, 16))
 
 
@@ -42,12 +48,18 @@ def attn_target(head_dim: int) -> str:
 
 
 def all_targets() -> List[str]:
-    return ["core"] + [attn_target(d) for d in ATTN_HEAD_DIMS]
+    return ["runtime", "core"] + [attn_target(d) for d in ATTN_HEAD_DIMS]
+
+
+def _is_host(target: str) -> bool:
+    return target == "runtime"
 
 
 def _plan(target: str) -> Tuple[List[str], List[str]]:
     """(sources, extra defines) of a target."""
     names = sorted(n for n in os.listdir(CSRC) if n.endswith(".hip"))
+    if target == "runtime":
+        return [os.path.join(CSRC, n) for n in RUNTIME_SOURCES], []
     if target == "core":
         return [os.path.join(CSRC, n) for n in names if n not in PER_HEAD_DIM], []
     if target.startswith("attn_d"):
@@ -61,12 +73,14 @@ def _plan(target: str) -> Tuple[List[str], List[str]]:
 def _digest(target: str) -> str:
     srcs, defines = _plan(target)
     h = hashlib.sha256()
-    headers = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith(".h"))
+    host = _is_host(target)
+    headers = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC)
+                     if n.endswith(".h") and (n in RUNTIME_HEADERS) == host)
     for p in srcs + headers:
         h.update(os.path.basename(p).encode())
         with open(p, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS + defines).encode())
+    h.update(" ".join((HOST_FLAGS if host else FLAGS) + defines).encode())
     return h.hexdigest()[:12]
 
 
@@ -111,13 +125,26 @@ def _hipcc() -> str:
                        "$ROCM_PATH/bin and /opt/rocm/bin)")
 
 
+def _host_compiler() -> str:
+    for c in (os.environ.get("CXX"), "g++", "c++", "clang++",
+              os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "llvm", "bin", "clang++")):
+        found = shutil.which(c) if c else None
+        if found:
+            return found
+    raise RuntimeError("no C++ compiler found for the host runtime (looked at $CXX, g++, c++, clang++ and "
+                       "$ROCM_PATH/llvm/bin/clang++)")
+
+
 def _say(msg: str) -> None:
     print(f"[inferrs_amd build] {msg}", file=sys.stderr, flush=True)
 
 
 def build(target: str = "core", verbose: bool = True, workers: Optional[int] = None) -> str:
     """Compile the sources of `target` and link its library; returns the path."""
-    hipcc = _hipcc()
+    host = _is_host(target)
+    hipcc = _host_compiler() if host else _hipcc()
+    flags = HOST_FLAGS if host else FLAGS
+    link_flags = [] if host else [f"--offload-arch={ARCH}"]
     out_dir = _writable_dir()
     name = _lib_name(target)
     srcs, defines = _plan(target)
@@ -125,14 +152,14 @@ def build(target: str = "core", verbose: bool = True, workers: Optional[int] = N
     os.makedirs(obj_dir, exist_ok=True)
     t0 = time.time()
     if verbose:
-        _say(f"{target}: compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
+        _say(f"{target}: compiling {len(srcs)} {'C++ sources' if host else f'HIP sources for {ARCH}'} into {out_dir}")
 
     def compile_one(src: str) -> str:
-        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
-        r = subprocess.run([hipcc, *FLAGS, *defines, "-I", CSRC, "-c", src, "-o", obj],
+        obj = os.path.join(obj_dir, os.path.splitext(os.path.basename(src))[0] + ".o")
+        r = subprocess.run([hipcc, *flags, *defines, "-I", CSRC, "-c", src, "-o", obj],
                            capture_output=True, text=True)
         if r.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
+            raise RuntimeError(f"{os.path.basename(hipcc)} failed on {src}:\n{r.stdout}\n{r.stderr}")
         if verbose:
             _say(f"  {target}: {os.path.basename(src)} done ({time.time() - t0:.0f} s)")
         return obj
@@ -141,10 +168,10 @@ def build(target: str = "core", verbose: bool = True, workers: Optional[int] = N
     with ThreadPoolExecutor(n) as pool:
         objs = list(pool.map(compile_one, srcs))
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.tmp")
-    r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp, *objs],
+    r = subprocess.run([hipcc, "-shared", "-fPIC", *link_flags, "-o", tmp, *objs],
                        capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed to link {name}:\n{r.stdout}\n{r.stderr}")
+        raise RuntimeError(f"{os.path.basename(hipcc)} failed to link {name}:\n{r.stdout}\n{r.stderr}")
     lib = os.path.join(out_dir, name)
     os.replace(tmp, lib)
     prefix = f"libinferrs_amd_{target}_"
