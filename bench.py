@@ -82,22 +82,16 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decod
     serving loop: scheduler, step function, greedy choice on the device."""
     import torch
     from inferrs_amd.engine import GenerationLoop
-    from inferrs_amd.engine.scheduler import RUNNING
+    from inferrs_amd.engine.scheduler import Request
     from inferrs_amd.sampling import SamplingParams
     start_len = context - steps - warmup
     loop = GenerationLoop(engine, max_batch_size=batch, max_tokens_per_step=max(batch, 16), decode_run=decode_run)
     params = SamplingParams.greedy(max_tokens=steps + warmup + 8, bypass_stop_tokens=True)
-    reqs = [loop.add([1 + i], params, request_id=f"d{i}") for i in range(batch)]
-    ids = [r.request_id for r in reqs]
+    ids = [f"d{i}" for i in range(batch)]
     # the requests enter as if their contexts had been run: random keys and values, and one generated token
     fill_context(engine, ids, start_len)
-    for r in reqs:
-        loop.scheduler.waiting.remove(r)
-        r.prompt = [1] * start_len
-        r.output = [1 + len(loop.scheduler.running)]
-        r.computed = start_len
-        r.status = RUNNING
-        loop.scheduler.running.append(r)
+    for i, sid in enumerate(ids):
+        loop.scheduler.adopt(Request(sid, [1] * start_len, params, output=[1 + i]))
     done_steps = 0
     while done_steps < warmup:
         loop.step(max_steps=warmup - done_steps)
@@ -132,6 +126,11 @@ def time_prefill(engine, n_tokens: int, runs: int, vocab: int):
     return best
 
 
+def note(msg: str) -> None:
+    """Progress goes to stderr; the one JSON line is all that stdout carries."""
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,8 +161,10 @@ def main() -> int:
     points_batches = [] if args.no_points or args.prefill_only else [1, 64]
     biggest = max([args.batch] + points_batches)
     num_pages = biggest * (-(-args.context // PAGE) + 1) + 8
+    note(f"random weights of {args.layers} layers and a cache of {num_pages} pages")
     engine = Engine.from_random(config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=num_pages,
                                 max_seqs=biggest + 1)
+    note(f"decode at batch {args.batch}, context {args.context}: {args.warmup} + {args.steps} steps")
 
     if args.prefill_only:
         t = time_prefill(engine, PREFILL_TOKENS, max(1, args.steps), raw["vocab_size"])
@@ -199,9 +200,11 @@ def main() -> int:
         points = {}
         for b in points_batches:
             steps = max(8, args.steps // 2)
+            note(f"decode at batch {b}: {steps} steps")
             el, _ = time_decode(engine, b, args.context, steps, min(args.warmup, 4), args.decode_run)
             points[f"decode_b{b}"] = round(b * steps / el, 2)
         record["points"] = points
+        note(f"prefill of {PREFILL_TOKENS} tokens")
         t = time_prefill(engine, PREFILL_TOKENS, 3, raw["vocab_size"])
         flops = prefill_flops(raw, PREFILL_TOKENS)
         record["prefill"] = {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS,

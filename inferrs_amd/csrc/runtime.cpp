@@ -214,6 +214,7 @@ struct Sched {
     std::vector<Req*> running;    // in order of admission
     std::vector<PlanEntry> plan;
     std::vector<int64_t> preempted, failed;
+    bool broken = false;          // the last plan met a misuse; the message is in the error channel
 
     bool is_running(const Req* r) const { return std::find(running.begin(), running.end(), r) != running.end(); }
     bool fits_alone(int n_tokens) const {
@@ -249,7 +250,7 @@ struct Sched {
             else ++i;
     }
     void make_plan(bool fresh) {
-        if (fresh) { plan.clear(); preempted.clear(); failed.clear(); }
+        if (fresh) { plan.clear(); preempted.clear(); failed.clear(); broken = false; }
         plan.clear();
         int budget = max_tokens_per_step;
         const size_t failed_before = failed.size(), preempted_before = preempted.size();
@@ -305,7 +306,10 @@ struct Sched {
                 continue;
             }
             const int n = std::min(std::min(r->total() - r->computed, prefill_chunk), budget);
-            if (cache->add_sequence(r->key) < 0) break;
+            if (cache->add_sequence(r->key) < 0) {        // the key is in use outside this scheduler, or no slot is left
+                broken = true;
+                break;
+            }
             // admitted only when all it has so far, and one token more, would fit now: a request that
             // is let in on its first portion alone tends to be preempted later
             const int all = r->total() + 1;
@@ -319,6 +323,7 @@ struct Sched {
             plan.push_back({r, r->computed, n, r->computed + n == r->total()});
             budget -= n;
         }
+        if (broken) return;
         if (plan.empty() && !running.empty() && failed.size() == failed_before && preempted.size() == preempted_before) {
             // every running request waits for pages that nobody will free: preempt the latest so that
             // the oldest can go on
@@ -667,6 +672,29 @@ int iar_sched_add(void* sched, int64_t key, const int* prompt, int n_prompt, int
     s->reqs.emplace(key, std::move(r));
     return 0;
 }
+int iar_sched_adopt(void* sched, int64_t key, const int* tokens, int n_tokens, int n_prompt, int max_tokens,
+                    int bypass_stop, const int* extra_stop, int n_extra) {
+    Sched* s = S(sched);
+    if (n_prompt < 1 || n_prompt > n_tokens) return fail(IAR_ERROR, "a request has at least one prompt token and no more than all its tokens");
+    if (n_tokens >= s->max_seq_len) return fail(IAR_ERROR, "the request has %d tokens, the limit is %d", n_tokens, s->max_seq_len - 1);
+    if (s->reqs.count(key)) return fail(IAR_ERROR, "a request of this key exists");
+    Sequence* seq = s->cache->find(key);
+    if (!seq) return fail(IAR_ERROR, "request is not live: only a request with a cache entry can be adopted");
+    if (seq->length >= n_tokens) return fail(IAR_ERROR, "the cache holds %d tokens of the request's %d: at least one must be left to feed", seq->length, n_tokens);
+    if ((int)s->running.size() >= s->max_batch_size) return fail(IAR_ERROR, "%d requests are running already", s->max_batch_size);
+    std::unique_ptr<Req> r(new Req());
+    r->key = key;
+    r->tokens.assign(tokens, tokens + n_tokens);
+    r->n_prompt = n_prompt;
+    r->computed = seq->length;
+    r->status = RUNNING;
+    r->max_tokens = max_tokens;
+    r->bypass_stop = bypass_stop != 0;
+    r->extra_stop.assign(extra_stop, extra_stop + n_extra);
+    s->running.push_back(r.get());
+    s->reqs.emplace(key, std::move(r));
+    return seq->length;
+}
 int iar_sched_num_waiting(void* sched) { return (int)S(sched)->waiting.size(); }
 int iar_sched_num_running(void* sched) { return (int)S(sched)->running.size(); }
 int iar_sched_waiting(void* sched, int64_t* out, int capacity) {
@@ -681,6 +709,11 @@ int iar_sched_running(void* sched, int64_t* out, int capacity) {
 }
 int iar_sched_plan(void* sched) {
     S(sched)->make_plan(true);
+    if (S(sched)->broken) {
+        // what was reserved for this plan's entries stays reserved: the caller has to end these requests
+        std::string why = g_error;
+        return fail(IAR_ERROR, "a waiting request cannot get a cache entry: %s", why.c_str());
+    }
     return (int)S(sched)->plan.size();
 }
 int iar_sched_plan_entries(void* sched, int64_t* keys, int* starts, int* counts, int* samples) {

@@ -74,6 +74,10 @@ void* iar_sched_create(void* cache, int max_batch_size, int max_tokens_per_step,
 void iar_sched_destroy(void* sched);
 int iar_sched_add(void* sched, int64_t key, const int* prompt, int n_prompt, int max_tokens, int bypass_stop,
                   const int* extra_stop, int n_extra);
+// A request that already has a cache entry (its first tokens were put there by other means) joins
+// the running requests: tokens = prompt then output so far.  Returns the number of cached tokens.
+int iar_sched_adopt(void* sched, int64_t key, const int* tokens, int n_tokens, int n_prompt, int max_tokens,
+                    int bypass_stop, const int* extra_stop, int n_extra);
 int iar_sched_num_waiting(void* sched);
 int iar_sched_num_running(void* sched);
 int iar_sched_waiting(void* sched, int64_t* out, int capacity);    // in queue order

@@ -137,6 +137,28 @@ class Scheduler:
         self._requests[key] = request
         self._grow(len(self._requests))
 
+    def adopt(self, request: Request) -> None:
+        """A request that already has a cache entry joins the running requests: its prompt and the
+        output so far are given, `computed` becomes what the cache holds of them (their keys and
+        values were put there by other means, e.g. a benchmark that fills a context)."""
+        name = request.request_id
+        if name not in self.cache.sequences:
+            raise ValueError(f"request {name!r} has no cache entry")
+        key = self.cache.names.pin(name)
+        p = request.params
+        extra = [int(t) for t in p.extra_stop_token_ids]
+        tokens = request.tokens
+        got = self._lib.iar_sched_adopt(self._ptr, key, native.ints(tokens), len(tokens), len(request.prompt),
+                                        int(p.max_tokens), int(bool(p.bypass_stop_tokens)), native.ints(extra), len(extra))
+        if got < 0:
+            self.cache.names.unpin(name, live=True)
+            raise ValueError(f"request {name!r}: {native.last_error()}")
+        request.arrival = self._arrivals
+        self._arrivals += 1
+        request.status, request.computed = RUNNING, got
+        self._requests[key] = request
+        self._grow(len(self._requests))
+
     def has_work(self) -> bool:
         return bool(self._lib.iar_sched_num_waiting(self._ptr) or self._lib.iar_sched_num_running(self._ptr))
 
@@ -165,6 +187,8 @@ class Scheduler:
         lib, ptr = self._lib, self._ptr
         plan = Plan()
         n = lib.iar_sched_plan(ptr)
+        if n < 0:
+            raise RuntimeError(native.last_error())
         for k in self._keys[:lib.iar_sched_plan_preempted(ptr, self._keys, self._room)]:
             r = self._requests[k]
             r.computed, r.status = 0, WAITING

@@ -50,6 +50,7 @@ _SIGNATURES = {
     "iar_sched_create": (c_void_p, [c_void_p, c_int, c_int, c_int, c_int, _PI, c_int]),
     "iar_sched_destroy": (None, [c_void_p]),
     "iar_sched_add": (c_int, [c_void_p, c_int64, _PI, c_int, c_int, c_int, _PI, c_int]),
+    "iar_sched_adopt": (c_int, [c_void_p, c_int64, _PI, c_int, c_int, c_int, c_int, _PI, c_int]),
     "iar_sched_num_waiting": (c_int, [c_void_p]),
     "iar_sched_num_running": (c_int, [c_void_p]),
     "iar_sched_waiting": (c_int, [c_void_p, _PK, c_int]),

@@ -159,3 +159,34 @@ def test_every_request_finishes_whatever_the_order_and_the_pool(seed):
             alone.output.append(token_for(alone))
         assert alone.output == r.output
     assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups) and cache.slots.num_free == 6
+
+
+def test_a_request_with_a_cache_entry_can_be_adopted():
+    cache, s = make(num_pages=16, page_size=4)
+    cache.add_sequence("a")
+    assert cache.reserve("a", 10)
+    cache.commit("a", 10)
+    a = Request("a", list(range(10)), SamplingParams.greedy(max_tokens=3), output=[77])
+    s.adopt(a)
+    assert a.status == "running" and a.computed == 10 and [r.request_id for r in s.running] == ["a"]
+    plan = s.plan()
+    assert [(e.request.request_id, e.tokens, e.samples) for e in plan.entries] == [("a", [77], True)]
+    assert s.commit(plan, {"a": 5}) == [] and a.output == [77, 5]
+    run(s, cache)
+    assert a.finish_reason == "length" and len(a.output) == 3
+    assert cache.groups[0].pool.num_free == 16 and not cache.names.names()
+    with pytest.raises(ValueError, match="no cache entry"):
+        s.adopt(Request("b", [1, 2], SamplingParams.greedy()))
+    cache.add_sequence("c")
+    assert cache.reserve("c", 2)
+    cache.commit("c", 2)
+    with pytest.raises(ValueError, match="at least one must be left"):
+        s.adopt(Request("c", [1, 2], SamplingParams.greedy()))
+
+
+def test_a_name_in_use_outside_the_scheduler_is_reported():
+    cache, s = make()
+    cache.add_sequence("a")                        # somebody else's request of the same name
+    s.add(req("a", 3))
+    with pytest.raises(RuntimeError, match="already live"):
+        s.plan()
