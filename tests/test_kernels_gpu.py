@@ -297,6 +297,26 @@ def test_skinny_rows_do_not_depend_on_the_batch():
     assert torch.equal(ops.gemm_skinny_bf16(dev(x[3:9].contiguous()), dev(w), torch.float32).cpu(), full[3:9])
 
 
+@pytest.mark.parametrize("dual", [False, True])
+def test_skinny_variants_for_tall_weights_agree_bit_for_bit(dual):
+    # a weight with more than two blocks a compute unit takes the variant that stages the activations
+    # through shared memory at 2 to 12 rows, and the plain one at 1 and at 16 rows
+    from inferrs_amd import ops
+    n, k = 8200, 520
+    x = randn(16, k, dtype=torch.bfloat16, seed=1)
+    w = randn(2 * n if dual else n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    full = ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32, dual=dual).cpu()
+    if dual:
+        gate = (x.double() @ w[:n].double().t()).to(torch.bfloat16).double()
+        want = gate / (1 + torch.exp(-gate)) * (x.double() @ w[n:].double().t()).to(torch.bfloat16).double()
+        close(full, want, 2 ** -7, "dual")
+    else:
+        close(full, x.double() @ w.double().t(), 2e-5, "tall")
+    for lo, hi in ((0, 1), (3, 9), (0, 12), (5, 7), (2, 15)):
+        part = ops.gemm_skinny_bf16(dev(x[lo:hi].contiguous()), dev(w), torch.float32, dual=dual).cpu()
+        assert torch.equal(part, full[lo:hi]), (lo, hi)
+
+
 def test_argmax_lowest_index_among_equal_maxima():
     from inferrs_amd import ops
     z = randn(4, 151936, dtype=torch.float32, seed=3)
