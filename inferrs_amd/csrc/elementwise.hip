@@ -101,7 +101,16 @@ __global__ __launch_bounds__(1024) void rmsnorm_bf16_vec_kernel(bf16_t* __restri
     const size_t base = (size_t)blockIdx.x * cols;
     const int nvec = cols / 8;
     float v[NORM_VECS][8];
+    float4 w0[NORM_VECS], w1[NORM_VECS];        // asked for now, used after the sum: one wait instead of two
     float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_VECS; ++i) {
+        const int vi = threadIdx.x + i * blockDim.x;
+        if (vi < nvec) {
+            w0[i] = *(const float4*)(w + (size_t)vi * 8);
+            w1[i] = *(const float4*)(w + (size_t)vi * 8 + 4);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < NORM_VECS; ++i) {
         const int vi = threadIdx.x + i * blockDim.x;
@@ -137,8 +146,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_bf16_vec_kernel(bf16_t* __restri
     for (int i = 0; i < NORM_VECS; ++i) {
         const int vi = threadIdx.x + i * blockDim.x;
         if (vi < nvec) {
-            const float4 w0 = *(const float4*)(w + (size_t)vi * 8), w1 = *(const float4*)(w + (size_t)vi * 8 + 4);
-            const float g[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+            const float g[8] = {w0[i].x, w0[i].y, w0[i].z, w0[i].w, w1[i].x, w1[i].y, w1[i].z, w1[i].w};
             uint32_t packed[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {

@@ -106,6 +106,33 @@ __global__ __launch_bounds__(QKV_THREADS) void qk_rope_kv_bf16_vec_kernel(
     const int tok = active ? (int)(unit / heads) : 0;
     const int hh = active ? (int)(unit % heads) : 0;
     const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);
+    // Everything that does not depend on the features is asked for before the first barrier, in
+    // 16-byte pieces: norm weights, and the angles when a thread's eight features lie on one
+    // side of the rotation's halves (else they are read one by one further down).
+    const float* nw = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+    const int half = rot / 2;
+    const bool vec_angles = interleaved ? rot % 8 == 0 : half % 8 == 0;
+    const bool rotates = active && cos_t != nullptr && kind != 2 && t * 8 < rot;
+    float gw[8], cs[8], sn[8];
+    if (active && nw != nullptr) {
+        const float4 g0 = *(const float4*)(nw + t * 8), g1 = *(const float4*)(nw + t * 8 + 4);
+        gw[0] = g0.x; gw[1] = g0.y; gw[2] = g0.z; gw[3] = g0.w; gw[4] = g1.x; gw[5] = g1.y; gw[6] = g1.z; gw[7] = g1.w;
+    }
+    if (rotates && vec_angles) {
+        if (interleaved) {
+            const size_t at = (size_t)tok * half + t * 4;
+            const float4 c0 = *(const float4*)(cos_t + at), s0 = *(const float4*)(sin_t + at);
+            cs[0] = cs[1] = c0.x; cs[2] = cs[3] = c0.y; cs[4] = cs[5] = c0.z; cs[6] = cs[7] = c0.w;
+            sn[0] = sn[1] = s0.x; sn[2] = sn[3] = s0.y; sn[4] = sn[5] = s0.z; sn[6] = sn[7] = s0.w;
+        } else {
+            const int e0 = t * 8;
+            const size_t at = (size_t)tok * half + (e0 < half ? e0 : e0 - half);
+            const float4 c0 = *(const float4*)(cos_t + at), c1 = *(const float4*)(cos_t + at + 4);
+            const float4 s0 = *(const float4*)(sin_t + at), s1 = *(const float4*)(sin_t + at + 4);
+            cs[0] = c0.x; cs[1] = c0.y; cs[2] = c0.z; cs[3] = c0.w; cs[4] = c1.x; cs[5] = c1.y; cs[6] = c1.z; cs[7] = c1.w;
+            sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+        }
+    }
     float v[8];
     float ss = 0.f;
     if (active) {
@@ -121,16 +148,12 @@ __global__ __launch_bounds__(QKV_THREADS) void qk_rope_kv_bf16_vec_kernel(
     }
     partial[threadIdx.x] = ss;
     __syncthreads();
-    const float* nw = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
     if (active && nw != nullptr) {
         float total = 0.f;
         for (int i = 0; i < tpu; ++i) total += partial[u * tpu + i];      // the same order in every thread
         const float scale = 1.0f / sqrtf(total / (float)d + eps);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float g = nw[t * 8 + j];
-            v[j] = scale * v[j] * (add_one ? 1.0f + g : g);
-        }
+        for (int j = 0; j < 8; ++j) v[j] = scale * v[j] * (add_one ? 1.0f + gw[j] : gw[j]);
     }
     if (active) {
 #pragma unroll
@@ -148,7 +171,6 @@ __global__ __launch_bounds__(QKV_THREADS) void qk_rope_kv_bf16_vec_kernel(
         return;
     }
     if (cos_t != nullptr) {
-        const int half = rot / 2;
         const float* row = rows + (size_t)u * tpu * 8;
         float o[8];
 #pragma unroll
@@ -159,7 +181,8 @@ __global__ __launch_bounds__(QKV_THREADS) void qk_rope_kv_bf16_vec_kernel(
                 const int i = interleaved ? e >> 1 : (e < half ? e : e - half);
                 const bool first = interleaved ? (e & 1) == 0 : e < half;
                 const int partner = interleaved ? e ^ 1 : (first ? e + half : e - half);
-                const float c = cos_t[(size_t)tok * half + i], s = sin_t[(size_t)tok * half + i];
+                const float c = vec_angles ? cs[j] : cos_t[(size_t)tok * half + i];
+                const float s = vec_angles ? sn[j] : sin_t[(size_t)tok * half + i];
                 o[j] = first ? v[j] * c - row[partner] * s : row[partner] * s + v[j] * c;
             }
         }
@@ -192,7 +215,8 @@ extern "C" int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const vo
     if (n == 0) return 0;
     const long long units = (long long)n * (slots ? nq + 2 * nkv : nq);
     const unsigned grid = (unsigned)((units + QK_WAVES - 1) / QK_WAVES);
-    const uintptr_t ptrs = (uintptr_t)q_out | (uintptr_t)qkv | (uintptr_t)(slots ? k_cache : nullptr);
+    const uintptr_t ptrs = (uintptr_t)q_out | (uintptr_t)qkv | (uintptr_t)(slots ? k_cache : nullptr) |
+                           (uintptr_t)q_norm_w | (uintptr_t)k_norm_w | (uintptr_t)cos_t | (uintptr_t)sin_t;
     if (dtype == IA_BF16 && d % 8 == 0 && d / 8 <= QKV_THREADS && (ptrs & 15) == 0) {
         const int units_per_block = QKV_THREADS / (d / 8);
         const unsigned vgrid = (unsigned)((units + units_per_block - 1) / units_per_block);
