@@ -27,6 +27,7 @@ class TensorSpec:
     """What a part expects under a name: the shape, and how random weights fill it."""
     shape: Tuple[int, ...]
     init: str = "matrix"       # "matrix": N(0, 0.02); "norm": 1 + N(0, 0.1); "table": integers
+    high: int = 0              # tables: random entries are drawn from 0..high-1 (0: no random fill)
 
 
 class WeightError(ValueError):

@@ -59,6 +59,21 @@ def normal_values(n: int, seed: int, mean: float, std: float) -> np.ndarray:
     return out
 
 
+def n_elements(shape) -> int:
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+def table_values(n: int, seed: int, high: int) -> np.ndarray:
+    """int32 [n]: element i is output i + 1 of the splitmix64 sequence started at seed, modulo `high`."""
+    with np.errstate(over="ignore"):
+        i = np.arange(1, n + 1, dtype=np.uint64)
+        h = _splitmix_out(np.uint64(seed & (2**64 - 1)) + i * _GOLDEN)
+    return (h % np.uint64(high)).astype(np.int32)
+
+
 def random_tensors(expected: Mapping[str, TensorSpec], seed: int,
                    dtype: torch.dtype = torch.bfloat16,
                    device: str = "cpu") -> Dict[str, torch.Tensor]:
@@ -70,16 +85,17 @@ def random_tensors(expected: Mapping[str, TensorSpec], seed: int,
     out: Dict[str, torch.Tensor] = {}
     for name, spec in expected.items():
         if spec.init == "table":
-            raise ValueError(f"no random fill is defined for integer table '{name}'")
+            if spec.high <= 0:
+                raise ValueError(f"no random fill is defined for integer table '{name}' (its TensorSpec gives no range)")
+            out[name] = torch.from_numpy(table_values(n_elements(spec.shape), _tensor_seed(seed, name), spec.high)
+                                         ).reshape(spec.shape).to(device)
+            continue
         mean, std = (1.0, NORM_STD) if spec.init == "norm" else (0.0, MATRIX_STD)
         tseed = _tensor_seed(seed, name)
         if on_gpu:
             out[name] = ops.fill_normal(spec.shape, tseed, mean, std, dtype, device)
         else:
-            n = 1
-            for s in spec.shape:
-                n *= int(s)
-            out[name] = torch.from_numpy(normal_values(n, tseed, mean, std)).reshape(spec.shape).to(dtype)
+            out[name] = torch.from_numpy(normal_values(n_elements(spec.shape), tseed, mean, std)).reshape(spec.shape).to(dtype)
     return out
 
 

@@ -334,3 +334,185 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype, page)
         elif dtype == "float32":
             cross = max(float(np.abs(got[r][i] - first[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
             assert cross < 2e-6, f"{mode} against whole: {cross:.3e}"
+
+
+# ---- a second toy architecture: a feed-forward with routing, another position encoding ----------
+
+@dataclass(frozen=True)
+class RoutedSpec:
+    """A feed-forward that routes: a router scores E experts in 32-bit, the best `top_k` share a token
+    by their renormalised softmax weights, and an integer table says which expert's weights stand
+    behind a router column.  Expert e: down_e(relu(up_e(h))^2)."""
+    hidden: int
+    intermediate: int
+    experts: int
+    top_k: int
+    kind: str = "toy_routed"
+
+
+@dataclass(frozen=True)
+class LinearAnglesSpec:
+    """A rotary position encoding with another law: angle[p, i] = p * alpha * (i + 1), pairs (2i, 2i+1)."""
+    head_dim: int
+    rot_dim: int
+    alpha: float
+    kind: str = "toy_linear_angles"
+
+
+def register_toy_routed():
+    from inferrs_amd import ops
+    from inferrs_amd.config import AttentionSpec, LayerSpec, ModelSpec, NormSpec, ScheduleEntry
+    from inferrs_amd.config.registry import register_architecture
+    from inferrs_amd.parts import FeedForward, Position, register_ffn, register_position
+    from inferrs_amd.weights import TensorSpec
+
+    @register_position("toy_linear_angles")
+    class LinearAngles(Position):
+        interleaved = True
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.spec, self.rot_dim = spec, spec.rot_dim
+            self.freq = (torch.arange(1, spec.rot_dim // 2 + 1, dtype=torch.float32) * spec.alpha).to(device)
+
+        def table(self, positions):
+            angle = positions.to(torch.float32)[:, None] * self.freq[None, :]     # 32-bit, as the rule asks
+            return torch.cos(angle).contiguous(), torch.sin(angle).contiguous()
+
+    @register_ffn("toy_routed")
+    class Routed(FeedForward):
+        @classmethod
+        def tensors(cls, spec):
+            e = spec.experts
+            return {"router.weight": TensorSpec((e, spec.hidden)),
+                    "remap": TensorSpec((e,), "table", high=e),
+                    "up.weight": TensorSpec((e * spec.intermediate, spec.hidden)),
+                    "down.weight": TensorSpec((e * spec.hidden, spec.intermediate))}
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.spec = spec
+            self.router = tensors["router.weight"].to(device=device, dtype=dtype).contiguous()
+            assert tensors["remap"].dtype == torch.int32                    # integer tables stay integers
+            self.remap = tensors["remap"].to(device)
+            self.up = [w.contiguous() for w in tensors["up.weight"].to(device=device, dtype=dtype).chunk(spec.experts)]
+            self.down = [w.contiguous() for w in tensors["down.weight"].to(device=device, dtype=dtype).chunk(spec.experts)]
+
+        def forward(self, ctx, h):
+            logits = ops.linear(h, self.router, torch.float32)               # router logits in 32-bit
+            best, cols = torch.topk(logits, self.spec.top_k, dim=-1)
+            weights = torch.softmax(best, dim=-1)
+            out = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
+            owner = self.remap[cols]                                         # [n, top_k] expert behind each chosen column
+            for e in range(self.spec.experts):
+                rows, slot = (owner == e).nonzero(as_tuple=True)
+                if rows.numel() == 0:
+                    continue
+                y = ops.linear(h[rows].contiguous(), self.up[e])
+                y = torch.relu(y.float()).square().to(h.dtype)
+                out.index_add_(0, rows, ops.linear(y, self.down[e]).float() * weights[rows, slot][:, None])
+            return out.to(h.dtype)
+
+    class RoutedConfig:
+        architecture = "ToyRoutedForCausalLM"
+        model_type = "toy_routed"
+
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def to_dict(self):
+            return dict(self.raw, architectures=[self.architecture], model_type=self.model_type)
+
+        def to_spec(self):
+            r = self.raw
+            h = r["hidden_size"]
+            norm = NormSpec(size=h, eps=r["eps"])
+            attn = AttentionSpec(hidden=h, n_heads=r["heads"], n_kv_heads=r["kv_heads"], head_dim=r["head_dim"],
+                                 position=LinearAnglesSpec(r["head_dim"], r["rot_dim"], r["alpha"]), qk_norm=None, window=None)
+            ffn = RoutedSpec(h, r["intermediate"], r["experts"], r["top_k"])
+
+            def layer(i):
+                p = f"blocks.{i}."
+                return LayerSpec(mixer=attn, ffn=ffn, norm_mixer=norm, norm_ffn=norm, mixer_prefix=p + "mixer.",
+                                 ffn_prefix=p + "ffn.", norm_mixer_name=p + "norm1.weight", norm_ffn_name=p + "norm2.weight")
+            layers = tuple(layer(i) for i in range(r["layers"]))
+            return ModelSpec(architecture=self.architecture, vocab_size=r["vocab"], hidden=h, layers=layers,
+                             schedule=tuple(ScheduleEntry(i) for i in range(r["layers"])), final_norm=norm,
+                             final_norm_name="norm.weight", embed_name="embed.weight", head_name=None, max_position=512)
+
+    register_architecture(RoutedConfig)
+    return RoutedConfig
+
+
+def toy_routed_plain(p, raw, ids):
+    """The second toy on a whole sequence in 64-bit: every step written out."""
+    t = len(ids)
+    x = p["embed.weight"][torch.as_tensor(ids)]
+    d, nq, nkv, rot = raw["head_dim"], raw["heads"], raw["kv_heads"], raw["rot_dim"]
+    # the engine forms the angles in 32-bit: the plain model takes the same angles, then goes on in 64-bit
+    angle = (torch.arange(t, dtype=torch.float32)[:, None] *
+             (torch.arange(1, rot // 2 + 1, dtype=torch.float32) * raw["alpha"])[None, :]).double()
+    cos, sin = torch.cos(angle), torch.sin(angle)
+
+    def rotate(v):          # pairs (2i, 2i+1) of the first rot features
+        a, b = v[..., 0:rot:2], v[..., 1:rot:2]
+        out = v.clone()
+        out[..., 0:rot:2] = a * cos - b * sin
+        out[..., 1:rot:2] = a * sin + b * cos
+        return out
+
+    for i in range(raw["layers"]):
+        pre = f"blocks.{i}."
+        h = pm.rms_norm(x, p[pre + "norm1.weight"], raw["eps"])
+        q = rotate(pm.linear(h, p[pre + "mixer.q_proj.weight"]).reshape(t, nq, d).transpose(0, 1))
+        k = rotate(pm.linear(h, p[pre + "mixer.k_proj.weight"]).reshape(t, nkv, d).transpose(0, 1))
+        v = pm.linear(h, p[pre + "mixer.v_proj.weight"]).reshape(t, nkv, d).transpose(0, 1)
+        k, v = pm.repeat_kv(k, nq // nkv), pm.repeat_kv(v, nq // nkv)
+        s = torch.matmul(q, k.transpose(1, 2)) / d ** 0.5
+        s = s.masked_fill(torch.arange(t)[None, :] > torch.arange(t)[:, None], float("-inf"))
+        x = x + pm.linear(torch.matmul(pm.softmax_last(s), v).transpose(0, 1).reshape(t, nq * d), p[pre + "mixer.o_proj.weight"])
+        h = pm.rms_norm(x, p[pre + "norm2.weight"], raw["eps"])
+        logits = pm.linear(h, p[pre + "ffn.router.weight"])
+        best, cols = torch.topk(logits, raw["top_k"], dim=-1)
+        weights = pm.softmax_last(best)
+        up = p[pre + "ffn.up.weight"].chunk(raw["experts"])
+        down = p[pre + "ffn.down.weight"].chunk(raw["experts"])
+        remap = p[pre + "ffn.remap"].long()
+        y = torch.zeros_like(x)
+        for row in range(t):
+            for slot in range(raw["top_k"]):
+                e = int(remap[cols[row, slot]])
+                y[row] += weights[row, slot] * pm.linear(torch.relu(pm.linear(h[row:row + 1], up[e])) ** 2, down[e])[0]
+        x = x + y
+    return pm.linear(pm.rms_norm(x, p["norm.weight"], raw["eps"]), p["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype,page,top_k", [("float32", 8, 2), ("bfloat16", 16, 4)])
+def test_toy_routed_feed_forward_and_position_encoding(tmp_path, dtype, page, top_k):
+    """A feed-forward with routing, a position encoding with another law and an integer table, all
+    defined in this file.  In bfloat16 every expert takes part (top_k = experts): a choice among
+    experts is not continuous, and rounding may choose otherwise than 64-bit arithmetic does."""
+    from inferrs_amd.engine import Engine, run_trace
+    from inferrs_amd.weights import write_random_model
+    RoutedConfig = register_toy_routed()
+    raw = dict(hidden_size=40, heads=5, kv_heads=1, head_dim=16, rot_dim=12, alpha=0.37, intermediate=56, vocab=89,
+               eps=1e-4, layers=2, experts=4, top_k=top_k)
+    folder = write_random_model(str(tmp_path / "routed"), RoutedConfig(raw), seed=9)
+    from safetensors.torch import load_file
+    loaded = load_file(os.path.join(folder, "model.safetensors"))
+    assert loaded["blocks.0.ffn.remap"].dtype == torch.int32 and int(loaded["blocks.0.ffn.remap"].max()) < 4
+    p = {k: (v if v.dtype == torch.int32 else v.double()) for k, v in loaded.items()}
+    reqs = {f"r{i}": random_tokens(n, 89, 60 + i) for i, n in enumerate([2, 37, 90])}
+    ref = {r: toy_routed_plain(p, raw, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for mode, trace in (("whole", tm.whole(reqs)), ("portions", tm.portions(reqs, [7, 2, 19])),
+                        ("mixed", tm.mixed(reqs, seed=5, max_live=3, decode_tail=8))):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-trace.max_tokens // page) + 2, max_seqs=4)
+        assert not eng.model.graph_safe                 # the toy parts did not say that they can be captured
+        run_trace(eng, trace.lines, str(tmp_path / mode), io.StringIO())
+        got = trace.read(str(tmp_path / mode), 89)
+        err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
+        assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
+        eng.cache.check_invariants()
