@@ -179,7 +179,7 @@ def main() -> int:
     achieved = nbytes / (elapsed / args.steps) / 1e9
 
     record = {
-        "metric": "decode tok/s at batch 8, context 8192 (Qwen3-8B)", "value": round(value, 2), "unit": "tok/s",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-8B)", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_key,
         "data": "synthetic: random-init weights, uniform-random token ids, cache pages of the context "

@@ -29,6 +29,8 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--device", default="auto", choices=["auto", "hip", "cuda"],
                    help="the one AMD GPU (there is no CPU path)")
     p.add_argument("--block-size", type=int, default=16, help="KV cache block size in tokens")
+    p.add_argument("--initial-blocks", type=int, default=16,
+                   help="initial KV cache blocks (the pool is allocated whole at the start: it never has fewer than this)")
     p.add_argument("--max-blocks", type=int, default=0, help="KV cache blocks (0 = from --paged-attention)")
     p.add_argument("--max-batch-size", type=int, default=32, help="maximum concurrent sequences")
     p.add_argument("--max-tokens-per-step", type=int, default=2048, help="token budget per scheduler step")
@@ -78,7 +80,7 @@ def load_engine(args):
     dtype = {"f32": "float32", "bf16": "bfloat16"}.get(args.dtype, args.dtype)
     options = dict(dtype=dtype, page_size=args.block_size, max_seqs=args.max_batch_size)
     if args.max_blocks > 0:
-        options["num_pages"] = args.max_blocks
+        options["num_pages"] = max(args.max_blocks, args.initial_blocks)
     else:
         options["memory_fraction"] = args.paged_attention
     print(f"inferrs-amd: loading {args.model} ({dtype})", file=sys.stderr, flush=True)
