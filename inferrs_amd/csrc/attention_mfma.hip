@@ -120,11 +120,44 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         uint4 k[2][KS];         // tile t, dim step ks: row r <-> key k0 + 8*(r/4) + 4t + r%4
         uint4 v[DB];            // dim block db: row r <-> dim 16 db + r, keys k0 + 8G .. +7
     };
-    auto load_step = [&](Operands& op, int k0) {
-        // Rows past the request's length are read from its last written slot instead (their
-        // scores are masked in the step): the pages behind them may not exist.  The two halves
-        // of a step lie in at most two pages, whose numbers are the same for every lane: they
-        // come through the scalar cache, and no load of a key waits for a load of its address.
+    // A step's 32 keys are two groups of 16 slots, each inside one page (page sizes are multiples of
+    // 16): a Place says where a group lies, and moves on without a division.
+    struct Place { int idx, off; };                  // page index in the block table, slot in that page
+    auto advance = [&](Place& at, int slots) {
+        at.off += slots;
+        while (at.off >= p.page) { at.off -= p.page; ++at.idx; }
+    };
+    // This lane's part of the addresses does not change from step to step: its key rows' slots inside
+    // their group, its piece of a row, and which of the two groups they belong to.
+    const bool k_second = r >= 8, v_second = G >= 2;
+    const uint32_t k_lane[2] = {(uint32_t)((((8 * (r >> 2) + (r & 3)) & 15) * HD + G * 8) * 2),
+                                (uint32_t)((((8 * (r >> 2) + 4 + (r & 3)) & 15) * HD + G * 8) * 2)};
+    const uint32_t v_lane = (uint32_t)((r * p.page + 8 * (G & 1)) * 2);
+    const size_t v_stride = (size_t)16 * p.page * 2;
+    auto load_step = [&](Operands& op, int k0, const Place& at) {
+        if (k0 + 32 <= kv_total) {
+            // every slot of the step is written: the pages' numbers and the groups' places are the same
+            // for all lanes (they come through the scalar cache), a lane adds its constant part
+            Place next = at;
+            advance(next, 16);
+            const int page_a = bt[at.idx], page_b = bt[next.idx];
+            const char* ka = (const char*)(p.k_cache + (((size_t)page_a * p.nkv + kvh) * p.page + at.off) * HD);
+            const char* kb = (const char*)(p.k_cache + (((size_t)page_b * p.nkv + kvh) * p.page + next.off) * HD);
+            const char* va = (const char*)(p.v_cache + ((size_t)page_a * p.nkv + kvh) * HD * p.page + at.off);
+            const char* vb = (const char*)(p.v_cache + ((size_t)page_b * p.nkv + kvh) * HD * p.page + next.off);
+            const char* kbase = k_second ? kb : ka;
+            const char* vbase = (v_second ? vb : va) + v_lane;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    op.k[t][ks] = (ks * 32 + G * 8 < HD) ? *(const uint4*)(kbase + k_lane[t] + ks * 64) : zero4();
+#pragma unroll
+            for (int db = 0; db < DB; ++db) op.v[db] = *(const uint4*)(vbase + db * v_stride);
+            return;
+        }
+        // The request's last step.  Rows past its length are read from its last written slot instead
+        // (their scores are masked in the step): the pages behind them may not exist.
         const int last_idx = (kv_total - 1) / p.page;
         const int idx_a = k0 / p.page;
         const int idx_b = (k0 + 16) / p.page < last_idx ? (k0 + 16) / p.page : last_idx;
@@ -224,25 +257,30 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         }
     };
 
-    // Variants that were tried and lost, each measured against this one in the same run (prompt of
-    // 2,048 and of 8,192 tokens, head size 128).  The counters say that the SIMDs are busy less than
-    // half of the time, with about ten vector instructions a matrix instruction and the matrix
-    // pipes at 13 %: the walk is bound by the latency of a step's chain (loads, first product, row
-    // maxima across lanes, exponentials, second product), which two waves a SIMD cover only in part.
-    // - Loading the next step's operands ahead of this step's products doubles the operand
-    //   registers, which costs a wave per SIMD, and that wave hid more latency.
-    // - Asking for the next keys right after the scores and for the next values right after the
-    //   second product (no register held twice): prompts 5 % slower.
-    // - Blocks of four waves that bring keys and values into shared memory once (a stage of 32 or
-    //   of 64 keys, the next stage on its way in registers, one barrier a stage): 0.5 and 0.95 of
-    //   the speed of independent waves that read the same pages through the L2; a third of the
-    //   shared memory's busy cycles were bank conflicts, and the barrier keeps the waves in step.
-    // - Moving the exponents' reference point only when the running maximum has risen by 2^8
-    //   (so that the accumulators are rescaled a few times a walk, not at most steps): no change.
+    // What bounds the walk of a long prompt, and what was tried (each variant measured against this
+    // one in the same run; prompts of 2,048 and 8,192 tokens, head size 128).  At 8,192 tokens a layer's
+    // waves ask the L2 for 121 M lines (15 GB, 12 TB/s) and the matrix pipes are busy 18 % of the time;
+    // with 16 columns a wave instead of 32 (twice the reads, the same arithmetic) the walk takes 1.9
+    // times as long: it is the L2's bandwidth.
+    // - Blocks of four waves that bring keys and values into shared memory once (stages of 64 keys, the
+    //   next stage on its way in registers, one barrier a stage, late and early tiles sharing a compute
+    //   unit) halved the L2's requests and were still 3 % slower: a third of the shared memory's busy
+    //   cycles were bank conflicts, and the waves wait for each other at every stage.
+    // - Loading the next step's operands ahead of this step's products doubles the operand registers,
+    //   which costs a wave per SIMD, and that wave hid more latency.  Asking for the next keys right
+    //   after the scores and for the next values right after the second product (no register held
+    //   twice): prompts 5 % slower.
+    // - Moving the exponents' reference point only when the running maximum has risen by 2^8 (the
+    //   accumulators are then rescaled a few times a walk, not at most steps), row maxima through
+    //   v_permlane swaps instead of shared memory, late and early column blocks as separate waves
+    //   instead of one after the other in a wave: within 1 % each.
+    // - Addresses without a division in the step (above): 1 % at 2,048 tokens.
+    Place at = {lo / p.page, lo % p.page};
     for (int k0 = lo; k0 < hi; k0 += 32) {
         Operands op;
-        load_step(op, k0);
+        load_step(op, k0, at);
         compute_step(op, k0);
+        advance(at, 32);
     }
 
     // ---- results: lane (col, G) holds dims 16 db + 4 G + i of its column ---------------------
