@@ -143,6 +143,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="length of the prompt of the prefill")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
     args = ap.parse_args()
@@ -167,10 +168,10 @@ def main() -> int:
     note(f"decode at batch {args.batch}, context {args.context}: {args.warmup} + {args.steps} steps")
 
     if args.prefill_only:
-        t = time_prefill(engine, PREFILL_TOKENS, max(1, args.steps), raw["vocab_size"])
-        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS,
+        t = time_prefill(engine, args.prefill_tokens, max(1, args.steps), raw["vocab_size"])
+        print(json.dumps({"prefill": {"value": round(args.prefill_tokens / t, 1), "tokens": args.prefill_tokens,
                                       "ms": round(t * 1e3, 3),
-                                      "frac": round(prefill_flops(raw, PREFILL_TOKENS) / t / PEAK_FLOPS[dtype_key], 4)}}))
+                                      "frac": round(prefill_flops(raw, args.prefill_tokens) / t / PEAK_FLOPS[dtype_key], 4)}}))
         return 0
     elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run)
     ms_per_step = elapsed / args.steps * 1e3
@@ -191,7 +192,7 @@ def main() -> int:
             "num_attention_heads": raw["num_attention_heads"], "num_key_value_heads": raw["num_key_value_heads"],
             "head_dim": raw["head_dim"], "vocab_size": raw["vocab_size"], "rope_theta": raw["rope_theta"],
             "rms_norm_eps": raw["rms_norm_eps"], "tie_word_embeddings": raw["tie_word_embeddings"],
-            "kv_page_size": PAGE, "prefill_tokens": PREFILL_TOKENS,
+            "kv_page_size": PAGE, "prefill_tokens": args.prefill_tokens,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
@@ -204,10 +205,10 @@ def main() -> int:
             el, _ = time_decode(engine, b, args.context, steps, min(args.warmup, 4), args.decode_run)
             points[f"decode_b{b}"] = round(b * steps / el, 2)
         record["points"] = points
-        note(f"prefill of {PREFILL_TOKENS} tokens")
-        t = time_prefill(engine, PREFILL_TOKENS, 3, raw["vocab_size"])
-        flops = prefill_flops(raw, PREFILL_TOKENS)
-        record["prefill"] = {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS,
+        note(f"prefill of {args.prefill_tokens} tokens")
+        t = time_prefill(engine, args.prefill_tokens, 3, raw["vocab_size"])
+        flops = prefill_flops(raw, args.prefill_tokens)
+        record["prefill"] = {"value": round(args.prefill_tokens / t, 1), "tokens": args.prefill_tokens,
                              "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS[dtype_key], 4)}
     print(json.dumps(record))
     return 0
