@@ -52,9 +52,11 @@ int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, co
                 const float* freq, const float* pres, const int* bias_ids, const float* bias_vals,
                 int nb, hipStream_t stream);
 long long ia_sample_workspace(int rows, int vocab);
+int ia_sample_max_top(void);
+// n_top, lp_out [rows, 1 + max_top], lp_ids [rows, max_top]: all null, or the log-probabilities asked for per row
 int ia_sample(int* out, const float* logits, void* workspace, int rows, int vocab,
               const float* temperature, const int* top_k, const float* top_p, const float* min_p,
-              const float* u, hipStream_t stream);
+              const float* u, const int* n_top, float* lp_out, int* lp_ids, hipStream_t stream);
 
 // Built per head size (-DIA_HEAD_DIM) into a library of its own.
 int ia_attention_mfma_head_dim(void);

@@ -271,11 +271,47 @@ __device__ int nth_with_key(const uint32_t* __restrict__ keys, int vocab, uint32
     return s_index;
 }
 
+// The first token after (prev_key, prev_idx) in the order of the reference's sorted list: keys
+// descending, equal keys by ascending index (its sort is stable).  Returns the index, or -1.
+__device__ int next_in_order(const uint32_t* __restrict__ keys, int vocab, uint32_t prev_key, int prev_idx,
+                             uint32_t* s_key, int* s_idx) {
+    uint32_t bk = 0u;
+    int bi = -1;
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const uint32_t k = keys[c];
+        if (!(k < prev_key || (k == prev_key && c > prev_idx))) continue;
+        if (bi < 0 || k > bk || (k == bk && c < bi)) { bk = k; bi = c; }
+    }
+#pragma unroll
+    for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
+        const uint32_t ok = (uint32_t)__shfl_xor((int)bk, o, IA_WAVE);
+        const int oi = __shfl_xor(bi, o, IA_WAVE);
+        if (oi >= 0 && (bi < 0 || ok > bk || (ok == bk && oi < bi))) { bk = ok; bi = oi; }
+    }
+    __syncthreads();
+    if ((threadIdx.x & (IA_WAVE - 1)) == 0) { s_key[threadIdx.x / IA_WAVE] = bk; s_idx[threadIdx.x / IA_WAVE] = bi; }
+    __syncthreads();
+    bk = 0u; bi = -1;
+    for (int w = 0; w < (int)(blockDim.x / IA_WAVE); ++w) {
+        const uint32_t ok = s_key[w];
+        const int oi = s_idx[w];
+        if (oi >= 0 && (bi < 0 || ok > bk || (ok == bk && oi < bi))) { bk = ok; bi = oi; }
+    }
+    __syncthreads();
+    return bi;
+}
+
+#define SAMPLE_MAX_TOP 20
+
 // workspace: [rows, 2, vocab] words: the keys, then the probabilities.
+// n_top (may be null): per row -1 = no log-probabilities, else how many of the list's first entries are
+// reported besides the drawn token's (sampler.rs:285-352).  lp_out [rows, 1 + SAMPLE_MAX_TOP]: the drawn
+// token's log-probability within the kept list, then the entries'; lp_ids [rows, SAMPLE_MAX_TOP]: their ids (-1: none).
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, uint32_t* __restrict__ workspace, int vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
-    const float* __restrict__ min_p, const float* __restrict__ u) {
+    const float* __restrict__ min_p, const float* __restrict__ u, const int* __restrict__ n_top,
+    float* __restrict__ lp_out, int* __restrict__ lp_ids) {
     __shared__ float scratch[32];
     __shared__ int s_counts[SAMPLE_THREADS];
     __shared__ float sv[16];
@@ -283,9 +319,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const int rowi = blockIdx.x;
     const float* row = logits + (size_t)rowi * vocab;
     float temp = temperature[rowi];
+    const int want_top = n_top != nullptr ? n_top[rowi] : -1;
+    if (want_top >= 0 && threadIdx.x < SAMPLE_MAX_TOP) {
+        lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + threadIdx.x] = -1;
+        lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + threadIdx.x] = -INFINITY;
+    }
     if (temp < 1e-5f) {
-        argmax_row(row, vocab, sv, si, out + rowi);
-        return;
+        if (want_top < 0) {
+            argmax_row(row, vocab, sv, si, out + rowi);
+            return;
+        }
+        temp = 1e-5f;           // with log-probabilities the reference takes no shortcut (sampler.rs:176, :232-239)
     }
     uint32_t* keys = workspace + (size_t)rowi * 2 * vocab;
     float* probs = (float*)(keys + vocab);
@@ -294,7 +338,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     float mx = -INFINITY;
     for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
         const float z = row[c] / temp;
-        keys[c] = order_key(z);
         probs[c] = z;
         mx = fmaxf(mx, z);
     }
@@ -310,8 +353,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         sum += e;
     }
     sum = block_sum(sum, scratch);
-    if (sum > 0.f)
-        for (int c = threadIdx.x; c < vocab; c += blockDim.x) probs[c] /= sum;
+    // The list is ordered by the probabilities themselves, as the reference sorts them: logits whose
+    // probabilities round to the same number (or vanish together) are ties, taken in index order.
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const float pr = sum > 0.f ? probs[c] / sum : probs[c];
+        probs[c] = pr;
+        keys[c] = order_key(pr);
+    }
     __syncthreads();
 
     // how long the kept prefix is (sampler.rs:256-283)
@@ -362,6 +410,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int token;
     if (!(filtered > 0.f)) {
         argmax_row(row, vocab, sv, si, out + rowi);
+        if (want_top >= 0 && threadIdx.x == 0) lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = -INFINITY;
         return;
     }
     const Prefix hit = shortest_prefix(keys, probs, vocab, u[rowi] * filtered, false, true, scratch);
@@ -388,18 +437,44 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         token = nth_with_key(keys, vocab, hit.key, hit.take, s_counts);
     }
     if (threadIdx.x == 0) out[rowi] = token;
+    if (want_top < 0) return;
+    // log-probabilities within the kept list: the drawn token's, then the list's first entries
+    if (threadIdx.x == 0) {
+        const float pt = probs[token];
+        lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = pt > 0.f ? logf(pt / filtered) : -INFINITY;
+    }
+    const int n_list = keep < vocab ? keep : vocab;
+    uint32_t prev_key = 0xffffffffu;
+    int prev_idx = -1;
+    uint32_t* s_key = (uint32_t*)scratch;
+    for (int i = 0; i < want_top && i < SAMPLE_MAX_TOP && i < n_list; ++i) {
+        const int idx = next_in_order(keys, vocab, prev_key, prev_idx, s_key, si);
+        if (idx < 0) break;
+        if (threadIdx.x == 0) {
+            const float pi = probs[idx];
+            lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + i] = idx;
+            lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + i] = pi > 0.f ? logf(pi / filtered) : -INFINITY;
+        }
+        prev_key = keys[idx];
+        prev_idx = idx;
+    }
 }
 
 extern "C" long long ia_sample_workspace(int rows, int vocab) { return (long long)rows * 2 * vocab; }
 
+extern "C" int ia_sample_max_top(void) { return SAMPLE_MAX_TOP; }
+
+// n_top, lp_out, lp_ids: all null, or all given (see sample_kernel).
 extern "C" int ia_sample(int* out, const float* logits, void* workspace, int rows, int vocab,
                          const float* temperature, const int* top_k, const float* top_p, const float* min_p,
-                         const float* u, hipStream_t stream) {
+                         const float* u, const int* n_top, float* lp_out, int* lp_ids, hipStream_t stream) {
     IA_CHECK(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
     IA_CHECK(workspace != nullptr || rows == 0, "sample: needs a workspace of rows * 2 * vocab words");
+    IA_CHECK((n_top == nullptr) == (lp_out == nullptr) && (n_top == nullptr) == (lp_ids == nullptr),
+             "sample: the arrays of the log-probabilities come together");
     if (rows == 0) return 0;
     sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, (uint32_t*)workspace, vocab, temperature,
-                                                       top_k, top_p, min_p, u);
+                                                       top_k, top_p, min_p, u, n_top, lp_out, lp_ids);
     IA_LAUNCH_CHECK("sample");
     return 0;
 }

@@ -19,6 +19,7 @@ class Generation:
     finish_reason: str
     error: Optional[str] = None
     preemptions: int = 0
+    logprobs: Optional[list] = None     # a TokenLogprob per token when the parameters asked for them
 
 
 class GenerationLoop:
@@ -90,8 +91,13 @@ class GenerationLoop:
                    for e in plan.entries]
         logits = self.engine.step(entries, commit=False)
         drawing = [e.request for e in plan.entries if e.samples]
-        tokens = self.sampler.sample(logits, [r.params for r in drawing], [r.tokens for r in drawing],
-                                     [r.seed for r in drawing])
+        tokens, infos = self.sampler.sample_with_logprobs(logits, [r.params for r in drawing],
+                                                          [r.tokens for r in drawing], [r.seed for r in drawing])
+        for r, info in zip(drawing, infos):
+            if info is not None:
+                # a request that was preempted draws its tokens again while it is recomputed: the same ones
+                del r.logprobs[len(r.output):]
+                r.logprobs.append(info)
         sampled: Dict[Hashable, int] = {r.request_id: t for r, t in zip(drawing, tokens)}
         done += self.scheduler.commit(plan, sampled)
         self.steps += 1
@@ -123,5 +129,6 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]], params=None, **lo
         raise ValueError("one SamplingParams for all prompts, or one per prompt")
     requests = [loop.add(p, sp, request_id=i) for i, (p, sp) in enumerate(zip(prompts, params))]
     loop.run()
-    return [Generation(r.request_id, r.prompt, list(r.output), r.finish_reason or "error", r.error, r.preemptions)
+    return [Generation(r.request_id, r.prompt, list(r.output), r.finish_reason or "error", r.error, r.preemptions,
+                       list(r.logprobs) if r.params.logprobs else None)
             for r in requests]

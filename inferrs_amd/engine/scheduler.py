@@ -49,6 +49,7 @@ class Request:
     error: Optional[str] = None
     preemptions: int = 0
     arrival: int = 0
+    logprobs: List[object] = field(default_factory=list)   # a TokenLogprob per output token, when asked for
 
     @property
     def tokens(self) -> List[int]:

@@ -441,21 +441,31 @@ def penalize(logits: torch.Tensor, window: Optional[torch.Tensor], repetition: t
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           min_p: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+           min_p: torch.Tensor, u: torch.Tensor, n_top: Optional[torch.Tensor] = None):
     """One token per row of float32 logits: greedy where temperature < 1e-5, else temperature,
-    top-k, top-p, min-p and the walk to the row's random number u in [0, 1)."""
-    _dev(logits, temperature, top_k, top_p, min_p, u)
+    top-k, top-p, min-p and the walk to the row's random number u in [0, 1).  With `n_top` (int32
+    per row: -1 none, else 0..20) also returns the log-probabilities within the kept list, float32
+    [rows, 1 + 20] (the drawn token's, then the list's first entries'), and those entries' ids, int32
+    [rows, 20] (-1: no entry): the result is then (tokens, log-probabilities, ids)."""
+    _dev(logits, temperature, top_k, top_p, min_p, u, n_top)
     _f32(logits, "logits"); _f32(temperature, "temperature"); _f32(top_p, "top_p"); _f32(min_p, "min_p"); _f32(u, "u")
     _i32(top_k, "top_k")
     rows, vocab = logits.shape
-    for t in (temperature, top_k, top_p, min_p, u):
+    for t in (temperature, top_k, top_p, min_p, u) + ((n_top,) if n_top is not None else ()):
         if t.numel() != rows:
             raise KernelError("sample: one parameter value per row of logits")
+    lib = library()
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    ws = torch.empty((library().ia_sample_workspace(rows, vocab),), dtype=torch.int32, device=logits.device)
-    _check(library().ia_sample(_p(out), _p(logits), _p(ws), rows, vocab, _p(temperature), _p(top_k), _p(top_p),
-                               _p(min_p), _p(u), _stream()))
-    return out
+    ws = torch.empty((lib.ia_sample_workspace(rows, vocab),), dtype=torch.int32, device=logits.device)
+    lp = ids = None
+    if n_top is not None:
+        _i32(n_top, "n_top")
+        most = lib.ia_sample_max_top()
+        lp = torch.empty((rows, 1 + most), dtype=torch.float32, device=logits.device)
+        ids = torch.empty((rows, most), dtype=torch.int32, device=logits.device)
+    _check(lib.ia_sample(_p(out), _p(logits), _p(ws), rows, vocab, _p(temperature), _p(top_k), _p(top_p),
+                         _p(min_p), _p(u), _p(n_top), _p(lp), _p(ids), _stream()))
+    return out if n_top is None else (out, lp, ids)
 
 
 def gated_silu_linear(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:

@@ -1,3 +1,3 @@
-from .params import SAMPLING_EPS, SamplingParams
+from .params import SAMPLING_EPS, SamplingParams, TokenLogprob
 from .rng import rand_f32, fresh_seed
 from .sampler import Sampler

@@ -21,6 +21,8 @@ class SamplingParams:
     max_tokens: int = 2048            # cap on generated tokens
     seed: Optional[int] = None        # None: a fresh seed per request
     logit_bias: Dict[int, float] = field(default_factory=dict)
+    logprobs: bool = False            # report the drawn token's log-probability within the kept list
+    top_logprobs: int = 0             # and the first 0..20 entries of that list (needs logprobs)
     extra_stop_token_ids: Tuple[int, ...] = ()
     bypass_stop_tokens: bool = False  # run to max_tokens whatever is generated (benchmarks)
 
@@ -37,6 +39,10 @@ class SamplingParams:
             raise ValueError(f"repeat_last_n must be >= 0, got {self.repeat_last_n}")
         if self.max_tokens < 1:
             raise ValueError(f"max_tokens must be >= 1, got {self.max_tokens}")
+        if not (0 <= self.top_logprobs <= 20):
+            raise ValueError(f"top_logprobs must lie in 0..20, got {self.top_logprobs}")
+        if self.top_logprobs and not self.logprobs:
+            raise ValueError("top_logprobs needs logprobs")
 
     @classmethod
     def greedy(cls, max_tokens: int = 2048, **kw) -> "SamplingParams":
@@ -51,4 +57,13 @@ class SamplingParams:
     @property
     def is_plain_greedy(self) -> bool:
         """The reference's fast path: arg max of the untouched logits (`sampler.rs:171-179`)."""
-        return self.temperature < SAMPLING_EPS and not self.has_penalty and not self.logit_bias
+        return self.temperature < SAMPLING_EPS and not self.has_penalty and not self.logit_bias and not self.logprobs
+
+
+@dataclass
+class TokenLogprob:
+    """What the reference reports for a drawn token (`sampler.rs:119-134`): its log-probability within
+    the list that top-k, top-p and min-p kept, and the first `top_logprobs` entries of that list."""
+    token_id: int
+    logprob: float
+    top_logprobs: Tuple[Tuple[int, float], ...] = ()

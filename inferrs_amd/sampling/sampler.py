@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from .params import SAMPLING_EPS, SamplingParams
+from .params import SAMPLING_EPS, SamplingParams, TokenLogprob
 from .rng import rand_f32
 
 
@@ -25,13 +25,19 @@ class Sampler:
                seeds: Sequence[int]) -> List[int]:
         """`logits` float32 [rows, vocab] on the device; row i belongs to a request with
         `params[i]`, whose prompt and output so far are `previous[i]` and whose seed is `seeds[i]`."""
+        return self.sample_with_logprobs(logits, params, previous, seeds)[0]
+
+    def sample_with_logprobs(self, logits: torch.Tensor, params: Sequence[SamplingParams],
+                             previous: Sequence[Sequence[int]], seeds: Sequence[int]):
+        """(tokens, per row a `TokenLogprob` or None): the log-probabilities for the rows whose
+        parameters ask for them (`sampler.rs:285-352`)."""
         rows = logits.shape[0]
         if not (len(params) == len(previous) == len(seeds) == rows):
             raise ValueError("one parameter set, token history and seed per row of logits")
         if rows == 0:
-            return []
+            return [], []
         if all(p.is_plain_greedy for p in params):
-            return ops.argmax(logits).cpu().tolist()
+            return ops.argmax(logits).cpu().tolist(), [None] * rows
 
         # penalties and bias, on a copy only if something is changed
         width = max((min(p.repeat_last_n, len(prev)) if p.has_penalty else 0) for p, prev in zip(params, previous))
@@ -65,6 +71,19 @@ class Sampler:
         # the step of a draw is the number of tokens before it (`sampler.rs:323-325`)
         u = np.asarray([rand_f32(seed, len(prev)) if p.temperature >= SAMPLING_EPS else 0.0
                         for p, prev, seed in zip(params, previous, seeds)], dtype=np.float32)
-        out = ops.sample(logits, self._dev(temperature), self._dev(top_k), self._dev(top_p), self._dev(min_p),
-                         self._dev(u))
-        return out.cpu().tolist()
+        if not any(p.logprobs for p in params):
+            out = ops.sample(logits, self._dev(temperature), self._dev(top_k), self._dev(top_p), self._dev(min_p),
+                             self._dev(u))
+            return out.cpu().tolist(), [None] * rows
+        n_top = np.asarray([p.top_logprobs if p.logprobs else -1 for p in params], dtype=np.int32)
+        out, lp, ids = ops.sample(logits, self._dev(temperature), self._dev(top_k), self._dev(top_p), self._dev(min_p),
+                                  self._dev(u), self._dev(n_top))
+        tokens, lp, ids = out.cpu().tolist(), lp.cpu().tolist(), ids.cpu().tolist()
+        infos = []
+        for i, p in enumerate(params):
+            if not p.logprobs:
+                infos.append(None)
+                continue
+            top = tuple((t, v) for t, v in zip(ids[i], lp[i][1:]) if t >= 0)[:p.top_logprobs]
+            infos.append(TokenLogprob(tokens[i], lp[i][0], top))
+        return tokens, infos

@@ -211,13 +211,14 @@ def rand_f32(seed: int, step: int) -> float:
 
 def sample(logits: torch.Tensor, previous: Sequence[int], *, temperature=0.7, top_p=0.9, top_k=50,
            min_p=0.0, repetition_penalty=1.1, repeat_last_n=64, frequency_penalty=0.0,
-           presence_penalty=0.0, seed: int = 0) -> int:
-    """inferrs/src/sampler.rs:146-335, step by step, for a seeded request."""
+           presence_penalty=0.0, seed: int = 0, logprobs: bool = False, top_logprobs: int = 0):
+    """inferrs/src/sampler.rs:146-352, step by step, for a seeded request.  With `logprobs` the result is
+    (token, its log-probability, [(id, log-probability)] of the kept list's first entries)."""
     z = logits.to(torch.float32).clone()
     vocab = z.numel()
     window = list(previous[-repeat_last_n:]) if repeat_last_n > 0 else []
     has_pen = (repetition_penalty != 1.0 or frequency_penalty != 0.0 or presence_penalty != 0.0) and window
-    if temperature < 1e-5 and not has_pen:
+    if temperature < 1e-5 and not has_pen and not logprobs:                 # :176
         return int(torch.argmax(z))
     if repetition_penalty not in (1.0, 0.0) and window:                    # :196-209
         for t in dict.fromkeys(window):
@@ -251,8 +252,11 @@ def sample(logits: torch.Tensor, previous: Sequence[int], *, temperature=0.7, to
     total = torch.tensor(0.0)
     for _, pr in kept:
         total = total + torch.tensor(pr, dtype=torch.float32)
+    denom = float(total) if total > 0 else 1.0                             # :286-292
+    top = [(i, math.log(pr / denom) if pr > 0 else -math.inf) for i, pr in kept[:top_logprobs]] if logprobs else []
     if total <= 0:
-        return kept[0][0] if kept else 0
+        first = kept[0][0] if kept else 0
+        return (first, -math.inf, top) if logprobs else first
     u = torch.tensor(rand_f32(seed, len(previous)), dtype=torch.float32)    # :323-335
     chosen = kept[-1][0]
     for i, pr in kept:
@@ -261,4 +265,7 @@ def sample(logits: torch.Tensor, previous: Sequence[int], *, temperature=0.7, to
             chosen = i
             break
         u = u - norm
-    return chosen
+    if not logprobs:
+        return chosen
+    pr = dict(kept)[chosen] / float(total)                                  # :339-352
+    return chosen, (math.log(pr) if pr > 0 else -math.inf), top

@@ -177,3 +177,29 @@ def test_runs_of_decode_steps_give_the_same_tokens_as_single_steps(tiny, dtype):
     first = results[1][0].index(results[1][0][20])
     assert results[8][0] == results[1][0][:first + 1]
     assert results[8][1] == results[1][1] and results[8][2] == results[1][2] and len(results[8][2]) == 23
+
+
+def test_generation_reports_log_probabilities(tiny):
+    """`logprobs` through the entry point: one record per generated token, consistent with the plain
+    model's softmax at that place (temperature 1, nothing filtered, so the kept list is the vocabulary)."""
+    import math
+    from inferrs_amd import SamplingParams
+    from inferrs_amd.engine import Engine
+    folder, cfg, params = tiny["B"]
+    eng = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=40, max_seqs=4)
+    prompt = random_tokens(9, cfg["vocab_size"], 71)
+    sp = SamplingParams(temperature=1.0, top_p=1.0, top_k=0, repetition_penalty=1.0, seed=3, max_tokens=6,
+                        logprobs=True, top_logprobs=4, bypass_stop_tokens=True)
+    plain = SamplingParams(temperature=1.0, top_p=1.0, top_k=0, repetition_penalty=1.0, seed=3, max_tokens=6,
+                           bypass_stop_tokens=True)
+    with_lp, without = eng.generate([prompt, prompt], [sp, plain])
+    assert with_lp.tokens == without.tokens and without.logprobs is None      # asking for them changes no draw
+    assert len(with_lp.logprobs) == 6
+    toks = list(prompt)
+    for tok, info in zip(with_lp.tokens, with_lp.logprobs):
+        logp = torch.log_softmax(pm.forward(cfg, params, toks)[-1], 0)
+        assert info.token_id == tok and info.logprob == pytest.approx(float(logp[tok]), abs=1e-4)
+        best = torch.topk(logp, 4)
+        assert [t for t, _ in info.top_logprobs] == best.indices.tolist()
+        assert [v for _, v in info.top_logprobs] == pytest.approx(best.values.tolist(), abs=1e-4)
+        toks.append(tok)

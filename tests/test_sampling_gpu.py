@@ -170,3 +170,54 @@ def test_sampling_params_defaults_are_the_reference_defaults():
     assert p.max_tokens == 2048 and p.seed is None and not p.bypass_stop_tokens
     with pytest.raises(ValueError):
         SamplingParams(top_p=0.0)
+
+
+LOGPROB_PARAMS = [
+    dict(temperature=0.7, top_p=1.0, top_k=0, repetition_penalty=1.0, top_logprobs=5),
+    dict(top_logprobs=20),                                                   # the reference's defaults: top-k 50, top-p 0.9
+    dict(temperature=1.0, top_p=1.0, top_k=3, repetition_penalty=1.3, repeat_last_n=16, top_logprobs=7),   # a list shorter than asked for
+    dict(temperature=0.0, top_p=1.0, top_k=0, repetition_penalty=1.0, top_logprobs=4),    # greedy: no shortcut with log-probabilities
+    dict(temperature=0.9, top_p=0.6, top_k=40, min_p=0.1, top_logprobs=0),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("vocab", [130, 2000, 151936])
+@pytest.mark.parametrize("kw", LOGPROB_PARAMS, ids=[str(i) for i in range(len(LOGPROB_PARAMS))])
+def test_log_probabilities_match_the_plain_transcription(vocab, kw):
+    """`logprobs` (inferrs/src/sampler.rs:285-352): the drawn token's log-probability within the list that
+    top-k, top-p and min-p kept, and the first `top_logprobs` entries of that list in its order."""
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    rows = 4 if vocab < 100000 else 2
+    zs, prevs, seeds, params = [], [], [], []
+    for i in range(rows):
+        z, prev = _case(vocab, 7000 + 10 * LOGPROB_PARAMS.index(kw) + i)
+        zs.append(z); prevs.append(prev[: 5 + 11 * i]); seeds.append(50 + i)
+        # a row without log-probabilities beside rows with them
+        params.append(SamplingParams(seed=seeds[-1], logprobs=i != 1, **(kw if i != 1 else {k: v for k, v in kw.items() if k != "top_logprobs"})))
+    tokens, infos = sampler.sample_with_logprobs(torch.stack(zs).to("cuda"), params, prevs, seeds)
+    assert infos[1] is None
+    full = {**dict(temperature=0.7, top_p=0.9, top_k=50, min_p=0.0, repetition_penalty=1.1, repeat_last_n=64,
+                   frequency_penalty=0.0, presence_penalty=0.0), **kw}
+    for i in range(rows):
+        if i == 1:
+            continue
+        want_token, want_lp, want_top = pm.sample(zs[i], prevs[i], seed=seeds[i], logprobs=True, **full)
+        info = infos[i]
+        assert info.token_id == tokens[i]
+        assert [t for t, _ in info.top_logprobs] == [t for t, _ in want_top]
+        for (_, got), (_, want) in zip(info.top_logprobs, want_top):
+            assert got == pytest.approx(want, abs=2e-3) or (math.isinf(got) and math.isinf(want))
+        if tokens[i] == want_token:            # they may part where u falls on a boundary (see above)
+            assert info.logprob == pytest.approx(want_lp, abs=2e-3) or (math.isinf(info.logprob) and math.isinf(want_lp))
+        if kw.get("temperature") == 0.0:
+            assert tokens[i] == int(torch.argmax(zs[i])) and info.logprob == pytest.approx(0.0, abs=1e-6)
+
+
+def test_log_probability_parameters_are_checked():
+    with pytest.raises(ValueError, match="needs logprobs"):
+        SamplingParams(top_logprobs=3)
+    with pytest.raises(ValueError, match="0..20"):
+        SamplingParams(logprobs=True, top_logprobs=21)
+    assert not SamplingParams.greedy(logprobs=True).is_plain_greedy and SamplingParams.greedy().is_plain_greedy
