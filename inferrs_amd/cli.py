@@ -131,7 +131,8 @@ def cmd_run(args) -> int:
 
     def answer(text: str) -> None:
         loop = GenerationLoop(engine, max_batch_size=args.max_batch_size,
-                              max_tokens_per_step=args.max_tokens_per_step, max_seq_len=args.max_seq_len or None)
+                              max_tokens_per_step=args.max_tokens_per_step, max_seq_len=args.max_seq_len or None,
+                              detokenize=codec.decode)
         req = loop.add(codec.encode(text, args.system), params)
         t0 = time.perf_counter()
         if codec.tokenizer is None:

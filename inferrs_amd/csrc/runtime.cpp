@@ -794,6 +794,22 @@ int iar_sched_request_output(void* sched, int64_t key, int* out, int capacity) {
     std::copy(r.tokens.begin() + r.n_prompt, r.tokens.begin() + r.n_prompt + n, out);
     return r.n_output();
 }
+int iar_sched_finish(void* sched, int64_t key) {
+    Sched* s = S(sched);
+    auto it = s->reqs.find(key);
+    if (it == s->reqs.end()) return fail(IAR_ERROR, "no such request");
+    Req* r = it->second.get();
+    if (r->status == FINISHED) return 0;
+    auto w = std::find(s->waiting.begin(), s->waiting.end(), r);
+    if (w != s->waiting.end()) s->waiting.erase(w);
+    auto run = std::find(s->running.begin(), s->running.end(), r);
+    if (run != s->running.end()) s->running.erase(run);
+    if (s->cache->find(key) && s->cache->free_sequence(key)) return IAR_ERROR;
+    int budget = 0;
+    s->drop_entries_of(r, budget);
+    r->status = FINISHED;
+    return 0;
+}
 int iar_sched_forget(void* sched, int64_t key) {
     Sched* s = S(sched);
     auto it = s->reqs.find(key);

@@ -99,6 +99,9 @@ int iar_sched_commit_decode(void* sched, int n, const int64_t* keys, const int* 
 // state of one request: 0 computed, 1 n output, 2 status (0 waiting, 1 running, 2 finished), 3 preemptions, 4 n prompt
 int iar_sched_request_state(void* sched, int64_t key, int* out5);
 int iar_sched_request_output(void* sched, int64_t key, int* out, int capacity);
+// End a waiting or running request now (a stop string matched, the client went away): its cache entry
+// is given back.  Entries of the current plan that belong to it are dropped.
+int iar_sched_finish(void* sched, int64_t key);
 int iar_sched_forget(void* sched, int64_t key);                     // drop a finished request's record
 
 #ifdef __cplusplus

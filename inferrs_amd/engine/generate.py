@@ -25,10 +25,13 @@ class Generation:
 class GenerationLoop:
     def __init__(self, engine: Engine, *, max_batch_size: int = 32, max_tokens_per_step: int = 2048,
                  prefill_chunk: Optional[int] = None, max_seq_len: Optional[int] = None,
-                 stop_token_ids: Optional[Sequence[int]] = None, decode_run: int = 8):
+                 stop_token_ids: Optional[Sequence[int]] = None, decode_run: int = 8,
+                 detokenize: Optional[Callable[[List[int]], str]] = None):
         """`decode_run`: when every running request decodes greedily and nobody waits, up to this
-        many decode steps are queued on the GPU at once (`Engine.decode_chain`); 1 switches it off."""
+        many decode steps are queued on the GPU at once (`Engine.decode_chain`); 1 switches it off.
+        `detokenize`: output token ids -> text, for requests with stop strings."""
         self.engine = engine
+        self.detokenize = detokenize
         self.decode_run = max(1, decode_run)
         limit = engine.spec.max_position if not max_seq_len else min(max_seq_len, engine.spec.max_position)
         self.scheduler = Scheduler(
@@ -48,6 +51,8 @@ class GenerationLoop:
         vocab = self.engine.spec.vocab_size
         if any((not isinstance(t, int)) or t < 0 or t >= vocab for t in prompt):
             raise ValueError(f"request {request_id!r}: token ids must be integers in 0..{vocab - 1}")
+        if any(params.stop_strings) and self.detokenize is None:
+            raise ValueError(f"request {request_id!r}: stop strings need a detokenizer (GenerationLoop(detokenize=...))")
         seed = params.seed if params.seed is not None else fresh_seed()
         req = Request(request_id, list(prompt), params, seed=seed)
         self.scheduler.add(req)
@@ -59,7 +64,8 @@ class GenerationLoop:
         running = list(sched.running)
         if max_steps < 2 or not running or sched.waiting or len(running) > sched.max_tokens_per_step:
             return None
-        if any(r.total - r.computed != 1 or not r.output or not r.params.is_plain_greedy for r in running):
+        if any(r.total - r.computed != 1 or not r.output or not r.params.is_plain_greedy or any(r.params.stop_strings)
+               for r in running):
             return None
         k = min(max_steps, min(min(r.params.max_tokens - len(r.output), sched.max_seq_len - r.total) for r in running))
         ids = [r.request_id for r in running]
@@ -100,8 +106,23 @@ class GenerationLoop:
                 r.logprobs.append(info)
         sampled: Dict[Hashable, int] = {r.request_id: t for r, t in zip(drawing, tokens)}
         done += self.scheduler.commit(plan, sampled)
+        # stop strings: the decoded output ends with one (`check_stop`, inferrs/src/engine.rs:866-887, where
+        # they come after the stop tokens and before the length)
+        for r in drawing:
+            if any(r.params.stop_strings) and r.finish_reason in (None, "length"):
+                text = self.detokenize(list(r.output))
+                if any(s and text.endswith(s) for s in r.params.stop_strings):
+                    if r.finish_reason is None:
+                        self.scheduler.finish(r, "stop")
+                        done.append(r)
+                    else:
+                        r.finish_reason = "stop"
         self.steps += 1
         return done
+
+    def cancel(self, request: Request) -> None:
+        """Nobody waits for this request any more: it ends with "cancelled" and gives back what it holds."""
+        self.scheduler.finish(request, "cancelled")
 
     def run(self, on_token: Optional[Callable[[Request, int], None]] = None) -> List[Request]:
         """Steps until nothing is waiting or running; returns everything that finished."""

@@ -182,6 +182,16 @@ class Scheduler:
         self._lib.iar_sched_forget(self._ptr, key)
         self.cache.names.unpin(r.request_id, live=False)
 
+    def finish(self, request: Request, reason: str) -> None:
+        """End a waiting or running request now, with `reason` ("stop" when a stop string matched,
+        "cancelled" when nobody waits for it any more): what it holds is given back."""
+        key = self.cache.names.find(request.request_id)
+        if key is None or key not in self._requests:
+            return                                      # finished already
+        if self._lib.iar_sched_finish(self._ptr, key):
+            raise RuntimeError(native.last_error())
+        self._finish(key, request, reason)
+
     # ---- planning ---------------------------------------------------------------------------
     def plan(self) -> Plan:
         """Decide the next step and reserve its pages.  May preempt or fail requests."""

@@ -65,6 +65,7 @@ _SIGNATURES = {
     "iar_sched_commit_decode": (c_int, [c_void_p, c_int, _PK, _PI, _PK, _PI, c_int]),
     "iar_sched_request_state": (c_int, [c_void_p, c_int64, _PI]),
     "iar_sched_request_output": (c_int, [c_void_p, c_int64, _PI, c_int]),
+    "iar_sched_finish": (c_int, [c_void_p, c_int64]),
     "iar_sched_forget": (c_int, [c_void_p, c_int64]),
 }
 

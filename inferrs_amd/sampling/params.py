@@ -24,6 +24,7 @@ class SamplingParams:
     logprobs: bool = False            # report the drawn token's log-probability within the kept list
     top_logprobs: int = 0             # and the first 0..20 entries of that list (needs logprobs)
     extra_stop_token_ids: Tuple[int, ...] = ()
+    stop_strings: Tuple[str, ...] = ()  # generation stops when the decoded output ends with one (needs a detokenizer)
     bypass_stop_tokens: bool = False  # run to max_tokens whatever is generated (benchmarks)
 
     def __post_init__(self):

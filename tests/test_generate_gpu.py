@@ -203,3 +203,38 @@ def test_generation_reports_log_probabilities(tiny):
         assert [t for t, _ in info.top_logprobs] == best.indices.tolist()
         assert [v for _, v in info.top_logprobs] == pytest.approx(best.values.tolist(), abs=1e-4)
         toks.append(tok)
+
+
+def test_stop_strings_and_cancellation(tiny):
+    """`stop_strings` (`check_stop`, inferrs/src/engine.rs:866-887): generation ends with "stop" as soon as the
+    decoded output ends with one of them; a request can also be cancelled between steps."""
+    from inferrs_amd import SamplingParams
+    from inferrs_amd.engine import Engine, GenerationLoop
+    folder, cfg, params = tiny["A"]
+    eng = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=64, max_seqs=4)
+    prompt = random_tokens(7, cfg["vocab_size"], 5)
+    free = eng.generate([prompt], SamplingParams.greedy(max_tokens=12, bypass_stop_tokens=True))[0].tokens
+    words = lambda ids: "".join(f"<{t}>" for t in ids)                     # a stand-in for a tokenizer
+    stop = f"<{free[4]}><{free[5]}>"                                       # two tokens long: matched across tokens
+    cut = next(i for i in range(1, 12) if words(free[:i + 1]).endswith(stop))
+    sp = SamplingParams.greedy(max_tokens=12, bypass_stop_tokens=True, stop_strings=("", "never", stop))
+    out = eng.generate([prompt, prompt], [sp, SamplingParams.greedy(max_tokens=12, bypass_stop_tokens=True)],
+                       detokenize=words)
+    assert out[0].tokens == free[:cut + 1] and out[0].finish_reason == "stop"
+    assert out[1].tokens == free and out[1].finish_reason == "length"
+    # a stop string at the very last allowed token still reads "stop"
+    last = eng.generate([prompt], SamplingParams.greedy(max_tokens=cut + 1, bypass_stop_tokens=True, stop_strings=(stop,)),
+                        detokenize=words)[0]
+    assert last.tokens == free[:cut + 1] and last.finish_reason == "stop"
+    with pytest.raises(ValueError, match="detokenizer"):
+        eng.generate([prompt], sp)
+    # cancellation
+    loop = GenerationLoop(eng)
+    a = loop.add(prompt, SamplingParams.greedy(max_tokens=50, bypass_stop_tokens=True))
+    b = loop.add(prompt, SamplingParams.greedy(max_tokens=6, bypass_stop_tokens=True))
+    loop.step()
+    loop.step()
+    loop.cancel(a)
+    loop.run()
+    assert a.finish_reason == "cancelled" and 0 < len(a.output) < 50 and b.output == free[:6]
+    assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups)

@@ -190,3 +190,20 @@ def test_a_name_in_use_outside_the_scheduler_is_reported():
     s.add(req("a", 3))
     with pytest.raises(RuntimeError, match="already live"):
         s.plan()
+
+
+def test_a_request_can_be_ended_from_outside():
+    cache, s = make(num_pages=16, page_size=4, max_tokens_per_step=8)
+    a, b, c = req("a", 6, 10), req("b", 20, 10), req("c", 3, 10)
+    for r in (a, b, c):
+        s.add(r)
+    plan = s.plan()                                  # a whole, the first two tokens of b
+    assert [(e.request.request_id, len(e.tokens)) for e in plan.entries] == [("a", 6), ("b", 2)]
+    s.finish(b, "cancelled")                         # while its portion is planned
+    assert b.finish_reason == "cancelled" and "b" not in cache.sequences
+    s.finish(c, "cancelled")                         # while it waits
+    assert c.status == "finished" and [r.request_id for r in s.waiting] == []
+    s.finish(c, "cancelled")                         # again: nothing happens
+    run(s, cache)
+    assert a.finish_reason == "length" and len(a.output) == 10
+    assert cache.groups[0].pool.num_free == 16 and not cache.names.names()
