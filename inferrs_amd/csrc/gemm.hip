@@ -10,6 +10,8 @@
 //     streams 16 weight rows in 16-byte pieces straight into MFMA 16x16x32 operands and
 //     the waves of a block split k between them; partial tiles are summed in a fixed order.
 //     A variant takes [gate; up] and writes silu(gate) * up.
+#include <type_traits>
+
 #include "common.h"
 #include "api.h"
 
@@ -214,6 +216,37 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                         for (int t = 0; t < RT; ++t)
                             acc[q][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                                 __builtin_bit_cast(bf16x8, a[i][q][t]), __builtin_bit_cast(bf16x8, b[i][u]), acc[q][t][u], 0, 0, 0);
+        }
+        if constexpr (!STAGE) {
+            // what the chunks leave: a chunk of 8 and one of 4 steps before single steps, each with its
+            // loads under way together (a wave's k range need not be a multiple of the chunk)
+            auto short_chunk = [&](auto steps) {
+                constexpr int C = decltype(steps)::value;
+                if (ks + C > pb) return;
+                uint4 a[C][NA][RT], b[C][MT];
+#pragma unroll
+                for (int i = 0; i < C; ++i) {
+#pragma unroll
+                    for (int q = 0; q < NA; ++q)
+#pragma unroll
+                        for (int t = 0; t < RT; ++t) a[i][q][t] = *(const uint4*)(wrow[q][t] + (ks + i) * SK_KSTEP);
+#pragma unroll
+                    for (int u = 0; u < MT; ++u) b[i][u] = *(const uint4*)(xrow[u] + (ks + i) * SK_KSTEP);
+                }
+#pragma unroll
+                for (int i = 0; i < C; ++i)
+#pragma unroll
+                    for (int u = 0; u < MT; ++u)
+#pragma unroll
+                        for (int q = 0; q < NA; ++q)
+#pragma unroll
+                            for (int t = 0; t < RT; ++t)
+                                acc[q][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                    __builtin_bit_cast(bf16x8, a[i][q][t]), __builtin_bit_cast(bf16x8, b[i][u]), acc[q][t][u], 0, 0, 0);
+                ks += C;
+            };
+            if constexpr (UNROLL > 8) short_chunk(std::integral_constant<int, 8>());
+            if constexpr (UNROLL > 4) short_chunk(std::integral_constant<int, 4>());
         }
         for (; ks < pb; ++ks) {
             const int k0 = ks * SK_KSTEP;
