@@ -46,18 +46,32 @@ struct AttnParams {
     const bf16_t* q;            // [n, nq, d]
     const bf16_t* k_cache;      // [pages, nkv, page, d]
     const bf16_t* v_cache;      // [pages, nkv, d, page]
+    bf16_t* k_cache_w;          // the same arrays for the fused form's writes
+    bf16_t* v_cache_w;
     const int* block_table;     // [seqs, max_pages]
     const int* cu_tokens;       // [seqs + 1]  request s owns tokens cu[s]..cu[s+1]
     const int* positions;       // [n]         absolute position of each token
     int max_pages, nq, nkv, page, window, splits, chunk, pair, seq_begin;
     float scale_log2;           // scale * log2(e)
+    // Decode steps with the per-head norm, the rotation and the cache write inside (FUSE): q is not
+    // read from `q` but formed from the projections' output, and the wave that walks a request's
+    // newest key forms that key and value, uses them and writes them to the cache.
+    const bf16_t* qkv;          // [n, (nq + 2 nkv) * d]: q heads, then k heads, then v heads
+    const float* q_norm_w;      // [d], or null: no norm
+    const float* k_norm_w;
+    const float* cos_t;         // [n, d / 2], or null: no rotation
+    const float* sin_t;
+    const int* slots;           // [n] cache slot of each token, or null: this layer writes no cache
+    float norm_eps;
+    int norm_add_one;
 };
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
 // One column block (16 * NB columns) of one request and key/value head, over one split of the keys.
-template <int NB>
+template <int NB, bool FUSE = false>
 __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, int kvh, int split, int seq) {
+    static_assert(!FUSE || (NB == 1 && HD % 64 == 0), "the fused form is for single tokens and head sizes in steps of 64");
     const int lane = threadIdx.x;
     const int r = lane & 15, G = lane >> 4;
     const int g = p.nq / p.nkv;
@@ -84,15 +98,74 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
     const int last_col = (col0 + 16 * NB <= n_cols ? col0 + 16 * NB : n_cols) - 1;
     const int pmin = kv_start + col0 / g, pmax = kv_start + last_col / g;
 
-    // Q^T operands stay in registers for the whole walk.
-    uint4 qreg[NB][KS];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
+    // FUSE: one head's row of the projections' output, normed and rotated as the separate kernel does
+    // it (32-bit throughout, one rounding at the end): lane (., G) holds the features ks * 32 + G * 8 ..
+    // + 8 of the row, and a feature's rotation partner, HD / 2 further on, lies in the same lane.
+    const int qkv_row = (p.nq + 2 * p.nkv) * HD;
+    auto normed_rotated = [&](const bf16_t* row, const float* norm_w, uint4 (&packed)[KS]) {
+        float f[KS][8];
+        float ss = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const int dim = ks * 32 + G * 8;
-            qreg[nb][ks] = (cvalid[nb] && dim < HD) ? *(const uint4*)(qrow + dim) : zero4();
+            const uint4 raw = *(const uint4*)(row + ks * 32 + G * 8);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                f[ks][2 * j] = __uint_as_float(w[j] << 16);
+                f[ks][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += f[ks][j] * f[ks][j];
+        }
+        if (norm_w != nullptr) {
+            ss += __shfl_xor(ss, 16, IA_WAVE);
+            ss += __shfl_xor(ss, 32, IA_WAVE);
+            const float scale = 1.0f / sqrtf(ss / (float)HD + p.norm_eps);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const float4 g0 = *(const float4*)(norm_w + ks * 32 + G * 8), g1 = *(const float4*)(norm_w + ks * 32 + G * 8 + 4);
+                const float gw[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[ks][j] = scale * f[ks][j] * (p.norm_add_one ? 1.0f + gw[j] : gw[j]);
+            }
+        }
+        if (p.cos_t != nullptr) {
+#pragma unroll
+            for (int ks = 0; ks < KS / 2; ++ks) {
+                // this token's angles for the lane's features of the first half
+                const size_t at = (size_t)t0 * (HD / 2) + ks * 32 + G * 8;
+                const float4 c0 = *(const float4*)(p.cos_t + at), c1 = *(const float4*)(p.cos_t + at + 4);
+                const float4 s0 = *(const float4*)(p.sin_t + at), s1 = *(const float4*)(p.sin_t + at + 4);
+                const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+                const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float a = f[ks][j], b = f[ks + KS / 2][j];
+                    f[ks][j] = a * c[j] - b * sn[j];
+                    f[ks + KS / 2][j] = a * sn[j] + b * c[j];
+                }
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            packed[ks] = make_uint4(pack_bf16x2(f[ks][0], f[ks][1]), pack_bf16x2(f[ks][2], f[ks][3]),
+                                    pack_bf16x2(f[ks][4], f[ks][5]), pack_bf16x2(f[ks][6], f[ks][7]));
+    };
+
+    // Q^T operands stay in registers for the whole walk.
+    uint4 qreg[NB][KS];
+    if constexpr (FUSE) {
+        // every lane forms a row (invalid columns their request's last head: never stored)
+        normed_rotated(p.qkv + (size_t)t0 * qkv_row + (size_t)head[0] * HD, p.q_norm_w, qreg[0]);
+    } else {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int dim = ks * 32 + G * 8;
+                qreg[nb][ks] = (cvalid[nb] && dim < HD) ? *(const uint4*)(qrow + dim) : zero4();
+            }
         }
     }
 
@@ -279,6 +352,43 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
     for (int k0 = lo; k0 < hi; k0 += 32) {
         Operands op;
         load_step(op, k0, at);
+        if constexpr (FUSE) {
+            // The step that holds the request's newest key (position kv_total - 1, this step's token): its
+            // slot of the cache is not written yet.  The key and value are formed here, put into the
+            // operands in place of what the loads brought, and written to the cache for the steps to come.
+            const int kk = kv_total - 1 - k0;
+            if (p.slots != nullptr && kk >= 0 && kk < 32) {
+                const int slot = p.slots[t0];
+                const int page = slot / p.page, off = slot - page * p.page;
+                uint4 knew[KS];
+                normed_rotated(p.qkv + (size_t)t0 * qkv_row + (size_t)(p.nq + kvh) * HD, p.k_norm_w, knew);
+                const int r_new = ((kk >> 3) << 2) | (kk & 3), t_new = (kk >> 2) & 1;
+                if (r == r_new) {
+                    bf16_t* krow = p.k_cache_w + (((size_t)page * p.nkv + kvh) * p.page + off) * HD + G * 8;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        if (t_new == 0) op.k[0][ks] = knew[ks]; else op.k[1][ks] = knew[ks];
+                        *(uint4*)(krow + ks * 32) = knew[ks];
+                    }
+                }
+                if (G == (kk >> 3)) {
+                    const bf16_t* vrow = p.qkv + (size_t)t0 * qkv_row + (size_t)(p.nq + p.nkv + kvh) * HD + r;
+                    bf16_t* vdst = p.v_cache_w + (((size_t)page * p.nkv + kvh) * HD + r) * p.page + off;
+                    const int j = kk & 7;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        const uint32_t bits = vrow[db * 16].bits;
+                        vdst[(size_t)db * 16 * p.page].bits = (uint16_t)bits;
+                        uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
+                        const uint32_t keep = (j & 1) ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (e == (j >> 1)) w[e] = (w[e] & keep) | ((j & 1) ? bits << 16 : bits);
+                        op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                }
+            }
+        }
         compute_step(op, k0);
         advance(at, 32);
     }
@@ -334,6 +444,17 @@ void attn_mfma_kernel(const AttnParams p) {
     if (late < early) return;
     attn_column_block<NB>(p, late, kvh, split, seq);
     if (early != late) attn_column_block<NB>(p, early, kvh, split, seq);
+}
+
+// Decode steps (one token a request) with the per-head norm, the rotation and the cache write inside.
+template <bool ENABLED = (HD % 64 == 0)>
+__global__ __launch_bounds__(IA_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1, HD > 64 ? 2 : 8)))
+void attn_mfma_fused_kernel(const AttnParams p) {
+    if constexpr (ENABLED) {
+        const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
+        if ((int)blockIdx.x < (p.nq / p.nkv + 15) / 16)
+            attn_column_block<1, true>(p, (int)blockIdx.x, kvh, split, p.seq_begin + blockIdx.z);
+    }
 }
 
 // Merges the partial results of the key splits of one (token, head): one block a row.  The
@@ -416,12 +537,17 @@ extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
 // token_begin + n_tokens of its n.  max_q_len: the most tokens any of them has in this step;
 // max_kv_len: their greatest length after it; `chunk`: keys per split (a multiple of 32,
 // splits * chunk >= max_kv_len).  The workspace is sized for all n tokens.
-extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
-                                 const void* v_cache, const int* block_table, const int* cu_tokens,
-                                 const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
-                                 int n_tokens, int max_q_len, int max_kv_len, int max_pages,
-                                 int nq, int nkv, int d, int page_size, int window, float scale,
-                                 int splits, int chunk, hipStream_t stream) {
+struct FusedArgs {
+    const void* qkv; const float* q_norm_w; const float* k_norm_w; const float* cos_t; const float* sin_t;
+    const int* slots; float eps; int add_one;
+};
+
+static int attention_launch(void* out, float* workspace, const void* q, const void* k_cache,
+                            const void* v_cache, const int* block_table, const int* cu_tokens,
+                            const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
+                            int n_tokens, int max_q_len, int max_kv_len, int max_pages,
+                            int nq, int nkv, int d, int page_size, int window, float scale,
+                            int splits, int chunk, const FusedArgs* fused, hipStream_t stream) {
     IA_CHECK(d == HD, "attention_mfma: built for head_dim %d, called with %d", HD, d);
     IA_CHECK(n >= 0 && n_seqs >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0,
              "attention_mfma: bad sizes n=%d seqs=%d nq=%d nkv=%d", n, n_seqs, nq, nkv);
@@ -443,6 +569,10 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
     p.q = (const bf16_t*)q;
     p.k_cache = (const bf16_t*)k_cache;
     p.v_cache = (const bf16_t*)v_cache;
+    p.k_cache_w = (bf16_t*)k_cache;
+    p.v_cache_w = (bf16_t*)v_cache;
+    p.qkv = nullptr; p.q_norm_w = p.k_norm_w = p.cos_t = p.sin_t = nullptr; p.slots = nullptr;
+    p.norm_eps = 0.f; p.norm_add_one = 0;
     p.block_table = block_table;
     p.cu_tokens = cu_tokens;
     p.positions = positions;
@@ -457,8 +587,21 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
     const int nb = cols > 16 ? 2 : 1;
     const long long col_blocks = (cols + 16 * nb - 1) / (16 * nb);
     const dim3 grid((unsigned)(p.pair ? (col_blocks + 1) / 2 : col_blocks), nkv * splits, n_seqs);
-    if (nb == 1) attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
-    else attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
+    if (fused != nullptr) {
+        IA_CHECK(HD % 64 == 0 && max_q_len == 1, "attention_mfma: the fused form takes single tokens and head sizes in "
+                 "steps of 64 (head size %d, %d tokens a request)", HD, max_q_len);
+        p.qkv = (const bf16_t*)fused->qkv;
+        p.q_norm_w = fused->q_norm_w; p.k_norm_w = fused->k_norm_w;
+        p.cos_t = fused->cos_t; p.sin_t = fused->sin_t; p.slots = fused->slots;
+        p.norm_eps = fused->eps; p.norm_add_one = fused->add_one;
+        // 16 columns a wave, whatever the number of query heads of a key/value head
+        const dim3 fgrid((unsigned)((cols + 15) / 16), nkv * splits, n_seqs);
+        attn_mfma_fused_kernel<><<<fgrid, IA_WAVE, 0, stream>>>(p);
+    } else if (nb == 1) {
+        attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
+    } else {
+        attn_mfma_kernel<2><<<grid, IA_WAVE, 0, stream>>>(p);
+    }
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
         attn_merge_kernel<<<(unsigned)((long long)n_tokens * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>(
@@ -466,4 +609,41 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
         IA_LAUNCH_CHECK("attention_merge");
     }
     return 0;
+}
+
+extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
+                                 const void* v_cache, const int* block_table, const int* cu_tokens,
+                                 const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
+                                 int n_tokens, int max_q_len, int max_kv_len, int max_pages,
+                                 int nq, int nkv, int d, int page_size, int window, float scale,
+                                 int splits, int chunk, hipStream_t stream) {
+    return attention_launch(out, workspace, q, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
+                            n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, max_pages, nq, nkv, d, page_size,
+                            window, scale, splits, chunk, nullptr, stream);
+}
+
+// Whether this head size has the fused decode form.
+extern "C" int ia_attention_mfma_has_fused(void) { return HD % 64 == 0 ? 1 : 0; }
+
+// Decode steps, one token a request: the per-head norm of q and k (weights may be null: none), the rotation
+// by each token's angles (cos, sin [n, d / 2], whole heads, halves paired; may be null: none) and the write
+// of the new key and value at `slots` (may be null: nothing is written and the cache is only read) happen
+// inside the attention kernel.  `qkv` [n, (nq + 2 nkv) * d] is the projections' output.
+extern "C" int ia_attention_mfma_decode_fused(void* out, float* workspace, const void* qkv, void* k_cache,
+                                              void* v_cache, const int* block_table, const int* cu_tokens,
+                                              const int* positions, const int* slots, const float* q_norm_w,
+                                              const float* k_norm_w, const float* cos_t, const float* sin_t,
+                                              float eps, int add_one, int n, int seq_begin, int n_seqs,
+                                              int token_begin, int n_tokens, int max_kv_len, int max_pages,
+                                              int nq, int nkv, int d, int page_size, int window, float scale,
+                                              int splits, int chunk, hipStream_t stream) {
+    IA_CHECK(qkv != nullptr && (q_norm_w == nullptr) == (k_norm_w == nullptr) && (cos_t == nullptr) == (sin_t == nullptr),
+             "attention_mfma_decode_fused: qkv is needed; norm weights and angle tables come in pairs");
+    IA_CHECK((((uintptr_t)qkv | (uintptr_t)q_norm_w | (uintptr_t)k_norm_w | (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0,
+             "attention_mfma_decode_fused: arrays must be 16-byte aligned");
+    IA_CHECK(n_seqs == n_tokens, "attention_mfma_decode_fused: one token a request (%d requests, %d tokens)", n_seqs, n_tokens);
+    const FusedArgs fused = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, slots, eps, add_one};
+    return attention_launch(out, workspace, nullptr, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
+                            n_seqs, token_begin, n_tokens, 1, max_kv_len, max_pages, nq, nkv, d, page_size,
+                            window, scale, splits, chunk, &fused, stream);
 }

@@ -315,6 +315,73 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     return out
 
 
+def attention_decode_fused_fits(dtype: torch.dtype, d: int, page_size: int, rot: int, interleaved: bool,
+                                has_rotation: bool) -> bool:
+    """Whether decode steps can take `attention_decode_fused`: what the matrix-core kernel takes, head sizes
+    in steps of 64, and a rotation (if any) of whole heads with halves paired."""
+    return (attention_mfma_fits(dtype, d, page_size) and d % 64 == 0
+            and (not has_rotation or (rot == d and not interleaved)))
+
+
+def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
+                           cu_tokens: torch.Tensor, block_table: torch.Tensor, *, nq: int, nkv: int, d: int,
+                           slots: Optional[torch.Tensor], q_norm_w: Optional[torch.Tensor],
+                           k_norm_w: Optional[torch.Tensor], eps: float, add_one: bool,
+                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], max_kv_len: int,
+                           window: Optional[int], scale: float, splits: Optional[int] = None,
+                           seqs: Optional[Tuple[int, int]] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Decode steps (one token a request) in one kernel: per-head norm of q and k, rotation, the write
+    of the new key and value at `slots` (None: the cache is only read) and the attention over the pages.
+    `qkv` [n, (nq + 2 nkv) * d] is the projections' output; request s owns token s.  Returns [n, nq, d]."""
+    _dev(qkv, k_cache, v_cache, positions, cu_tokens, block_table, slots, q_norm_w, k_norm_w, cos, sin, out)
+    _i32(positions, "positions"); _i32(cu_tokens, "cu_tokens"); _i32(block_table, "block_table")
+    _f32(q_norm_w, "q_norm weight"); _f32(k_norm_w, "k_norm weight"); _f32(cos, "cos"); _f32(sin, "sin")
+    n = qkv.shape[0]
+    page_size = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, nkv, page_size, d, qkv.dtype, "attention_decode_fused")
+    if not attention_decode_fused_fits(qkv.dtype, d, page_size, d, False, cos is not None):
+        raise KernelError(f"attention_decode_fused: takes bfloat16, head sizes in steps of 64 and page sizes in "
+                          f"steps of 16; got {qkv.dtype}, head size {d}, page size {page_size}")
+    if qkv.dim() != 2 or qkv.shape[1] != (nq + 2 * nkv) * d or nq % nkv:
+        raise KernelError(f"attention_decode_fused: qkv has shape {tuple(qkv.shape)}, expected [n, {(nq + 2 * nkv) * d}]")
+    all_seqs = cu_tokens.numel() - 1
+    seq_begin, n_seqs = seqs if seqs is not None else (0, all_seqs)
+    if (positions.numel() != n or block_table.dim() != 2 or block_table.shape[0] < all_seqs or seq_begin < 0
+            or seq_begin + n_seqs > all_seqs or seq_begin + n_seqs > n):
+        raise KernelError("attention_decode_fused: positions, cu_tokens, block_table and the range do not fit the batch")
+    if max_kv_len > block_table.shape[1] * page_size:
+        raise KernelError(f"attention_decode_fused: max_kv_len {max_kv_len} does not fit {block_table.shape[1]} pages")
+    for w, name in ((q_norm_w, "q_norm"), (k_norm_w, "k_norm")):
+        if w is not None and w.numel() != d:
+            raise KernelError(f"attention_decode_fused: {name} weight has {w.numel()} entries, head_dim is {d}")
+    if (q_norm_w is None) != (k_norm_w is None) or (cos is None) != (sin is None):
+        raise KernelError("attention_decode_fused: norm weights and angle tables come in pairs")
+    if cos is not None and (cos.shape != (n, d // 2) or sin.shape != cos.shape):
+        raise KernelError(f"attention_decode_fused: rotary tables must be [{n}, {d // 2}]")
+    if slots is not None:
+        _i32(slots, "slots")
+        if slots.numel() != n:
+            raise KernelError(f"attention_decode_fused: {slots.numel()} slots for {n} tokens")
+    if out is None:
+        out = torch.empty((n, nq, d), dtype=qkv.dtype, device=qkv.device)
+    elif tuple(out.shape) != (n, nq, d) or out.dtype != qkv.dtype:
+        raise KernelError("attention_decode_fused: `out` must be [n, nq, d] in the dtype of qkv")
+    if splits is None:
+        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, 1, max_kv_len)
+    else:
+        chunk = -(-(-(-max_kv_len // splits)) // 32) * 32
+    target = _build.attn_target(d)
+    lib = library(target)
+    ws_floats = lib.ia_attention_mfma_workspace(n, nq, splits)
+    ws = torch.empty((ws_floats,), dtype=torch.float32, device=qkv.device) if ws_floats else None
+    _check(lib.ia_attention_mfma_decode_fused(
+        _p(out), _p(ws), _p(qkv), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions), _p(slots),
+        _p(q_norm_w), _p(k_norm_w), _p(cos), _p(sin), ctypes.c_float(eps), int(add_one), n, seq_begin, n_seqs,
+        seq_begin, n_seqs, max_kv_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
+        ctypes.c_float(scale), splits, chunk, _stream()), target)
+    return out
+
+
 # ---- matrix products --------------------------------------------------------------------------
 
 SKINNY_MAX_ROWS = 16          # beyond this the vendor's GEMM reads the weights faster

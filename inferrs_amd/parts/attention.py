@@ -70,6 +70,16 @@ class Attention(Mixer):
         qkv = self.qkv(h)
         table = ctx.position_table(self.position)
         cos, sin = table if table is not None else (None, None)
+        if ctx.max_q_len == 1 and ops.attention_decode_fused_fits(qkv.dtype, s.head_dim, group.page_size,
+                                                                   self.position.rot_dim, self.position.interleaved,
+                                                                   cos is not None):
+            # decode steps: norm, rotation, cache write and attention in one kernel
+            a = ops.attention_decode_fused(
+                qkv, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table, nq=s.n_heads,
+                nkv=s.n_kv_heads, d=s.head_dim, slots=group.slots if cache.writable else None,
+                q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one,
+                cos=cos, sin=sin, max_kv_len=ctx.max_kv_len, window=s.window, scale=s.softmax_scale)
+            return self.o(a.view(a.shape[0], s.n_heads * s.head_dim))
         q = ops.qk_rope_kv(
             qkv, s.n_heads, s.n_kv_heads, s.head_dim,
             q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one,

@@ -342,3 +342,50 @@ def test_fill_normal_equals_the_host_fill(dtype):
     z = (ops.fill_normal((n,), 7, 0.0, 1.0, torch.float32, "cuda").cpu()).double()
     assert abs(float(z.mean())) < 0.01 and abs(float(z.std()) - 1.0) < 0.01
     assert abs(float((z ** 4).mean()) - 3.0) < 0.1                      # the fourth moment of a normal
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,window", [
+    (32, 8, 128, 16, None), (4, 2, 64, 16, None), (40, 2, 64, 32, None), (6, 3, 192, 16, 37), (2, 1, 256, 48, None)])
+@pytest.mark.parametrize("norm,rope,write", [(True, True, True), (False, True, True), (True, False, True), (True, True, False)])
+def test_attention_decode_fused_is_the_three_kernels_in_one(nq, nkv, d, page, window, norm, rope, write):
+    """Decode steps: per-head norm, rotation, cache write and attention in one kernel against the separate
+    kernels (the same arithmetic but for the order of the norm's sum of squares): the results agree to
+    the rounding of bfloat16, and the cache holds the same new keys and values."""
+    from inferrs_amd import ops
+    dtype = torch.bfloat16
+    lens = [300, 17, 1000, 33, 64, 1]                       # lengths after the step; the last token of each is this step's
+    q, kc, vc, positions, token_seq, table = attention_case(dtype, nq, nkv, d, page, lens, [1] * len(lens), 23)
+    n = len(lens)
+    qkv = randn(n, (nq + 2 * nkv) * d, dtype=dtype, seed=5)
+    qw = (1 + 0.3 * randn(d, dtype=torch.float32, seed=6)) if norm else None
+    kw = (1 + 0.3 * randn(d, dtype=torch.float32, seed=7)) if norm else None
+    cos = sin = None
+    if rope:
+        inv = 1.0 / (10000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        ang = positions.float()[:, None] * inv[None, :]
+        cos, sin = torch.cos(ang), torch.sin(ang)
+    slots = torch.tensor([int(table[s, (l - 1) // page]) * page + (l - 1) % page for s, l in enumerate(lens)], dtype=torch.int32)
+    cu = torch.arange(n + 1, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    dv = lambda t: None if t is None else dev(t)
+    # the separate kernels
+    k1, v1 = dev(kc), dev(vc)
+    q1 = ops.qk_rope_kv(dev(qkv), nq, nkv, d, q_norm_w=dv(qw), k_norm_w=dv(kw), eps=1e-5, add_one=False, cos=dv(cos),
+                        sin=dv(sin), rot=d if rope else 0, interleaved=False, k_cache=k1, v_cache=v1,
+                        slots=dev(slots) if write else None, page_size=page)
+    for splits in (None, 1, 4):
+        want = ops.attention_mfma(q1, k1, v1, dev(positions), dev(cu), dev(table), max_q_len=1, max_kv_len=max(lens),
+                                  window=window, scale=scale, splits=splits).float().cpu()
+        k2, v2 = dev(kc), dev(vc)
+        if not write:                                       # a layer that reads another's cache: the new key is there already
+            k2.copy_(k1); v2.copy_(v1)
+        got = ops.attention_decode_fused(dev(qkv), k2, v2, dev(positions), dev(cu), dev(table), nq=nq, nkv=nkv, d=d,
+                                         slots=dev(slots) if write else None, q_norm_w=dv(qw), k_norm_w=dv(kw), eps=1e-5,
+                                         add_one=False, cos=dv(cos), sin=dv(sin), max_kv_len=max(lens), window=window,
+                                         scale=scale, splits=splits).float().cpu()
+        close(got, want, 2 ** -7, f"fused splits={splits}")
+        if write:
+            assert torch.equal(v2, v1)
+            # keys: the same but for a last bit here and there (the sum of squares is added up in another order)
+            dk = (k2.float() - k1.float()).abs()
+            assert float(dk.max()) <= 2 ** -7 * float(k1.float().abs().max()) and float((dk > 0).float().mean()) < 1e-3
