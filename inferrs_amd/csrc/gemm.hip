@@ -114,7 +114,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // two rows a load), puts it into its own corner of shared memory and reads the operand layout from
 // there.  Measured on the logits head at 8 rows: 4.8 -> 5.9 TB/s.
 #define SK_STAGE_PAD 16     // bytes between staged rows, against bank conflicts
-template <int MT, int RT, bool DUAL, bool STAGE>
+// STAGE: 0, or the k steps of a staged chunk (8 or 16).
+template <int MT, int RT, bool DUAL, int STAGE>
 __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     void* __restrict__ out, int out_f32, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     int M, int N, int K, int kper, int m_base, int rot_mul) {
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     // A chunk of k steps has all its loads under way before its first product: a wave is one of
     // few on its SIMD when the weight is small, and what it has in flight is what hides the memory's
     // latency.
-    constexpr int UNROLL = STAGE ? 8 : (NA * RT * MT >= 8) ? 2 : (NA * RT * MT >= 4 ? 4 : (NA * RT * MT == 2 ? 8 : 16));
+    constexpr int UNROLL = STAGE ? STAGE : (NA * RT * MT >= 8) ? 2 : (NA * RT * MT >= 4 ? 4 : (NA * RT * MT == 2 ? 8 : 16));
     constexpr int STAGE_PITCH = UNROLL * 2 * SK_KSTEP + SK_STAGE_PAD;      // bytes of a staged row
     constexpr int STAGE_LANES = UNROLL * 4;                               // lanes that bring one row
     const int stage_rows = M - m_base < 16 ? M - m_base : 16;
@@ -370,6 +371,7 @@ static int skinny_waves(int N, int K, int rt, int tiles_per_wave) {
 }
 
 #define SK_STAGE_LDS_MOST (96 * 1024)
+#define SK_STAGE16_LDS_MOST (160 * 1024)     // one block a compute unit: all of its shared memory
 
 template <int MT, int RT, bool DUAL>
 static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* w, int M, int N, int K,
@@ -383,12 +385,13 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
     if constexpr (MT == 1) {
         const int rows = M - m_base < 16 ? M - m_base : 16;
         const size_t staged = tiles + (size_t)waves * rows * (8 * 2 * SK_KSTEP + SK_STAGE_PAD);
+        const size_t staged16 = tiles + (size_t)waves * rows * (16 * 2 * SK_KSTEP + SK_STAGE_PAD);
         // Staging pays where blocks stream for long: with at least two blocks for every compute unit
         // (a weight that one round of blocks covers is read in one burst, and what counts there is
         // how much a wave has in flight), with 2 to 12 batch rows (one row is one cache line a load
         // anyway; beyond 12 the staging area leaves too few blocks on a compute unit), and with whole
         // chunks of 8 k steps in a wave's range.  Measured at 8 rows: gate|up 46 -> 40 us, logits head
-        // 261 -> 224 us; down and o (one round of blocks) are better off without.
+        // 261 -> 224 us.
         static int cus = 0;
         if (cus == 0) {
             int dev = 0;
@@ -399,18 +402,37 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
         if (g_stage && rows >= 2 && rows <= 12 && (int)grid >= 2 * cus && kper >= 8 && staged <= SK_STAGE_LDS_MOST) {
             static bool raised = false;       // per instantiation: shared memory beyond 64 KiB has to be asked for
             if (!raised) {
-                const hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, RT, DUAL, true>,
+                const hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, RT, DUAL, 8>,
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, SK_STAGE_LDS_MOST);
                 IA_CHECK(e == hipSuccess, "gemm_skinny: cannot ask for %d bytes of shared memory: %s",
                          SK_STAGE_LDS_MOST, hipGetErrorString(e));
                 raised = true;
             }
-            gemm_skinny_kernel<MT, RT, DUAL, true><<<grid, waves * IA_WAVE, staged, stream>>>(
+            gemm_skinny_kernel<MT, RT, DUAL, 8><<<grid, waves * IA_WAVE, staged, stream>>>(
                 out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
             return 0;
         }
+        if constexpr (!DUAL && RT == 1) {
+            // A weight that one round of blocks covers (o, down, qkv): chunks of 16 steps, so that a wave has
+            // as much in flight as without staging, and all of a compute unit's shared memory for its one
+            // block.  Measured at 8 rows: down 25.6 -> 22.3 us, o 11.5 -> 9.9, qkv 16.8 -> 14.2; at 16 rows
+            // 30.4 -> 24.5, 12.9 -> 10.6, 19.1 -> 16.8.
+            if (g_stage && rows >= 2 && (int)grid < 2 * cus && kper % 16 == 0 && staged16 <= SK_STAGE16_LDS_MOST) {
+                static bool raised16 = false;
+                if (!raised16) {
+                    const hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, RT, DUAL, 16>,
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, SK_STAGE16_LDS_MOST);
+                    IA_CHECK(e == hipSuccess, "gemm_skinny: cannot ask for %d bytes of shared memory: %s",
+                             SK_STAGE16_LDS_MOST, hipGetErrorString(e));
+                    raised16 = true;
+                }
+                gemm_skinny_kernel<MT, RT, DUAL, 16><<<grid, waves * IA_WAVE, staged16, stream>>>(
+                    out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
+                return 0;
+            }
+        }
     }
-    gemm_skinny_kernel<MT, RT, DUAL, false><<<grid, waves * IA_WAVE, waves > 1 ? tiles : 0, stream>>>(
+    gemm_skinny_kernel<MT, RT, DUAL, 0><<<grid, waves * IA_WAVE, waves > 1 ? tiles : 0, stream>>>(
         out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
     return 0;
 }

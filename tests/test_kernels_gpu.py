@@ -297,6 +297,20 @@ def test_skinny_rows_do_not_depend_on_the_batch():
     assert torch.equal(ops.gemm_skinny_bf16(dev(x[3:9].contiguous()), dev(w), torch.float32).cpu(), full[3:9])
 
 
+def test_skinny_variants_for_one_round_weights_agree_bit_for_bit():
+    # a weight of fewer than two blocks a compute unit whose waves take whole chunks of 16 k steps: staged at 2
+    # rows and more, plain at one row
+    from inferrs_amd import ops
+    n, k = 4096, 4096
+    x = randn(16, k, dtype=torch.bfloat16, seed=1)
+    w = randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    full = ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32).cpu()
+    close(full, x.double() @ w.double().t(), 2e-5, "one round")
+    for lo, hi in ((0, 1), (7, 8), (3, 9), (0, 12), (2, 15)):
+        part = ops.gemm_skinny_bf16(dev(x[lo:hi].contiguous()), dev(w), torch.float32).cpu()
+        assert torch.equal(part, full[lo:hi]), (lo, hi)
+
+
 @pytest.mark.parametrize("dual", [False, True])
 def test_skinny_variants_for_tall_weights_agree_bit_for_bit(dual):
     # a weight with more than two blocks a compute unit takes the variant that stages the activations
