@@ -147,6 +147,56 @@ def test_qk_rope_kv(dtype, nq, nkv, d, rot, interleaved, normed):
     assert torch.equal(vc_d.cpu().float(), want_v.to(dtype).float()), "values are copied as they are"
 
 
+@pytest.mark.parametrize("nq,nkv,d,page", [(8, 2, 128, 16), (3, 3, 64, 8), (2, 1, 256, 16), (5, 5, 48, 24),
+                                            (4, 4, 128, 4)])
+@pytest.mark.parametrize("layout", ["aligned", "shifted", "two requests", "shuffled"])
+def test_qk_rope_kv_values_of_a_prompt_portion(nq, nkv, d, page, layout):
+    """Steps with prompt portions write the values eight tokens at a time where their slots are
+    neighbours in a page; every arrangement of the slots must end in the same cache."""
+    from inferrs_amd import ops
+    dtype, n, pages = torch.bfloat16, 43, 24
+    g = torch.Generator().manual_seed(21)
+    if layout == "aligned":
+        slots = torch.arange(n) + 2 * page
+    elif layout == "shifted":
+        slots = torch.arange(n) + page + 3
+    elif layout == "two requests":        # 19 tokens of one request, 24 of another, pages apart
+        first_free = (page + 24 + page - 1) // page * page
+        slots = torch.cat([torch.arange(19) + first_free + page + 5, torch.arange(24) + page])
+    else:
+        slots = torch.randperm(pages * page, generator=g)[:n]
+    slots = slots.to(torch.int32)
+    assert int(slots.max()) < pages * page and len(set(slots.tolist())) == n
+    qkv = randn(n, (nq + 2 * nkv) * d, dtype=dtype, seed=22, scale=2.0)
+    qw, kw = randn(d, dtype=torch.float32, seed=23), randn(d, dtype=torch.float32, seed=24)
+    cos, sin = torch.rand(n, d // 2, generator=g), torch.rand(n, d // 2, generator=g)
+    kc = torch.full((pages, nkv, page, d), 7.0, dtype=dtype)
+    vc = torch.full((pages, nkv, d, page), 7.0, dtype=dtype)
+    kc_d, vc_d = dev(kc), dev(vc)
+    q = ops.qk_rope_kv(dev(qkv), nq, nkv, d, q_norm_w=dev(qw), k_norm_w=dev(kw), eps=1e-6, add_one=False,
+                       cos=dev(cos), sin=dev(sin), rot=d, interleaved=False, k_cache=kc_d, v_cache=vc_d,
+                       slots=dev(slots), page_size=page)
+    rq, rk, rv = ref_qk_rope(qkv, nq, nkv, d, qw, kw, 1e-6, False, cos, sin, d, False)
+    close(q, rq, tol(dtype, 3e-6), "q")
+    want_k, want_v = kc.float().clone(), vc.float().clone()
+    for t in range(n):
+        s = int(slots[t])
+        want_k[s // page, :, s % page] = rk[t]
+        want_v[s // page, :, :, s % page] = rv[t]
+    close(kc_d, want_k, tol(dtype, 3e-6), "k cache")
+    assert torch.equal(vc_d.cpu().float(), want_v.to(dtype).float()), "values are copied as they are"
+    # the kernel that decode steps use (a thread a head, values token by token) gives the same bits
+    kc_1, vc_1 = dev(kc), dev(vc)
+    ops.library().ia_qk_rope_kv_tune(0, 0)
+    try:
+        q_1 = ops.qk_rope_kv(dev(qkv), nq, nkv, d, q_norm_w=dev(qw), k_norm_w=dev(kw), eps=1e-6, add_one=False,
+                             cos=dev(cos), sin=dev(sin), rot=d, interleaved=False, k_cache=kc_1, v_cache=vc_1,
+                             slots=dev(slots), page_size=page)
+    finally:
+        ops.library().ia_qk_rope_kv_tune(1, 1)
+    assert torch.equal(q, q_1) and torch.equal(kc_d, kc_1) and torch.equal(vc_d, vc_1)
+
+
 def ref_attention(q, kc, vc, positions, token_seq, table, window, scale):
     n, nq, d = q.shape
     nkv, page = kc.shape[1], kc.shape[2]
