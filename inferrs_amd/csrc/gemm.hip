@@ -373,6 +373,19 @@ static int skinny_waves(int N, int K, int rt, int tiles_per_wave) {
 #define SK_STAGE_LDS_MOST (96 * 1024)
 #define SK_STAGE16_LDS_MOST (160 * 1024)     // one block a compute unit: all of its shared memory
 
+// Shared memory beyond 64 KiB has to be asked for, once per instantiation.
+template <int MT, int RT, bool DUAL, int STAGE>
+static int skinny_ask_shared(int bytes) {
+    static bool asked = false;
+    if (!asked) {
+        const hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, RT, DUAL, STAGE>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        IA_CHECK(e == hipSuccess, "gemm_skinny: cannot ask for %d bytes of shared memory: %s", bytes, hipGetErrorString(e));
+        asked = true;
+    }
+    return 0;
+}
+
 template <int MT, int RT, bool DUAL>
 static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* w, int M, int N, int K,
                          int m_base, hipStream_t stream) {
@@ -384,14 +397,8 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
     const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
     if constexpr (MT == 1) {
         const int rows = M - m_base < 16 ? M - m_base : 16;
-        const size_t staged = tiles + (size_t)waves * rows * (8 * 2 * SK_KSTEP + SK_STAGE_PAD);
+        const size_t staged8 = tiles + (size_t)waves * rows * (8 * 2 * SK_KSTEP + SK_STAGE_PAD);
         const size_t staged16 = tiles + (size_t)waves * rows * (16 * 2 * SK_KSTEP + SK_STAGE_PAD);
-        // Staging pays where blocks stream for long: with at least two blocks for every compute unit
-        // (a weight that one round of blocks covers is read in one burst, and what counts there is
-        // how much a wave has in flight), with 2 to 12 batch rows (one row is one cache line a load
-        // anyway; beyond 12 the staging area leaves too few blocks on a compute unit), and with whole
-        // chunks of 8 k steps in a wave's range.  Measured at 8 rows: gate|up 46 -> 40 us, logits head
-        // 261 -> 224 us.
         static int cus = 0;
         if (cus == 0) {
             int dev = 0;
@@ -399,33 +406,32 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
                 hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
                 cus = 256;
         }
-        if (g_stage && rows >= 2 && rows <= 12 && (int)grid >= 2 * cus && kper >= 8 && staged <= SK_STAGE_LDS_MOST) {
-            static bool raised = false;       // per instantiation: shared memory beyond 64 KiB has to be asked for
-            if (!raised) {
-                const hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, RT, DUAL, 8>,
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, SK_STAGE_LDS_MOST);
-                IA_CHECK(e == hipSuccess, "gemm_skinny: cannot ask for %d bytes of shared memory: %s",
-                         SK_STAGE_LDS_MOST, hipGetErrorString(e));
-                raised = true;
-            }
-            gemm_skinny_kernel<MT, RT, DUAL, 8><<<grid, waves * IA_WAVE, staged, stream>>>(
+        int stage = 0;
+        if (g_stage && rows >= 2 && (int)grid >= 2 * cus) {
+            // Staging pays where blocks stream for long: with at least two blocks for every compute unit,
+            // with 2 to 12 batch rows (one row is one cache line a load anyway; beyond 12 the staging area
+            // leaves too few blocks on a compute unit), and with whole chunks of 8 k steps in a wave's
+            // range.  Measured at 8 rows: gate|up 46 -> 40 us, logits head 261 -> 224 us.
+            if (rows <= 12 && kper >= 8 && staged8 <= SK_STAGE_LDS_MOST) stage = 8;
+        } else if (g_stage && rows >= 2 && !DUAL && RT == 1) {
+            // A weight that one round of blocks covers (o, down, qkv) is read in one burst, and what counts
+            // is how much a wave has in flight: chunks of 16 steps, as much as without staging, and up to
+            // all of a compute unit's shared memory for its block.  Measured at 8 rows: down 25.6 -> 22.3 us,
+            // o 11.5 -> 9.9, qkv 16.8 -> 14.2; at 16 rows 30.4 -> 24.5, 12.9 -> 10.6, 19.1 -> 16.8.  (From 9 rows on
+            // the area leaves room for one block of qkv's 384 on a compute unit, and they go in two rounds;
+            // chunks of 8, which keep it one round, were no faster: 15.8 against 16.4 us at 10 rows, 17.4
+            // against 16.7 at 16.)
+            if (kper % 16 == 0 && staged16 <= SK_STAGE16_LDS_MOST) stage = 16;
+        }
+        if (stage == 8) {
+            if (skinny_ask_shared<MT, RT, DUAL, 8>(SK_STAGE_LDS_MOST)) return 1;
+            gemm_skinny_kernel<MT, RT, DUAL, 8><<<grid, waves * IA_WAVE, staged8, stream>>>(
                 out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
             return 0;
         }
         if constexpr (!DUAL && RT == 1) {
-            // A weight that one round of blocks covers (o, down, qkv): chunks of 16 steps, so that a wave has
-            // as much in flight as without staging, and all of a compute unit's shared memory for its one
-            // block.  Measured at 8 rows: down 25.6 -> 22.3 us, o 11.5 -> 9.9, qkv 16.8 -> 14.2; at 16 rows
-            // 30.4 -> 24.5, 12.9 -> 10.6, 19.1 -> 16.8.
-            if (g_stage && rows >= 2 && (int)grid < 2 * cus && kper % 16 == 0 && staged16 <= SK_STAGE16_LDS_MOST) {
-                static bool raised16 = false;
-                if (!raised16) {
-                    const hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, RT, DUAL, 16>,
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, SK_STAGE16_LDS_MOST);
-                    IA_CHECK(e == hipSuccess, "gemm_skinny: cannot ask for %d bytes of shared memory: %s",
-                             SK_STAGE16_LDS_MOST, hipGetErrorString(e));
-                    raised16 = true;
-                }
+            if (stage == 16) {
+                if (skinny_ask_shared<MT, RT, DUAL, 16>(SK_STAGE16_LDS_MOST)) return 1;
                 gemm_skinny_kernel<MT, RT, DUAL, 16><<<grid, waves * IA_WAVE, staged16, stream>>>(
                     out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
                 return 0;

@@ -384,7 +384,12 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 
 # ---- matrix products --------------------------------------------------------------------------
 
-SKINNY_MAX_ROWS = 16          # beyond this the vendor's GEMM reads the weights faster
+# Beyond this many rows the vendor's GEMM reads the weights faster.  Measured at the sizes of an 8 B model
+# (us: qkv, o, gate|up with SiLU, down, logits head): 12 rows 16.2, 10.2, 41.5, 23.7, 233 here against 14.8,
+# 12.5, 46.3, 21.5, 260 there (92 against 95 a layer); 14 rows 17.3, 10.6, 48.4, 24.7, 286 against 14.7, 12.5,
+# 46.7, 21.6, 261 (101 against 95): past 12 rows the staging area of the activations no longer fits beside
+# enough blocks on a compute unit.
+SKINNY_MAX_ROWS = 12
 
 
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -443,9 +448,9 @@ def widen(x: torch.Tensor) -> torch.Tensor:
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
-    skinny MFMA kernel for up to 16 rows, the vendor's GEMM beyond that (the reference uses
+    skinny MFMA kernel for up to SKINNY_MAX_ROWS rows, the vendor's GEMM beyond that (the reference uses
     cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
-    the skinny kernel's accumulators for up to 16 rows; beyond that it is the vendor's bfloat16
+    the skinny kernel's accumulators for those few rows; beyond that it is the vendor's bfloat16
     result widened, which is what the reference does for every row (its logits are computed in
     the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`)."""
     out_dtype = out_dtype or x.dtype

@@ -313,7 +313,7 @@ def test_gemm_tiled_float32_is_true_32_bit(m, n, k):
     assert torch.equal(ops.linear(dev(x[:1]), dev(w)).cpu(), ops.linear(dev(x), dev(w)).cpu()[:1])
 
 
-@pytest.mark.parametrize("m", [1, 2, 8, 16, 17, 33, 64, 65, 200])
+@pytest.mark.parametrize("m", [1, 2, 8, 12, 13, 16, 17, 33, 64, 65, 200])
 @pytest.mark.parametrize("n,k", [(130, 40), (515, 136), (4096, 4096), (1000, 12288), (16, 8)])
 @pytest.mark.parametrize("out_dtype", DTYPES)
 def test_linear_bfloat16(m, n, k, out_dtype):
@@ -322,8 +322,8 @@ def test_linear_bfloat16(m, n, k, out_dtype):
     want = x.double() @ w.double().t()
     got = ops.linear(dev(x), dev(w), out_dtype)
     assert got.dtype == out_dtype
-    # beyond 16 rows a 32-bit result is the bfloat16 one widened
-    close(got, want, tol(out_dtype, 2e-5) if m <= 16 else 2 ** -8, f"linear {m}x{n}x{k}")
+    # beyond the skinny kernel's rows a 32-bit result is the vendor's bfloat16 one widened
+    close(got, want, tol(out_dtype, 2e-5) if m <= ops.SKINNY_MAX_ROWS else 2 ** -8, f"linear {m}x{n}x{k}")
 
 
 @pytest.mark.parametrize("m", [1, 8, 17, 40, 64])
