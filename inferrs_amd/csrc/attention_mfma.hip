@@ -51,7 +51,7 @@ struct AttnParams {
     const int* block_table;     // [seqs, max_pages]
     const int* cu_tokens;       // [seqs + 1]  request s owns tokens cu[s]..cu[s+1]
     const int* positions;       // [n]         absolute position of each token
-    int max_pages, nq, nkv, page, window, splits, chunk, pair, seq_begin;
+    int max_pages, nq, nkv, page, window, splits, chunk, pair, seq_begin;   // pair: see the kernels
     float scale_log2;           // scale * log2(e)
     // Decode steps with the per-head norm, the rotation and the cache write inside (FUSE): q is not
     // read from `q` but formed from the projections' output, and the wave that walks a request's
@@ -457,6 +457,279 @@ void attn_mfma_fused_kernel(const AttnParams p) {
     }
 }
 
+// ---- prompt portions, head size 128: blocks of four waves that share keys and values ----------
+// A block owns 128 columns of one request and key/value head (32 columns a wave) and walks the keys in
+// stages of 64.  A stage's keys and values come from the cache pages straight into shared memory
+// (global_load_lds, 16 bytes a lane: no register holds them on the way), the next stage while this
+// one is multiplied, and every wave reads its MFMA operands from there: the L2 is asked for a key once
+// a block instead of once a wave.  A load instruction fills 1 KiB of shared memory in lane order, so
+// the lane picks the piece it fetches such that the layout comes out swizzled:
+//   keys    row of 256 bytes a key, the 16-byte piece c of key k at place c ^ ((k & 3) | ((k >> 3) & 3) << 2)
+//   values  row of 128 bytes a feature (64 keys), the piece c of feature f at place c ^ ((f >> 1) & 7)
+// and the 16 lanes that read an operand together (16 rows, the same piece) hit 16 different banks.
+#define TILE_WAVES 4
+#define TILE_COLS (TILE_WAVES * 32)
+#define TILE_STAGE 64
+#define TILE_K_BYTES (TILE_STAGE * HD * 2)
+#define TILE_BUF_BYTES (2 * TILE_K_BYTES)
+
+template <bool ENABLED = (HD == 128)>
+__global__ __launch_bounds__(TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attn_tile_kernel(const AttnParams p) {
+    if constexpr (ENABLED) {
+        // Two stages, as two arrays: the compiler then knows that the loads on their way into one do not
+        // touch the other, and does not wait for them before it reads an operand.
+        __shared__ __align__(16) char stage_a[TILE_BUF_BYTES];
+        __shared__ __align__(16) char stage_b[TILE_BUF_BYTES];
+        const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+        const int r = lane & 15, G = lane >> 4;
+        const int kvh = blockIdx.y, seq = p.seq_begin + blockIdx.z;
+        const int g = p.nq / p.nkv;
+        const int t0 = p.cu_tokens[seq], q_len = p.cu_tokens[seq + 1] - t0;
+        const int n_cols = q_len * g;
+        const int n_tiles = (n_cols + TILE_COLS - 1) / TILE_COLS;
+        if ((int)blockIdx.x >= n_tiles) return;
+        // Long walks first.  When all blocks fit on the chip at once (two a compute unit), the second half
+        // of them, which joins the first half on its compute units, brings short walks first: a compute
+        // unit's two blocks then end together (one prompt of 2,048 tokens: 103 -> 88 us).
+        const unsigned linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const bool second = p.pair > 0 && ((linear / (unsigned)p.pair) & 1u) != 0;
+        const int bcol0 = (second ? (int)blockIdx.x : n_tiles - 1 - (int)blockIdx.x) * TILE_COLS;
+        const int kv_start = p.positions[t0];
+        const int kv_total = kv_start + q_len;
+        const int* bt = p.block_table + (size_t)seq * p.max_pages;
+        const int blast = (bcol0 + TILE_COLS <= n_cols ? bcol0 + TILE_COLS : n_cols) - 1;
+        const int bpmin = kv_start + bcol0 / g, bpmax = kv_start + blast / g;
+        int lo = p.window > 0 ? (bpmin - p.window + 1 > 0 ? bpmin - p.window + 1 : 0) : 0;
+        lo &= ~(TILE_STAGE - 1);
+        const int stages = (bpmax + 1 - lo + TILE_STAGE - 1) / TILE_STAGE;
+
+        // this wave's columns (a wave without any still brings its share of the stages)
+        const int col0 = bcol0 + wave * 32;
+        const bool has_cols = col0 < n_cols;
+        int tq[2], head[2], pos[2];
+        bool cvalid[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const int c = col0 + nb * 16 + r;
+            cvalid[nb] = c < n_cols;
+            const int cc = cvalid[nb] ? c : n_cols - 1;
+            tq[nb] = cc / g;
+            head[nb] = kvh * g + (cc - tq[nb] * g);
+            pos[nb] = kv_start + tq[nb];
+        }
+        const int wlast = (col0 + 32 <= n_cols ? col0 + 32 : n_cols) - 1;
+        const int pmin = kv_start + (has_cols ? col0 : 0) / g, pmax = has_cols ? kv_start + wlast / g : -1;
+        const int wlo = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;
+
+        uint4 qreg[2][KS];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) qreg[nb][ks] = cvalid[nb] ? *(const uint4*)(qrow + ks * 32 + G * 8) : zero4();
+        }
+        f32x4 acc[2][DB];
+        float m[2], l[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            m[nb] = -INFINITY;
+            l[nb] = 0.f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+
+        // ---- a stage on its way: wave w brings keys 16 w .. + 16 and features 32 w .. + 32 ----------
+        // Groups of 16 keys past the request's length are read from the group of its last key instead
+        // (their scores are masked and their values zeroed below): the pages behind may not exist.
+        // Lane j looks up the page of the stage's j-th group of 16 keys (j < 4; the other lanes repeat them) a
+        // stage ahead of its use, so that nobody waits for the block table.
+        auto pages_for = [&](int s, int& page, int& off) {
+            const int key0 = lo + s * TILE_STAGE + 16 * (lane & 3);
+            const int k = key0 < kv_total ? key0 : (kv_total - 1) & ~15;
+            const int idx = k / p.page;
+            page = bt[idx];
+            off = k - idx * p.page;
+        };
+        auto issue = [&](char* buf, int page_l, int off_l) {
+            {
+                const int page = __shfl(page_l, wave, IA_WAVE), off = __shfl(off_l, wave, IA_WAVE);
+                const char* krows = (const char*)(p.k_cache + (((size_t)page * p.nkv + kvh) * p.page + off) * HD);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int row = 4 * c + (lane >> 4), key = 16 * wave + row;
+                    const int piece = (lane & 15) ^ ((key & 3) | (((key >> 3) & 3) << 2));
+                    __builtin_amdgcn_global_load_lds(
+                        (const void __attribute__((address_space(1)))*)(krows + row * (HD * 2) + piece * 16),
+                        (void __attribute__((address_space(3)))*)(buf + (16 * wave + 4 * c) * (HD * 2)), 16, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int f = 32 * wave + 8 * c + (lane >> 3);
+                const int piece = (lane & 7) ^ ((f >> 1) & 7);
+                const int page = __shfl(page_l, piece >> 1, IA_WAVE), off = __shfl(off_l, piece >> 1, IA_WAVE);
+                const char* src = (const char*)(p.v_cache + (((size_t)page * p.nkv + kvh) * HD + f) * p.page + off + (piece & 1) * 8);
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)src,
+                    (void __attribute__((address_space(3)))*)(buf + TILE_K_BYTES + (32 * wave + 8 * c) * (TILE_STAGE * 2)),
+                    16, 0, 0);
+            }
+        };
+        // values of keys past the request's length may hold anything at all: a lane zeroes them in the
+        // pieces that it brought itself, once they have arrived
+        auto zero_tail = [&](int s, char* buf) {
+            const int kb = lo + s * TILE_STAGE;
+            if (kb + TILE_STAGE <= kv_total) return;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int f = 32 * wave + 8 * c + (lane >> 3);
+                const int piece = (lane & 7) ^ ((f >> 1) & 7);
+                const int first_bad = kv_total - (kb + 8 * piece);
+                if (first_bad >= 8) continue;
+                uint4* at = (uint4*)(buf + TILE_K_BYTES + (32 * wave + 8 * c) * (TILE_STAGE * 2) + lane * 16);
+                const uint4 v = *at;
+                uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j >= first_bad) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                *at = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        };
+
+        // this lane's places in a stage: they do not change from stage to stage
+        uint32_t k_at[2][2];            // [step of 32 keys][tile t]: the row's start and what the pieces are xor-ed with
+        uint32_t k_xor;
+        {
+            const int kl = 8 * (r >> 2) + (r & 3);
+            k_xor = (uint32_t)((kl & 3) | (((kl >> 3) & 3) << 2));
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) k_at[u][t] = (uint32_t)((32 * u + kl + 4 * t) * (HD * 2));
+        }
+
+        int page_l, off_l;
+        auto stage = [&](int s, char* buf, char* other) {
+            __builtin_amdgcn_s_waitcnt(0);                 // this wave's part of stage s has arrived
+            zero_tail(s, buf);
+            __syncthreads();                               // everybody's has, and everybody is done with stage s - 1
+            if (s + 1 < stages) {
+                issue(other, page_l, off_l);
+                if (s + 2 < stages) pages_for(s + 2, page_l, off_l);
+            }
+            const int kb = lo + s * TILE_STAGE;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int k0 = kb + 32 * u;
+                if (k0 > pmax || k0 + 31 < wlo) continue;  // nothing of this step is visible to this wave's columns
+                const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
+                uint4 kop[2][KS];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        kop[t][ks] = *(const uint4*)(buf + k_at[u][t] + (((uint32_t)(ks * 4 + G) ^ k_xor) * 16));
+                uint4 pb[2];
+                float alpha[2];
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    f32x4 sacc[2];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks)
+                            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                __builtin_bit_cast(bf16x8, kop[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), sacc[t], 0, 0, 0);
+                    }
+                    float sc[8];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sc[4 * t + i] = sacc[t][i];
+                    if (edge) {
+                        const int kbase_idx = k0 + 8 * G;
+                        const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const int key = kbase_idx + j;
+                            if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
+                        }
+                    }
+                    float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, IA_WAVE));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, IA_WAVE));
+                    // The exponents' reference point moves only when the step's maximum has passed it by 2^8
+                    // (probabilities then reach 2^8 at most, which 32-bit sums and bfloat16 operands hold as
+                    // well as 1): the accumulators are rescaled a few times a walk instead of at most steps.
+                    const float cand = mx * p.scale_log2;
+                    const bool rise = cand > m[nb] + 8.0f;              // also the first finite maximum after -inf
+                    const float m_new = rise ? cand : m[nb];
+                    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                    alpha[nb] = rise ? __builtin_amdgcn_exp2f(m[nb] - m_use) : 1.0f;
+                    float pr[8], psum = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], p.scale_log2, -m_use));
+                        psum += pr[j];
+                    }
+                    l[nb] = l[nb] * alpha[nb] + psum;
+                    m[nb] = m_new;
+                    pb[nb].x = pack_bf16x2(pr[0], pr[1]);
+                    pb[nb].y = pack_bf16x2(pr[2], pr[3]);
+                    pb[nb].z = pack_bf16x2(pr[4], pr[5]);
+                    pb[nb].w = pack_bf16x2(pr[6], pr[7]);
+                    if (__any(alpha[nb] != 1.0f)) {
+#pragma unroll
+                        for (int db = 0; db < DB; ++db) {
+                            acc[nb][db][0] *= alpha[nb]; acc[nb][db][1] *= alpha[nb];
+                            acc[nb][db][2] *= alpha[nb]; acc[nb][db][3] *= alpha[nb];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const int f = 16 * db + r;
+                    const uint4 vop = *(const uint4*)(buf + TILE_K_BYTES + f * (TILE_STAGE * 2) +
+                                                      (((4 * u + G) ^ ((f >> 1) & 7)) * 16));
+#pragma unroll
+                    for (int nb = 0; nb < 2; ++nb)
+                        acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, vop), __builtin_bit_cast(bf16x8, pb[nb]), acc[nb][db], 0, 0, 0);
+                }
+            }
+        };
+        pages_for(0, page_l, off_l);
+        issue(stage_a, page_l, off_l);
+        if (stages > 1) pages_for(1, page_l, off_l);
+        for (int s = 0; s < stages; s += 2) {
+            stage(s, stage_a, stage_b);
+            if (s + 1 < stages) stage(s + 1, stage_b, stage_a);
+        }
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            float lt = l[nb];
+            lt += __shfl_xor(lt, 16, IA_WAVE);
+            lt += __shfl_xor(lt, 32, IA_WAVE);
+            if (!cvalid[nb]) continue;
+            const float inv = 1.0f / lt;
+            bf16_t* o = p.out + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD + 4 * G;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                uint2 w;
+                w.x = pack_bf16x2(acc[nb][db][0] * inv, acc[nb][db][1] * inv);
+                w.y = pack_bf16x2(acc[nb][db][2] * inv, acc[nb][db][3] * inv);
+                *(uint2*)(o + 16 * db) = w;
+            }
+        }
+    }
+}
+
+static int g_tiles = 1;
+// Measurement switch: 0 keeps prompt portions on the kernel of single waves.
+extern "C" void ia_attention_mfma_tiles(int on) { g_tiles = on; }
+
 // Merges the partial results of the key splits of one (token, head): one block a row.  The
 // partial results were written by other compute units, so every read is a long way off: the
 // block's waves share the splits between them (wave w takes splits w, w + waves, ...) and
@@ -597,6 +870,18 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         // 16 columns a wave, whatever the number of query heads of a key/value head
         const dim3 fgrid((unsigned)((cols + 15) / 16), nkv * splits, n_seqs);
         attn_mfma_fused_kernel<><<<fgrid, IA_WAVE, 0, stream>>>(p);
+    } else if (HD == 128 && g_tiles && splits == 1 && cols >= TILE_COLS) {
+        // portions of prompts: blocks of four waves that share the keys through shared memory
+        const dim3 tgrid((unsigned)((cols + TILE_COLS - 1) / TILE_COLS), nkv, n_seqs);
+        static int cus = 0;
+        if (cus == 0) {
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+                cus = 256;
+        }
+        p.pair = (long long)tgrid.x * tgrid.y * tgrid.z <= 2LL * cus ? cus : 0;     // the tile kernel's use of the field
+        attn_tile_kernel<><<<tgrid, TILE_WAVES * IA_WAVE, 0, stream>>>(p);
     } else if (nb == 1) {
         attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
     } else {

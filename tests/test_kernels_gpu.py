@@ -215,6 +215,29 @@ def ref_attention(q, kc, vc, positions, token_seq, table, window, scale):
     return out
 
 
+def ref_attention_dense(q, kc, vc, positions, token_seq, table, window, scale):
+    """The same formula, request by request on dense copies of its keys and values (for long cases)."""
+    n, nq, d = q.shape
+    nkv, page = kc.shape[1], kc.shape[2]
+    out = torch.zeros(n, nq, d)
+    for s in token_seq.unique().tolist():
+        rows = (token_seq == s).nonzero().flatten()
+        pos = positions[rows].long()
+        length = int(pos.max()) + 1
+        pages = table[s, :-(-length // page)].long()
+        k = kc[pages].float().permute(1, 0, 2, 3).reshape(nkv, -1, d)[:, :length]           # [nkv, L, d]
+        v = vc[pages].float().permute(1, 0, 3, 2).reshape(nkv, -1, d)[:, :length]           # [nkv, L, d]
+        k, v = k.repeat_interleave(nq // nkv, 0), v.repeat_interleave(nq // nkv, 0)         # [nq, L, d]
+        sc = torch.einsum("thd,hjd->thj", q[rows].float(), k) * scale
+        j = torch.arange(length)
+        hidden = j[None, :] > pos[:, None]
+        if window:
+            hidden |= j[None, :] < (pos[:, None] - window + 1)
+        sc = sc.masked_fill(hidden[:, None, :], float("-inf"))
+        out[rows] = torch.einsum("thj,hjd->thd", torch.softmax(sc, -1), v)
+    return out
+
+
 def attention_case(dtype, nq, nkv, d, page, lens, q_lens, seed, needle=False):
     """Requests with `lens` cached tokens of which the last `q_lens` are this step's queries,
     pages handed out in a shuffled order."""
@@ -254,6 +277,7 @@ def test_attention_generic(dtype, nq, nkv, d, page, window):
                                 window=window, scale=scale)
     want = ref_attention(q, kc, vc, positions, token_seq, table, window, scale)
     close(got, want, tol(dtype, 5e-6, 2 ** -7), "attention")
+    close(ref_attention_dense(q, kc, vc, positions, token_seq, table, window, scale), want, 1e-5, "the two references")
 
 
 @pytest.mark.parametrize("nq,nkv,d,page,window", [
@@ -280,6 +304,40 @@ def test_attention_mfma(nq, nkv, d, page, window, lens, q_lens):
                                  max_q_len=max(q_lens), max_kv_len=max(lens), window=window, scale=scale,
                                  splits=splits)
         close(got, want, 2 ** -7, f"attention_mfma splits={splits}")
+
+
+@pytest.mark.parametrize("nq,nkv,page,window", [(8, 2, 16, None), (4, 4, 32, None), (10, 2, 48, None), (8, 2, 16, 150),
+                                                (32, 8, 16, None)])
+@pytest.mark.parametrize("lens,q_lens", [
+    ([333], [333]),                                       # a whole prompt
+    ([700, 90], [130, 64]),                               # late portions of long prompts
+    ([64, 65, 127, 128], [64, 65, 127, 128]),             # around the size of a stage of keys
+    ([500, 40, 260], [37, 40, 1])])                       # short portions and a single token beside a long one
+def test_attention_mfma_prompt_portions_head_size_128(nq, nkv, page, window, lens, q_lens):
+    """Head size 128 with 128 columns or more: blocks of four waves that share keys and values through
+    shared memory, against the reference and against the kernel of single waves."""
+    from inferrs_amd import ops
+    dtype, d = torch.bfloat16, 128
+    q, kc, vc, positions, token_seq, table = attention_case(dtype, nq, nkv, d, page, lens, q_lens, 17, needle=True)
+    for s, l in enumerate(lens):
+        for j in range(l, -(-l // page) * page):
+            kc[int(table[s, j // page]), :, j % page] = float("nan")
+            vc[int(table[s, j // page]), :, :, j % page] = float("nan")
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    want = ref_attention_dense(q, kc, vc, positions, token_seq, table, window, scale)
+    args = (dev(q), dev(kc), dev(vc), dev(positions), dev(cu), dev(table))
+    kw = dict(max_q_len=max(q_lens), max_kv_len=max(lens), window=window, scale=scale, splits=1)
+    got = ops.attention_mfma(*args, **kw)
+    close(got, want, 2 ** -7, "blocks of four waves")
+    lib = ops.library("attn_d128")
+    lib.ia_attention_mfma_tiles(0)
+    try:
+        single = ops.attention_mfma(*args, **kw)
+    finally:
+        lib.ia_attention_mfma_tiles(1)
+    close(single, want, 2 ** -7, "single waves")
+    close(got, single.float().cpu(), 2 ** -7, "the two kernels")
 
 
 def test_attention_mfma_refuses_what_it_cannot_take():
