@@ -457,6 +457,37 @@ void attn_mfma_fused_kernel(const AttnParams p) {
     }
 }
 
+// The maximum / the sum over the four lanes that hold a column's values (lanes l, l ^ 16, l ^ 32, l ^ 48), in all
+// of them, by swaps between rows of 16 lanes and between the halves of the wave: no trip through shared memory.
+// (the maximum instructions themselves, which return the other operand when one is a NaN: fmaxf() puts
+// an instruction in front of each operand that turns a signalling NaN into a quiet one)
+__device__ __forceinline__ float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float column_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    x = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const uint32_t w = __float_as_uint(x);
+    auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_sum(float x) {
+    const uint32_t u = __float_as_uint(x);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const uint32_t w = __float_as_uint(x);
+    auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // ---- prompt portions, head size 128: blocks of four waves that share keys and values ----------
 // A block owns 128 columns of one request and key/value head (32 columns a wave) and walks the keys in
 // stages of 64.  A stage's keys and values come from the cache pages straight into shared memory
@@ -657,9 +688,8 @@ void attn_tile_kernel(const AttnParams p) {
                             if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
                         }
                     }
-                    float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-                    mx = fmaxf(mx, __shfl_xor(mx, 16, IA_WAVE));
-                    mx = fmaxf(mx, __shfl_xor(mx, 32, IA_WAVE));
+                    float mx = max2(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], max3(sc[5], sc[6], sc[7])));
+                    mx = column_max(mx);
                     // The exponents' reference point moves only when the step's maximum has passed it by 2^8
                     // (probabilities then reach 2^8 at most, which 32-bit sums and bfloat16 operands hold as
                     // well as 1): the accumulators are rescaled a few times a walk instead of at most steps.
@@ -709,9 +739,7 @@ void attn_tile_kernel(const AttnParams p) {
         }
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
-            float lt = l[nb];
-            lt += __shfl_xor(lt, 16, IA_WAVE);
-            lt += __shfl_xor(lt, 32, IA_WAVE);
+            const float lt = column_sum(l[nb]);
             if (!cvalid[nb]) continue;
             const float inv = 1.0f / lt;
             bf16_t* o = p.out + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD + 4 * G;
