@@ -496,7 +496,8 @@ __device__ __forceinline__ float column_sum(float x) {
 // a block instead of once a wave.  A load instruction fills 1 KiB of shared memory in lane order, so
 // the lane picks the piece it fetches such that the layout comes out swizzled:
 //   keys    row of 256 bytes a key, the 16-byte piece c of key k at place c ^ ((k & 3) | ((k >> 3) & 3) << 2)
-//   values  row of 128 bytes a feature (64 keys), the piece c of feature f at place c ^ ((f >> 1) & 7)
+//   values  by groups of 16 keys: row of 32 bytes a feature, its two halves swapped in every other block of
+//           eight features
 // and the 16 lanes that read an operand together (16 rows, the same piece) hit 16 different banks.
 #define TILE_WAVES 4
 #define TILE_COLS (TILE_WAVES * 32)
@@ -573,52 +574,51 @@ void attn_tile_kernel(const AttnParams p) {
         // ---- a stage on its way: wave w brings keys 16 w .. + 16 and features 32 w .. + 32 ----------
         // Groups of 16 keys past the request's length are read from the group of its last key instead
         // (their scores are masked and their values zeroed below): the pages behind may not exist.
-        // Lane j looks up the page of the stage's j-th group of 16 keys (j < 4; the other lanes repeat them) a
-        // stage ahead of its use, so that nobody waits for the block table.
+        // Wave w brings the stage's w-th group of 16 keys and their values: one place in one page, the same
+        // for all its lanes, looked up a stage ahead of its use so that nobody waits for the block table.
+        // What a lane adds to that place does not change from stage to stage.
+        const int wave_s = __builtin_amdgcn_readfirstlane(wave);
         auto pages_for = [&](int s, int& page, int& off) {
-            const int key0 = lo + s * TILE_STAGE + 16 * (lane & 3);
+            const int key0 = lo + s * TILE_STAGE + 16 * wave_s;
             const int k = key0 < kv_total ? key0 : (kv_total - 1) & ~15;
             const int idx = k / p.page;
             page = bt[idx];
             off = k - idx * p.page;
         };
-        auto issue = [&](char* buf, int page_l, int off_l) {
-            {
-                const int page = __shfl(page_l, wave, IA_WAVE), off = __shfl(off_l, wave, IA_WAVE);
-                const char* krows = (const char*)(p.k_cache + (((size_t)page * p.nkv + kvh) * p.page + off) * HD);
+        uint32_t k_from[4];             // keys: chunk c is rows 4 c .. + 4 of the group, a lane's piece swizzled
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int row = 4 * c + (lane >> 4), key = 16 * wave + row;
-                    const int piece = (lane & 15) ^ ((key & 3) | (((key >> 3) & 3) << 2));
-                    __builtin_amdgcn_global_load_lds(
-                        (const void __attribute__((address_space(1)))*)(krows + row * (HD * 2) + piece * 16),
-                        (void __attribute__((address_space(3)))*)(buf + (16 * wave + 4 * c) * (HD * 2)), 16, 0, 0);
-                }
-            }
+        for (int c = 0; c < 4; ++c) {
+            const int row = 4 * c + (lane >> 4), key = 16 * wave + row;
+            const int piece = (lane & 15) ^ ((key & 3) | (((key >> 3) & 3) << 2));
+            k_from[c] = (uint32_t)(row * (HD * 2) + piece * 16);
+        }
+        // values: chunk c is features 32 c .. + 32, two lanes a feature (its 16 keys), the halves swapped in
+        // every other block of eight features
+        const uint32_t v_from = (uint32_t)(((lane >> 1) * p.page + (((lane & 1) ^ ((lane >> 4) & 1)) * 8)) * 2);
+        auto issue = [&](char* buf, int page, int off) {
+            const char* krows = (const char*)(p.k_cache + (((size_t)page * p.nkv + kvh) * p.page + off) * HD);
+            const char* vrows = (const char*)(p.v_cache + ((size_t)page * p.nkv + kvh) * HD * p.page + off);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int f = 32 * wave + 8 * c + (lane >> 3);
-                const int piece = (lane & 7) ^ ((f >> 1) & 7);
-                const int page = __shfl(page_l, piece >> 1, IA_WAVE), off = __shfl(off_l, piece >> 1, IA_WAVE);
-                const char* src = (const char*)(p.v_cache + (((size_t)page * p.nkv + kvh) * HD + f) * p.page + off + (piece & 1) * 8);
+            for (int c = 0; c < 4; ++c)
                 __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)src,
-                    (void __attribute__((address_space(3)))*)(buf + TILE_K_BYTES + (32 * wave + 8 * c) * (TILE_STAGE * 2)),
-                    16, 0, 0);
-            }
+                    (const void __attribute__((address_space(1)))*)(krows + k_from[c]),
+                    (void __attribute__((address_space(3)))*)(buf + (16 * wave_s + 4 * c) * (HD * 2)), 16, 0, 0);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(vrows + (size_t)c * 32 * p.page * 2 + v_from),
+                    (void __attribute__((address_space(3)))*)(buf + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024), 16, 0, 0);
         };
         // values of keys past the request's length may hold anything at all: a lane zeroes them in the
         // pieces that it brought itself, once they have arrived
         auto zero_tail = [&](int s, char* buf) {
             const int kb = lo + s * TILE_STAGE;
             if (kb + TILE_STAGE <= kv_total) return;
+            const int first_bad = kv_total - (kb + 16 * wave_s + 8 * ((lane & 1) ^ ((lane >> 4) & 1)));
+            if (first_bad >= 8) return;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                const int f = 32 * wave + 8 * c + (lane >> 3);
-                const int piece = (lane & 7) ^ ((f >> 1) & 7);
-                const int first_bad = kv_total - (kb + 8 * piece);
-                if (first_bad >= 8) continue;
-                uint4* at = (uint4*)(buf + TILE_K_BYTES + (32 * wave + 8 * c) * (TILE_STAGE * 2) + lane * 16);
+                uint4* at = (uint4*)(buf + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024 + lane * 16);
                 const uint4 v = *at;
                 uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -640,6 +640,8 @@ void attn_tile_kernel(const AttnParams p) {
                 for (int t = 0; t < 2; ++t) k_at[u][t] = (uint32_t)((32 * u + kl + 4 * t) * (HD * 2));
         }
 
+        // values: group of 16 keys (G >> 1 of the step's two), feature row of 32 bytes, the half G & 1 swapped as written
+        const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HD * 2) + r * 32 + (((G & 1) ^ ((r >> 3) & 1)) * 16));
         int page_l, off_l;
         auto stage = [&](int s, char* buf, char* other) {
             __builtin_amdgcn_s_waitcnt(0);                 // this wave's part of stage s has arrived
@@ -650,35 +652,52 @@ void attn_tile_kernel(const AttnParams p) {
                 if (s + 2 < stages) pages_for(s + 2, page_l, off_l);
             }
             const int kb = lo + s * TILE_STAGE;
+            // Steps of 32 keys.  A wave's operands are asked for a phase ahead of their use: the values of a
+            // step before its softmax is worked out, the keys of the next step before this step's second
+            // product, so that the shared memory's latency passes behind arithmetic.
+            bool live[2];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int k0 = kb + 32 * u;
-                if (k0 > pmax || k0 + 31 < wlo) continue;  // nothing of this step is visible to this wave's columns
-                const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
-                uint4 kop[2][KS];
+            for (int u = 0; u < 2; ++u)        // something of the step is visible to this wave's columns
+                live[u] = !(kb + 32 * u > pmax || kb + 32 * u + 31 < wlo);
+            uint4 kop[2][KS];
+            auto read_keys = [&](int u) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
                         kop[t][ks] = *(const uint4*)(buf + k_at[u][t] + (((uint32_t)(ks * 4 + G) ^ k_xor) * 16));
-                uint4 pb[2];
-                float alpha[2];
+            };
+            if (live[0]) read_keys(0);
+            else if (live[1]) read_keys(1);
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
-                    f32x4 sacc[2];
+            for (int u = 0; u < 2; ++u) {
+                if (!live[u]) continue;
+                const int k0 = kb + 32 * u;
+                const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
+                f32x4 sacc[2][2];
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                        sacc[nb][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int ks = 0; ks < KS; ++ks)
-                            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                                __builtin_bit_cast(bf16x8, kop[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), sacc[t], 0, 0, 0);
+                            sacc[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                __builtin_bit_cast(bf16x8, kop[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), sacc[nb][t], 0, 0, 0);
                     }
+                uint4 vop[DB];
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HD * 2) + db * 512 + v_at);
+                __builtin_amdgcn_sched_barrier(0);
+                uint4 pb[2];
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
                     float sc[8];
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) sc[4 * t + i] = sacc[t][i];
+                        for (int i = 0; i < 4; ++i) sc[4 * t + i] = sacc[nb][t][i];
                     if (edge) {
                         const int kbase_idx = k0 + 8 * G;
                         const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
@@ -697,37 +716,35 @@ void attn_tile_kernel(const AttnParams p) {
                     const bool rise = cand > m[nb] + 8.0f;              // also the first finite maximum after -inf
                     const float m_new = rise ? cand : m[nb];
                     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                    alpha[nb] = rise ? __builtin_amdgcn_exp2f(m[nb] - m_use) : 1.0f;
+                    const float alpha = rise ? __builtin_amdgcn_exp2f(m[nb] - m_use) : 1.0f;
                     float pr[8], psum = 0.f;
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
                         pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], p.scale_log2, -m_use));
                         psum += pr[j];
                     }
-                    l[nb] = l[nb] * alpha[nb] + psum;
+                    l[nb] = l[nb] * alpha + psum;
                     m[nb] = m_new;
                     pb[nb].x = pack_bf16x2(pr[0], pr[1]);
                     pb[nb].y = pack_bf16x2(pr[2], pr[3]);
                     pb[nb].z = pack_bf16x2(pr[4], pr[5]);
                     pb[nb].w = pack_bf16x2(pr[6], pr[7]);
-                    if (__any(alpha[nb] != 1.0f)) {
+                    if (__any(alpha != 1.0f)) {
 #pragma unroll
                         for (int db = 0; db < DB; ++db) {
-                            acc[nb][db][0] *= alpha[nb]; acc[nb][db][1] *= alpha[nb];
-                            acc[nb][db][2] *= alpha[nb]; acc[nb][db][3] *= alpha[nb];
+                            acc[nb][db][0] *= alpha; acc[nb][db][1] *= alpha;
+                            acc[nb][db][2] *= alpha; acc[nb][db][3] *= alpha;
                         }
                     }
                 }
+                if (u == 0 && live[1]) read_keys(1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const int f = 16 * db + r;
-                    const uint4 vop = *(const uint4*)(buf + TILE_K_BYTES + f * (TILE_STAGE * 2) +
-                                                      (((4 * u + G) ^ ((f >> 1) & 7)) * 16));
+                for (int db = 0; db < DB; ++db)
 #pragma unroll
                     for (int nb = 0; nb < 2; ++nb)
                         acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8, vop), __builtin_bit_cast(bf16x8, pb[nb]), acc[nb][db], 0, 0, 0);
-                }
+                            __builtin_bit_cast(bf16x8, vop[db]), __builtin_bit_cast(bf16x8, pb[nb]), acc[nb][db], 0, 0, 0);
             }
         };
         pages_for(0, page_l, off_l);
