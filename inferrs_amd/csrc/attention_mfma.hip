@@ -515,7 +515,8 @@ void attn_tile_kernel(const AttnParams p) {
         __shared__ __align__(16) char stage_b[TILE_BUF_BYTES];
         const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
         const int r = lane & 15, G = lane >> 4;
-        const int kvh = blockIdx.y, seq = p.seq_begin + blockIdx.z;
+        const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
+        const int seq = p.seq_begin + blockIdx.z;
         const int g = p.nq / p.nkv;
         const int t0 = p.cu_tokens[seq], q_len = p.cu_tokens[seq + 1] - t0;
         const int n_cols = q_len * g;
@@ -524,8 +525,9 @@ void attn_tile_kernel(const AttnParams p) {
         // Long walks first.  When all blocks fit on the chip at once (two a compute unit), the second half
         // of them, which joins the first half on its compute units, brings short walks first: a compute
         // unit's two blocks then end together (one prompt of 2,048 tokens: 103 -> 88 us).
-        const unsigned linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-        const bool second = p.pair > 0 && ((linear / (unsigned)p.pair) & 1u) != 0;
+        // (the order is one for all tiles of a request, key/value head and split: each tile is walked once)
+        const unsigned first_of_row = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const bool second = p.pair > 0 && ((first_of_row / (unsigned)p.pair) & 1u) != 0;
         const int bcol0 = (second ? (int)blockIdx.x : n_tiles - 1 - (int)blockIdx.x) * TILE_COLS;
         const int kv_start = p.positions[t0];
         const int kv_total = kv_start + q_len;
@@ -534,7 +536,13 @@ void attn_tile_kernel(const AttnParams p) {
         const int bpmin = kv_start + bcol0 / g, bpmax = kv_start + blast / g;
         int lo = p.window > 0 ? (bpmin - p.window + 1 > 0 ? bpmin - p.window + 1 : 0) : 0;
         lo &= ~(TILE_STAGE - 1);
-        const int stages = (bpmax + 1 - lo + TILE_STAGE - 1) / TILE_STAGE;
+        int hi = bpmax + 1;
+        if (p.splits > 1) {             // this block's share of the keys (`chunk` is a multiple of a stage)
+            const int c_lo = split * p.chunk, c_hi = c_lo + p.chunk;
+            lo = lo > c_lo ? lo : c_lo;
+            hi = hi < c_hi ? hi : c_hi;
+        }
+        const int stages = hi > lo ? (hi - lo + TILE_STAGE - 1) / TILE_STAGE : 0;
 
         // this wave's columns (a wave without any still brings its share of the stages)
         const int col0 = bcol0 + wave * 32;
@@ -629,17 +637,13 @@ void attn_tile_kernel(const AttnParams p) {
         };
 
         // this lane's places in a stage: they do not change from stage to stage
-        uint32_t k_at[2][2];            // [step of 32 keys][tile t]: the row's start and what the pieces are xor-ed with
-        uint32_t k_xor;
+        uint32_t k_at[KS];              // keys: the lane's row of tile 0 of step 0 and its swizzled piece of dim step ks
         {
             const int kl = 8 * (r >> 2) + (r & 3);
-            k_xor = (uint32_t)((kl & 3) | (((kl >> 3) & 3) << 2));
+            const uint32_t k_xor = (uint32_t)((kl & 3) | (((kl >> 3) & 3) << 2));
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) k_at[u][t] = (uint32_t)((32 * u + kl + 4 * t) * (HD * 2));
+            for (int ks = 0; ks < KS; ++ks) k_at[ks] = (uint32_t)(kl * (HD * 2)) + (((uint32_t)(ks * 4 + G) ^ k_xor) * 16);
         }
-
         // values: group of 16 keys (G >> 1 of the step's two), feature row of 32 bytes, the half G & 1 swapped as written
         const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HD * 2) + r * 32 + (((G & 1) ^ ((r >> 3) & 1)) * 16));
         int page_l, off_l;
@@ -665,7 +669,7 @@ void attn_tile_kernel(const AttnParams p) {
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        kop[t][ks] = *(const uint4*)(buf + k_at[u][t] + (((uint32_t)(ks * 4 + G) ^ k_xor) * 16));
+                        kop[t][ks] = *(const uint4*)(buf + (32 * u + 4 * t) * (HD * 2) + k_at[ks]);
             };
             if (live[0]) read_keys(0);
             else if (live[1]) read_keys(1);
@@ -747,9 +751,11 @@ void attn_tile_kernel(const AttnParams p) {
                             __builtin_bit_cast(bf16x8, vop[db]), __builtin_bit_cast(bf16x8, pb[nb]), acc[nb][db], 0, 0, 0);
             }
         };
-        pages_for(0, page_l, off_l);
-        issue(stage_a, page_l, off_l);
-        if (stages > 1) pages_for(1, page_l, off_l);
+        if (stages > 0) {
+            pages_for(0, page_l, off_l);
+            issue(stage_a, page_l, off_l);
+            if (stages > 1) pages_for(1, page_l, off_l);
+        }
         for (int s = 0; s < stages; s += 2) {
             stage(s, stage_a, stage_b);
             if (s + 1 < stages) stage(s + 1, stage_b, stage_a);
@@ -758,14 +764,27 @@ void attn_tile_kernel(const AttnParams p) {
         for (int nb = 0; nb < 2; ++nb) {
             const float lt = column_sum(l[nb]);
             if (!cvalid[nb]) continue;
-            const float inv = 1.0f / lt;
-            bf16_t* o = p.out + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD + 4 * G;
+            const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
+            if (p.splits == 1) {
+                const float inv = 1.0f / lt;
+                bf16_t* o = p.out + row * HD + 4 * G;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                uint2 w;
-                w.x = pack_bf16x2(acc[nb][db][0] * inv, acc[nb][db][1] * inv);
-                w.y = pack_bf16x2(acc[nb][db][2] * inv, acc[nb][db][3] * inv);
-                *(uint2*)(o + 16 * db) = w;
+                for (int db = 0; db < DB; ++db) {
+                    uint2 w;
+                    w.x = pack_bf16x2(acc[nb][db][0] * inv, acc[nb][db][1] * inv);
+                    w.y = pack_bf16x2(acc[nb][db][2] * inv, acc[nb][db][3] * inv);
+                    *(uint2*)(o + 16 * db) = w;
+                }
+            } else {
+                // for the merge: sums and accumulators relative to the exponents' reference point m
+                float* o = p.part_o + (row * p.splits + split) * HD + 4 * G;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) *(f32x4*)(o + 16 * db) = acc[nb][db];
+                if (G == 0) {
+                    float* ml = p.part_ml + (row * p.splits + split) * 2;
+                    ml[0] = m[nb];
+                    ml[1] = lt;
+                }
             }
         }
     }
@@ -844,6 +863,42 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
     }
 }
 
+// The same merge for steps with many rows and few splits (portions of prompts): a wave a row, every lane
+// with the splits' maxima and sums of its row and HD / 64 features.
+#define MERGE_ROWS_WAVES 4
+__global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_kernel(
+    bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
+    size_t first_row, size_t n_rows) {
+    constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
+    const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+    const size_t local = (size_t)blockIdx.x * MERGE_ROWS_WAVES + wave;
+    if (local >= n_rows) return;
+    const size_t row = first_row + local;
+    const float* ml = part_ml + row * splits * 2;
+    const float* po = part_o + row * splits * HD;
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml[2 * s]);
+    float total = 0.f, o[PER];
+#pragma unroll
+    for (int t = 0; t < PER; ++t) o[t] = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float ms = ml[2 * s];
+        const float w = ms == -INFINITY ? 0.f : exp2f(ms - mx);          // a split that held no key of this row
+        total += ml[2 * s + 1] * w;
+#pragma unroll
+        for (int t = 0; t < PER; ++t) {
+            const int e = lane + t * IA_WAVE;
+            if (e < HD) o[t] = fmaf(po[(size_t)s * HD + e], w, o[t]);
+        }
+    }
+    const float inv = 1.0f / total;
+#pragma unroll
+    for (int t = 0; t < PER; ++t) {
+        const int e = lane + t * IA_WAVE;
+        if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(o[t] * inv);
+    }
+}
+
 extern "C" int ia_attention_mfma_head_dim(void) { return HD; }
 
 // Floats of workspace that `splits` > 1 needs: partial outputs, then maxima and sums.
@@ -915,9 +970,9 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         // 16 columns a wave, whatever the number of query heads of a key/value head
         const dim3 fgrid((unsigned)((cols + 15) / 16), nkv * splits, n_seqs);
         attn_mfma_fused_kernel<><<<fgrid, IA_WAVE, 0, stream>>>(p);
-    } else if (HD == 128 && g_tiles && splits == 1 && cols >= TILE_COLS) {
+    } else if (HD == 128 && g_tiles && cols >= TILE_COLS && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
-        const dim3 tgrid((unsigned)((cols + TILE_COLS - 1) / TILE_COLS), nkv, n_seqs);
+        const dim3 tgrid((unsigned)((cols + TILE_COLS - 1) / TILE_COLS), nkv * splits, n_seqs);
         static int cus = 0;
         if (cus == 0) {
             int dev = 0;
@@ -934,8 +989,14 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     }
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
-        attn_merge_kernel<<<(unsigned)((long long)n_tokens * nq), MERGE_WAVES * IA_WAVE, 0, stream>>>(
-            (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq);
+        const long long rows = (long long)n_tokens * nq;
+        if (rows >= 4096 && splits <= 16)
+            attn_merge_rows_kernel<<<(unsigned)((rows + MERGE_ROWS_WAVES - 1) / MERGE_ROWS_WAVES), MERGE_ROWS_WAVES * IA_WAVE,
+                                     0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq,
+                                                  (size_t)rows);
+        else
+            attn_merge_kernel<<<(unsigned)rows, MERGE_WAVES * IA_WAVE, 0, stream>>>(
+                (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq);
         IA_LAUNCH_CHECK("attention_merge");
     }
     return 0;

@@ -253,10 +253,22 @@ def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int) -> bool:
     return dtype == torch.bfloat16 and d in _build.ATTN_HEAD_DIMS and page_size % 16 == 0
 
 
-def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: int) -> Tuple[int, int]:
+ATTN_TILE_COLS = 128           # head size 128, prompt portions: columns a block of four waves
+ATTN_TILE_BLOCKS = 512         # blocks wanted (two a compute unit) before the keys stop being split
+ATTN_TILE_MIN_CHUNK = 512      # fewest keys a block's share is worth (eight stages of 64)
+
+
+def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: int, d: int = 0) -> Tuple[int, int]:
     """(splits, keys per split) for the matrix-core kernel: the keys are split between waves
     when the batch alone has too few (request, kv head, column block) items to fill the chip."""
     cols = max_q_len * g
+    if d == 128 and cols >= ATTN_TILE_COLS:
+        items = n_seqs * nkv * -(-cols // ATTN_TILE_COLS)
+        splits = 1
+        while items * splits < ATTN_TILE_BLOCKS and max_kv_len >= 2 * splits * ATTN_TILE_MIN_CHUNK and splits < 128:
+            splits *= 2
+        chunk = -(-max_kv_len // splits)
+        return splits, -(-chunk // 64) * 64
     col_blocks = 1 if cols <= 16 else -(-cols // 32)
     items = n_seqs * nkv * col_blocks
     splits = 1
@@ -301,9 +313,9 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     elif out.shape != q.shape or out.dtype != q.dtype:
         raise KernelError("attention_mfma: `out` must have the shape and dtype of q")
     if splits is None:
-        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len)
+        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len, d)
     else:
-        chunk = -(-(-(-max_kv_len // splits)) // 32) * 32
+        chunk = -(-(-(-max_kv_len // splits)) // 64) * 64
     target = _build.attn_target(d)
     lib = library(target)
     ws_floats = lib.ia_attention_mfma_workspace(n, nq, splits)

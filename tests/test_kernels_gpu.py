@@ -330,6 +330,8 @@ def test_attention_mfma_prompt_portions_head_size_128(nq, nkv, page, window, len
     kw = dict(max_q_len=max(q_lens), max_kv_len=max(lens), window=window, scale=scale, splits=1)
     got = ops.attention_mfma(*args, **kw)
     close(got, want, 2 ** -7, "blocks of four waves")
+    for splits in (None, 2, 3):                        # the keys shared out between blocks and merged
+        close(ops.attention_mfma(*args, **dict(kw, splits=splits)), want, 2 ** -7, f"blocks of four waves, splits={splits}")
     lib = ops.library("attn_d128")
     lib.ia_attention_mfma_tiles(0)
     try:
@@ -338,6 +340,21 @@ def test_attention_mfma_prompt_portions_head_size_128(nq, nkv, page, window, len
         lib.ia_attention_mfma_tiles(1)
     close(single, want, 2 ** -7, "single waves")
     close(got, single.float().cpu(), 2 ** -7, "the two kernels")
+
+
+def test_attention_mfma_prompt_that_half_fills_the_chip():
+    """Between one and two blocks a compute unit the second half of the blocks walks its tiles in the other
+    order; with 47 tiles a row of the grid that half does not begin at a row's start."""
+    from inferrs_amd import ops
+    dtype, d, nq, nkv, page = torch.bfloat16, 128, 32, 8, 16
+    lens = q_lens = [1500]
+    q, kc, vc, positions, token_seq, table = attention_case(dtype, nq, nkv, d, page, lens, q_lens, 19, needle=True)
+    cu = torch.tensor([0, 1500], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    want = ref_attention_dense(q, kc, vc, positions, token_seq, table, None, scale)
+    got = ops.attention_mfma(dev(q), dev(kc), dev(vc), dev(positions), dev(cu), dev(table), max_q_len=1500,
+                             max_kv_len=1500, window=None, scale=scale, splits=1)
+    close(got, want, 2 ** -7, "47 x 8 blocks")
 
 
 def test_attention_mfma_refuses_what_it_cannot_take():
