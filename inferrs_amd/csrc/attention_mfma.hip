@@ -500,9 +500,11 @@ __device__ __forceinline__ float column_sum(float x) {
 // a block instead of once a wave.  A load instruction fills 1 KiB of shared memory in lane order, so
 // the lane picks the piece it fetches such that the layout comes out swizzled:
 //   keys    row of 256 bytes a key, the 16-byte piece c of key k at place c ^ ((k & 3) | ((k >> 3) & 3) << 2)
-//   values  by groups of 16 keys: row of 32 bytes a feature, its two halves swapped in every other block of
-//           eight features
-// and the 16 lanes that read an operand together (16 rows, the same piece) hit 16 different banks.
+//   values  by groups of 16 keys: row of 32 bytes a feature, as the cache page holds it
+// The swizzle of the keys spreads the 16 rows that a read takes at the same place over the banks (rows of 256
+// bytes would all begin in the same one).  The counters show no bank conflict for either array
+// (SQ_LDS_BANK_CONFLICT = 0); values with their halves swapped in every other block of eight features, which
+// looked as good on paper, cost two extra cycles a read.
 // Measured against the kernel of single waves (one request, 32 query and 8 key/value heads): a prompt of
 // 2,048 tokens 118 -> 80 us, of 8,192 tokens 1.20 -> 0.74 ms (750 TFLOP/s of the causal half); a portion of
 // 512 tokens at 8,192 (keys split four ways) 181 -> 106 us.  Timing-only variants of the kernel show no
@@ -611,9 +613,9 @@ void attn_tile_kernel(const AttnParams p) {
             const int piece = (lane & 15) ^ ((key & 3) | (((key >> 3) & 3) << 2));
             k_from[c] = (uint32_t)(row * (HD * 2) + piece * 16);
         }
-        // values: chunk c is features 32 c .. + 32, two lanes a feature (its 16 keys), the halves swapped in
-        // every other block of eight features
-        const uint32_t v_from = (uint32_t)(((lane >> 1) * p.page + (((lane & 1) ^ ((lane >> 4) & 1)) * 8)) * 2);
+        // values: chunk c is features 32 c .. + 32, two lanes a feature (its 16 keys)
+        const int v_half = lane & 1;                                            // which eight keys the lane's piece holds
+        const uint32_t v_from = (uint32_t)(((lane >> 1) * p.page + v_half * 8) * 2);
         auto issue = [&](char* buf, int page, int off) {
             const char* krows = (const char*)(p.k_cache + (((size_t)page * p.nkv + kvh) * p.page + off) * HD);
             const char* vrows = (const char*)(p.v_cache + ((size_t)page * p.nkv + kvh) * HD * p.page + off);
@@ -633,7 +635,7 @@ void attn_tile_kernel(const AttnParams p) {
         auto zero_tail = [&](int s, char* buf) {
             const int kb = lo + s * TILE_STAGE;
             if (kb + TILE_STAGE <= kv_total) return;
-            const int first_bad = kv_total - (kb + 16 * wave_s + 8 * ((lane & 1) ^ ((lane >> 4) & 1)));
+            const int first_bad = kv_total - (kb + 16 * wave_s + 8 * v_half);
             if (first_bad >= 8) return;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
@@ -655,8 +657,8 @@ void attn_tile_kernel(const AttnParams p) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) k_at[ks] = (uint32_t)(kl * (HD * 2)) + (((uint32_t)(ks * 4 + G) ^ k_xor) * 16);
         }
-        // values: group of 16 keys (G >> 1 of the step's two), feature row of 32 bytes, the half G & 1 swapped as written
-        const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HD * 2) + r * 32 + (((G & 1) ^ ((r >> 3) & 1)) * 16));
+        // values: group of 16 keys (G >> 1 of the step's two), feature row of 32 bytes, half G & 1
+        const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HD * 2) + r * 32 + (G & 1) * 16);
         int page_l, off_l;
         auto stage = [&](int s, char* buf, char* other) {
             __builtin_amdgcn_s_waitcnt(0);                 // this wave's part of stage s has arrived
