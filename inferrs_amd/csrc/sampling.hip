@@ -303,6 +303,124 @@ __device__ int next_in_order(const uint32_t* __restrict__ keys, int vocab, uint3
 
 #define SAMPLE_MAX_TOP 20
 
+// With a top_k of up to SAMPLE_FAST_K every filter works on the first top_k entries of the ordered list, so
+// the row's top_k tokens are picked out first (three histograms over the key's bits find the k-th largest
+// key; equal keys are taken by ascending index), sorted in shared memory, and one thread then does what the
+// reference does with its sorted list, in its order and with its sums (sampler.rs:256-335): six passes over
+// the row instead of the hundred of the bisections below (16 rows of 152 k: 4.5 ms -> 0.2 ms).
+#define SAMPLE_FAST_K 1024
+__device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__ keys, const float* __restrict__ probs,
+                             int vocab, int rowi, int k, float tp, float mp, float u, int want_top,
+                             float* __restrict__ lp_out, int* __restrict__ lp_ids, int* s_counts) {
+    __shared__ int hist[2048];
+    __shared__ unsigned long long cand[SAMPLE_FAST_K];      // (key, ~index): larger is earlier in the list
+    __shared__ int s_bin, s_above, s_n;
+    // ---- the k-th largest key, 11 + 11 + 10 bits at a time
+    uint32_t prefix = 0u;
+    int prefix_bits = 0, need = k;
+    for (int level = 0; level < 3; ++level) {
+        const int bits = level < 2 ? 11 : 10;
+        const int shift = 32 - prefix_bits - bits;
+        for (int i = threadIdx.x; i < 2048; i += blockDim.x) hist[i] = 0;
+        __syncthreads();
+        for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+            const uint32_t key = keys[c];
+            if (prefix_bits == 0 || (key >> (32 - prefix_bits)) == prefix)
+                atomicAdd(&hist[(key >> shift) & ((1u << bits) - 1u)], 1);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int cum = 0, b = (1 << bits) - 1;
+            for (; b > 0; --b) {
+                if (cum + hist[b] >= need) break;
+                cum += hist[b];
+            }
+            s_bin = b;
+            s_above = cum;
+        }
+        __syncthreads();
+        need -= s_above;
+        prefix = (prefix << bits) | (uint32_t)s_bin;
+        prefix_bits += bits;
+        __syncthreads();
+    }
+    const uint32_t kth = prefix;                            // `need` (>= 1) of the tokens with this key belong to the list
+    const int ties = hist[kth & 1023u];
+    __syncthreads();
+    int last_tie = vocab;                                   // ties up to this index are taken
+    if (ties > need) last_tie = nth_with_key(keys, vocab, kth, need, s_counts);
+    if (threadIdx.x == 0) s_n = 0;
+    __syncthreads();
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const uint32_t key = keys[c];
+        if (key > kth || (key == kth && c <= last_tie)) {
+            const int slot = atomicAdd(&s_n, 1);
+            if (slot < SAMPLE_FAST_K) cand[slot] = ((unsigned long long)key << 32) | (uint32_t)~(uint32_t)c;
+        }
+    }
+    __syncthreads();
+    const int n = s_n < k ? s_n : k;                        // = k
+    int padded = 2;
+    while (padded < n) padded <<= 1;
+    for (int i = n + threadIdx.x; i < padded; i += blockDim.x) cand[i] = 0ull;
+    // ---- bitonic sort, descending
+    for (int size = 2; size <= padded; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int t = threadIdx.x; t < padded / 2; t += blockDim.x) {
+                const int i = 2 * t - (t & (stride - 1)), j = i + stride;
+                const bool down = (i & size) == 0;
+                const unsigned long long a = cand[i], b = cand[j];
+                if ((a < b) == down) { cand[i] = b; cand[j] = a; }
+            }
+        }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    // ---- the reference's steps 7 to 12 on its sorted list
+    auto index_of = [&](int i) { return (int)~(uint32_t)(cand[i] & 0xffffffffull); };
+    int len = n;
+    if (tp < 1.0f) {
+        float cumsum = 0.f;
+        for (int i = 0; i < len; ++i) {
+            cumsum += probs[index_of(i)];
+            if (cumsum >= tp) { len = i + 1; break; }
+        }
+    }
+    if (mp > 0.0f && len > 0) {
+        const float threshold = probs[index_of(0)] * mp;
+        int cut = 0;
+        while (cut < len && probs[index_of(cut)] >= threshold) ++cut;
+        if (cut > 0) len = cut;
+    }
+    float filtered = 0.f;
+    for (int i = 0; i < len; ++i) filtered += probs[index_of(i)];
+    const float denom = filtered > 0.f ? filtered : 1.0f;
+    if (want_top >= 0)
+        for (int i = 0; i < want_top && i < SAMPLE_MAX_TOP && i < len; ++i) {
+            const float pi = probs[index_of(i)];
+            lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + i] = index_of(i);
+            lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + i] = pi > 0.f ? logf(pi / denom) : -INFINITY;
+        }
+    if (!(filtered > 0.f)) {
+        out[rowi] = len > 0 ? index_of(0) : 0;
+        if (want_top >= 0) lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = -INFINITY;
+        return;
+    }
+    float rng = u;
+    int at = len - 1;
+    for (int i = 0; i < len; ++i) {
+        const float norm = probs[index_of(i)] / filtered;
+        if (rng < norm) { at = i; break; }
+        rng -= norm;
+    }
+    const int token = index_of(at);
+    out[rowi] = token;
+    if (want_top >= 0) {
+        const float pt = probs[token] / filtered;
+        lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = pt > 0.f ? logf(pt) : -INFINITY;
+    }
+}
+
 // workspace: [rows, 2, vocab] words: the keys, then the probabilities.
 // n_top (may be null): per row -1 = no log-probabilities, else how many of the list's first entries are
 // reported besides the drawn token's (sampler.rs:285-352).  lp_out [rows, 1 + SAMPLE_MAX_TOP]: the drawn
@@ -311,7 +429,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, uint32_t* __restrict__ workspace, int vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
     const float* __restrict__ min_p, const float* __restrict__ u, const int* __restrict__ n_top,
-    float* __restrict__ lp_out, int* __restrict__ lp_ids) {
+    float* __restrict__ lp_out, int* __restrict__ lp_ids, int fast_top_k) {
     __shared__ float scratch[32];
     __shared__ int s_counts[SAMPLE_THREADS];
     __shared__ float sv[16];
@@ -362,9 +480,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
     __syncthreads();
 
+    const int k = top_k[rowi];
+    if (fast_top_k && k > 0 && k < vocab && k <= SAMPLE_FAST_K) {
+        sample_top_k(out, keys, probs, vocab, rowi, k, top_p[rowi], min_p[rowi], u[rowi], want_top, lp_out, lp_ids, s_counts);
+        return;
+    }
     // how long the kept prefix is (sampler.rs:256-283)
     int keep = vocab;
-    const int k = top_k[rowi];
     if (k > 0 && k < keep) keep = k;
     const float tp = top_p[rowi];
     if (tp < 1.0f) {
@@ -462,6 +584,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
 extern "C" long long ia_sample_workspace(int rows, int vocab) { return (long long)rows * 2 * vocab; }
 
+static int g_sample_fast = 1;
+// Measurement and test switch: 0 sends rows with a top_k through the bisections as well.
+extern "C" void ia_sample_tune(int fast_top_k) { g_sample_fast = fast_top_k; }
+
 extern "C" int ia_sample_max_top(void) { return SAMPLE_MAX_TOP; }
 
 // n_top, lp_out, lp_ids: all null, or all given (see sample_kernel).
@@ -474,7 +600,7 @@ extern "C" int ia_sample(int* out, const float* logits, void* workspace, int row
              "sample: the arrays of the log-probabilities come together");
     if (rows == 0) return 0;
     sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, (uint32_t*)workspace, vocab, temperature,
-                                                       top_k, top_p, min_p, u, n_top, lp_out, lp_ids);
+                                                       top_k, top_p, min_p, u, n_top, lp_out, lp_ids, g_sample_fast);
     IA_LAUNCH_CHECK("sample");
     return 0;
 }

@@ -95,6 +95,37 @@ def test_sampler_matches_the_plain_transcription(vocab, kw):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("vocab,top_k", [(387, 1), (387, 50), (387, 386), (5000, 700), (151936, 50), (151936, 1024)])
+def test_rows_with_a_top_k_take_the_same_tokens_on_both_paths(vocab, top_k):
+    """Rows with a top_k up to 1,024 pick their top_k tokens out and walk them as the reference walks its sorted
+    list; the other rows (and these, with the switch off) find the same prefixes by bisection over the keys."""
+    from inferrs_amd import ops
+    g = torch.Generator().manual_seed(vocab + top_k)
+    rows = 24
+    logits = (torch.randn(rows, vocab, generator=g) * 2.5).to(torch.bfloat16).float()      # coarse values: many ties
+    temperature = torch.linspace(0.5, 1.5, rows)
+    top_p = torch.tensor([1.0, 0.9, 0.6] * (rows // 3))
+    min_p = torch.tensor([0.0, 0.0, 0.0, 0.1] * (rows // 4))
+    u = torch.rand(rows, generator=g)
+    k = torch.full((rows,), top_k, dtype=torch.int32)
+    n_top = torch.full((rows,), 5, dtype=torch.int32)
+    args = [t.to("cuda") for t in (logits, temperature, k, top_p, min_p, u, n_top)]
+    fast = ops.sample(*args)
+    ops.library().ia_sample_tune(0)
+    try:
+        slow = ops.sample(*args)
+    finally:
+        ops.library().ia_sample_tune(1)
+    same = (fast[0] == slow[0]).cpu()
+    # sequential sums there, tree sums here: a row may part where u lies within their rounding of a boundary
+    assert int(same.sum()) >= rows - 1, (fast[0].tolist(), slow[0].tolist())
+    assert torch.equal(fast[2].cpu()[same], slow[2].cpu()[same]), "the lists' first entries"
+    lp_f, lp_s = fast[1].cpu()[same], slow[1].cpu()[same]
+    finite = torch.isfinite(lp_s)
+    assert torch.equal(torch.isfinite(lp_f), finite) and float((lp_f[finite] - lp_s[finite]).abs().max()) < 1e-4
+
+
+@pytest.mark.gpu
 def test_mixed_rows_do_not_influence_each_other():
     from inferrs_amd.sampling import Sampler
     sampler = Sampler("cuda:0")
