@@ -345,3 +345,29 @@ def test_real_layer_sizes(tmp_path):
             assert err <= tol, f"{dtype} {mode}: {err:.3e} at {where}"
             del eng
             torch.cuda.empty_cache()
+
+
+def test_real_layer_sizes_long_prompt_in_portions(tmp_path):
+    """The same layer over a prompt of 1,100 tokens, whole and in portions of 300, 37 and 512 tokens: with head
+    size 128 these steps take the attention kernel of four-wave blocks, and the late portions (few tiles, more
+    than 1,024 keys) its form that shares the keys out between blocks and merges them."""
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1031, hidden_size=4096,
+               intermediate_size=12288, num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8,
+               head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+               max_position_embeddings=4096, hidden_act="silu")
+    folder = write_model(str(tmp_path / "layer8b"), raw, seed=22)
+    cfg, params = pm.read_model(folder, torch.float64)
+    reqs = {"long": random_tokens(1100, raw["vocab_size"], 400)}
+    ref = {r: pm.forward(cfg, params, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    del params
+    from inferrs_amd.engine import Engine, run_trace
+    for mode, trace in (("whole", tm.whole(reqs)), ("portions", tm.portions(reqs, (300, 37, 512)))):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=-(-trace.max_tokens // 16) + 1, max_seqs=2)
+        out_dir = str(tmp_path / mode)
+        run_trace(eng, trace.lines, out_dir, io.StringIO())
+        eng.cache.check_invariants()
+        got = trace.read(out_dir, raw["vocab_size"])
+        err, where = worst(got, ref, reqs)
+        assert err <= 2e-2, f"{mode}: {err:.3e} at {where}"
+        del eng
+        torch.cuda.empty_cache()
