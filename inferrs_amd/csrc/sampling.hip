@@ -17,7 +17,9 @@
 // the tokens equal to K (taken by ascending index), and the threshold for "the shortest
 // prefix whose weight reaches a target" is found by bisection over the 32 bits of the key,
 // one block-wide sum per bit.  Sums are tree sums in a fixed order; they differ from the
-// reference's sequential sums by rounding only.
+// reference's sequential sums by rounding only.  Rows with a top_k of up to 1,024 take a
+// shorter way (sample_top_k): their first top_k tokens are picked out and sorted, and the
+// reference's steps run on that list as it runs them.
 #include "common.h"
 #include "api.h"
 
