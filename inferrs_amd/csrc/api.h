@@ -51,6 +51,7 @@ int ia_argmax(int* out, const float* logits, void* workspace, int rows, int voca
 int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, const float* rep,
                 const float* freq, const float* pres, const int* bias_ids, const float* bias_vals,
                 int nb, hipStream_t stream);
+int ia_window_push(int* window, int rows, int w, const int* caps, const int* tokens, hipStream_t stream);
 long long ia_sample_workspace(int rows, int vocab);
 int ia_sample_max_top(void);
 // n_top, lp_out [rows, 1 + max_top], lp_ids [rows, max_top]: all null, or the log-probabilities asked for per row

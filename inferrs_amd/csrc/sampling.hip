@@ -168,6 +168,34 @@ extern "C" int ia_penalize(float* logits, int rows, int vocab, const int* window
     return 0;
 }
 
+// A row's window after it has drawn `tokens[row]`: the last `caps[row]` tokens of its prompt and output
+// (entries from caps[row] on stay -1; caps[row] = 0: the row has no window).  For runs of decode steps that
+// are queued without the host in between.
+__global__ void window_push_kernel(int* __restrict__ window, int w, const int* __restrict__ caps,
+                                   const int* __restrict__ tokens, int rows) {
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows) return;
+    int* win = window + (size_t)row * w;
+    const int cap = caps[row] < w ? caps[row] : w;
+    if (cap <= 0) return;
+    int held = 0;
+    while (held < cap && win[held] >= 0) ++held;
+    if (held < cap) {
+        win[held] = tokens[row];
+        return;
+    }
+    for (int i = 0; i + 1 < cap; ++i) win[i] = win[i + 1];
+    win[cap - 1] = tokens[row];
+}
+
+extern "C" int ia_window_push(int* window, int rows, int w, const int* caps, const int* tokens, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && w > 0, "window_push: bad sizes rows=%d w=%d", rows, w);
+    if (rows == 0) return 0;
+    window_push_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(window, w, caps, tokens, rows);
+    IA_LAUNCH_CHECK("window_push");
+    return 0;
+}
+
 // ---- sampling -------------------------------------------------------------------------------
 #define SAMPLE_THREADS 512
 

@@ -169,13 +169,15 @@ class Engine:
         entry = self._graphs.get((len(seq_ids), len(seq_ids), pad_pages))
         return entry is not None and entry != "seen"
 
-    def decode_chain(self, seq_ids: Sequence[Hashable], tokens: Sequence[int], steps: int) -> Optional[List[List[int]]]:
-        """`steps` greedy decode steps of the same requests, queued back to back: every step's
-        arg max is written on the device where the next step reads its token ids, so the host
-        prepares and queues step i+1 while step i runs and waits once at the end.  The requests
-        hold reserved pages for `steps` more tokens; nothing is committed here.  Returns the chosen
-        tokens `[steps][requests]`, or None when this shape has no captured graph yet (the caller
-        then takes single steps)."""
+    def decode_chain(self, seq_ids: Sequence[Hashable], tokens: Sequence[int], steps: int,
+                     pick=None) -> Optional[List[List[int]]]:
+        """`steps` decode steps of the same requests, queued back to back: every step's choice
+        (the arg max, or `pick(logits, step, out)` writing int32 tokens into `out` on the device) is
+        written on the device where the next step reads its token ids, so the host prepares and
+        queues step i+1 while step i runs and waits once at the end.  The requests hold reserved
+        pages for `steps` more tokens; nothing is committed here.  Returns the chosen tokens
+        `[steps][requests]`, or None when this shape has no captured graph yet (the caller then
+        takes single steps)."""
         if not self.chain_ready(seq_ids, steps):
             return None
         pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
@@ -188,7 +190,10 @@ class Engine:
             if self.builder.generation != generation:
                 raise RuntimeError("the staging buffer moved under a captured graph")
             graph.replay()
-            ops.argmax(logits, out=chosen[i])
+            if pick is None:
+                ops.argmax(logits, out=chosen[i])
+            else:
+                pick(logits, i, chosen[i])
             ctx.token_ids.copy_(chosen[i])            # the next step's token ids, on the device
             self.graph_replays += 1
         return chosen.cpu().tolist()

@@ -27,8 +27,9 @@ class GenerationLoop:
                  prefill_chunk: Optional[int] = None, max_seq_len: Optional[int] = None,
                  stop_token_ids: Optional[Sequence[int]] = None, decode_run: int = 8,
                  detokenize: Optional[Callable[[List[int]], str]] = None):
-        """`decode_run`: when every running request decodes greedily and nobody waits, up to this
-        many decode steps are queued on the GPU at once (`Engine.decode_chain`); 1 switches it off.
+        """`decode_run`: when every running request decodes and nobody waits, up to this many decode
+        steps are queued on the GPU at once (`Engine.decode_chain`; draws included, their random
+        numbers and penalty windows kept on the device); 1 switches it off.
         `detokenize`: output token ids -> text, for requests with stop strings."""
         self.engine = engine
         self.detokenize = detokenize
@@ -64,7 +65,8 @@ class GenerationLoop:
         running = list(sched.running)
         if max_steps < 2 or not running or sched.waiting or len(running) > sched.max_tokens_per_step:
             return None
-        if any(r.total - r.computed != 1 or not r.output or not r.params.is_plain_greedy or any(r.params.stop_strings)
+        # (log-probabilities and stop strings are looked at step by step)
+        if any(r.total - r.computed != 1 or not r.output or r.params.logprobs or any(r.params.stop_strings)
                for r in running):
             return None
         k = min(max_steps, min(min(r.params.max_tokens - len(r.output), sched.max_seq_len - r.total) for r in running))
@@ -73,7 +75,10 @@ class GenerationLoop:
             return None
         for i in ids:
             self.engine.cache.reserve(i, k)
-        tokens = self.engine.decode_chain(ids, [r.tokens[-1] for r in running], k)
+        draw = self.sampler.begin_chain([r.params for r in running], [r.tokens for r in running],
+                                        [r.seed for r in running], k)
+        tokens = self.engine.decode_chain(ids, [r.tokens[-1] for r in running], k,
+                                          pick=None if draw.greedy else draw.pick)
         done: List[Request] = []
         for i in range(k):
             done += sched.commit_decode(running, tokens[i])

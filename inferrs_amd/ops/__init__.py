@@ -524,6 +524,18 @@ def penalize(logits: torch.Tensor, window: Optional[torch.Tensor], repetition: t
     return logits
 
 
+def window_push(window: torch.Tensor, caps: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """In place: every row's penalty window [rows, w] (int32, -1 = empty) takes the row's new token; row i
+    keeps its last caps[i] tokens (0: no window)."""
+    _dev(window, caps, tokens)
+    _i32(window, "window"); _i32(caps, "caps"); _i32(tokens, "tokens")
+    rows, w = window.shape
+    if caps.numel() != rows or tokens.numel() != rows or not window.is_contiguous():
+        raise KernelError("window_push: one cap and one token per row of a contiguous window")
+    _check(library().ia_window_push(_p(window), rows, w, _p(caps), _p(tokens), _stream()))
+    return window
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            min_p: torch.Tensor, u: torch.Tensor, n_top: Optional[torch.Tensor] = None):
     """One token per row of float32 logits: greedy where temperature < 1e-5, else temperature,

@@ -21,6 +21,11 @@ class Sampler:
     def _dev(self, array: np.ndarray) -> torch.Tensor:
         return torch.from_numpy(array).to(self.device, non_blocking=False)
 
+    def begin_chain(self, params: Sequence[SamplingParams], previous: Sequence[Sequence[int]],
+                    seeds: Sequence[int], steps: int) -> "ChainDraw":
+        """The draws of the next `steps` decode steps of these requests, prepared for the device."""
+        return ChainDraw(self, params, previous, seeds, steps)
+
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], previous: Sequence[Sequence[int]],
                seeds: Sequence[int]) -> List[int]:
         """`logits` float32 [rows, vocab] on the device; row i belongs to a request with
@@ -87,3 +92,63 @@ class Sampler:
             top = tuple((t, v) for t, v in zip(ids[i], lp[i][1:]) if t >= 0)[:p.top_logprobs]
             infos.append(TokenLogprob(tokens[i], lp[i][0], top))
         return tokens, infos
+
+
+class ChainDraw:
+    """The draws of a run of decode steps that are queued without the host in between: what
+    `Sampler.sample` works out from the token lists at every step is kept on the device here, the
+    random numbers of all steps (they depend on seed and step only) and every row's penalty window,
+    which takes the row's new token after each draw.  The tokens are those of single steps."""
+
+    def __init__(self, sampler: "Sampler", params: Sequence[SamplingParams], previous: Sequence[Sequence[int]],
+                 seeds: Sequence[int], steps: int):
+        if any(p.logprobs for p in params):
+            raise ValueError("log-probabilities are reported step by step, not from a run of steps")
+        rows = len(params)
+        self.greedy = all(p.is_plain_greedy for p in params)
+        if self.greedy:
+            return
+        dev = sampler._dev
+        caps = np.asarray([p.repeat_last_n if p.has_penalty else 0 for p in params], dtype=np.int32)
+        width = int(caps.max()) if rows else 0
+        n_bias = max(len(p.logit_bias) for p in params)
+        self.window = self.caps = self.bias_ids = self.bias_vals = None
+        self.penalized = bool(width or n_bias)
+        if self.penalized:
+            rep, freq, pres = np.ones(rows, np.float32), np.zeros(rows, np.float32), np.zeros(rows, np.float32)
+            window = np.full((rows, max(width, 1)), -1, dtype=np.int32)
+            for i, (p, prev) in enumerate(zip(params, previous)):
+                if p.has_penalty:
+                    tail = list(prev[-p.repeat_last_n:])
+                    window[i, :len(tail)] = tail
+                    rep[i], freq[i], pres[i] = p.repetition_penalty, p.frequency_penalty, p.presence_penalty
+            if width:
+                self.window, self.caps = dev(window), dev(caps)
+            self.rep, self.freq, self.pres = dev(rep), dev(freq), dev(pres)
+            if n_bias:
+                ids = np.full((rows, n_bias), -1, dtype=np.int32)
+                vals = np.zeros((rows, n_bias), dtype=np.float32)
+                for i, p in enumerate(params):
+                    for j, (tid, b) in enumerate(sorted(p.logit_bias.items())):
+                        ids[i, j], vals[i, j] = int(tid), float(b)
+                self.bias_ids, self.bias_vals = dev(ids), dev(vals)
+        self.temperature = dev(np.asarray([p.temperature for p in params], dtype=np.float32))
+        self.top_k = dev(np.asarray([p.top_k for p in params], dtype=np.int32))
+        self.top_p = dev(np.asarray([p.top_p for p in params], dtype=np.float32))
+        self.min_p = dev(np.asarray([p.min_p for p in params], dtype=np.float32))
+        # the step of a draw is the number of tokens before it (`sampler.rs:323-325`)
+        self.u = dev(np.asarray([[rand_f32(seed, len(prev) + i) if p.temperature >= SAMPLING_EPS else 0.0
+                                  for p, prev, seed in zip(params, previous, seeds)] for i in range(steps)],
+                                dtype=np.float32).reshape(steps, rows))
+
+    def pick(self, logits: torch.Tensor, step: int, out: torch.Tensor) -> None:
+        """The tokens of the run's `step`-th step from its logits, into `out` (int32 [rows], on the device)."""
+        if self.greedy:
+            ops.argmax(logits, out=out)
+            return
+        if self.penalized:
+            logits = logits.clone()
+            ops.penalize(logits, self.window, self.rep, self.freq, self.pres, self.bias_ids, self.bias_vals)
+        out.copy_(ops.sample(logits, self.temperature, self.top_k, self.top_p, self.min_p, self.u[step]))
+        if self.window is not None:
+            ops.window_push(self.window, self.caps, out)

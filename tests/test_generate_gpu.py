@@ -179,6 +179,37 @@ def test_runs_of_decode_steps_give_the_same_tokens_as_single_steps(tiny, dtype):
     assert results[8][1] == results[1][1] and results[8][2] == results[1][2] and len(results[8][2]) == 23
 
 
+def test_runs_of_decode_steps_draw_the_same_tokens_as_single_steps(tiny):
+    """Requests that draw (temperature, top-k, top-p, min-p, penalties over a window that fills up and then
+    moves, a logit bias; a greedy one with a penalty among them) also decode several steps at a time: the
+    random numbers of the run and the penalty windows live on the device, and the tokens are those of
+    single steps."""
+    from inferrs_amd.engine import Engine, GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 500 + n) for n in (7, 30, 12, 3)]
+    sps = [SamplingParams(seed=11, max_tokens=45),                                           # the reference's defaults
+           SamplingParams(seed=12, max_tokens=45, temperature=1.2, top_k=0, top_p=0.8, repetition_penalty=1.0,
+                          frequency_penalty=0.3, presence_penalty=0.2, repeat_last_n=9),
+           SamplingParams(seed=13, max_tokens=31, temperature=0.0, repetition_penalty=1.4, repeat_last_n=20),
+           SamplingParams(seed=14, max_tokens=45, temperature=0.9, top_k=12, min_p=0.05, repetition_penalty=1.0,
+                          logit_bias={5: 2.0, 17: -3.0})]
+    results = {}
+    for run in (1, 8):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=64, max_seqs=5)
+        loop = GenerationLoop(eng, decode_run=run, stop_token_ids=[])
+        reqs = [loop.add(p, s) for p, s in zip(prompts, sps)]
+        loop.run()
+        results[run] = [list(r.output) for r in reqs]
+        if run == 8:
+            assert eng.graph_replays > 20
+        eng.cache.check_invariants()
+        assert not eng.cache.sequences
+    assert results[8] == results[1]
+    assert [len(o) for o in results[8]] == [45, 45, 31, 45]
+
+
 def test_generation_reports_log_probabilities(tiny):
     """`logprobs` through the entry point: one record per generated token, consistent with the plain
     model's softmax at that place (temperature 1, nothing filtered, so the kept list is the vocabulary)."""
