@@ -197,7 +197,7 @@ extern "C" int ia_window_push(int* window, int rows, int w, const int* caps, con
 }
 
 // ---- sampling -------------------------------------------------------------------------------
-#define SAMPLE_THREADS 512
+#define SAMPLE_THREADS 1024
 
 // Keys order like the values they come from; NaN sorts below everything.
 __device__ __forceinline__ uint32_t order_key(float z) {
@@ -337,8 +337,25 @@ __device__ int next_in_order(const uint32_t* __restrict__ keys, int vocab, uint3
 // the row's top_k tokens are picked out first (three histograms over the key's bits find the k-th largest
 // key; equal keys are taken by ascending index), sorted in shared memory, and one thread then does what the
 // reference does with its sorted list, in its order and with its sums (sampler.rs:256-335): six passes over
-// the row instead of the hundred of the bisections below (16 rows of 152 k: 4.5 ms -> 0.2 ms).
+// the row instead of the hundred of the bisections below (16 rows of 152 k: 2.5 ms -> 0.16 ms).
 #define SAMPLE_FAST_K 1024
+// f(index, key) for all keys of a row, this thread's share, four loads under way at a time.
+template <typename F>
+__device__ __forceinline__ void for_each_key(const uint32_t* __restrict__ keys, int vocab, F f) {
+    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
+        uint32_t k[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            k[j] = c < vocab ? keys[c] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            if (c < vocab) f(c, k[j]);
+        }
+    }
+}
 __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__ keys, const float* __restrict__ probs,
                              int vocab, int rowi, int k, float tp, float mp, float u, int want_top,
                              float* __restrict__ lp_out, int* __restrict__ lp_ids, int* s_counts) {
@@ -353,20 +370,36 @@ __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
         const int shift = 32 - prefix_bits - bits;
         for (int i = threadIdx.x; i < 2048; i += blockDim.x) hist[i] = 0;
         __syncthreads();
-        for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-            const uint32_t key = keys[c];
+        for_each_key(keys, vocab, [&](int, uint32_t key) {
             if (prefix_bits == 0 || (key >> (32 - prefix_bits)) == prefix)
                 atomicAdd(&hist[(key >> shift) & ((1u << bits) - 1u)], 1);
-        }
+        });
         __syncthreads();
-        if (threadIdx.x == 0) {
-            int cum = 0, b = (1 << bits) - 1;
-            for (; b > 0; --b) {
-                if (cum + hist[b] >= need) break;
-                cum += hist[b];
+        // the highest bin at which the count from the top reaches `need`: lane l of the first wave adds up
+        // bins top - 32 l - 31 .. top - 32 l, the lanes' sums are scanned, and the lane where the count is
+        // reached walks its own bins
+        if (threadIdx.x < IA_WAVE) {
+            const int n_bins = 1 << bits, per = n_bins / IA_WAVE;
+            const int top = n_bins - 1 - (int)threadIdx.x * per;
+            int mine = 0;
+            for (int i = 0; i < per; ++i) mine += hist[top - i];
+            int upto = mine;                                   // inclusive scan over the lanes
+#pragma unroll
+            for (int o = 1; o < IA_WAVE; o <<= 1) {
+                const int other = __shfl_up(upto, o, IA_WAVE);
+                if ((int)threadIdx.x >= o) upto += other;
             }
-            s_bin = b;
-            s_above = cum;
+            const unsigned long long reached = __ballot(upto >= need);
+            const int first = reached ? __ffsll((long long)reached) - 1 : IA_WAVE - 1;
+            if ((int)threadIdx.x == first) {
+                int cum = upto - mine, b = top;
+                for (; b > top - per + 1; --b) {
+                    if (cum + hist[b] >= need) break;
+                    cum += hist[b];
+                }
+                s_bin = b;
+                s_above = cum;
+            }
         }
         __syncthreads();
         need -= s_above;
@@ -381,13 +414,12 @@ __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
     if (ties > need) last_tie = nth_with_key(keys, vocab, kth, need, s_counts);
     if (threadIdx.x == 0) s_n = 0;
     __syncthreads();
-    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-        const uint32_t key = keys[c];
+    for_each_key(keys, vocab, [&](int c, uint32_t key) {
         if (key > kth || (key == kth && c <= last_tie)) {
             const int slot = atomicAdd(&s_n, 1);
             if (slot < SAMPLE_FAST_K) cand[slot] = ((unsigned long long)key << 32) | (uint32_t)~(uint32_t)c;
         }
-    }
+    });
     __syncthreads();
     const int n = s_n < k ? s_n : k;                        // = k
     int padded = 2;
@@ -405,6 +437,9 @@ __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
             }
         }
     __syncthreads();
+    __shared__ float cprob[SAMPLE_FAST_K];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) cprob[i] = probs[(int)~(uint32_t)(cand[i] & 0xffffffffull)];
+    __syncthreads();
     if (threadIdx.x != 0) return;
     // ---- the reference's steps 7 to 12 on its sorted list
     auto index_of = [&](int i) { return (int)~(uint32_t)(cand[i] & 0xffffffffull); };
@@ -412,22 +447,22 @@ __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
     if (tp < 1.0f) {
         float cumsum = 0.f;
         for (int i = 0; i < len; ++i) {
-            cumsum += probs[index_of(i)];
+            cumsum += cprob[i];
             if (cumsum >= tp) { len = i + 1; break; }
         }
     }
     if (mp > 0.0f && len > 0) {
-        const float threshold = probs[index_of(0)] * mp;
+        const float threshold = cprob[0] * mp;
         int cut = 0;
-        while (cut < len && probs[index_of(cut)] >= threshold) ++cut;
+        while (cut < len && cprob[cut] >= threshold) ++cut;
         if (cut > 0) len = cut;
     }
     float filtered = 0.f;
-    for (int i = 0; i < len; ++i) filtered += probs[index_of(i)];
+    for (int i = 0; i < len; ++i) filtered += cprob[i];
     const float denom = filtered > 0.f ? filtered : 1.0f;
     if (want_top >= 0)
         for (int i = 0; i < want_top && i < SAMPLE_MAX_TOP && i < len; ++i) {
-            const float pi = probs[index_of(i)];
+            const float pi = cprob[i];
             lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + i] = index_of(i);
             lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + i] = pi > 0.f ? logf(pi / denom) : -INFINITY;
         }
@@ -439,14 +474,14 @@ __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
     float rng = u;
     int at = len - 1;
     for (int i = 0; i < len; ++i) {
-        const float norm = probs[index_of(i)] / filtered;
+        const float norm = cprob[i] / filtered;
         if (rng < norm) { at = i; break; }
         rng -= norm;
     }
     const int token = index_of(at);
     out[rowi] = token;
     if (want_top >= 0) {
-        const float pt = probs[token] / filtered;
+        const float pt = cprob[at] / filtered;
         lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = pt > 0.f ? logf(pt) : -INFINITY;
     }
 }
@@ -483,11 +518,24 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     float* probs = (float*)(keys + vocab);
 
     // temperature, softmax (sampler.rs:232-249)
+    // (the passes over the row keep four loads under way; a thread's sums run in the order of its indices)
     float mx = -INFINITY;
-    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-        const float z = row[c] / temp;
-        probs[c] = z;
-        mx = fmaxf(mx, z);
+    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
+        float z[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            z[j] = c < vocab ? row[c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            if (c < vocab) {
+                z[j] = z[j] / temp;
+                probs[c] = z[j];
+                mx = fmaxf(mx, z[j]);
+            }
+        }
     }
     mx = wave_max(mx);
     __syncthreads();
@@ -495,18 +543,42 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     __syncthreads();
     for (int w = 0; w < SAMPLE_THREADS / IA_WAVE; ++w) mx = fmaxf(mx, scratch[w]);
     float sum = 0.f;
-    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-        const float e = expf(probs[c] - mx);
-        probs[c] = e;
-        sum += e;
+    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
+        float z[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            z[j] = c < vocab ? probs[c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            if (c < vocab) {
+                const float e = expf(z[j] - mx);
+                probs[c] = e;
+                sum += e;
+            }
+        }
     }
     sum = block_sum(sum, scratch);
     // The list is ordered by the probabilities themselves, as the reference sorts them: logits whose
     // probabilities round to the same number (or vanish together) are ties, taken in index order.
-    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-        const float pr = sum > 0.f ? probs[c] / sum : probs[c];
-        probs[c] = pr;
-        keys[c] = order_key(pr);
+    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
+        float e[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            e[j] = c < vocab ? probs[c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            if (c < vocab) {
+                const float pr = sum > 0.f ? e[j] / sum : e[j];
+                probs[c] = pr;
+                keys[c] = order_key(pr);
+            }
+        }
     }
     __syncthreads();
 
