@@ -114,11 +114,35 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // two rows a load), puts it into its own corner of shared memory and reads the operand layout from
 // there.  Measured on the logits head at 8 rows: 4.8 -> 5.9 TB/s.
 #define SK_STAGE_PAD 16     // bytes between staged rows, against bank conflicts
+
+// A residual stream around the product, so that no kernel of its own adds and norms between two
+// products (decode steps: such a kernel is all launch and latency).  The norm of a row,
+// x * rsqrt(mean(x^2) + eps) * g, is split in two: the product before the norm forms x * g while it
+// has the row's new values at hand, and the product after it applies the row's scale to its sums.
+//   resid / sums_out / scaled_out / next_w: the product is not stored but added to `resid` [M, N] in place, as
+//     the add kernel would (the product rounded to the storage precision, the sum formed in 32-bit and
+//     rounded); the block writes the sum of squares of its 16 features of every new row to
+//     sums_out[row][block] and the new values times next_w (or 1 + next_w) to scaled_out [M, N].
+//   sums_in: x holds such scaled rows, and sums_in[row][0 .. n_sums) their sums of squares: every sum of
+//     the product is multiplied by rsqrt(sum of the row's sums_in / K + eps) before it is rounded.
+// One rounding of the normed value, as in the norm kernel, at another place (before the scale instead of
+// after it); the sum of squares is added up in another order than there.
+struct SkinnyStream {
+    bf16_t* resid;
+    float* sums_out;
+    bf16_t* scaled_out;
+    const float* next_w;
+    const float* sums_in;
+    int n_sums;
+    float eps;
+    int add_one;
+};
+
 // STAGE: 0, or the k steps of a staged chunk (8 or 16).
 template <int MT, int RT, bool DUAL, int STAGE>
 __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     void* __restrict__ out, int out_f32, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-    int M, int N, int K, int kper, int m_base, int rot_mul) {
+    int M, int N, int K, int kper, int m_base, int rot_mul, const SkinnyStream st) {
     constexpr int NA = DUAL ? 2 : 1;
     static_assert(!STAGE || MT == 1, "staging holds one tile of batch rows");
     extern __shared__ f32x4 red[];      // [waves][NA][RT][MT][64], then with STAGE [waves][rows][chunk of x]
@@ -166,6 +190,29 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     constexpr int STAGE_LANES = UNROLL * 4;                               // lanes that bring one row
     const int stage_rows = M - m_base < 16 ? M - m_base : 16;
     char* const stage = (char*)(red + (size_t)waves * NA * RT * MT * IA_WAVE) + (size_t)wave * stage_rows * STAGE_PITCH;
+    // What the end of the kernel needs of a stream is asked for now, so that its way from memory lies behind the
+    // product: the rows' sums of squares (a row a wave, 16 bytes a lane), and for the wave that stores, the
+    // stream's old values and the next norm's weights.
+    __shared__ float ss_row[16];
+    constexpr int SS_ROWS = (16 + 7) / 8;                   // rows a wave when eight waves share out sixteen
+    float4 ss_mine[SS_ROWS];
+    const bool ss_wide = st.sums_in != nullptr && (st.n_sums & 3) == 0 && st.n_sums <= 4 * IA_WAVE;
+    if (ss_wide) {                                          // (a stream has one tile of batch rows)
+#pragma unroll
+        for (int j = 0; j < SS_ROWS; ++j) {
+            const int m = wave + j * waves;
+            ss_mine[j] = (m < stage_rows && 4 * lane < st.n_sums)
+                             ? *(const float4*)(st.sums_in + (size_t)(m_base + m) * st.n_sums + 4 * lane)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    uint2 resid_old = make_uint2(0u, 0u);
+    float4 next_w4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool resid_ahead = st.resid != nullptr && wave == 0 && (N & 3) == 0 && n0 + 4 * g + 3 < N && m_base + r < M;
+    if (resid_ahead) {
+        resid_old = *(const uint2*)(st.resid + (size_t)(m_base + r) * N + n0 + 4 * g);
+        if (st.scaled_out != nullptr) next_w4 = *(const float4*)(st.next_w + n0 + 4 * g);
+    }
     const int whole = K / SK_KSTEP;                         // steps that lie inside K entirely
     const int ke = ks1 < whole ? ks1 : whole;
     const int len = ke - ks0;
@@ -282,6 +329,26 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                 }
         }
     }
+    if (st.sums_in != nullptr) {
+        // every row's sum of squares, a row a wave: a lane's four neighbours first, then across the lanes
+        auto one_by_one = [&](int m) {
+            float ss = 0.f;
+            for (int b = lane; b < st.n_sums; b += IA_WAVE) ss += st.sums_in[(size_t)(m_base + m) * st.n_sums + b];
+            return ss;
+        };
+#pragma unroll
+        for (int j = 0; j < SS_ROWS; ++j) {
+            const int m = wave + j * waves;
+            if (m >= stage_rows) continue;
+            float ss = ss_wide ? ((ss_mine[j].x + ss_mine[j].y) + ss_mine[j].z) + ss_mine[j].w : one_by_one(m);
+            ss = wave_sum(ss);
+            if (lane == 0) ss_row[m] = ss;
+        }
+        for (int m = wave + SS_ROWS * waves; m < stage_rows; m += waves) {
+            const float ss = wave_sum(one_by_one(m));
+            if (lane == 0) ss_row[m] = ss;
+        }
+    }
     if (waves > 1) {
 #pragma unroll
         for (int q = 0; q < NA; ++q)
@@ -290,6 +357,8 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
 #pragma unroll
                 for (int u = 0; u < MT; ++u)
                     red[(((wave * NA + q) * RT + t) * MT + u) * IA_WAVE + lane] = acc[q][t][u];
+        __syncthreads();
+    } else if (st.sums_in != nullptr) {
         __syncthreads();
     }
     // the tiles are shared out between the waves for the sum and the store
@@ -313,6 +382,58 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                 }
             }
             const int m = m_base + u * 16 + r;
+            if constexpr (MT == 1) {
+                if (st.sums_in != nullptr) {
+                    const float scale = 1.0f / sqrtf(ss_row[r < stage_rows ? r : 0] / (float)K + st.eps);
+#pragma unroll
+                    for (int q = 0; q < NA; ++q) { s[q][0] *= scale; s[q][1] *= scale; s[q][2] *= scale; s[q][3] *= scale; }
+                }
+            }
+            if constexpr (!DUAL && RT == 1 && MT == 1) {
+                if (st.resid != nullptr) {
+                    // (all lanes of the wave stay for the sums; rows and features outside add nothing)
+                    const int nb = n0 + 4 * g;
+                    float sq = 0.f;
+                    if (resid_ahead) {
+                        const uint16_t old[4] = {(uint16_t)resid_old.x, (uint16_t)(resid_old.x >> 16),
+                                                 (uint16_t)resid_old.y, (uint16_t)(resid_old.y >> 16)};
+                        const float gw[4] = {next_w4.x, next_w4.y, next_w4.z, next_w4.w};
+                        uint16_t h[4], hw[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float product = bf16_bits_to_f32(f32_to_bf16_bits(s[0][i]));
+                            h[i] = f32_to_bf16_bits(product + bf16_bits_to_f32(old[i]));
+                            const float hf = bf16_bits_to_f32(h[i]);
+                            sq += hf * hf;
+                            hw[i] = f32_to_bf16_bits(hf * (st.add_one ? 1.0f + gw[i] : gw[i]));
+                        }
+                        *(uint2*)(st.resid + (size_t)m * N + nb) =
+                            make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+                        if (st.scaled_out != nullptr)
+                            *(uint2*)(st.scaled_out + (size_t)m * N + nb) =
+                                make_uint2((uint32_t)hw[0] | ((uint32_t)hw[1] << 16), (uint32_t)hw[2] | ((uint32_t)hw[3] << 16));
+                    } else if (m < M) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            if (nb + i >= N) continue;
+                            bf16_t* at = st.resid + (size_t)m * N + nb + i;
+                            const float product = bf16_bits_to_f32(f32_to_bf16_bits(s[0][i]));
+                            const uint16_t h = f32_to_bf16_bits(product + bf16_bits_to_f32(at->bits));
+                            at->bits = h;
+                            const float hf = bf16_bits_to_f32(h);
+                            sq += hf * hf;
+                            if (st.scaled_out != nullptr) {
+                                const float gw = st.next_w[nb + i];
+                                st.scaled_out[(size_t)m * N + nb + i].bits = f32_to_bf16_bits(hf * (st.add_one ? 1.0f + gw : gw));
+                            }
+                        }
+                    }
+                    sq += __shfl_xor(sq, 16, IA_WAVE);
+                    sq += __shfl_xor(sq, 32, IA_WAVE);
+                    if (g == 0 && m < M) st.sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
+                    continue;
+                }
+            }
             if (m >= M) continue;
             const int nb = n0 + t * 16 + 4 * g;
             float v[4];
@@ -372,6 +493,7 @@ static int skinny_waves(int N, int K, int rt, int tiles_per_wave) {
 
 #define SK_STAGE_LDS_MOST (96 * 1024)
 #define SK_STAGE16_LDS_MOST (160 * 1024)     // one block a compute unit: all of its shared memory
+#define SK_SCALES_RESERVE 256                // the rows' sums of squares: static shared memory beside the launch's own area
 
 // Shared memory beyond 64 KiB has to be asked for, once per instantiation.
 template <int MT, int RT, bool DUAL, int STAGE>
@@ -386,9 +508,20 @@ static int skinny_ask_shared(int bytes) {
     return 0;
 }
 
+static int skinny_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    return cus;
+}
+
 template <int MT, int RT, bool DUAL>
 static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* w, int M, int N, int K,
-                         int m_base, hipStream_t stream) {
+                         int m_base, const SkinnyStream& st, hipStream_t stream) {
     const int waves = skinny_waves(N, K, RT, (DUAL ? 2 : 1) * RT * MT);
     const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
     const int kper = (ksteps + waves - 1) / waves;
@@ -399,20 +532,14 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
         const int rows = M - m_base < 16 ? M - m_base : 16;
         const size_t staged8 = tiles + (size_t)waves * rows * (8 * 2 * SK_KSTEP + SK_STAGE_PAD);
         const size_t staged16 = tiles + (size_t)waves * rows * (16 * 2 * SK_KSTEP + SK_STAGE_PAD);
-        static int cus = 0;
-        if (cus == 0) {
-            int dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-                cus = 256;
-        }
+        const int cus = skinny_cus();
         int stage = 0;
         if (g_stage && rows >= 2 && (int)grid >= 2 * cus) {
             // Staging pays where blocks stream for long: with at least two blocks for every compute unit,
             // with 2 to 12 batch rows (one row is one cache line a load anyway; beyond 12 the staging area
             // leaves too few blocks on a compute unit), and with whole chunks of 8 k steps in a wave's
             // range.  Measured at 8 rows: gate|up 46 -> 40 us, logits head 261 -> 224 us.
-            if (rows <= 12 && kper >= 8 && staged8 <= SK_STAGE_LDS_MOST) stage = 8;
+            if (rows <= 12 && kper >= 8 && staged8 <= SK_STAGE_LDS_MOST - SK_SCALES_RESERVE) stage = 8;
         } else if (g_stage && rows >= 2 && !DUAL && RT == 1) {
             // A weight that one round of blocks covers (o, down, qkv) is read in one burst, and what counts
             // is how much a wave has in flight: chunks of 16 steps, as much as without staging, and up to
@@ -421,36 +548,44 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
             // the area leaves room for one block of qkv's 384 on a compute unit, and they go in two rounds;
             // chunks of 8, which keep it one round, were no faster: 15.8 against 16.4 us at 10 rows, 17.4
             // against 16.7 at 16.)
-            if (kper % 16 == 0 && staged16 <= SK_STAGE16_LDS_MOST) stage = 16;
+            if (kper % 16 == 0 && staged16 <= SK_STAGE16_LDS_MOST - SK_SCALES_RESERVE) stage = 16;
         }
         if (stage == 8) {
-            if (skinny_ask_shared<MT, RT, DUAL, 8>(SK_STAGE_LDS_MOST)) return 1;
+            if (skinny_ask_shared<MT, RT, DUAL, 8>(SK_STAGE_LDS_MOST - SK_SCALES_RESERVE)) return 1;
             gemm_skinny_kernel<MT, RT, DUAL, 8><<<grid, waves * IA_WAVE, staged8, stream>>>(
-                out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
+                out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul, st);
             return 0;
         }
         if constexpr (!DUAL && RT == 1) {
             if (stage == 16) {
-                if (skinny_ask_shared<MT, RT, DUAL, 16>(SK_STAGE16_LDS_MOST)) return 1;
+                if (skinny_ask_shared<MT, RT, DUAL, 16>(SK_STAGE16_LDS_MOST - SK_SCALES_RESERVE)) return 1;
                 gemm_skinny_kernel<MT, RT, DUAL, 16><<<grid, waves * IA_WAVE, staged16, stream>>>(
-                    out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
+                    out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul, st);
                 return 0;
             }
         }
     }
     gemm_skinny_kernel<MT, RT, DUAL, 0><<<grid, waves * IA_WAVE, waves > 1 ? tiles : 0, stream>>>(
-        out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul);
+        out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul, st);
     return 0;
 }
 
-// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` out[M, N] = silu(x . w[0:N]^T) * (x . w[N:2N]^T).
-extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
-                                   int out_dtype, int dual, hipStream_t stream) {
+static int skinny_product(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype, int dual,
+                          const SkinnyStream& st, hipStream_t stream) {
     IA_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     IA_CHECK(K % 8 == 0, "gemm_skinny: K=%d must be a multiple of 8 (use the tiled product)", K);
     IA_CHECK(out_dtype == IA_F32 || out_dtype == IA_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
     IA_CHECK((((uintptr_t)x | (uintptr_t)w) & 15) == 0, "gemm_skinny: x and w must be 16-byte aligned");
     IA_CHECK((((uintptr_t)out) & 15) == 0, "gemm_skinny: out must be 16-byte aligned");
+    const bool streams = st.resid != nullptr || st.sums_in != nullptr;
+    IA_CHECK(!streams || (M <= 16 && N < 65536), "gemm_skinny: a residual stream around the product takes up to 16 rows "
+             "and fewer than 65536 features, got M=%d N=%d", M, N);
+    IA_CHECK(st.resid == nullptr || (!dual && st.sums_out != nullptr && (st.scaled_out == nullptr) == (st.next_w == nullptr)),
+             "gemm_skinny: the sum into a residual stream is for plain products, needs a place for the sums of squares, "
+             "and the next norm's weight together with a place for the scaled rows");
+    IA_CHECK(st.sums_in == nullptr || st.n_sums > 0, "gemm_skinny: scaled rows come with their sums of squares");
+    IA_CHECK((((uintptr_t)st.resid | (uintptr_t)st.scaled_out | (uintptr_t)st.next_w) & 15) == 0,
+             "gemm_skinny: the stream's arrays must be 16-byte aligned");
     if (M == 0) return 0;
     const int out_f32 = out_dtype == IA_F32;
     const bf16_t* xb = (const bf16_t*)x;
@@ -459,19 +594,43 @@ extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int 
         const int rows = M - m_base;
         int rc = 0;
         if (dual) {
-            if (rows <= 16) rc = launch_skinny<1, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
-            else if (rows <= 32) rc = launch_skinny<2, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
-            else rc = launch_skinny<4, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            if (rows <= 16) rc = launch_skinny<1, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
+            else if (rows <= 32) rc = launch_skinny<2, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
+            else rc = launch_skinny<4, 1, true>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
         } else {
             // very tall weights (a logits head) have blocks to spare: two row tiles a wave halve the
             // loads of the activations
-            if (rows <= 16 && N >= 65536) rc = launch_skinny<1, 2, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
-            else if (rows <= 16) rc = launch_skinny<1, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
-            else if (rows <= 32) rc = launch_skinny<2, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
-            else rc = launch_skinny<4, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, stream);
+            if (rows <= 16 && N >= 65536) rc = launch_skinny<1, 2, false>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
+            else if (rows <= 16) rc = launch_skinny<1, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
+            else if (rows <= 32) rc = launch_skinny<2, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
+            else rc = launch_skinny<4, 1, false>(out, out_f32, xb, wb, M, N, K, m_base, st, stream);
         }
         if (rc) return rc;
         IA_LAUNCH_CHECK("gemm_skinny");
     }
     return 0;
+}
+
+// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` out[M, N] = silu(x . w[0:N]^T) * (x . w[N:2N]^T).
+extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
+                                   int out_dtype, int dual, hipStream_t stream) {
+    const SkinnyStream none = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0};
+    return skinny_product(out, x, w, M, N, K, out_dtype, dual, none, stream);
+}
+
+// Blocks of the plain product with N output features: the columns of its sums of squares.
+extern "C" int ia_gemm_skinny_blocks(int N) { return (N + 15) / 16; }
+
+// The product with a residual stream around it (up to 16 rows; see SkinnyStream).
+//   resid != null (plain products): resid[M, N] += product in place, nothing goes to `out` (may be null);
+//     sums_out[M][ia_gemm_skinny_blocks(N)] receives the sums of squares of the new rows, block by block, and
+//     scaled_out[M, N] (may be null, with next_w) the new rows times next_w [N] (1 + next_w with add_one).
+//   sums_in != null: x [M, K] holds such scaled rows and sums_in[M][n_sums] their sums of squares; the
+//     product's sums are multiplied by rsqrt(sum / K + eps) before anything else happens to them.
+extern "C" int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype,
+                                     int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
+                                     int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream) {
+    const SkinnyStream st = {(bf16_t*)resid, sums_out, (bf16_t*)scaled_out, next_w, sums_in, n_sums, eps, add_one};
+    IA_CHECK(out != nullptr || resid != nullptr, "gemm_skinny: no place for the result");
+    return skinny_product(out, x, w, M, N, K, out_dtype, dual, st, stream);
 }

@@ -48,6 +48,8 @@ class StepContext:
     n_single: int = 0            # the first n_single requests bring one token each (they come first)
     max_kv_single: int = 0       # the greatest length among those, after the step
     max_kv_multi: int = 0        # and among the others
+    stream: Optional[torch.Tensor] = None   # set by a block around a part that may add its output to it itself
+    stream_norm: Any = None                 # and the norm part that will read the stream next
     _tables: Dict[Any, Any] = field(default_factory=dict)
 
     @property

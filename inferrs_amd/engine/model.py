@@ -76,18 +76,22 @@ class DecoderModel:
         """Runs the step's tokens through every stop of the schedule (which appends to the
         caches) and returns float32 logits `[n_want, vocab]`."""
         x = ops.embed_gather(self.embed, ctx.token_ids)
-        pending: Optional[torch.Tensor] = None
+        pending = None                               # a block's output that is not added to x yet
         for stop, e in enumerate(self.spec.schedule):
             cache = storage.layers.get(self.spec.cache_stop(stop))
             if cache is not None and e.cache_of is not None:
                 cache = cache.reader()
-            x, pending = self.blocks[e.layer].forward(ctx, x, pending, cache)
+            after = self.spec.schedule[stop + 1].layer if stop + 1 < len(self.spec.schedule) else None
+            next_norm = self.blocks[after].norm_mixer if after is not None else None
+            x, pending = self.blocks[e.layer].forward(ctx, x, pending, cache, next_norm)
         n_want = ctx.want_rows.numel()
         if n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         xs = ops.gather_rows(x, ctx.want_rows)
-        ps = ops.gather_rows(pending, ctx.want_rows)
-        h = self.final_norm.add_forward(xs, ps)
+        if isinstance(pending, ops.Added):           # the last block has added its output to x itself
+            h = self.final_norm.forward(xs)
+        else:
+            h = self.final_norm.add_forward(xs, ops.gather_rows(pending, ctx.want_rows))
         return self.head(h, out_dtype=torch.float32)
 
     def weight_bytes(self) -> int:

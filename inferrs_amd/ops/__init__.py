@@ -458,7 +458,89 @@ def widen(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+# ---- a residual stream around the skinny product ---------------------------------------------
+# Decode steps have a few rows, and a kernel of its own that adds a product to the stream and norms the
+# sum is all launch and latency.  The product before such a norm can add itself to the stream
+# (`linear_add`): it leaves every row's sum of squares, block by block, and the new rows times the
+# norm's weight; the product after the norm (`linear` / `gated_silu_linear` given `NormedRows`) takes
+# those rows and multiplies its sums by the row's scale, rsqrt(mean of squares + eps).
+
+STREAM_MAX_ROWS = 12          # rows up to which the products take over the sums and norms of a step
+
+
+class Added:
+    """What a part returns instead of its output when it has added it to the step's stream itself:
+    `sums` [rows, blocks] are the partial sums of squares of the stream's new rows and `scaled` the
+    new rows times the weight of `norm` (the norm part that comes next), or None."""
+    __slots__ = ("sums", "scaled", "norm")
+
+    def __init__(self, sums: torch.Tensor, scaled: Optional[torch.Tensor] = None, norm=None):
+        self.sums, self.scaled, self.norm = sums, scaled, norm
+
+
+class NormedRows:
+    """Rows of a stream `x` whose norm, rmsnorm(x; weight, eps), is left to the product that reads them:
+    `scaled` = x * weight (rounded once) and `sums` [rows, blocks] the rows' sums of squares."""
+    __slots__ = ("x", "scaled", "sums", "weight", "eps", "add_one")
+
+    def __init__(self, x: torch.Tensor, scaled: torch.Tensor, sums: torch.Tensor, weight: torch.Tensor, eps: float,
+                 add_one: bool):
+        self.x, self.scaled, self.sums, self.weight = x, scaled, sums, weight
+        self.eps, self.add_one = float(eps), bool(add_one)
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    @property
+    def dtype(self):
+        return self.x.dtype
+
+    def materialize(self) -> torch.Tensor:
+        return rmsnorm(self.x, self.weight, self.eps, self.add_one)
+
+
+def _stream_product(x: torch.Tensor, w: torch.Tensor, n: int, out_dtype, dual: bool, resid=None, sums_out=None,
+                    scaled_out=None, next_w=None, add_one: bool = False, sums_in=None, eps: float = 0.0):
+    m, k = x.shape
+    out = None if resid is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _check(library().ia_gemm_skinny_stream(
+        _p(out), _p(x), _p(w), m, n, k, _DT[out_dtype], int(dual), _p(resid), _p(sums_out), _p(scaled_out), _p(next_w),
+        int(add_one), _p(sums_in), sums_in.shape[1] if sums_in is not None else 0, ctypes.c_float(eps), _stream()))
+    return out
+
+
+def _takes_normed_rows(x: NormedRows, w: torch.Tensor, n: int) -> bool:
+    m, k = x.scaled.shape
+    return (m <= SKINNY_MAX_ROWS and x.scaled.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] == k
+            and skinny_fits(x.scaled, w) and n < 65536 and x.sums.dtype == torch.float32 and x.sums.shape[0] == m
+            and x.sums.is_contiguous() and x.scaled.is_contiguous())
+
+
+def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=None):
+    """resid += x . w^T in place, as `add_rmsnorm` would add the product (rounded, then summed in 32-bit
+    and rounded), by the skinny kernel itself.  Returns (sums, scaled): the partial sums of squares of the
+    new rows [rows, blocks], and the new rows times the weight of `next_norm` (a norm part with `weight`
+    and `add_one`; None: no such rows); or None when this product cannot (the caller then forms it and
+    lets the norm add it)."""
+    m, k = x.shape
+    n = w.shape[0]
+    if (m > SKINNY_MAX_ROWS or m == 0 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k
+            or not skinny_fits(x, w) or n >= 65536 or resid.dtype != torch.bfloat16 or tuple(resid.shape) != (m, n)
+            or not resid.is_contiguous()):
+        return None
+    next_w = getattr(next_norm, "weight", None)
+    if next_w is not None and (next_w.dtype != torch.float32 or next_w.numel() != n):
+        next_w = None
+    _dev(x, w, resid, next_w)
+    sums = torch.empty((m, library().ia_gemm_skinny_blocks(n)), dtype=torch.float32, device=x.device)
+    scaled = torch.empty_like(resid) if next_w is not None else None
+    _stream_product(x, w, n, torch.bfloat16, False, resid=resid, sums_out=sums, scaled_out=scaled, next_w=next_w,
+                    add_one=bool(getattr(next_norm, "add_one", False)))
+    return sums, scaled
+
+
+def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
     skinny MFMA kernel for up to SKINNY_MAX_ROWS rows, the vendor's GEMM beyond that (the reference uses
     cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
@@ -466,6 +548,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     result widened, which is what the reference does for every row (its logits are computed in
     the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`)."""
     out_dtype = out_dtype or x.dtype
+    if isinstance(x, NormedRows):
+        if _takes_normed_rows(x, w, w.shape[0]):
+            _dev(x.scaled, w, x.sums)
+            return _stream_product(x.scaled, w, w.shape[0], out_dtype, False, sums_in=x.sums, eps=x.eps)
+        x = x.materialize()
     if x.dtype == torch.float32:
         return gemm_tiled(x, w, out_dtype)
     m, k = x.shape
@@ -564,9 +651,15 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return out if n_top is None else (out, lp, ids)
 
 
-def gated_silu_linear(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(x . gate^T) * (x . up^T) for w_gate_up = [gate; up]: one fused kernel for few bfloat16
     rows, else the product followed by the element-wise kernel."""
+    if isinstance(x, NormedRows):
+        if w_gate_up.shape[0] % 2 == 0 and _takes_normed_rows(x, w_gate_up, w_gate_up.shape[0] // 2):
+            _dev(x.scaled, w_gate_up, x.sums)
+            return _stream_product(x.scaled, w_gate_up, w_gate_up.shape[0] // 2, x.scaled.dtype, True,
+                                   sums_in=x.sums, eps=x.eps)
+        x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
         return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True)
     return silu_mul(linear(x, w_gate_up))

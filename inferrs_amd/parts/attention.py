@@ -23,6 +23,8 @@ from .linear import Linear
 @register_mixer("attention")
 class Attention(Mixer):
     graph_safe = True
+    takes_normed_rows = True      # the q|k|v product norms the rows it is given as `ops.NormedRows`
+    adds_to_stream = True         # the output projection adds itself to `ctx.stream` where it can
 
     @classmethod
     def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorSpec]:
@@ -64,7 +66,16 @@ class Attention(Mixer):
             self.norm_eps, self.norm_add_one = 0.0, False
         self.position = part_class("position", spec.position)(spec.position, {}, dtype, device)
 
-    def forward(self, ctx, h: torch.Tensor, cache) -> torch.Tensor:
+    def _project(self, ctx, a: torch.Tensor):
+        """The output projection: added to the step's stream by the product itself where that can be."""
+        if getattr(ctx, "stream", None) is not None:
+            norm = getattr(ctx, "stream_norm", None)
+            added = ops.linear_add(a, self.o.weight, ctx.stream, norm)
+            if added is not None:
+                return ops.Added(added[0], added[1], norm)
+        return self.o(a)
+
+    def forward(self, ctx, h, cache):
         s = self.spec
         group = ctx.groups[cache.group]
         qkv = self.qkv(h)
@@ -79,7 +90,7 @@ class Attention(Mixer):
                 nkv=s.n_kv_heads, d=s.head_dim, slots=group.slots if cache.writable else None,
                 q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one,
                 cos=cos, sin=sin, max_kv_len=ctx.max_kv_len, window=s.window, scale=s.softmax_scale)
-            return self.o(a.view(a.shape[0], s.n_heads * s.head_dim))
+            return self._project(ctx, a.view(a.shape[0], s.n_heads * s.head_dim))
         q = ops.qk_rope_kv(
             qkv, s.n_heads, s.n_kv_heads, s.head_dim,
             q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one,
@@ -104,4 +115,4 @@ class Attention(Mixer):
         else:
             a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
                                       window=s.window, scale=s.softmax_scale)
-        return self.o(a.view(a.shape[0], s.n_heads * s.head_dim))
+        return self._project(ctx, a.view(a.shape[0], s.n_heads * s.head_dim))

@@ -12,6 +12,15 @@ as `forward(ctx, h, cache)`; a feed-forward as `forward(ctx, h)`; a norm as
 `forward(x)` or `add_forward(x, delta)` (adds `delta` into `x` in place and
 returns the normalised sum); a position encoding as `table(positions)` whose
 result the mixer hands to its kernels.
+
+Two optional abilities, for steps of a few rows (decode), where a kernel of its own for "add to
+the stream and norm" is all launch and latency: a mixer or feed-forward with `adds_to_stream = True`
+finds the stream in `ctx.stream` (and in `ctx.stream_norm` the norm part that reads it next) and may
+add its output to it itself, returning `ops.Added` (the new rows' partial sums of squares, and the
+rows times that norm's weight) instead of the output; one with `takes_normed_rows = True` may be
+handed `ops.NormedRows` instead of normed rows, whose norm its first product finishes (`ops.linear`
+and `ops.gated_silu_linear` take them; `.materialize()` gives plain rows).  A norm takes part if it
+offers `rows_for_product(x, added)`.  Parts without these attributes are run as ever.
 """
 from __future__ import annotations
 

@@ -16,6 +16,8 @@ from .linear import Linear
 @register_ffn("gated_mlp")
 class GatedMlp(FeedForward):
     graph_safe = True
+    takes_normed_rows = True      # the gate|up product norms the rows it is given as `ops.NormedRows`
+    adds_to_stream = True         # the down product adds itself to `ctx.stream` where it can
 
     @classmethod
     def tensors(cls, spec: GatedMlpSpec) -> Dict[str, TensorSpec]:
@@ -32,5 +34,11 @@ class GatedMlp(FeedForward):
         self.gate_up = Linear([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dtype, device)
         self.down = Linear([tensors["down_proj.weight"]], dtype, device)
 
-    def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
-        return self.down(ops.gated_silu_linear(h, self.gate_up.weight))
+    def forward(self, ctx, h):
+        act = ops.gated_silu_linear(h, self.gate_up.weight)
+        if getattr(ctx, "stream", None) is not None:
+            norm = getattr(ctx, "stream_norm", None)
+            added = ops.linear_add(act, self.down.weight, ctx.stream, norm)
+            if added is not None:
+                return ops.Added(added[0], added[1], norm)
+        return self.down(act)

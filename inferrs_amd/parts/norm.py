@@ -32,3 +32,8 @@ class RMSNorm(Norm):
 
     def add_forward(self, x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, self.add_one)
+
+    def rows_for_product(self, x: torch.Tensor, added: "ops.Added") -> ops.NormedRows:
+        """The norm of a stream's rows left to the product that reads them: `added` holds the rows times
+        this norm's weight and their sums of squares."""
+        return ops.NormedRows(x, added.scaled, added.sums, self.weight, self.eps, self.add_one)

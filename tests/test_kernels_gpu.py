@@ -414,6 +414,70 @@ def test_gated_silu_linear(m, n, k):
     close(ops.silu_mul(ops.linear(dev(x), dev(w))), want, 2 ** -7, "two kernels")
 
 
+class _Norm:
+    """What the products need of a norm part."""
+    def __init__(self, weight, add_one=False):
+        self.weight, self.add_one, self.eps = weight, add_one, 1e-6
+
+
+@pytest.mark.parametrize("m", [1, 2, 8, 12])
+@pytest.mark.parametrize("n,k,n2,add_one", [(4096, 4096, 6144, False), (4096, 12288, 6144, False), (2560, 1024, 520, True),
+                                            (144, 4096, 4096, False), (200, 40, 72, False)])
+def test_products_around_a_residual_stream(m, n, k, n2, add_one):
+    """A product that adds itself to the stream (leaving the rows' sums of squares and the rows times the next
+    norm's weight), and the product after it, which finishes the norm by scaling its sums: the stream holds
+    the bits that the add kernel would leave, and the second product is the product of the normed rows up to
+    where the one rounding of a normed value happens."""
+    from inferrs_amd import ops
+    x = randn(m, k, dtype=torch.bfloat16, seed=31)
+    w = randn(n, k, dtype=torch.bfloat16, seed=32, scale=0.03)
+    stream = randn(m, n, dtype=torch.bfloat16, seed=33)
+    norm_w = (0.0 if add_one else 1.0) + 0.1 * randn(n, dtype=torch.float32, seed=34)
+    w2 = randn(n2, n, dtype=torch.bfloat16, seed=35, scale=0.03)
+    w3 = randn(2 * n2, n, dtype=torch.bfloat16, seed=36, scale=0.03)
+    # the two-kernel way
+    plain_stream = dev(stream)
+    plain_rows = ops.add_rmsnorm(plain_stream, ops.linear(dev(x), dev(w)), dev(norm_w), 1e-6, add_one)
+    # the products' way
+    fused_stream = dev(stream)
+    norm = _Norm(dev(norm_w), add_one)
+    sums, scaled = ops.linear_add(dev(x), dev(w), fused_stream, norm)
+    assert tuple(sums.shape) == (m, -(-n // 16)) and scaled.shape == fused_stream.shape
+    assert torch.equal(fused_stream, plain_stream), "the stream after the sum"
+    new_rows = fused_stream.float().cpu().double()
+    want_sums = torch.nn.functional.pad(new_rows.pow(2), (0, -n % 16)).view(m, -1, 16).sum(-1)
+    close(sums, want_sums, 1e-5, "sums of squares")
+    gain = norm_w.double() + (1.0 if add_one else 0.0)
+    assert torch.equal(scaled.cpu(), (new_rows * gain).to(torch.float32).to(torch.bfloat16)), "rows times the weight"
+    rows = ops.NormedRows(fused_stream, scaled, sums, norm.weight, 1e-6, add_one)
+    assert torch.equal(rows.materialize(), plain_rows)
+    exact = new_rows / torch.sqrt(new_rows.pow(2).mean(-1, keepdim=True) + 1e-6) * gain
+    g = (exact @ w3[:n2].double().t()).to(torch.bfloat16).double()
+    refs = {"product": exact @ w2.double().t(),
+            "gated product": g / (1 + torch.exp(-g)) * (exact @ w3[n2:].double().t()).to(torch.bfloat16).double()}
+    for what, got, want in (("product", ops.linear(rows, dev(w2)), ops.linear(plain_rows, dev(w2))),
+                            ("gated product", ops.gated_silu_linear(rows, dev(w3)), ops.gated_silu_linear(plain_rows, dev(w3)))):
+        close(want, refs[what], 2 ** -6, what + " of the two kernels")
+        close(got, refs[what], 2 ** -6, what + " with the norm's end inside")
+    # without a next norm: sums only
+    only = ops.linear_add(dev(x), dev(w), dev(stream))
+    assert only[1] is None and torch.equal(only[0], sums)
+
+
+def test_products_leave_the_stream_alone_where_they_cannot_take_it():
+    from inferrs_amd import ops
+    # 13 rows and more, or a 32-bit stream: the product does not add itself
+    big = randn(13, 64, dtype=torch.bfloat16, seed=3)
+    assert ops.linear_add(dev(big), dev(randn(64, 64, dtype=torch.bfloat16, seed=4)), dev(randn(13, 64, dtype=torch.bfloat16, seed=5))) is None
+    x, w = randn(3, 40, dtype=torch.float32, seed=1), randn(64, 40, dtype=torch.float32, seed=2)
+    assert ops.linear_add(dev(x), dev(w), dev(torch.zeros(3, 64))) is None
+    # a product of 65536 features and more (a logits head) norms the rows first
+    xs = randn(2, 64, dtype=torch.bfloat16, seed=6)
+    rows = ops.NormedRows(dev(xs), dev(xs), dev((xs.float() ** 2).sum(-1, keepdim=True)), dev(torch.ones(64)), 1e-6, False)
+    head = dev(randn(65536, 64, dtype=torch.bfloat16, seed=7))
+    assert torch.equal(ops.linear(rows, head), ops.linear(ops.rmsnorm(dev(xs), dev(torch.ones(64)), 1e-6, False), head))
+
+
 def test_skinny_rows_do_not_depend_on_the_batch():
     from inferrs_amd import ops
     x, w = randn(16, 4096, dtype=torch.bfloat16, seed=1), randn(77, 4096, dtype=torch.bfloat16, seed=2)
