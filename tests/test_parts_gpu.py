@@ -516,3 +516,37 @@ def test_toy_routed_feed_forward_and_position_encoding(tmp_path, dtype, page, to
         err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
         assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
         eng.cache.check_invariants()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_steps_of_a_few_rows_with_and_without_the_products_taking_the_norms(tmp_path, name):
+    """Steps of up to 12 bfloat16 rows leave the sums into the stream and the norms to the products around
+    them; with that switched off the same steps run the norm kernels.  One rounding of a normed value either
+    way, at different places: the logits agree to bfloat16's precision, and both agree with the plain model."""
+    import plain_model as pm
+    from tiny_configs import TINY, random_tokens, write_model
+    from inferrs_amd import ops
+    from inferrs_amd.engine import Engine, Entry
+    raw = TINY[name]
+    folder = write_model(str(tmp_path / name), raw, seed=41)
+    cfg, params = pm.read_model(folder)
+    prompts = {f"r{i}": random_tokens(n, raw["vocab_size"], 700 + i) for i, n in enumerate([9, 5, 11])}
+    want = {r: pm.forward(cfg, params, t) for r, t in prompts.items()}
+    outs = {}
+    for most in (12, 0):
+        saved, ops.STREAM_MAX_ROWS = ops.STREAM_MAX_ROWS, most
+        try:
+            eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=16, max_seqs=4)
+            rows = [eng.step([Entry(r, t[:4], [3]) for r, t in prompts.items()])]           # 12 rows in one step
+            for i in range(4, 9):                                                           # then three rows a step
+                rows.append(eng.step([Entry(r, [t[i]], [0]) for r, t in prompts.items() if i < len(t)]))
+            outs[most] = rows
+        finally:
+            ops.STREAM_MAX_ROWS = saved
+    scale = max(float(w.abs().max()) for w in want.values())
+    for a, b in zip(outs[12], outs[0]):
+        assert float((a - b).abs().max()) <= 2e-2 * scale
+    for most in (12, 0):
+        first = outs[most][0].cpu()
+        for j, (r, t) in enumerate(prompts.items()):
+            assert float((first[j] - want[r][3]).abs().max()) <= 3e-2 * scale, (most, r)
