@@ -45,6 +45,13 @@ int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, 
                   int out_dtype, hipStream_t stream);
 int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
                         int out_dtype, int dual, hipStream_t stream);
+// The skinny product with a residual stream around it (decode steps; see gemm.hip): adds itself to `resid`
+// and leaves the rows' sums of squares and the rows times the next norm's weight, and / or takes such rows
+// and finishes their norm.
+int ia_gemm_skinny_blocks(int N);
+int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype,
+                          int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
+                          int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream);
 
 long long ia_argmax_workspace(int rows, int vocab);
 int ia_argmax(int* out, const float* logits, void* workspace, int rows, int vocab, hipStream_t stream);
