@@ -19,7 +19,8 @@
 // one block-wide sum per bit.  Sums are tree sums in a fixed order; they differ from the
 // reference's sequential sums by rounding only.  Rows with a top_k of up to 1,024 take a
 // shorter way (sample_top_k): their first top_k tokens are picked out and sorted, and the
-// reference's steps run on that list as it runs them.
+// reference's steps run on that list as it runs them.  Rows without a top_k try that way with
+// the first 1,024 tokens of their list and take the long one when the list does not end there.
 #include "common.h"
 #include "api.h"
 
@@ -356,12 +357,15 @@ __device__ __forceinline__ void for_each_key(const uint32_t* __restrict__ keys, 
         }
     }
 }
-__device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__ keys, const float* __restrict__ probs,
-                             int vocab, int rowi, int k, float tp, float mp, float u, int want_top,
+// `open`: the row has no top_k; k tokens are only the beginning of its list, whose weight is `total`.  The steps
+// then succeed if top_p or min_p end the list within these k, or else the walk ends there; if not, nothing is
+// written and false comes back (the caller goes the long way).
+__device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__ keys, const float* __restrict__ probs,
+                             int vocab, int rowi, int k, bool open, float total, float tp, float mp, float u, int want_top,
                              float* __restrict__ lp_out, int* __restrict__ lp_ids, int* s_counts) {
     __shared__ int hist[2048];
     __shared__ unsigned long long cand[SAMPLE_FAST_K];      // (key, ~index): larger is earlier in the list
-    __shared__ int s_bin, s_above, s_n;
+    __shared__ int s_bin, s_above, s_n, s_done;
     // ---- the k-th largest key, 11 + 11 + 10 bits at a time
     uint32_t prefix = 0u;
     int prefix_bits = 0, need = k;
@@ -440,50 +444,69 @@ __device__ void sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
     __shared__ float cprob[SAMPLE_FAST_K];
     for (int i = threadIdx.x; i < n; i += blockDim.x) cprob[i] = probs[(int)~(uint32_t)(cand[i] & 0xffffffffull)];
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    // ---- the reference's steps 7 to 12 on its sorted list
-    auto index_of = [&](int i) { return (int)~(uint32_t)(cand[i] & 0xffffffffull); };
-    int len = n;
-    if (tp < 1.0f) {
-        float cumsum = 0.f;
-        for (int i = 0; i < len; ++i) {
-            cumsum += cprob[i];
-            if (cumsum >= tp) { len = i + 1; break; }
+    if (threadIdx.x == 0) {
+        // ---- the reference's steps 7 to 12 on its sorted list
+        auto index_of = [&](int i) { return (int)~(uint32_t)(cand[i] & 0xffffffffull); };
+        bool ended = !open, done = true;                    // ended: the list's end lies within these n tokens
+        int len = n;
+        if (tp < 1.0f) {
+            float cumsum = 0.f;
+            bool found = false;
+            for (int i = 0; i < len; ++i) {
+                cumsum += cprob[i];
+                if (cumsum >= tp) { len = i + 1; found = true; break; }
+            }
+            if (found) ended = true;
+            else if (open) done = false;                    // the nucleus is longer than what was picked out
         }
-    }
-    if (mp > 0.0f && len > 0) {
-        const float threshold = cprob[0] * mp;
-        int cut = 0;
-        while (cut < len && cprob[cut] >= threshold) ++cut;
-        if (cut > 0) len = cut;
-    }
-    float filtered = 0.f;
-    for (int i = 0; i < len; ++i) filtered += cprob[i];
-    const float denom = filtered > 0.f ? filtered : 1.0f;
-    if (want_top >= 0)
-        for (int i = 0; i < want_top && i < SAMPLE_MAX_TOP && i < len; ++i) {
-            const float pi = cprob[i];
-            lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + i] = index_of(i);
-            lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + i] = pi > 0.f ? logf(pi / denom) : -INFINITY;
+        if (done && mp > 0.0f && len > 0) {
+            const float threshold = cprob[0] * mp;
+            int cut = 0;
+            while (cut < len && cprob[cut] >= threshold) ++cut;
+            if (cut < len) { if (cut > 0) len = cut; ended = true; }
+            else if (!ended) done = false;                  // every picked token passes: the cut lies further on
         }
-    if (!(filtered > 0.f)) {
-        out[rowi] = len > 0 ? index_of(0) : 0;
-        if (want_top >= 0) lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = -INFINITY;
-        return;
+        float filtered = total;
+        if (done && ended) {
+            filtered = 0.f;
+            for (int i = 0; i < len; ++i) filtered += cprob[i];
+        }
+        int at = -1;
+        if (done && filtered > 0.f) {
+            float rng = u;
+            for (int i = 0; i < len; ++i) {
+                const float norm = cprob[i] / filtered;
+                if (rng < norm) { at = i; break; }
+                rng -= norm;
+            }
+            if (at < 0) {
+                if (ended) at = len - 1;
+                else done = false;                          // the walk goes on beyond what was picked out
+            }
+        }
+        if (done) {
+            const float denom = filtered > 0.f ? filtered : 1.0f;
+            if (want_top >= 0)
+                for (int i = 0; i < want_top && i < SAMPLE_MAX_TOP && i < len; ++i) {
+                    const float pi = cprob[i];
+                    lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + i] = index_of(i);
+                    lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + i] = pi > 0.f ? logf(pi / denom) : -INFINITY;
+                }
+            if (!(filtered > 0.f)) {
+                out[rowi] = len > 0 ? index_of(0) : 0;
+                if (want_top >= 0) lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = -INFINITY;
+            } else {
+                out[rowi] = index_of(at);
+                if (want_top >= 0) {
+                    const float pt = cprob[at] / filtered;
+                    lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = pt > 0.f ? logf(pt) : -INFINITY;
+                }
+            }
+        }
+        s_done = done ? 1 : 0;
     }
-    float rng = u;
-    int at = len - 1;
-    for (int i = 0; i < len; ++i) {
-        const float norm = cprob[i] / filtered;
-        if (rng < norm) { at = i; break; }
-        rng -= norm;
-    }
-    const int token = index_of(at);
-    out[rowi] = token;
-    if (want_top >= 0) {
-        const float pt = cprob[at] / filtered;
-        lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP)] = pt > 0.f ? logf(pt) : -INFINITY;
-    }
+    __syncthreads();
+    return s_done != 0;
 }
 
 // workspace: [rows, 2, vocab] words: the keys, then the probabilities.
@@ -584,8 +607,28 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
     const int k = top_k[rowi];
     if (fast_top_k && k > 0 && k < vocab && k <= SAMPLE_FAST_K) {
-        sample_top_k(out, keys, probs, vocab, rowi, k, top_p[rowi], min_p[rowi], u[rowi], want_top, lp_out, lp_ids, s_counts);
+        sample_top_k(out, keys, probs, vocab, rowi, k, false, 0.f, top_p[rowi], min_p[rowi], u[rowi], want_top, lp_out,
+                     lp_ids, s_counts);
         return;
+    }
+    if (fast_top_k && (k <= 0 || k >= vocab) && vocab > SAMPLE_FAST_K) {
+        // without a top_k: the list's first 1,024 tokens, which hold the nucleus, the min_p cut or the walk's end
+        // for all but flat distributions; its weight is the sum the long way would use
+        float t = 0.f;
+        for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
+            float pr[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = c0 + j * (int)blockDim.x;
+                pr[j] = c < vocab ? probs[c] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) t += pr[j];
+        }
+        const float total = block_sum(t, scratch);
+        if (sample_top_k(out, keys, probs, vocab, rowi, SAMPLE_FAST_K, true, total, top_p[rowi], min_p[rowi], u[rowi],
+                         want_top, lp_out, lp_ids, s_counts))
+            return;
     }
     // how long the kept prefix is (sampler.rs:256-283)
     int keep = vocab;

@@ -95,10 +95,13 @@ def test_sampler_matches_the_plain_transcription(vocab, kw):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("vocab,top_k", [(387, 1), (387, 50), (387, 386), (5000, 700), (151936, 50), (151936, 1024)])
+@pytest.mark.parametrize("vocab,top_k", [(387, 1), (387, 50), (387, 386), (5000, 700), (151936, 50), (151936, 1024),
+                                         (5000, 0), (151936, 0)])
 def test_rows_with_a_top_k_take_the_same_tokens_on_both_paths(vocab, top_k):
     """Rows with a top_k up to 1,024 pick their top_k tokens out and walk them as the reference walks its sorted
-    list; the other rows (and these, with the switch off) find the same prefixes by bisection over the keys."""
+    list; the other rows (and these, with the switch off) find the same prefixes by bisection over the keys.
+    Rows without a top_k try the same with the first 1,024 tokens of their list and go the long way when neither
+    the nucleus, nor the min_p cut, nor the walk ends within those (here: the rows with a high temperature)."""
     from inferrs_amd import ops
     g = torch.Generator().manual_seed(vocab + top_k)
     rows = 24
