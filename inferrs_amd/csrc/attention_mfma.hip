@@ -879,9 +879,13 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
     }
 }
 
-// The same merge for steps with many rows and few splits (portions of prompts): a wave a row, every lane
-// with the splits' maxima and sums of its row and HD / 64 features.
+// The same merge for steps with many rows and few splits (portions of prompts, decode steps of many
+// requests): a wave a row, every lane with the splits' maxima and sums of its row and HD / 64 features.
+// Kernel times at head size 128, context 8,192, 32 heads (the block-a-row kernel against this one):
+// 512 rows of 8 splits 4.9 against 7.6 us, 1,024 rows of 4 splits 7.0 against 5.1, 2,048 rows of 4 splits
+// 12.2 against 5.0.
 #define MERGE_ROWS_WAVES 4
+#define MERGE_ROWS_FROM 1024
 __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
     size_t first_row, size_t n_rows) {
@@ -1006,7 +1010,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     IA_LAUNCH_CHECK("attention_mfma");
     if (splits > 1) {
         const long long rows = (long long)n_tokens * nq;
-        if (rows >= 4096 && splits <= 16)
+        if (rows >= MERGE_ROWS_FROM && splits <= 16)
             attn_merge_rows_kernel<<<(unsigned)((rows + MERGE_ROWS_WAVES - 1) / MERGE_ROWS_WAVES), MERGE_ROWS_WAVES * IA_WAVE,
                                      0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq,
                                                   (size_t)rows);
