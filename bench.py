@@ -2,7 +2,7 @@
 """Decode and prefill throughput of the engine on one MI355X, Qwen3-8B layer sizes, bfloat16,
 random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--shape 8B|14B|32B] [--layers L]
 
 A step is one decode step of the whole batch: the step function over one token per request,
 greedy choice of the next token on the device, and feeding it back.  The requests' caches are
@@ -29,7 +29,10 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_si
                 hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
                 num_attention_heads=32, num_key_value_heads=8, head_dim=128, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
-FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+# The larger dense models of the family differ in these sizes only.
+QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64)
+SHAPES = {"8B": QWEN3_8B, "14B": QWEN3_14B, "32B": QWEN3_32B}
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 PREFILL_TOKENS = 2048
@@ -138,7 +141,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS,
+    ap.add_argument("--shape", default="8B", choices=sorted(SHAPES), help="layer sizes of this Qwen3 model")
+    ap.add_argument("--layers", type=int, default=None,
                     help="run fewer layers than the model has (recorded in the config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -155,11 +159,22 @@ def main() -> int:
     from inferrs_amd.config import Qwen3Config
     from inferrs_amd.engine import Engine
 
-    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    full_layers = SHAPES[args.shape]["num_hidden_layers"]
+    if args.layers is None:
+        args.layers = full_layers
+    raw = dict(SHAPES[args.shape], num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     esize = 2 if args.dtype == "bfloat16" else 4
     points_batches = [] if args.no_points or args.prefill_only else [1, 64]
+    # a point whose cache would not fit beside the weights is left out (batch 64 at a context of 32 k and more)
+    per_token = 2 * raw["num_key_value_heads"] * raw["head_dim"] * args.layers * esize
+    weights = (matmul_params(raw) * args.layers + 2 * raw["vocab_size"] * raw["hidden_size"]) * esize
+    room = 0.9 * torch.cuda.get_device_properties(0).total_memory - weights
+    for b in list(points_batches):
+        if b * (args.context + PAGE) * per_token > room:
+            note(f"batch {b} at context {args.context} does not fit this GPU's memory: point left out")
+            points_batches.remove(b)
     biggest = max([args.batch] + points_batches)
     num_pages = biggest * (-(-args.context // PAGE) + 1) + 8
     note(f"random weights of {args.layers} layers and a cache of {num_pages} pages")
@@ -180,14 +195,14 @@ def main() -> int:
     achieved = nbytes / (elapsed / args.steps) / 1e9
 
     record = {
-        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-8B)", "value": round(value, 2), "unit": "tok/s",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-{args.shape})", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_key,
         "data": "synthetic: random-init weights, uniform-random token ids, cache pages of the context "
                 "filled with random keys and values",
         "config": {
-            "model": "Qwen3-8B shape", "global_batch": args.batch, "seq_len": args.context,
-            "parallelism": "single GPU", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+            "model": f"Qwen3-{args.shape} shape", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single GPU", "layers": args.layers, "layers_of_model": full_layers,
             "hidden_size": raw["hidden_size"], "intermediate_size": raw["intermediate_size"],
             "num_attention_heads": raw["num_attention_heads"], "num_key_value_heads": raw["num_key_value_heads"],
             "head_dim": raw["head_dim"], "vocab_size": raw["vocab_size"], "rope_theta": raw["rope_theta"],

@@ -48,7 +48,10 @@ int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, i
 // The skinny product with a residual stream around it (decode steps; see gemm.hip): adds itself to `resid`
 // and leaves the rows' sums of squares and the rows times the next norm's weight, and / or takes such rows
 // and finishes their norm.
+// (the sums of squares come block by block: ia_gemm_skinny_blocks(N) blocks of ia_gemm_skinny_block_rows(N)
+// neighbouring features each, a choice that depends on N and on the chip's number of compute units)
 int ia_gemm_skinny_blocks(int N);
+int ia_gemm_skinny_block_rows(int N);
 int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype,
                           int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
                           int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream);

@@ -142,14 +142,14 @@ struct SkinnyStream {
 template <int MT, int RT, bool DUAL, int STAGE>
 __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     void* __restrict__ out, int out_f32, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-    int M, int N, int K, int kper, int m_base, int rot_mul, const SkinnyStream st) {
+    int M, int N, int K, int kper, int rpb, int m_base, int rot_mul, const SkinnyStream st) {
     constexpr int NA = DUAL ? 2 : 1;
     static_assert(!STAGE || MT == 1, "staging holds one tile of batch rows");
     extern __shared__ f32x4 red[];      // [waves][NA][RT][MT][64], then with STAGE [waves][rows][chunk of x]
     const int lane = threadIdx.x & (IA_WAVE - 1);
     const int wave = threadIdx.x / IA_WAVE;
     const int waves = blockDim.x / IA_WAVE;
-    const int n0 = blockIdx.x * 16 * RT;
+    const int n0 = blockIdx.x * rpb;
     const int r = lane & 15, g = lane >> 4;
     const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
     const int ks0 = wave * kper, ks1 = ks0 + kper < ksteps ? ks0 + kper : ksteps;
@@ -159,7 +159,9 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     for (int a = 0; a < NA; ++a)
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
-            const int n = n0 + t * 16 + r;
+            // (rows beyond the block's share or beyond N read the last row inside both: their sums are never stored)
+            const int j = t * 16 + r < rpb ? t * 16 + r : rpb - 1;
+            const int n = n0 + j;
             wrow[a][t] = w + ((size_t)a * N + (n < N ? n : N - 1)) * K + g * 8;
         }
     // Batch rows beyond M are read from row 0: their columns of the result are never stored.
@@ -208,7 +210,8 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     }
     uint2 resid_old = make_uint2(0u, 0u);
     float4 next_w4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    const bool resid_ahead = st.resid != nullptr && wave == 0 && (N & 3) == 0 && n0 + 4 * g + 3 < N && m_base + r < M;
+    const bool resid_ahead = st.resid != nullptr && wave == 0 && ((N | n0) & 3) == 0 && n0 + 4 * g + 3 < N &&
+                             4 * g + 3 < rpb && m_base + r < M;
     if (resid_ahead) {
         resid_old = *(const uint2*)(st.resid + (size_t)(m_base + r) * N + n0 + 4 * g);
         if (st.scaled_out != nullptr) next_w4 = *(const float4*)(st.next_w + n0 + 4 * g);
@@ -415,7 +418,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                     } else if (m < M) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            if (nb + i >= N) continue;
+                            if (nb + i >= N || 4 * g + i >= rpb) continue;
                             bf16_t* at = st.resid + (size_t)m * N + nb + i;
                             const float product = bf16_bits_to_f32(f32_to_bf16_bits(s[0][i]));
                             const uint16_t h = f32_to_bf16_bits(product + bf16_bits_to_f32(at->bits));
@@ -449,7 +452,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                     v[i] = s[0][i];
                 }
             }
-            if (nb + 3 < N && (N & 3) == 0) {
+            if (nb + 3 < N && ((N | n0) & 3) == 0 && t * 16 + 4 * g + 3 < rpb) {
                 if (out_f32) {
                     *(f32x4*)((float*)out + (size_t)m * N + nb) = (f32x4){v[0], v[1], v[2], v[3]};
                 } else {
@@ -461,7 +464,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (nb + i >= N) continue;
+                    if (nb + i >= N || t * 16 + 4 * g + i >= rpb) continue;
                     if (out_f32) ((float*)out)[(size_t)m * N + nb + i] = v[i];
                     else ((bf16_t*)out)[(size_t)m * N + nb + i].bits = f32_to_bf16_bits(v[i]);
                 }
@@ -478,9 +481,45 @@ extern "C" void ia_gemm_skinny_tune(int target_waves, int min_ksteps, int rot_mu
     g_stage = stage;
 }
 
-// How many waves share k: a function of the weight's shape and of the row tiling only.
-static int skinny_waves(int N, int K, int rt, int tiles_per_wave) {
-    const int groups = (N + 16 * rt - 1) / (16 * rt);
+static int skinny_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    return cus;
+}
+
+// Output features a block owns (one tile of rows a wave: 8 to 16 of the tile's 16).  A weight whose blocks of 16
+// go round the compute units once or twice and leave a round partly filled (5,120 features: 320 blocks on 256
+// units) is read at the pace of the units that got two; smaller blocks fill the rounds (10 features: 512 blocks).
+// Depends on the number of features and the chip alone.
+static int skinny_rows_per_block(int N, int rt) {
+    if (rt != 1) return 16 * rt;
+    const int cus = skinny_cus();
+    if ((N + 15) / 16 >= 8 * cus) return 16;
+    // rows of the fullest compute unit; the largest block within a sixteenth of the best (smaller blocks spend
+    // more of their time starting and adding up)
+    auto fullest = [&](int rows) { return ((N + rows - 1) / rows + cus - 1) / cus * rows; };
+    int least = fullest(16);
+    for (int rows = 15; rows >= 8; --rows) least = fullest(rows) < least ? fullest(rows) : least;
+    int best = 16;
+    while (fullest(best) * 16 > least * 17) --best;
+    return best;
+}
+
+// How many waves share k, and how many k steps each takes: a function of the weight's shape, of the row
+// tiling and of the chip only.
+#define SK_CHUNK 16     // k steps of the longest chunk a wave has in flight
+// Weights whose blocks go round the compute units three times or more stream for long (gate|up, a logits head);
+// the others are read in one burst.
+static bool skinny_tall(int blocks) { return blocks >= 3 * skinny_cus(); }
+
+static void skinny_split(int N, int K, int rt, int tiles_per_wave, int* waves_out, int* kper_out) {
+    const int rpb = skinny_rows_per_block(N, rt);
+    const int groups = (N + rpb - 1) / rpb;
     const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
     // the waves' tiles meet in shared memory: at most 64 KiB of it
     const int most = 65536 / (tiles_per_wave * IA_WAVE * (int)sizeof(f32x4));
@@ -488,7 +527,29 @@ static int skinny_waves(int N, int K, int rt, int tiles_per_wave) {
     while (waves * 2 <= SK_MAX_WAVES && waves * 2 <= most && ksteps / (waves * 2) >= g_min_ksteps &&
            (groups * waves < g_target_waves || waves < g_min_waves))
         waves *= 2;
-    return waves;
+    int kper = (ksteps + waves - 1) / waves;
+    // A range that is no multiple of the chunk ends in short chunks and single steps, each of which waits
+    // for the memory on its own, and keeps the staged variants out (a width of 5,120 leaves 20 steps to each of
+    // eight waves).  Long rows are shared out in whole chunks instead.  Tall weights: chunks of 8 steps (what
+    // their staged variant takes) between no more waves than by the rule above, since blocks of more than eight
+    // waves streamed slower (24,576 x 5,120 at 8 rows: 7 waves of 24 steps 55.7 us, 10 of 16 62.5, 5 of 32 62.9).
+    // The others: chunks of 16 between as many waves, up to 12, as make the longest range shortest (5,120 -> 10
+    // waves of 16 steps, 17,408 -> 12 of 48, 25,600 -> 10 of 80; 5,120 x 5,120 at 8 rows 20.7 -> 17.6 us).  The
+    // last wave takes what is left.
+    if (ksteps >= 8 * SK_CHUNK && kper % SK_CHUNK != 0) {
+        const bool tall = skinny_tall(groups);
+        const int unit = tall ? 8 : SK_CHUNK;
+        const int chunks = (ksteps + unit - 1) / unit;
+        // (12 waves: what leaves the staging area of 12 batch rows inside a compute unit's shared memory)
+        const int top = tall ? waves : (most < 12 ? most : 12);
+        int best = (chunks + waves - 1) / waves;
+        for (int w = waves + 1; w <= top; ++w)
+            if ((chunks + w - 1) / w < best) best = (chunks + w - 1) / w;
+        kper = best * unit;
+        waves = (ksteps + kper - 1) / kper;
+    }
+    *waves_out = waves;
+    *kper_out = kper;
 }
 
 #define SK_STAGE_LDS_MOST (96 * 1024)
@@ -508,40 +569,28 @@ static int skinny_ask_shared(int bytes) {
     return 0;
 }
 
-static int skinny_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-    }
-    return cus;
-}
-
 template <int MT, int RT, bool DUAL>
 static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* w, int M, int N, int K,
                          int m_base, const SkinnyStream& st, hipStream_t stream) {
-    const int waves = skinny_waves(N, K, RT, (DUAL ? 2 : 1) * RT * MT);
-    const int ksteps = (K + SK_KSTEP - 1) / SK_KSTEP;
-    const int kper = (ksteps + waves - 1) / waves;
+    int waves, kper;
+    skinny_split(N, K, RT, (DUAL ? 2 : 1) * RT * MT, &waves, &kper);
     // the kernel places the staging area behind the tiles of all waves, also when there is one wave
     const size_t tiles = (size_t)waves * (DUAL ? 2 : 1) * RT * MT * IA_WAVE * sizeof(f32x4);
-    const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
+    const int rpb = skinny_rows_per_block(N, RT);
+    const unsigned grid = (unsigned)((N + rpb - 1) / rpb);
     if constexpr (MT == 1) {
         const int rows = M - m_base < 16 ? M - m_base : 16;
         const size_t staged8 = tiles + (size_t)waves * rows * (8 * 2 * SK_KSTEP + SK_STAGE_PAD);
         const size_t staged16 = tiles + (size_t)waves * rows * (16 * 2 * SK_KSTEP + SK_STAGE_PAD);
-        const int cus = skinny_cus();
         int stage = 0;
-        if (g_stage && rows >= 2 && (int)grid >= 2 * cus) {
-            // Staging pays where blocks stream for long: with at least two blocks for every compute unit,
+        if (g_stage && rows >= 2 && skinny_tall((int)grid)) {
+            // Staging pays where blocks stream for long: with at least three blocks for every compute unit,
             // with 2 to 12 batch rows (one row is one cache line a load anyway; beyond 12 the staging area
             // leaves too few blocks on a compute unit), and with whole chunks of 8 k steps in a wave's
             // range.  Measured at 8 rows: gate|up 46 -> 40 us, logits head 261 -> 224 us.
             if (rows <= 12 && kper >= 8 && staged8 <= SK_STAGE_LDS_MOST - SK_SCALES_RESERVE) stage = 8;
         } else if (g_stage && rows >= 2 && !DUAL && RT == 1) {
-            // A weight that one round of blocks covers (o, down, qkv) is read in one burst, and what counts
+            // A weight that one or two rounds of blocks cover (o, down, qkv) is read in one burst, and what counts
             // is how much a wave has in flight: chunks of 16 steps, as much as without staging, and up to
             // all of a compute unit's shared memory for its block.  Measured at 8 rows: down 25.6 -> 22.3 us,
             // o 11.5 -> 9.9, qkv 16.8 -> 14.2; at 16 rows 30.4 -> 24.5, 12.9 -> 10.6, 19.1 -> 16.8.  (From 9 rows on
@@ -553,20 +602,20 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
         if (stage == 8) {
             if (skinny_ask_shared<MT, RT, DUAL, 8>(SK_STAGE_LDS_MOST - SK_SCALES_RESERVE)) return 1;
             gemm_skinny_kernel<MT, RT, DUAL, 8><<<grid, waves * IA_WAVE, staged8, stream>>>(
-                out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul, st);
+                out, out_f32, x, w, M, N, K, kper, rpb, m_base, g_rot_mul, st);
             return 0;
         }
         if constexpr (!DUAL && RT == 1) {
             if (stage == 16) {
                 if (skinny_ask_shared<MT, RT, DUAL, 16>(SK_STAGE16_LDS_MOST - SK_SCALES_RESERVE)) return 1;
                 gemm_skinny_kernel<MT, RT, DUAL, 16><<<grid, waves * IA_WAVE, staged16, stream>>>(
-                    out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul, st);
+                    out, out_f32, x, w, M, N, K, kper, rpb, m_base, g_rot_mul, st);
                 return 0;
             }
         }
     }
     gemm_skinny_kernel<MT, RT, DUAL, 0><<<grid, waves * IA_WAVE, waves > 1 ? tiles : 0, stream>>>(
-        out, out_f32, x, w, M, N, K, kper, m_base, g_rot_mul, st);
+        out, out_f32, x, w, M, N, K, kper, rpb, m_base, g_rot_mul, st);
     return 0;
 }
 
@@ -619,7 +668,13 @@ extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int 
 }
 
 // Blocks of the plain product with N output features: the columns of its sums of squares.
-extern "C" int ia_gemm_skinny_blocks(int N) { return (N + 15) / 16; }
+// Features of a block of the plain product.
+extern "C" int ia_gemm_skinny_block_rows(int N) { return skinny_rows_per_block(N, 1); }
+
+extern "C" int ia_gemm_skinny_blocks(int N) {
+    const int rpb = skinny_rows_per_block(N, 1);
+    return (N + rpb - 1) / rpb;
+}
 
 // The product with a residual stream around it (up to 16 rows; see SkinnyStream).
 //   resid != null (plain products): resid[M, N] += product in place, nothing goes to `out` (may be null);

@@ -442,10 +442,11 @@ def test_products_around_a_residual_stream(m, n, k, n2, add_one):
     fused_stream = dev(stream)
     norm = _Norm(dev(norm_w), add_one)
     sums, scaled = ops.linear_add(dev(x), dev(w), fused_stream, norm)
-    assert tuple(sums.shape) == (m, -(-n // 16)) and scaled.shape == fused_stream.shape
+    per = ops.library().ia_gemm_skinny_block_rows(n)              # features a block: 16, fewer where that fills the chip evenly
+    assert 8 <= per <= 16 and tuple(sums.shape) == (m, -(-n // per)) and scaled.shape == fused_stream.shape
     assert torch.equal(fused_stream, plain_stream), "the stream after the sum"
     new_rows = fused_stream.float().cpu().double()
-    want_sums = torch.nn.functional.pad(new_rows.pow(2), (0, -n % 16)).view(m, -1, 16).sum(-1)
+    want_sums = torch.nn.functional.pad(new_rows.pow(2), (0, -n % per)).view(m, -1, per).sum(-1)
     close(sums, want_sums, 1e-5, "sums of squares")
     gain = norm_w.double() + (1.0 if add_one else 0.0)
     assert torch.equal(scaled.cpu(), (new_rows * gain).to(torch.float32).to(torch.bfloat16)), "rows times the weight"
