@@ -197,15 +197,20 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
     // stream's old values and the next norm's weights.
     __shared__ float ss_row[16];
     constexpr int SS_ROWS = (16 + 7) / 8;                   // rows a wave when eight waves share out sixteen
-    float4 ss_mine[SS_ROWS];
-    const bool ss_wide = st.sums_in != nullptr && (st.n_sums & 3) == 0 && st.n_sums <= 4 * IA_WAVE;
+    constexpr int SS_VEC = 2;                               // 16-byte pieces a lane: rows of up to 512 sums
+    float4 ss_mine[SS_ROWS][SS_VEC];
+    const bool ss_wide = st.sums_in != nullptr && (st.n_sums & 3) == 0 && st.n_sums <= 4 * IA_WAVE * SS_VEC;
     if (ss_wide) {                                          // (a stream has one tile of batch rows)
 #pragma unroll
         for (int j = 0; j < SS_ROWS; ++j) {
             const int m = wave + j * waves;
-            ss_mine[j] = (m < stage_rows && 4 * lane < st.n_sums)
-                             ? *(const float4*)(st.sums_in + (size_t)(m_base + m) * st.n_sums + 4 * lane)
-                             : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int v = 0; v < SS_VEC; ++v) {
+                const int at = 4 * (lane + v * IA_WAVE);
+                ss_mine[j][v] = (m < stage_rows && at < st.n_sums)
+                                    ? *(const float4*)(st.sums_in + (size_t)(m_base + m) * st.n_sums + at)
+                                    : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
         }
     }
     uint2 resid_old = make_uint2(0u, 0u);
@@ -343,7 +348,15 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
         for (int j = 0; j < SS_ROWS; ++j) {
             const int m = wave + j * waves;
             if (m >= stage_rows) continue;
-            float ss = ss_wide ? ((ss_mine[j].x + ss_mine[j].y) + ss_mine[j].z) + ss_mine[j].w : one_by_one(m);
+            float ss;
+            if (ss_wide) {
+                ss = ((ss_mine[j][0].x + ss_mine[j][0].y) + ss_mine[j][0].z) + ss_mine[j][0].w;
+#pragma unroll
+                for (int v = 1; v < SS_VEC; ++v)
+                    ss += ((ss_mine[j][v].x + ss_mine[j][v].y) + ss_mine[j][v].z) + ss_mine[j][v].w;
+            } else {
+                ss = one_by_one(m);
+            }
             ss = wave_sum(ss);
             if (lane == 0) ss_row[m] = ss;
         }

@@ -389,7 +389,8 @@ def test_gemm_tiled_float32_is_true_32_bit(m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 2, 8, 12, 13, 16, 17, 33, 64, 65, 200])
-@pytest.mark.parametrize("n,k", [(130, 40), (515, 136), (4096, 4096), (1000, 12288), (16, 8)])
+# (5,120 features: blocks of 10; 5,120 wide: k shared out between 10 waves)
+@pytest.mark.parametrize("n,k", [(130, 40), (515, 136), (4096, 4096), (1000, 12288), (16, 8), (5120, 5120), (7170, 5128)])
 @pytest.mark.parametrize("out_dtype", DTYPES)
 def test_linear_bfloat16(m, n, k, out_dtype):
     from inferrs_amd import ops
@@ -401,8 +402,17 @@ def test_linear_bfloat16(m, n, k, out_dtype):
     close(got, want, tol(out_dtype, 2e-5) if m <= ops.SKINNY_MAX_ROWS else 2 ** -8, f"linear {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("m", [1, 12])
+@pytest.mark.parametrize("n,k", [(5120, 17408), (5120, 25600), (10240, 5120)])
+def test_linear_bfloat16_long_rows(m, n, k):
+    """Widths whose k steps do not divide evenly between the waves: the last wave takes what is left."""
+    from inferrs_amd import ops
+    x, w = randn(m, k, dtype=torch.bfloat16, seed=1), randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    close(ops.linear(dev(x), dev(w), torch.float32), x.double() @ w.double().t(), 2e-5, f"linear {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("m", [1, 8, 17, 40, 64])
-@pytest.mark.parametrize("n,k", [(130, 40), (12288, 4096), (200, 136)])
+@pytest.mark.parametrize("n,k", [(130, 40), (12288, 4096), (200, 136), (17408, 5120)])
 def test_gated_silu_linear(m, n, k):
     from inferrs_amd import ops
     x = randn(m, k, dtype=torch.bfloat16, seed=1)
@@ -422,6 +432,7 @@ class _Norm:
 
 @pytest.mark.parametrize("m", [1, 2, 8, 12])
 @pytest.mark.parametrize("n,k,n2,add_one", [(4096, 4096, 6144, False), (4096, 12288, 6144, False), (2560, 1024, 520, True),
+                                            (5120, 8192, 7168, False),
                                             (144, 4096, 4096, False), (200, 40, 72, False)])
 def test_products_around_a_residual_stream(m, n, k, n2, add_one):
     """A product that adds itself to the stream (leaving the rows' sums of squares and the rows times the next
