@@ -396,12 +396,13 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 
 # ---- matrix products --------------------------------------------------------------------------
 
-# Beyond this many rows the vendor's GEMM reads the weights faster.  Measured at the sizes of an 8 B model
-# (us: qkv, o, gate|up with SiLU, down, logits head): 12 rows 16.2, 10.2, 41.5, 23.7, 233 here against 14.8,
-# 12.5, 46.3, 21.5, 260 there (92 against 95 a layer); 14 rows 17.3, 10.6, 48.4, 24.7, 286 against 14.7, 12.5,
-# 46.7, 21.6, 261 (101 against 95): past 12 rows the staging area of the activations no longer fits beside
-# enough blocks on a compute unit.
-SKINNY_MAX_ROWS = 12
+# Beyond this many rows (one tile of MFMA columns) the vendor's GEMM reads the weights faster.  From 13 to 16
+# rows the single products are about even (us at the sizes of an 8 B model, qkv, o, gate|up with SiLU, down:
+# 16.9, 11.4, 49.6, 24.7 here against about 15, 12.5, 46.4, 22.5 there at 16 rows: past 12 rows the staging area
+# of the activations no longer fits beside enough blocks on a compute unit), but only these products take over
+# the sums and norms of the residual stream: a decode step of 13 requests at a context of 2,048 5.70 -> 5.37 ms,
+# of 16 requests 5.47 -> 5.37.
+SKINNY_MAX_ROWS = 16
 
 
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -465,7 +466,7 @@ def widen(x: torch.Tensor) -> torch.Tensor:
 # norm's weight; the product after the norm (`linear` / `gated_silu_linear` given `NormedRows`) takes
 # those rows and multiplies its sums by the row's scale, rsqrt(mean of squares + eps).
 
-STREAM_MAX_ROWS = 12          # rows up to which the products take over the sums and norms of a step
+STREAM_MAX_ROWS = 16          # rows up to which the products take over the sums and norms of a step
 
 
 class Added:

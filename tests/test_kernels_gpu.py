@@ -430,7 +430,7 @@ class _Norm:
         self.weight, self.add_one, self.eps = weight, add_one, 1e-6
 
 
-@pytest.mark.parametrize("m", [1, 2, 8, 12])
+@pytest.mark.parametrize("m", [1, 2, 8, 12, 13, 16])
 @pytest.mark.parametrize("n,k,n2,add_one", [(4096, 4096, 6144, False), (4096, 12288, 6144, False), (2560, 1024, 520, True),
                                             (5120, 8192, 7168, False),
                                             (144, 4096, 4096, False), (200, 40, 72, False)])
@@ -478,9 +478,10 @@ def test_products_around_a_residual_stream(m, n, k, n2, add_one):
 
 def test_products_leave_the_stream_alone_where_they_cannot_take_it():
     from inferrs_amd import ops
-    # 13 rows and more, or a 32-bit stream: the product does not add itself
-    big = randn(13, 64, dtype=torch.bfloat16, seed=3)
-    assert ops.linear_add(dev(big), dev(randn(64, 64, dtype=torch.bfloat16, seed=4)), dev(randn(13, 64, dtype=torch.bfloat16, seed=5))) is None
+    # more rows than the skinny product takes, or a 32-bit stream: the product does not add itself
+    many = ops.SKINNY_MAX_ROWS + 1
+    big = randn(many, 64, dtype=torch.bfloat16, seed=3)
+    assert ops.linear_add(dev(big), dev(randn(64, 64, dtype=torch.bfloat16, seed=4)), dev(randn(many, 64, dtype=torch.bfloat16, seed=5))) is None
     x, w = randn(3, 40, dtype=torch.float32, seed=1), randn(64, 40, dtype=torch.float32, seed=2)
     assert ops.linear_add(dev(x), dev(w), dev(torch.zeros(3, 64))) is None
     # a product of 65536 features and more (a logits head) norms the rows first
