@@ -45,6 +45,9 @@ int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, 
                   int out_dtype, hipStream_t stream);
 int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
                         int out_dtype, int dual, hipStream_t stream);
+// Large bfloat16 products in tiles of 256 x 256 (gemm_mfma.hip); K a multiple of 64; with `dual` w is [gate; up]
+// and out = silu(x . gate^T) * (x . up^T).
+int ia_gemm_mfma_bf16(void* out, const void* x, const void* w, int M, int N, int K, int dual, hipStream_t stream);
 // The skinny product with a residual stream around it (decode steps; see gemm.hip): adds itself to `resid`
 // and leaves the rows' sums of squares and the rows times the next norm's weight, and / or takes such rows
 // and finishes their norm.

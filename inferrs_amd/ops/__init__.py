@@ -405,6 +405,38 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 SKINNY_MAX_ROWS = 16
 
 
+# Who multiplies more bfloat16 rows than the skinny kernel takes: "library" (the vendor's GEMM, as the reference's
+# products go to cuBLAS) or "own" (the tiled matrix-core kernel of this package, where the width is a multiple of
+# 64).  The library is faster at the sizes of an 8 B model (2,048 rows: 84, 60, 335 with SiLU and 168 us for qkv, o,
+# gate|up and down against 125, 119, 435 and 323 us), so it is the default; INFERRS_AMD_LARGE_PRODUCTS=own
+# runs the model without it.
+LARGE_PRODUCTS = os.environ.get("INFERRS_AMD_LARGE_PRODUCTS", "library")
+
+
+def _own_large(x: torch.Tensor, w: torch.Tensor) -> bool:
+    if LARGE_PRODUCTS not in ("library", "own"):
+        raise KernelError(f"INFERRS_AMD_LARGE_PRODUCTS / ops.LARGE_PRODUCTS: 'library' or 'own', not {LARGE_PRODUCTS!r}")
+    return (LARGE_PRODUCTS == "own" and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 64 == 0
+            and x.is_contiguous() and w.is_contiguous())
+
+
+def gemm_mfma_bf16(x: torch.Tensor, w: torch.Tensor, dual: bool = False) -> torch.Tensor:
+    """x [m, k] . w[n, k]^T in bfloat16 by the tiled matrix-core kernel (k a multiple of 64); with `dual`
+    w is [gate; up] and the result silu(x . gate^T) * (x . up^T)."""
+    _dev(x, w)
+    m, k = x.shape
+    rows, k2 = w.shape
+    if k2 != k or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or k % 64 or (dual and rows % 2):
+        raise KernelError(f"gemm_mfma: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
+    if not (x.is_contiguous() and w.is_contiguous()):
+        raise KernelError("gemm_mfma: operands must be contiguous")
+    n = rows // 2 if dual else rows
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    if m:
+        _check(library().ia_gemm_mfma_bf16(_p(out), _p(x), _p(w), m, n, k, int(dual), _stream()))
+    return out
+
+
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     _dev(x, w)
     m, k = x.shape
@@ -564,7 +596,7 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch
     _dev(x, w)
     if w.shape[1] != k or w.dtype != x.dtype:
         raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
-    y = torch.nn.functional.linear(x, w)
+    y = gemm_mfma_bf16(x, w) if _own_large(x, w) else torch.nn.functional.linear(x, w)
     return widen(y) if out_dtype == torch.float32 else y
 
 
@@ -663,4 +695,6 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
         x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
         return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True)
+    if w_gate_up.shape[0] % 2 == 0 and x.dtype == torch.bfloat16 and skinny_fits(x, w_gate_up) and _own_large(x, w_gate_up):
+        return gemm_mfma_bf16(x, w_gate_up, dual=True)
     return silu_mul(linear(x, w_gate_up))

@@ -402,6 +402,30 @@ def test_linear_bfloat16(m, n, k, out_dtype):
     close(got, want, tol(out_dtype, 2e-5) if m <= ops.SKINNY_MAX_ROWS else 2 ** -8, f"linear {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("dual", [False, True])
+@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (255, 250, 64), (256, 256, 128), (257, 260, 192), (777, 1002, 320),
+                                   (2048, 1536, 4096), (300, 130, 1024)])
+def test_tiled_matrix_core_product(m, n, k, dual):
+    """The tiled kernel for many rows, alone: sizes that fill no tile, one and several stages of k, features that
+    are no multiple of four (single stores), with and without the activation inside."""
+    from inferrs_amd import ops
+    x = randn(m, k, dtype=torch.bfloat16, seed=1)
+    w = randn((2 if dual else 1) * n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    got = ops.gemm_mfma_bf16(dev(x), dev(w), dual)
+    assert got.shape == (m, n) and got.dtype == torch.bfloat16
+    want = x.double() @ w.double().t()
+    if dual:
+        gate, up = want[:, :n].to(torch.bfloat16).double(), want[:, n:].to(torch.bfloat16).double()
+        want = gate / (1 + torch.exp(-gate)) * up
+    close(got, want, 2 ** -7, f"tiled {m}x{n}x{k} dual={dual}")
+
+
+def test_tiled_matrix_core_product_refuses_other_widths():
+    from inferrs_amd import ops
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mfma_bf16(dev(randn(32, 40, dtype=torch.bfloat16)), dev(randn(16, 40, dtype=torch.bfloat16)))
+
+
 @pytest.mark.parametrize("m", [1, 12])
 @pytest.mark.parametrize("n,k", [(5120, 17408), (5120, 25600), (10240, 5120)])
 def test_linear_bfloat16_long_rows(m, n, k):

@@ -347,6 +347,25 @@ def test_real_layer_sizes(tmp_path):
             torch.cuda.empty_cache()
 
 
+def test_own_large_products_through_the_engine(models, tmp_path):
+    """The model without the vendor's GEMM: every cutting with the package's own tiled kernel for the products of
+    many rows (widths that are multiples of 64: tiny configuration A; other widths stay with the library)."""
+    from inferrs_amd import ops
+    folder, raw, reqs, ref = pick(models, "A", False, "bfloat16")
+    limit = bound(folder, reqs, ref, "bfloat16")
+    calls = []
+    saved, ops.LARGE_PRODUCTS, inner = ops.LARGE_PRODUCTS, "own", ops.gemm_mfma_bf16
+    ops.gemm_mfma_bf16 = lambda *a, **k: (calls.append(1), inner(*a, **k))[1]
+    try:
+        for mode, trace in traces(reqs).items():
+            got = replay(folder, raw, "A", "bfloat16", trace, str(tmp_path / f"own_{mode}"))
+            err, where = worst(got, ref, reqs)
+            assert err <= limit, f"{mode}: {err:.3e} at {where}"
+    finally:
+        ops.LARGE_PRODUCTS, ops.gemm_mfma_bf16 = saved, inner
+    assert calls, "the tiled kernel never ran"
+
+
 def test_real_layer_sizes_long_prompt_in_portions(tmp_path):
     """The same layer over a prompt of 1,100 tokens, whole and in portions of 300, 37 and 512 tokens: with head
     size 128 these steps take the attention kernel of four-wave blocks, and the late portions (few tiles, more
