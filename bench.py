@@ -10,6 +10,14 @@ brought to the benchmark's context length by filling their pages with random key
 (decode time does not depend on their content); the prefill figure is measured separately
 on a 2,048-token prompt through the same step function.  One JSON line is printed.
 
+    python bench.py --workload mixed16|concurrent32 [--shape ...] [--decode-tokens T]
+
+runs requests through the serving loop instead (scheduler, prompt portions beside decode tokens, greedy
+choice): `mixed16` is 16 requests with prompts of 128 to 4,096 random tokens in portions of 512 at the
+14B shape, `concurrent32` 32 requests of 1,024 prompt tokens at the 32B shape; every request decodes
+`--decode-tokens` tokens.  Its JSON line gives tokens a second over the whole run, the prompts' and the
+decoded tokens' rates apart, and the time to a request's first token.
+
 The reference measures the same quantities with `inferrs bench` (`inferrs/src/bench.rs:40-224`,
 `Engine::bench_generate`, `inferrs/src/engine.rs:2557-2641`): synthetic prompt, stop tokens
 ignored, device-synchronised wall time.
@@ -129,6 +137,72 @@ def time_prefill(engine, n_tokens: int, runs: int, vocab: int):
     return best
 
 
+WORKLOADS = {
+    # name: (shape, requests, shortest prompt, longest prompt, portion, decode tokens)
+    "mixed16": ("14B", 16, 128, 4096, 512, 128),
+    "concurrent32": ("32B", 32, 1024, 1024, 1024, 256),
+}
+
+
+def run_workload(engine, lengths, portion: int, decode_tokens: int, budget: int, vocab: int, seed: int):
+    """All requests arrive at once and run to their last token.  Returns (seconds, seconds to each
+    request's first token, loop steps, seconds until the last prompt was through)."""
+    import torch
+    from inferrs_amd.engine import GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    loop = GenerationLoop(engine, max_batch_size=len(lengths), max_tokens_per_step=budget, prefill_chunk=portion)
+    g = torch.Generator().manual_seed(seed)
+    params = SamplingParams.greedy(max_tokens=decode_tokens, bypass_stop_tokens=True)
+    requests = [loop.add(torch.randint(0, vocab, (n,), generator=g).tolist(), params) for n in lengths]
+    first = {}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while loop.scheduler.has_work():
+        loop.step()
+        now = time.perf_counter() - t0          # (a step's tokens are on the host when it returns)
+        for r in requests:
+            if r.output and r.request_id not in first:
+                first[r.request_id] = now
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    if any(len(r.output) != decode_tokens for r in requests):
+        raise RuntimeError("a request ended early")
+    return elapsed, [first[r.request_id] for r in requests], loop.steps, max(first.values())
+
+
+def workload_main(args, raw, engine_factory) -> int:
+    import random
+    _, n_req, lo, hi, portion, _ = WORKLOADS[args.workload]
+    rnd = random.Random(0)
+    lengths = [rnd.randint(lo, hi) for _ in range(n_req)]
+    decode_tokens = args.decode_tokens
+    budget = max(2048, portion)
+    pages = sum(-(-(n + decode_tokens + 1) // PAGE) + 1 for n in lengths) + 8
+    note(f"{args.workload}: {n_req} requests, {sum(lengths)} prompt tokens, {decode_tokens} decoded tokens each")
+    engine = engine_factory(pages, n_req + 1)
+    run_workload(engine, lengths, portion, min(decode_tokens, 16), budget, raw["vocab_size"], seed=1)      # warm-up
+    runs = [run_workload(engine, lengths, portion, decode_tokens, budget, raw["vocab_size"], seed=2 + i)
+            for i in range(max(1, args.steps if args.steps < 16 else 3))]
+    elapsed, firsts, steps, prompts_done = min(runs, key=lambda r: r[0])
+    p_tok, d_tok = sum(lengths), n_req * decode_tokens
+    print(json.dumps({
+        "metric": f"tokens/s of the serving loop, workload {args.workload} (Qwen3-{args.shape})",
+        "value": round((p_tok + d_tok) / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "runs": len(runs),
+        "seconds": round(elapsed, 4), "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random-init weights, uniform-random token ids, stop tokens ignored",
+        "config": {"model": f"Qwen3-{args.shape} shape", "layers": args.layers, "requests": n_req,
+                   "prompt_tokens": p_tok, "shortest_prompt": min(lengths), "longest_prompt": max(lengths),
+                   "portion": portion, "tokens_per_step": budget, "decode_tokens": decode_tokens, "kv_page_size": PAGE},
+        "loop_steps": steps,
+        "first_token_s": {"mean": round(sum(firsts) / len(firsts), 4), "max": round(max(firsts), 4)},
+        # until the last request has its first token the steps are mostly prompt portions, after it only decode steps
+        "prompt_phase": {"seconds": round(prompts_done, 4), "prompt_tok_s": round(p_tok / prompts_done, 1)},
+        "decode_phase": {"seconds": round(elapsed - prompts_done, 4),
+                         "tok_s": round(n_req * (decode_tokens - 1) / max(elapsed - prompts_done, 1e-9), 1)},
+    }))
+    return 0
+
+
 def note(msg: str) -> None:
     """Progress goes to stderr; the one JSON line is all that stdout carries."""
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
@@ -141,7 +215,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
-    ap.add_argument("--shape", default="8B", choices=sorted(SHAPES), help="layer sizes of this Qwen3 model")
+    ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="layer sizes of this Qwen3 model (8B)")
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="run requests through the serving loop instead of timing decode steps")
+    ap.add_argument("--decode-tokens", type=int, default=None, help="tokens every request of a workload decodes")
     ap.add_argument("--layers", type=int, default=None,
                     help="run fewer layers than the model has (recorded in the config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
@@ -159,6 +236,8 @@ def main() -> int:
     from inferrs_amd.config import Qwen3Config
     from inferrs_amd.engine import Engine
 
+    if args.shape is None:
+        args.shape = WORKLOADS[args.workload][0] if args.workload else "8B"
     full_layers = SHAPES[args.shape]["num_hidden_layers"]
     if args.layers is None:
         args.layers = full_layers
@@ -166,6 +245,12 @@ def main() -> int:
     config = Qwen3Config.from_dict(raw)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     esize = 2 if args.dtype == "bfloat16" else 4
+    if args.workload:
+        if args.decode_tokens is None:
+            args.decode_tokens = WORKLOADS[args.workload][5]
+        note(f"random weights of {args.layers} layers")
+        return workload_main(args, raw, lambda pages, seqs: Engine.from_random(
+            config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=pages, max_seqs=seqs))
     points_batches = [] if args.no_points or args.prefill_only else [1, 64]
     # a point whose cache would not fit beside the weights is left out (batch 64 at a context of 32 k and more)
     per_token = 2 * raw["num_key_value_heads"] * raw["head_dim"] * args.layers * esize

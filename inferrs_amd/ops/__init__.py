@@ -396,12 +396,10 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 
 # ---- matrix products --------------------------------------------------------------------------
 
-# Beyond this many rows (one tile of MFMA columns) the vendor's GEMM reads the weights faster.  From 13 to 16
-# rows the single products are about even (us at the sizes of an 8 B model, qkv, o, gate|up with SiLU, down:
-# 16.9, 11.4, 49.6, 24.7 here against about 15, 12.5, 46.4, 22.5 there at 16 rows: past 12 rows the staging area
-# of the activations no longer fits beside enough blocks on a compute unit), but only these products take over
-# the sums and norms of the residual stream: a decode step of 13 requests at a context of 2,048 5.70 -> 5.37 ms,
-# of 16 requests 5.47 -> 5.37.
+# Beyond this many rows (one tile of MFMA columns) the vendor's GEMM reads the weights faster.  Up to 16 rows the
+# skinny products also take over the sums and norms of the residual stream; a decode step at a context of 2,048
+# and the sizes of an 8 B model takes 5.11 ms with 12 requests, 5.32 with 13 and 5.46 with 16 (5.54 and 5.44 with
+# the vendor's GEMM and norm kernels of their own from 13 rows on; at the 14B shape 9.7 against 10.9 ms at 14 rows).
 SKINNY_MAX_ROWS = 16
 
 
