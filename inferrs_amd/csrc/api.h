@@ -48,6 +48,9 @@ int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, i
 // Large bfloat16 products in tiles of 256 x 256 (gemm_mfma.hip); K a multiple of 64; with `dual` w is [gate; up]
 // and out = silu(x . gate^T) * (x . up^T).
 int ia_gemm_mfma_bf16(void* out, const void* x, const void* w, int M, int N, int K, int dual, hipStream_t stream);
+// Tuning knobs of the skinny product (tests switch the staged variants off with stage = 0); the defaults are
+// (2048, 8, 5, 8, 1).
+void ia_gemm_skinny_tune(int target_waves, int min_ksteps, int rot_mul, int min_waves, int stage);
 // The skinny product with a residual stream around it (decode steps; see gemm.hip): adds itself to `resid`
 // and leaves the rows' sums of squares and the rows times the next norm's weight, and / or takes such rows
 // and finishes their norm.

@@ -596,15 +596,15 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
         const size_t staged8 = tiles + (size_t)waves * rows * (8 * 2 * SK_KSTEP + SK_STAGE_PAD);
         const size_t staged16 = tiles + (size_t)waves * rows * (16 * 2 * SK_KSTEP + SK_STAGE_PAD);
         int stage = 0;
-        if (g_stage && rows >= 2 && skinny_tall((int)grid)) {
-            // Staging pays where blocks stream for long: with at least three blocks for every compute unit, from 2
-            // batch rows on (one row is one cache line a load anyway), with whole chunks of 8 k steps in a wave's
+        if (g_stage && rows >= 1 && skinny_tall((int)grid)) {
+            // Staging pays where blocks stream for long: with at least three blocks for every compute unit (also with
+            // one batch row: gate|up 39.2 -> 37.0 us, a decode step of one request 3.97 -> 3.84 ms), with whole chunks of 8 k steps in a wave's
             // range, and while the staging area leaves room for two blocks on a compute unit (eight waves: up to 15
             // rows; at 16 rows, one block a unit, a decode step at the sizes of an 8 B model took 5.73 ms against
             // 5.44 without staging; seven waves, a width of 5,120: all 16).  Measured at 8 rows: gate|up 46 -> 40 us,
             // logits head 261 -> 224 us; at 14 rows a decode step of the 14B shape 10.9 -> 9.7 ms.
             if (kper >= 8 && staged8 <= SK_STAGE_LDS_MOST - SK_SCALES_RESERVE) stage = 8;
-        } else if (g_stage && rows >= 2 && !DUAL && RT == 1) {
+        } else if (g_stage && rows >= 1 && !DUAL && RT == 1) {
             // A weight that one or two rounds of blocks cover (o, down, qkv) is read in one burst, and what counts
             // is how much a wave has in flight: chunks of 16 steps, as much as without staging, and up to
             // all of a compute unit's shared memory for its block.  Measured at 8 rows: down 25.6 -> 22.3 us,

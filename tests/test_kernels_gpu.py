@@ -523,24 +523,38 @@ def test_skinny_rows_do_not_depend_on_the_batch():
     assert torch.equal(ops.gemm_skinny_bf16(dev(x[3:9].contiguous()), dev(w), torch.float32).cpu(), full[3:9])
 
 
+def _without_staging(fn):
+    """The skinny product's plain variant: the tuning entry switches the staged ones off (and on again)."""
+    from inferrs_amd import ops
+    lib = ops.library()
+    lib.ia_gemm_skinny_tune(2048, 8, 5, 8, 0)
+    try:
+        return fn()
+    finally:
+        lib.ia_gemm_skinny_tune(2048, 8, 5, 8, 1)
+
+
 def test_skinny_variants_for_one_round_weights_agree_bit_for_bit():
-    # a weight of fewer than two blocks a compute unit whose waves take whole chunks of 16 k steps: staged at 2
-    # rows and more, plain at one row
+    # a weight of fewer than three blocks a compute unit whose waves take whole chunks of 16 k steps: its
+    # activations are staged through shared memory; the plain variant gives the same bits
     from inferrs_amd import ops
     n, k = 4096, 4096
     x = randn(16, k, dtype=torch.bfloat16, seed=1)
     w = randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
     full = ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32).cpu()
     close(full, x.double() @ w.double().t(), 2e-5, "one round")
+    assert torch.equal(_without_staging(lambda: ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32).cpu()), full)
     for lo, hi in ((0, 1), (7, 8), (3, 9), (0, 12), (2, 15)):
         part = ops.gemm_skinny_bf16(dev(x[lo:hi].contiguous()), dev(w), torch.float32).cpu()
         assert torch.equal(part, full[lo:hi]), (lo, hi)
+        assert torch.equal(_without_staging(lambda: ops.gemm_skinny_bf16(dev(x[lo:hi].contiguous()), dev(w), torch.float32).cpu()),
+                           part), (lo, hi)
 
 
 @pytest.mark.parametrize("dual", [False, True])
 def test_skinny_variants_for_tall_weights_agree_bit_for_bit(dual):
-    # a weight with more than two blocks a compute unit takes the variant that stages the activations
-    # through shared memory at 2 to 12 rows, and the plain one at 1 and at 16 rows
+    # a weight with three blocks a compute unit and more takes the variant that stages the activations through
+    # shared memory while two blocks fit a compute unit, the plain one beyond; both give the same bits
     from inferrs_amd import ops
     n, k = 8200, 520
     x = randn(16, k, dtype=torch.bfloat16, seed=1)
@@ -552,6 +566,7 @@ def test_skinny_variants_for_tall_weights_agree_bit_for_bit(dual):
         close(full, want, 2 ** -7, "dual")
     else:
         close(full, x.double() @ w.double().t(), 2e-5, "tall")
+    assert torch.equal(_without_staging(lambda: ops.gemm_skinny_bf16(dev(x), dev(w), torch.float32, dual=dual).cpu()), full)
     for lo, hi in ((0, 1), (3, 9), (0, 12), (5, 7), (2, 15)):
         part = ops.gemm_skinny_bf16(dev(x[lo:hi].contiguous()), dev(w), torch.float32, dual=dual).cpu()
         assert torch.equal(part, full[lo:hi]), (lo, hi)
