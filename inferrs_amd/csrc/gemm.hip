@@ -543,22 +543,16 @@ static void skinny_split(int N, int K, int rt, int tiles_per_wave, int* waves_ou
     int kper = (ksteps + waves - 1) / waves;
     // A range that is no multiple of the chunk ends in short chunks and single steps, each of which waits
     // for the memory on its own, and keeps the staged variants out (a width of 5,120 leaves 20 steps to each of
-    // eight waves).  Long rows are shared out in whole chunks instead.  Tall weights: chunks of 8 steps (what
-    // their staged variant takes) between no more waves than by the rule above, since blocks of more than eight
-    // waves streamed slower (24,576 x 5,120 at 8 rows: 7 waves of 24 steps 55.7 us, 10 of 16 62.5, 5 of 32 62.9).
-    // The others: chunks of 16 between as many waves, up to 12, as make the longest range shortest (5,120 -> 10
-    // waves of 16 steps, 17,408 -> 12 of 48, 25,600 -> 10 of 80; 5,120 x 5,120 at 8 rows 20.7 -> 17.6 us).  The
+    // eight waves).  Long rows are shared out in whole chunks instead, of 8 steps for tall weights (what their
+    // staged variant takes) and of 16 for the others, between no more waves than by the rule above: blocks of more
+    // than eight waves streamed slower (24,576 x 5,120 at 8 rows: 7 waves of 24 steps 55.7 us, 10 of 16 62.5;
+    // 5,120 x 17,408 at one row: 7 waves of 80 steps 35.0 us, 12 of 48 38.6; 5,120 x 5,120 at 8 rows: 5 waves of
+    // 32 steps 14.4 us, 10 of 16 16.0), and their staging areas leave room for one block a compute unit only.  The
     // last wave takes what is left.
     if (ksteps >= 8 * SK_CHUNK && kper % SK_CHUNK != 0) {
-        const bool tall = skinny_tall(groups);
-        const int unit = tall ? 8 : SK_CHUNK;
+        const int unit = skinny_tall(groups) ? 8 : SK_CHUNK;
         const int chunks = (ksteps + unit - 1) / unit;
-        // (12 waves: what leaves the staging area of 12 batch rows inside a compute unit's shared memory)
-        const int top = tall ? waves : (most < 12 ? most : 12);
-        int best = (chunks + waves - 1) / waves;
-        for (int w = waves + 1; w <= top; ++w)
-            if ((chunks + w - 1) / w < best) best = (chunks + w - 1) / w;
-        kper = best * unit;
+        kper = (chunks + waves - 1) / waves * unit;
         waves = (ksteps + kper - 1) / kper;
     }
     *waves_out = waves;
