@@ -538,7 +538,10 @@ static void skinny_split(int N, int K, int rt, int tiles_per_wave, int* waves_ou
     const int most = 65536 / (tiles_per_wave * IA_WAVE * (int)sizeof(f32x4));
     // (a logits head, two row tiles a wave, has blocks to spare: half as many waves with ranges twice as long read it
     // faster, 151,936 x 4,096 at 8 rows 228 -> 215 us, and leave room for the staging area of 16 rows, 296 -> 240 us)
-    const int min_waves = rt == 2 ? (g_min_waves + 1) / 2 : g_min_waves;
+    // So does a tall weight whose halved number of waves still takes whole chunks of 16 steps: gate|up of
+    // 2 x 12,288 x 4,096 at 8 rows 40.1 -> 38.8 us, at 16 rows 49.4 -> 42.8 (5,120 wide it does not: 72.4 -> 74.4 us).
+    const int half = (g_min_waves + 1) / 2;
+    const int min_waves = (rt == 2 || (skinny_tall(groups) && ksteps % (SK_CHUNK * half) == 0)) ? half : g_min_waves;
     int waves = 1;
     while (waves * 2 <= SK_MAX_WAVES && waves * 2 <= most && ksteps / (waves * 2) >= g_min_ksteps &&
            (groups * waves < g_target_waves || waves < min_waves))

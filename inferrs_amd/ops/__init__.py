@@ -398,7 +398,7 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 
 # Beyond this many rows (one tile of MFMA columns) the vendor's GEMM reads the weights faster.  Up to 16 rows the
 # skinny products also take over the sums and norms of the residual stream; a decode step at a context of 2,048
-# and the sizes of an 8 B model takes 5.11 ms with 12 requests, 5.32 with 13 and 5.46 with 16 (5.54 and 5.44 with
+# and the sizes of an 8 B model takes 5.02 ms with 12 requests, 5.20 with 13 and 5.22 with 16 (5.54 and 5.44 with
 # the vendor's GEMM and norm kernels of their own from 13 rows on; at the 14B shape 9.7 against 10.9 ms at 14 rows).
 SKINNY_MAX_ROWS = 16
 
