@@ -317,18 +317,20 @@ def test_captured_steps_of_many_requests_equal_eager_ones(models, tmp_path, n_re
     assert max(errs) <= 2 ** -6, f"replays differ from eager steps: {errs}"
 
 
-def test_real_layer_sizes(tmp_path):
+@pytest.mark.parametrize("hidden,heads,intermediate", [(4096, 32, 12288), (5120, 40, 17408)], ids=["8B", "14B"])
+def test_real_layer_sizes(tmp_path, hidden, heads, intermediate):
     """One layer with the sizes of Qwen3-8B (hidden 4096, 32 query and 8 key/value heads of 128,
-    intermediate 12288) and a small vocabulary: the kernels' serving shapes (the skinny products of
-    6144, 4096 and 2 x 12288 rows, among them the variant that stages the activations; attention over
-    head size 128 with four query heads a key/value head) against the plain implementation, whole,
-    with a decoded tail and mixed.  bfloat16 within 2 % of the largest logit (the tiny models'
-    measured bounds are 1 to 3 %), 32-bit within 1e-5."""
-    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1031, hidden_size=4096,
-               intermediate_size=12288, num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8,
+    intermediate 12288) or Qwen3-14B (5120, 40 query heads: five a key/value head, 17408) and a small
+    vocabulary: the kernels' serving shapes (the skinny products of 6144, 4096 and 2 x 12288 rows, among
+    them the variant that stages the activations; at the 14B sizes blocks of 10 and 14 features, k shared
+    out between five and seven waves, rows of 512 sums of squares; attention over head size 128) against
+    the plain implementation, whole, with a decoded tail and mixed.  bfloat16 within 2 % of the largest
+    logit (the tiny models' measured bounds are 1 to 3 %), 32-bit within 1e-5."""
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1031, hidden_size=hidden,
+               intermediate_size=intermediate, num_hidden_layers=1, num_attention_heads=heads, num_key_value_heads=8,
                head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
                max_position_embeddings=4096, hidden_act="silu")
-    folder = write_model(str(tmp_path / "layer8b"), raw, seed=21)
+    folder = write_model(str(tmp_path / "layer"), raw, seed=21)
     cfg, params = pm.read_model(folder, torch.float64)
     reqs = {f"r{i}": random_tokens(n, raw["vocab_size"], 300 + i) for i, n in enumerate([3, 40, 90])}
     ref = {r: pm.forward(cfg, params, t).numpy().astype(np.float32) for r, t in reqs.items()}
