@@ -189,10 +189,30 @@ __global__ void window_push_kernel(int* __restrict__ window, int w, const int* _
     win[cap - 1] = tokens[row];
 }
 
+// The same for windows of up to 64 entries (the reference's default, `repeat_last_n`), a wave a row and a lane an
+// entry: one thread that moves 64 entries one after the other took 17 us.
+__global__ __launch_bounds__(IA_WAVE) void window_push_wave_kernel(int* __restrict__ window, int w, const int* __restrict__ caps,
+                                                                   const int* __restrict__ tokens) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    int* win = window + (size_t)row * w;
+    const int cap = caps[row] < w ? caps[row] : w;
+    if (cap <= 0) return;
+    const int mine = lane < cap ? win[lane] : -1;
+    const unsigned long long empty = __ballot(lane < cap && mine < 0);
+    const int held = empty ? __ffsll((long long)empty) - 1 : cap;
+    const int next = __shfl_down(mine, 1, IA_WAVE);
+    if (held < cap) {
+        if (lane == held) win[lane] = tokens[row];
+    } else if (lane < cap) {
+        win[lane] = lane + 1 < cap ? next : tokens[row];
+    }
+}
+
 extern "C" int ia_window_push(int* window, int rows, int w, const int* caps, const int* tokens, hipStream_t stream) {
     IA_CHECK(rows >= 0 && w > 0, "window_push: bad sizes rows=%d w=%d", rows, w);
     if (rows == 0) return 0;
-    window_push_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(window, w, caps, tokens, rows);
+    if (w <= IA_WAVE) window_push_wave_kernel<<<rows, IA_WAVE, 0, stream>>>(window, w, caps, tokens);
+    else window_push_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(window, w, caps, tokens, rows);
     IA_LAUNCH_CHECK("window_push");
     return 0;
 }

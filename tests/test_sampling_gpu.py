@@ -255,3 +255,35 @@ def test_log_probability_parameters_are_checked():
     with pytest.raises(ValueError, match="0..20"):
         SamplingParams(logprobs=True, top_logprobs=21)
     assert not SamplingParams.greedy(logprobs=True).is_plain_greedy and SamplingParams.greedy().is_plain_greedy
+
+
+@pytest.mark.parametrize("w", [1, 5, 64, 100])
+def test_window_push_alone(w):
+    """A row's penalty window takes its new token: appended while the row's cap is not reached, else the oldest
+    entry goes; rows without a window stay as they are.  Windows of up to 64 entries take a wave a row, wider
+    ones a thread a row."""
+    import torch
+    from inferrs_amd import ops
+    g = torch.Generator().manual_seed(w)
+    rows = 9
+    caps = torch.tensor([0, 1, w, max(1, w // 2), w, w + 7, 2, w, 3], dtype=torch.int32)
+    held = [0, 1, 0, max(1, w // 2), w, w, 1, max(0, w - 1), 0]
+    window = torch.full((rows, w), -1, dtype=torch.int32)
+    for r in range(rows):
+        n = min(held[r], min(int(caps[r]), w))
+        window[r, :n] = torch.randint(0, 1000, (n,), generator=g, dtype=torch.int32)
+    tokens = torch.randint(0, 1000, (rows,), generator=g, dtype=torch.int32)
+    want = window.clone()
+    for r in range(rows):
+        cap = min(int(caps[r]), w)
+        if cap <= 0:
+            continue
+        have = int((want[r, :cap] >= 0).sum())
+        if have < cap:
+            want[r, have] = tokens[r]
+        else:
+            want[r, :cap - 1] = want[r, 1:cap].clone()
+            want[r, cap - 1] = tokens[r]
+    dev = "cuda:0"
+    got = ops.window_push(window.to(dev), caps.to(dev), tokens.to(dev)).cpu()
+    assert torch.equal(got, want)
