@@ -257,6 +257,7 @@ def test_log_probability_parameters_are_checked():
     assert not SamplingParams.greedy(logprobs=True).is_plain_greedy and SamplingParams.greedy().is_plain_greedy
 
 
+@pytest.mark.gpu
 @pytest.mark.parametrize("w", [1, 5, 64, 100])
 def test_window_push_alone(w):
     """A row's penalty window takes its new token: appended while the row's cap is not reached, else the oldest
