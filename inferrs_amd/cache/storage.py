@@ -1,9 +1,11 @@
 """Device arrays behind the cache manager's bookkeeping.
 
 Paged groups: per layer a key array `[pages, n_kv_heads, page_size, head_dim]` and a value array
-`[pages, n_kv_heads, head_dim, page_size]` (values are kept transposed inside a page: the
+`[pages, n_kv_heads, value_dim, page_size]` (values are kept transposed inside a page: the
 attention kernels multiply probabilities into them along the slots) in the model's precision,
-so one page of one head is `page_size * head_dim` contiguous elements.  (The reference keeps `[pages * page_size, n_kv_heads, head_dim]` per layer,
+so one page of one head is `page_size * head_dim` contiguous elements.  Keys and values of one
+width share one allocation; a mixer whose values are wider or narrower than its keys
+(`PagedKV.v_head_dim`) gets two.  (The reference keeps `[pages * page_size, n_kv_heads, head_dim]` per layer,
 `inferrs-models/src/kv_cache.rs:249-270`, and gathers it into a dense copy per pass; here the
 attention kernels read pages through the block table.)  Pages are not cleared on reuse:
 attention never reads beyond a request's length.
@@ -42,13 +44,18 @@ class CacheStorage:
         self.arrays = []
         for g in manager.groups:
             need = g.need
-            arr = torch.zeros((len(g.layers), 2, max(g.pool.num_pages, 1), need.n_kv_heads,
-                               manager.page_size, need.head_dim), dtype=dtype, device=device)
-            self.arrays.append(arr)
+            pages, ps = max(g.pool.num_pages, 1), manager.page_size
+            if need.value_dim == need.head_dim:
+                arr = torch.zeros((len(g.layers), 2, pages, need.n_kv_heads, ps, need.head_dim), dtype=dtype, device=device)
+                self.arrays.append(arr)
+                keys, values = arr[:, 0], arr[:, 1]
+            else:
+                keys = torch.zeros((len(g.layers), pages, need.n_kv_heads, ps, need.head_dim), dtype=dtype, device=device)
+                values = torch.zeros((len(g.layers), pages, need.n_kv_heads, ps, need.value_dim), dtype=dtype, device=device)
+                self.arrays += [keys, values]
             for i, layer in enumerate(g.layers):
-                self.layers[layer] = LayerCache(
-                    layer, g.index, arr[i, 0],
-                    arr[i, 1].view(arr.shape[2], need.n_kv_heads, need.head_dim, manager.page_size))
+                self.layers[layer] = LayerCache(layer, g.index, keys[i],
+                                                values[i].view(pages, need.n_kv_heads, need.value_dim, ps))
         for st in manager.states:
             arr = torch.zeros((manager.max_seqs, *st.need.shape), dtype=st.need.dtype, device=device)
             self.arrays.append(arr)
@@ -57,6 +64,17 @@ class CacheStorage:
     def clear_state_slot(self, slot: int) -> None:
         for st in self.manager.states:
             self.layers[st.layer].state[slot].zero_()
+
+    @staticmethod
+    def page_bytes(manager: CacheManager, dtype: torch.dtype) -> int:
+        """Bytes that one more page in every group costs, over all layers."""
+        esize = torch.empty((), dtype=dtype).element_size()
+        return sum(len(g.layers) * g.need.page_elements(manager.page_size) * esize for g in manager.groups)
+
+    @staticmethod
+    def state_bytes(manager: CacheManager) -> int:
+        """Bytes of the fixed-size state arrays: every request slot of every layer that keeps such state."""
+        return sum(manager.max_seqs * st.need.bytes_per_request() for st in manager.states)
 
     def bytes(self) -> int:
         return sum(a.numel() * a.element_size() for a in self.arrays)

@@ -92,18 +92,20 @@ def load_engine(args):
 class TokenCodec:
     """Text <-> token ids through the folder's tokenizer.json when there is one; plain ids else."""
 
-    def __init__(self, model_dir: str):
+    def __init__(self, model_dir: str, config=None):
+        from .chat import detect_template
         self.tokenizer = None
+        self.template = "plain"
         path = os.path.join(model_dir, "tokenizer.json")
         if os.path.isfile(path):
             from tokenizers import Tokenizer
             self.tokenizer = Tokenizer.from_file(path)
+            self.template = detect_template(model_dir, config)
 
     def encode(self, text: str, system: Optional[str] = None) -> List[int]:
         if self.tokenizer is not None:
-            if system:
-                text = f"<|im_start|>system\n{system}<|im_end|>\n<|im_start|>user\n{text}<|im_end|>\n<|im_start|>assistant\n"
-            return self.tokenizer.encode(text).ids
+            from .chat import render
+            return self.tokenizer.encode(render(self.template, text, system)).ids
         if system:
             raise SystemExit("inferrs-amd: --system needs a tokenizer.json in the model folder")
         try:
@@ -122,7 +124,7 @@ def cmd_run(args) -> int:
     from .engine import GenerationLoop
     from .sampling import SamplingParams
     engine = load_engine(args)
-    codec = TokenCodec(args.model)
+    codec = TokenCodec(args.model, getattr(engine, "config", None))
     params = SamplingParams(
         temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p,
         repetition_penalty=args.repetition_penalty, repeat_last_n=args.repeat_last_n,

@@ -13,37 +13,12 @@ activation is SiLU.
 """
 from __future__ import annotations
 
-import json
-import os
 from dataclasses import dataclass, asdict
-from typing import Any, Dict, Tuple
+from typing import Any, Dict, Optional, Tuple
 
+from .base import ConfigError, eos_ids as _eos_ids, opt_number as _opt_number, require_int as _require_int
 from .spec import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec,
                    PositionSpec, SpecError, default_schedule)
-
-
-class ConfigError(ValueError):
-    pass
-
-
-def _require_int(raw: Dict[str, Any], key: str, minimum: int = 1) -> int:
-    if key not in raw or raw[key] is None:
-        raise ConfigError(f"config.json: required key '{key}' is missing")
-    v = raw[key]
-    if isinstance(v, bool) or not isinstance(v, int):
-        raise ConfigError(f"config.json: '{key}' must be an integer, got {v!r}")
-    if v < minimum:
-        raise ConfigError(f"config.json: '{key}' must be >= {minimum}, got {v}")
-    return v
-
-
-def _opt_number(raw: Dict[str, Any], key: str, default: float) -> float:
-    v = raw.get(key)
-    if v is None:
-        return float(default)
-    if isinstance(v, bool) or not isinstance(v, (int, float)):
-        raise ConfigError(f"config.json: '{key}' must be a number, got {v!r}")
-    return float(v)
 
 
 @dataclass(frozen=True)
@@ -63,6 +38,7 @@ class Qwen3Config:
 
     architecture = "Qwen3ForCausalLM"
     model_type = "qwen3"
+    chat_template = "chatml"        # the family's prompts (`inferrs_amd.chat`), when the folder does not say
 
     @classmethod
     def from_dict(cls, raw: Dict[str, Any]) -> "Qwen3Config":
@@ -87,15 +63,7 @@ class Qwen3Config:
             tie = True
         if not isinstance(tie, bool):
             raise ConfigError(f"config.json: 'tie_word_embeddings' must be a boolean, got {tie!r}")
-        eos = raw.get("eos_token_id")
-        if eos is None:
-            eos_ids: Tuple[int, ...] = ()
-        elif isinstance(eos, int) and not isinstance(eos, bool):
-            eos_ids = (eos,)
-        elif isinstance(eos, list) and all(isinstance(e, int) for e in eos):
-            eos_ids = tuple(eos)
-        else:
-            raise ConfigError(f"config.json: 'eos_token_id' must be an integer or a list, got {eos!r}")
+        eos_ids = _eos_ids(raw)
         maxpos = raw.get("max_position_embeddings")
         maxpos = 40960 if maxpos is None else _require_int(raw, "max_position_embeddings")
         cfg = cls(
@@ -152,10 +120,9 @@ class Qwen3Config:
                                     position=position, qk_norm=head_norm, window=None),
                 ffn=GatedMlpSpec(hidden=self.hidden_size, intermediate=self.intermediate_size,
                                  activation="silu"),
-                norm_mixer=layer_norm, norm_ffn=layer_norm,
-                mixer_prefix=p + "self_attn.", ffn_prefix=p + "mlp.",
-                norm_mixer_name=p + "input_layernorm.weight",
-                norm_ffn_name=p + "post_attention_layernorm.weight",
+                norms=(layer_norm, layer_norm),
+                norm_names=(p + "input_layernorm.weight", p + "post_attention_layernorm.weight"),
+                mixer_prefix=p + "self_attn.", ffn_prefix=p + "mlp.", arrangement="pre_norm",
             ))
         spec = ModelSpec(
             architecture=self.architecture, vocab_size=self.vocab_size, hidden=self.hidden_size,
@@ -166,17 +133,3 @@ class Qwen3Config:
             max_position=self.max_position_embeddings, eos_token_ids=self.eos_token_ids)
         spec.validate()
         return spec
-
-
-def read_config_json(model_dir: str) -> Dict[str, Any]:
-    path = os.path.join(model_dir, "config.json")
-    if not os.path.isfile(path):
-        raise ConfigError(f"config.json not found in {model_dir}")
-    try:
-        with open(path, "r", encoding="utf-8") as f:
-            raw = json.load(f)
-    except json.JSONDecodeError as e:
-        raise ConfigError(f"Failed to parse config.json in {model_dir}: {e}") from e
-    if not isinstance(raw, dict):
-        raise ConfigError(f"config.json in {model_dir} must hold a JSON object")
-    return raw

@@ -17,7 +17,8 @@ from __future__ import annotations
 
 from typing import Any, Dict, Optional, Type
 
-from .qwen3 import ConfigError, Qwen3Config, read_config_json
+from .base import ConfigError, read_config_json
+from .qwen3 import Qwen3Config
 from .spec import ModelSpec
 
 _BY_ARCHITECTURE: Dict[str, Type] = {}

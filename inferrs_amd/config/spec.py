@@ -75,16 +75,39 @@ class GatedMlpSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One residual block: which parts, and the tensor-name prefixes they load from."""
+    """One residual block: which parts, how they are arranged, and the tensor names they load from.
+
+    `arrangement` names a registered block class (`parts.register_block`), which says how many
+    norms it has and where they stand: "pre_norm" has two, before the mixer and before the
+    feed-forward.  `norms[i]` loads its weight from `norm_names[i]`."""
     mixer: Any
     ffn: Any
-    norm_mixer: NormSpec
-    norm_ffn: NormSpec
+    norms: Tuple[NormSpec, ...]
+    norm_names: Tuple[str, ...]
     mixer_prefix: str
     ffn_prefix: str
-    norm_mixer_name: str
-    norm_ffn_name: str
     arrangement: str = "pre_norm"
+
+
+@dataclass(frozen=True)
+class EmbeddingSpec:
+    """Token ids -> rows of the stream.  kind "embedding": a gather from a [vocab, hidden] table."""
+    vocab_size: int
+    hidden: int
+    name: str
+    kind: str = "embedding"
+
+
+@dataclass(frozen=True)
+class HeadSpec:
+    """Normed rows -> logits.  kind "lm_head": a product with a [vocab, hidden] matrix stored under
+    `name`; when the file has no such tensor (or `name` is None) the embedding table serves.
+    `required`: a random model is written with a matrix of its own."""
+    vocab_size: int
+    hidden: int
+    name: Optional[str]
+    required: bool = True
+    kind: str = "lm_head"
 
 
 @dataclass(frozen=True)
@@ -107,13 +130,21 @@ class ModelSpec:
     hidden: int
     layers: Tuple[LayerSpec, ...]
     schedule: Tuple[ScheduleEntry, ...]
-    final_norm: NormSpec
-    final_norm_name: str
+    final_norm: Optional[NormSpec]      # None: the head reads the stream as it is
+    final_norm_name: Optional[str]
     embed_name: str
     head_name: Optional[str]            # None: logits use the embedding table
     max_position: int
     head_required: bool = True          # False: use `head_name` if the file has it, else the table
     eos_token_ids: Tuple[int, ...] = field(default_factory=tuple)
+    embedding: Any = None               # a spec whose `kind` names a registered embedding part; None: EmbeddingSpec
+    head: Any = None                    # likewise for the logits head; None: HeadSpec
+
+    def __post_init__(self):
+        if self.embedding is None:
+            object.__setattr__(self, "embedding", EmbeddingSpec(self.vocab_size, self.hidden, self.embed_name))
+        if self.head is None:
+            object.__setattr__(self, "head", HeadSpec(self.vocab_size, self.hidden, self.head_name, self.head_required))
 
     def validate(self) -> None:
         n = len(self.layers)
@@ -121,6 +152,11 @@ class ModelSpec:
             raise SpecError("a model needs at least one layer")
         if not self.schedule:
             raise SpecError("the schedule is empty")
+        if (self.final_norm is None) != (self.final_norm_name is None):
+            raise SpecError("a final norm and the name of its weight come together")
+        for i, layer in enumerate(self.layers):
+            if len(layer.norms) != len(layer.norm_names):
+                raise SpecError(f"layer {i}: {len(layer.norms)} norms but {len(layer.norm_names)} names for their weights")
         for i, e in enumerate(self.schedule):
             if not (0 <= e.layer < n):
                 raise SpecError(f"schedule stop {i} names layer {e.layer}, outside 0..{n - 1}")

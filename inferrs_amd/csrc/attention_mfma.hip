@@ -181,7 +181,8 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         for (int db = 0; db < DB; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
-    int lo = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;
+    const int window_floor = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;   // first key any column sees
+    int lo = window_floor;
     int hi = pmax + 1;
     if (p.splits > 1) {
         const int c_lo = split * p.chunk, c_hi = c_lo + p.chunk;
@@ -267,6 +268,23 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
                         if (j >= first_bad) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                    op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+            }
+        }
+        if (p.window > 0 && k0 < window_floor) {
+            // The walk starts at a multiple of 32 below the first key that any column sees: the keys in between
+            // may lie in pages that the window has passed and the request has given back (the block table then
+            // names some other page, which holds anything at all).  Their scores are masked below; their values
+            // are zeroed here, for the same reason as the slots beyond the length.
+            const int first_good = window_floor - (k0 + 8 * G);     // keys below this index are outside every window
+            if (first_good > 0) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (j < first_good) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
                     op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
                 }
             }
@@ -550,7 +568,8 @@ void attn_tile_kernel(const AttnParams p) {
         const int* bt = p.block_table + (size_t)seq * p.max_pages;
         const int blast = (bcol0 + TILE_COLS <= n_cols ? bcol0 + TILE_COLS : n_cols) - 1;
         const int bpmin = kv_start + bcol0 / g, bpmax = kv_start + blast / g;
-        int lo = p.window > 0 ? (bpmin - p.window + 1 > 0 ? bpmin - p.window + 1 : 0) : 0;
+        const int bfloor = p.window > 0 ? (bpmin - p.window + 1 > 0 ? bpmin - p.window + 1 : 0) : 0;   // first key the block sees
+        int lo = bfloor;
         lo &= ~(TILE_STAGE - 1);
         int hi = bpmax + 1;
         if (p.splits > 1) {             // this block's share of the keys (`chunk` is a multiple of a stage)
@@ -635,11 +654,14 @@ void attn_tile_kernel(const AttnParams p) {
         };
         // values of keys past the request's length may hold anything at all: a lane zeroes them in the
         // pieces that it brought itself, once they have arrived
+        // So may the values of keys below the block's window, between the stage's start and the first key that any
+        // of its columns sees: the window has passed them, and their pages may have been given back.
         auto zero_tail = [&](int s, char* buf) {
             const int kb = lo + s * TILE_STAGE;
-            if (kb + TILE_STAGE <= kv_total) return;
-            const int first_bad = kv_total - (kb + 16 * wave_s + 8 * v_half);
-            if (first_bad >= 8) return;
+            const int mine = kb + 16 * wave_s + 8 * v_half;          // the first of this lane's eight keys
+            const int first_bad = kb + TILE_STAGE <= kv_total ? 8 : kv_total - mine;
+            const int first_good = kb < bfloor ? bfloor - mine : 0;
+            if (first_bad >= 8 && first_good <= 0) return;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 uint4* at = (uint4*)(buf + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024 + lane * 16);
@@ -647,7 +669,7 @@ void attn_tile_kernel(const AttnParams p) {
                 uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (j >= first_bad) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                    if (j >= first_bad || j < first_good) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
                 *at = make_uint4(w[0], w[1], w[2], w[3]);
             }
         };

@@ -215,6 +215,7 @@ struct Sched {
     std::vector<PlanEntry> plan;
     std::vector<int64_t> preempted, failed;
     bool broken = false;          // the last plan met a misuse; the message is in the error channel
+    std::unordered_set<int64_t> left_out;   // decodes that found no budget in the last plan: served first in the next
 
     bool is_running(const Req* r) const { return std::find(running.begin(), running.end(), r) != running.end(); }
     bool fits_alone(int n_tokens) const {
@@ -260,9 +261,13 @@ struct Sched {
         std::vector<Req*> decoding;
         for (Req* r : running)
             if (r->total() - r->computed == 1 && r->n_output() > 0) decoding.push_back(r);
+        // (a budget smaller than the number of decoding requests must not starve the late ones: whoever was
+        // left out last time goes first, in admission order, then the others)
+        std::stable_partition(decoding.begin(), decoding.end(), [&](Req* r) { return left_out.count(r->key) != 0; });
+        left_out.clear();
         for (Req* r : decoding) {
             if (!is_running(r)) continue;                 // preempted while serving an earlier one
-            if (budget < 1) break;
+            if (budget < 1) { left_out.insert(r->key); continue; }
             bool ok = true;
             while (cache->reserve(*cache->find(r->key), 1) != 0) {
                 Req* victim = preempt_latest(r);
@@ -627,7 +632,7 @@ int iar_build_step(void* cache, int n_entries, const int64_t* keys, const int* q
                 slots[cu[j] + q] = page * ps + pos % ps;
             }
             const int copy = std::min((int)t.size(), max_pages);
-            for (int q = 0; q < copy; ++q) table[(long long)j * max_pages + q] = t[q] < 0 ? 0 : t[q];   // released pages are never read
+            for (int q = 0; q < copy; ++q) table[(long long)j * max_pages + q] = t[q] < 0 ? 0 : t[q];   // (a released entry names page 0: kernels that round a window's start down may load from it, and use nothing of it)
         }
     }
     meta[0] = (int)total; meta[1] = n; meta[2] = n_entries; meta[3] = n_want; meta[4] = max_pages; meta[5] = max_q;

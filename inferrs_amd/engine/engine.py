@@ -10,18 +10,23 @@ everything earlier comes from the cache that previous steps left.
 """
 from __future__ import annotations
 
+import logging
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import torch
 
 from .. import ops
 from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..config.base import folder_stop_ids
 from ..config.registry import load_config
 from ..parts.assemble import generated_tensors, model_tensors
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
 from .batch import StepBuilder, StepError
 from .model import DecoderModel, parse_dtype
+
+
+log = logging.getLogger("inferrs_amd")
 
 
 class Entry:
@@ -53,11 +58,14 @@ class Engine:
         if num_pages is None and cache_tokens is not None:
             num_pages = -(-cache_tokens // page_size)
         if num_pages is None:
-            esize = 4 if model.dtype == torch.float32 else 2
-            per_page = sum(len(g.layers) * 2 * g.need.n_kv_heads * g.need.head_dim * page_size * esize
-                           for g in probe.groups)
+            # the budget pays for the fixed-size state of every request slot first, pages get the rest
+            per_page = CacheStorage.page_bytes(probe, model.dtype)
             free, _total = torch.cuda.mem_get_info(self.device)
-            num_pages = max(1, int(free * memory_fraction) // max(per_page, 1))
+            budget = int(free * memory_fraction) - CacheStorage.state_bytes(probe)
+            if budget < per_page:
+                raise OutOfPages(f"{memory_fraction:.2f} of the free GPU memory ({free >> 20} MiB) does not hold the "
+                                 f"per-request state of {max_seqs} requests and one page of {per_page} bytes")
+            num_pages = max(1, budget // max(per_page, 1))
             # more than every request slot at the longest sequence is never used
             num_pages = min(num_pages, max_seqs * -(-model.spec.max_position // page_size))
         self.cache = CacheManager(needs, page_size, num_pages, max_seqs)
@@ -66,19 +74,30 @@ class Engine:
         # Decode steps (one token a request) are launch-bound: each distinct shape is captured
         # into a HIP graph the second time it is seen and replayed from then on.
         self.use_graphs = use_graphs and model.graph_safe
+        self.unused_tensors: List[str] = []
+        self.stop_token_ids: Tuple[int, ...] = tuple(model.spec.eos_token_ids)
         self._graphs: Dict[Tuple[int, int, int], object] = {}
+        self._graphs_generation = self.builder.generation    # the staging buffer the graphs were captured over
         self.graph_replays = 0
 
     # ---- construction -----------------------------------------------------------------------
     @classmethod
-    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", strict: bool = False, **kw) -> "Engine":
+        """`strict`: tensors of the folder that the model does not read are an error instead of a note."""
         config = load_config(model_dir)
         spec = config.to_spec()
         expected, optional = model_tensors(spec)
-        tensors = load_weights(model_dir, expected, optional)
+        unused: List[str] = []
+        tensors = load_weights(model_dir, expected, optional, strict=strict, unused=unused)
+        if unused:
+            log.info("%s: %d tensors are not read by %s: %s", model_dir, len(unused), spec.architecture,
+                     ", ".join(unused[:8]) + (" ..." if len(unused) > 8 else ""))
         model = DecoderModel(spec, tensors, parse_dtype(dtype), device)
         eng = cls(model, **kw)
         eng.config = config
+        eng.unused_tensors = unused
+        # what ends a request of this folder's model: config.json's ids and what the files beside it declare
+        eng.stop_token_ids = folder_stop_ids(model_dir, spec.eos_token_ids)
         return eng
 
     @classmethod
@@ -165,6 +184,7 @@ class Engine:
         captured graph whose context bucket holds them to the end."""
         if not self.use_graphs or steps < 1 or not seq_ids:
             return False
+        self._drop_stale_graphs()
         pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
         entry = self._graphs.get((len(seq_ids), len(seq_ids), pad_pages))
         return entry is not None and entry != "seen"
@@ -198,6 +218,14 @@ class Engine:
             self.graph_replays += 1
         return chosen.cpu().tolist()
 
+    def _drop_stale_graphs(self) -> None:
+        """Captured graphs hold the address of the step builder's device buffer.  Any step, also one
+        that is not a decode step (a long prompt portion), may have made that buffer grow and move
+        since: graphs captured over the old one are dropped before any of them is looked up."""
+        if self._graphs_generation != self.builder.generation:
+            self._graphs.clear()
+            self._graphs_generation = self.builder.generation
+
     def _decode_step(self, triples) -> torch.Tensor:
         """One token a request, through a captured graph when this shape has been seen before.
         The block tables are padded to the bucket's width, so that every kernel argument is the
@@ -206,10 +234,9 @@ class Engine:
         longest = self.cache.max_length([t[0] for t in triples]) + 1
         pad_pages = self._bucket_pages(longest)
         n_want = sum(len(t[2]) for t in triples)
-        generation = self.builder.generation
+        self._drop_stale_graphs()
         ctx = self.builder.build(triples, pad_pages=pad_pages)
-        if self.builder.generation != generation:
-            self._graphs.clear()                        # the staging buffer moved: captured addresses are stale
+        self._drop_stale_graphs()                       # (the buffer may have moved in this very build)
         key = (len(triples), n_want, pad_pages)
         entry = self._graphs.get(key)
         if entry is None:

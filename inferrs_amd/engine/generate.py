@@ -38,7 +38,7 @@ class GenerationLoop:
         self.scheduler = Scheduler(
             engine.cache, max_batch_size=min(max_batch_size, engine.cache.max_seqs),
             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk, max_seq_len=limit,
-            stop_token_ids=engine.spec.eos_token_ids if stop_token_ids is None else stop_token_ids)
+            stop_token_ids=engine.stop_token_ids if stop_token_ids is None else stop_token_ids)
         self.sampler = Sampler(engine.device)
         self.steps = 0
         self._next_id = 0

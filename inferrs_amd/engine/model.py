@@ -9,9 +9,8 @@ import torch
 
 from .. import ops
 from ..config.spec import ModelSpec
-from ..parts.base import part_class
-from ..parts.block import Block
-from ..parts.linear import Linear, to_compute
+from ..parts.base import block_class, part_class
+from ..parts.linear import Linear
 from .batch import StepContext
 
 DTYPES = {"float32": torch.float32, "f32": torch.float32, "fp32": torch.float32,
@@ -35,32 +34,29 @@ class DecoderModel:
         on any device.  Entries are dropped from the dict as they are taken over."""
         spec.validate()
         self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
-        self.embed = to_compute(tensors[spec.embed_name], dtype, device)
-        head = tensors.pop(spec.head_name, None) if spec.head_name is not None else None
-        if head is not None:
-            self.head = Linear([head], dtype, device)
-        else:
-            self.head = Linear.__new__(Linear)           # logits share the embedding table
-            self.head.weight = self.embed
-            self.head.out_features, self.head.in_features = self.embed.shape
-        del head
-        tensors.pop(spec.embed_name, None)
+
+        def take(names) -> Dict[str, torch.Tensor]:
+            return {n: tensors.pop(n) for n in list(names) if n in tensors}
+
+        embedding_cls = part_class("embedding", spec.embedding)
+        self.embedding = embedding_cls(spec.embedding, take(embedding_cls.tensors(spec.embedding)), dtype, device)
+        head_cls = part_class("head", spec.head)
+        self.head = head_cls(spec.head, take(head_cls.tensors(spec.head)), dtype, device, embedding=self.embedding)
         self.blocks = []
         for layer in spec.layers:
-            names = [n for n in tensors if n.startswith(layer.mixer_prefix) or n.startswith(layer.ffn_prefix)
-                     or n in (layer.norm_mixer_name, layer.norm_ffn_name)]
-            self.blocks.append(Block(layer, {n: tensors[n] for n in names}, dtype, device))
-            for n in names:
-                del tensors[n]
-        self.final_norm = part_class("norm", spec.final_norm)(
-            spec.final_norm, {"weight": tensors.pop(spec.final_norm_name)}, dtype, device)
+            cls = block_class(layer)
+            self.blocks.append(cls(layer, take(cls.tensors(layer)), dtype, device))
+        self.final_norm = None
+        if spec.final_norm is not None:
+            self.final_norm = part_class("norm", spec.final_norm)(
+                spec.final_norm, {"weight": tensors.pop(spec.final_norm_name)}, dtype, device)
 
     @property
     def graph_safe(self) -> bool:
         """Whether every part allows a decode step to be captured and replayed."""
-        parts = [self.final_norm]
+        parts = [self.embedding, self.head, self.final_norm]
         for b in self.blocks:
-            parts += [b.mixer, b.ffn, b.norm_mixer, b.norm_ffn, getattr(b.mixer, "position", None)]
+            parts += list(b.parts())
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
     def cache_needs(self) -> Dict[int, object]:
@@ -75,24 +71,27 @@ class DecoderModel:
     def forward(self, ctx: StepContext, storage) -> torch.Tensor:
         """Runs the step's tokens through every stop of the schedule (which appends to the
         caches) and returns float32 logits `[n_want, vocab]`."""
-        x = ops.embed_gather(self.embed, ctx.token_ids)
+        x = self.embedding.forward(ctx)
         pending = None                               # a block's output that is not added to x yet
         for stop, e in enumerate(self.spec.schedule):
             cache = storage.layers.get(self.spec.cache_stop(stop))
             if cache is not None and e.cache_of is not None:
                 cache = cache.reader()
             after = self.spec.schedule[stop + 1].layer if stop + 1 < len(self.spec.schedule) else None
-            next_norm = self.blocks[after].norm_mixer if after is not None else None
+            next_norm = self.blocks[after].first_norm if after is not None else None
             x, pending = self.blocks[e.layer].forward(ctx, x, pending, cache, next_norm)
         n_want = ctx.want_rows.numel()
         if n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         xs = ops.gather_rows(x, ctx.want_rows)
-        if isinstance(pending, ops.Added):           # the last block has added its output to x itself
+        added = pending is None or isinstance(pending, ops.Added)   # the last block has left nothing to add
+        if self.final_norm is None:
+            h = xs if added else ops.add_inplace(xs, ops.gather_rows(pending, ctx.want_rows))
+        elif added:
             h = self.final_norm.forward(xs)
         else:
             h = self.final_norm.add_forward(xs, ops.gather_rows(pending, ctx.want_rows))
-        return self.head(h, out_dtype=torch.float32)
+        return self.head.forward(h)
 
     def weight_bytes(self) -> int:
         seen, total = set(), 0
@@ -100,12 +99,15 @@ class DecoderModel:
             nonlocal total
             if t is not None and t.data_ptr() not in seen:
                 seen.add(t.data_ptr()); total += t.numel() * t.element_size()
-        add(self.embed); add(self.head.weight); add(self.final_norm.weight)
+        parts = [self.embedding, self.head, self.final_norm]
         for b in self.blocks:
-            for part in (b.mixer, b.ffn, b.norm_mixer, b.norm_ffn):
-                for v in vars(part).values():
-                    if isinstance(v, torch.Tensor):
-                        add(v)
-                    elif isinstance(v, Linear):
-                        add(v.weight)
+            parts += list(b.parts())
+        for part in parts:
+            if part is None:
+                continue
+            for v in vars(part).values():
+                if isinstance(v, torch.Tensor):
+                    add(v)
+                elif isinstance(v, Linear):
+                    add(v.weight)
         return total

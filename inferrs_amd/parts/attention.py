@@ -47,8 +47,13 @@ class Attention(Mixer):
     def __init__(self, spec: AttentionSpec, tensors: Dict[str, torch.Tensor], dtype, device):
         if spec.n_heads % spec.n_kv_heads:
             raise SpecError(f"attention: {spec.n_heads} heads are not a multiple of {spec.n_kv_heads} kv heads")
-        if spec.head_dim % 16 or not (16 <= spec.head_dim <= 512):
-            raise SpecError(f"attention: head_dim {spec.head_dim} must be a multiple of 16 in 16..512")
+        # (the matrix-core kernels take head sizes in steps of 16 up to 256 in bfloat16; every other size, and the
+        # 32-bit path, runs on the plain kernels, which take any size up to 512)
+        if not (1 <= spec.head_dim <= 512):
+            raise SpecError(f"attention: head_dim {spec.head_dim} is outside 1..512, the range of the attention kernels")
+        rot = getattr(spec.position, "rot_dim", 0) if getattr(spec.position, "kind", "none") != "none" else 0
+        if rot % 2 or rot > spec.head_dim:
+            raise SpecError(f"attention: the rotated part of a head ({rot}) must be even and within head_dim {spec.head_dim}")
         if spec.window is not None and spec.window < 1:
             raise SpecError(f"attention: window {spec.window} must be >= 1")
         if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:

@@ -36,10 +36,20 @@ from ..weights.loader import TensorSpec
 
 @dataclass(frozen=True)
 class PagedKV:
-    """Keys and values of every cached position, in pages; `window` keeps only the last ones."""
+    """Keys and values of every cached position, in pages; `window` keeps only the last ones.
+    `head_dim` is the width of a key; values have `v_head_dim` (None: the same)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    def page_elements(self, page_size: int) -> int:
+        """Elements that one page of one layer holds (keys and values of all heads)."""
+        return self.n_kv_heads * page_size * (self.head_dim + self.value_dim)
 
 
 @dataclass(frozen=True)
@@ -48,10 +58,17 @@ class FixedState:
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
 
+    def bytes_per_request(self) -> int:
+        n = 1
+        for s in self.shape:
+            n *= int(s)
+        return n * torch.empty((), dtype=self.dtype).element_size()
+
 
 # ---- registries -----------------------------------------------------------------------------
 
-_TABLES: Dict[str, Dict[str, type]] = {"mixer": {}, "ffn": {}, "norm": {}, "position": {}}
+_TABLES: Dict[str, Dict[str, type]] = {"mixer": {}, "ffn": {}, "norm": {}, "position": {}, "block": {},
+                                       "embedding": {}, "head": {}}
 
 
 def _register(table: str, kind: str) -> Callable[[type], type]:
@@ -76,6 +93,28 @@ def register_norm(kind: str):
 
 def register_position(kind: str):
     return _register("position", kind)
+
+
+def register_block(arrangement: str):
+    """A block class: how a layer's mixer, feed-forward and norms are arranged around the stream.
+    Looked up by `LayerSpec.arrangement`."""
+    return _register("block", arrangement)
+
+
+def register_embedding(kind: str):
+    return _register("embedding", kind)
+
+
+def register_head(kind: str):
+    return _register("head", kind)
+
+
+def block_class(layer_spec: Any) -> type:
+    try:
+        return _TABLES["block"][layer_spec.arrangement]
+    except KeyError:
+        raise KeyError(f"no block is registered for the arrangement {layer_spec.arrangement!r}; "
+                       f"known: {sorted(_TABLES['block'])}") from None
 
 
 def part_class(table: str, spec: Any) -> type:
@@ -129,3 +168,46 @@ class Position(Part):
     def table(self, positions: torch.Tensor):
         """Whatever the mixer's kernels need for these positions (None for no encoding)."""
         return None
+
+
+class BlockBase:
+    """One layer around the residual stream.  A block class offers
+
+      * `tensors(layer_spec) -> {full tensor name: TensorSpec}` (a classmethod),
+      * `__init__(layer_spec, tensors, dtype, device)` with `tensors` keyed by those names,
+      * `forward(ctx, x, pending, cache, next_norm) -> (x, pending)`: `x` is the stream, `pending` what the
+        block before has left to be added to it (None, a tensor, or `ops.Added` when it is in already), `cache`
+        the mixer's `LayerCache`, `next_norm` the `first_norm` of the block that runs next (or the model's
+        final norm's stand-in None); the block returns the stream and what IT leaves to be added,
+      * `first_norm`: the norm part that reads the stream first in this block, or None (only a block before
+        it that prepares rows for exactly this norm looks at it),
+      * `parts()`: every part it holds, for the model's questions (may a step be captured, bytes of weights).
+    """
+    first_norm = None
+
+    @classmethod
+    def tensors(cls, layer_spec) -> Dict[str, TensorSpec]:
+        raise NotImplementedError
+
+    def parts(self):
+        return []
+
+    def forward(self, ctx, x, pending, cache, next_norm=None):
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    """Token ids -> the stream's first rows: `forward(ctx) -> [n_tokens, hidden]`; `table` is the
+    [vocab, hidden] matrix a tied logits head may share (None if there is none to share)."""
+    table = None
+
+    def forward(self, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Normed rows -> 32-bit logits: `__init__(spec, tensors, dtype, device, embedding)` (the embedding
+    part, for a tied head) and `forward(rows) -> float32 [rows, vocab]`."""
+
+    def forward(self, rows: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError

@@ -1,39 +1,73 @@
 """One residual block.  Arrangement "pre_norm" as in the reference
 (`inferrs-models/src/models/qwen3.rs:284-300`):
 
-    x = x + mixer(norm_mixer(x));  x = x + ffn(norm_ffn(x))
+    x = x + mixer(norm_0(x));  x = x + ffn(norm_1(x))
 
 The sums are formed in 32-bit inside the norm kernel that follows them, so a block takes
 the stream `x` together with the not-yet-added output of the block before it and returns
 the same pair.  In steps of a few rows the products around a norm can take over both the sum
 and the norm (`ops.Added`, `ops.NormedRows`).
+
+Other arrangements (norms after the parts, four norms around them, parts side by side) are other
+classes under `register_block`; the model asks the table by `LayerSpec.arrangement`.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Tuple
+from typing import Dict, Tuple
 
 import torch
 
 from .. import ops
 from ..config.spec import LayerSpec, SpecError
-from .base import part_class
+from ..weights.loader import TensorSpec
+from .base import BlockBase, part_class, register_block
 
 
-class Block:
+def sub_tensors(tensors: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tensor]:
+    return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
+
+
+def part_tensors(layer: LayerSpec, n_norms: int) -> Dict[str, TensorSpec]:
+    """The tensors of a layer's mixer, feed-forward and `n_norms` norms, by full name."""
+    if len(layer.norms) != n_norms or len(layer.norm_names) != n_norms:
+        raise SpecError(f"the arrangement {layer.arrangement!r} has {n_norms} norms, the layer names {len(layer.norms)}")
+    out: Dict[str, TensorSpec] = {}
+    for local, ts in part_class("mixer", layer.mixer).tensors(layer.mixer).items():
+        out[layer.mixer_prefix + local] = ts
+    for local, ts in part_class("ffn", layer.ffn).tensors(layer.ffn).items():
+        out[layer.ffn_prefix + local] = ts
+    for name, nspec in zip(layer.norm_names, layer.norms):
+        (ts,) = part_class("norm", nspec).tensors(nspec).values()
+        out[name] = ts
+    return out
+
+
+def build_parts(layer: LayerSpec, tensors: Dict[str, torch.Tensor], dtype, device):
+    """(mixer, feed-forward, [norms]) of a layer."""
+    mixer = part_class("mixer", layer.mixer)(layer.mixer, sub_tensors(tensors, layer.mixer_prefix), dtype, device)
+    ffn = part_class("ffn", layer.ffn)(layer.ffn, sub_tensors(tensors, layer.ffn_prefix), dtype, device)
+    norms = [part_class("norm", nspec)(nspec, {"weight": tensors[name]}, dtype, device)
+             for name, nspec in zip(layer.norm_names, layer.norms)]
+    return mixer, ffn, norms
+
+
+@register_block("pre_norm")
+class Block(BlockBase):
+    N_NORMS = 2
+
+    @classmethod
+    def tensors(cls, spec: LayerSpec) -> Dict[str, TensorSpec]:
+        return part_tensors(spec, cls.N_NORMS)
+
     def __init__(self, spec: LayerSpec, tensors: Dict[str, torch.Tensor], dtype, device):
-        if spec.arrangement != "pre_norm":
-            raise SpecError(f"unknown block arrangement {spec.arrangement!r}")
+        if len(spec.norms) != self.N_NORMS:
+            raise SpecError(f"a pre-norm block has two norms, the layer names {len(spec.norms)}")
         self.spec = spec
+        self.mixer, self.ffn, (self.norm_mixer, self.norm_ffn) = build_parts(spec, tensors, dtype, device)
+        self.first_norm = self.norm_mixer
 
-        def sub(prefix: str) -> Dict[str, torch.Tensor]:
-            return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
-
-        self.mixer = part_class("mixer", spec.mixer)(spec.mixer, sub(spec.mixer_prefix), dtype, device)
-        self.ffn = part_class("ffn", spec.ffn)(spec.ffn, sub(spec.ffn_prefix), dtype, device)
-        self.norm_mixer = part_class("norm", spec.norm_mixer)(
-            spec.norm_mixer, {"weight": tensors[spec.norm_mixer_name]}, dtype, device)
-        self.norm_ffn = part_class("norm", spec.norm_ffn)(
-            spec.norm_ffn, {"weight": tensors[spec.norm_ffn_name]}, dtype, device)
+    def parts(self):
+        return [self.mixer, self.ffn, self.norm_mixer, self.norm_ffn, getattr(self.mixer, "position", None)]
 
     def forward(self, ctx, x: torch.Tensor, pending, cache, next_norm=None) -> Tuple[torch.Tensor, object]:
         # Steps of a few bfloat16 rows (decode): a part that says `adds_to_stream` may add its output to
@@ -52,6 +86,13 @@ class Block:
         out = self.ffn.forward(ctx, h2)
         ctx.stream = ctx.stream_norm = None
         return x, out
+
+
+def settle(x: torch.Tensor, pending) -> torch.Tensor:
+    """The stream with `pending` added (in place): for arrangements and model ends that do not begin with a norm."""
+    if pending is not None and not isinstance(pending, ops.Added):
+        ops.add_inplace(x, pending)
+    return x
 
 
 def normed(norm, x: torch.Tensor, pending, lazy: bool = False):

@@ -4,8 +4,12 @@ The reference reads each tensor eagerly by name and fails on the first one
 that is missing (`CannotFindTensor`, `candle-core/src/safetensors.rs:501-515`)
 or has another shape (`shape mismatch for {name}`,
 `candle-nn/src/var_builder.rs:509-518`).  Here the whole folder is checked
-first and ONE error lists every missing tensor, every unexpected one and every
-wrong shape, so a bad checkpoint is diagnosed in one go.
+first and ONE error lists every missing tensor and every wrong shape, so a bad
+checkpoint is diagnosed in one go; it lists the tensors that the model does not
+read as well ("unexpected tensors"), since a misnamed tensor is one missing and one
+unexpected.  Such tensors alone are no error, as in the reference
+(`candle-nn/src/var_builder.rs:501-529` reads what it is asked for): they are
+returned as a note for the caller to log, unless `strict=True` makes them fatal.
 
 Tensors keep the precision they are stored in: bfloat16 stays bfloat16, a
 tensor stored in 32-bit stays 32-bit, half precision is widened to 32-bit
@@ -69,10 +73,13 @@ def _keep_precision(t: torch.Tensor) -> torch.Tensor:
 
 
 def load_weights(model_dir: str, expected: Mapping[str, TensorSpec],
-                 optional: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
+                 optional: Iterable[str] = (), strict: bool = False,
+                 unused: Optional[List[str]] = None) -> Dict[str, torch.Tensor]:
     """Read every expected tensor from the folder's safetensors files (CPU tensors).
 
-    `optional` names may be absent; when present they are checked like the rest.
+    `optional` names may be absent; when present they are checked like the rest.  Tensors of the
+    files that the model does not read are appended to `unused` (when given) and, with `strict`,
+    make the load fail.
     """
     optional_set: Set[str] = set(optional)
     files = [SafetensorsFile(p) for p in weight_files(model_dir)]
@@ -93,7 +100,10 @@ def load_weights(model_dir: str, expected: Mapping[str, TensorSpec],
                 wrong_shape.append((name, tuple(spec.shape), tuple(e.shape)))
             if e.dtype not in _FLOAT and not (spec.init == "table" and e.dtype in _INT):
                 wrong_dtype.append((name, e.dtype))
-        if missing or unexpected or wrong_shape or wrong_dtype:
+        if unused is not None:
+            unused.extend(unexpected)
+        # (the error names the unexpected tensors too: a misnamed tensor shows up as one missing and one unexpected)
+        if missing or wrong_shape or wrong_dtype or (strict and unexpected):
             raise WeightError(model_dir, missing, unexpected, wrong_shape, wrong_dtype)
         out: Dict[str, torch.Tensor] = {}
         for name in expected:

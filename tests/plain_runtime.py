@@ -324,6 +324,7 @@ class Scheduler:
         self.running: List[Request] = []            # in order of admission
         self.finished: Dict[Hashable, Request] = {}
         self._arrivals = 0
+        self._left_out: set = set()                 # decodes that found no budget in the last plan
 
     # ---- requests ---------------------------------------------------------------------------
     def add(self, request: Request) -> None:
@@ -354,11 +355,16 @@ class Scheduler:
 
         # 1. decodes: running requests with exactly one token left to feed
         decoding = [r for r in self.running if r.total - r.computed == 1 and r.output]
+        # whoever was left out for lack of budget last time goes first, then the others (admission order)
+        decoding = ([r for r in decoding if r.request_id in self._left_out]
+                    + [r for r in decoding if r.request_id not in self._left_out])
+        self._left_out = set()
         for r in decoding:
             if r not in self.running:               # preempted while serving an earlier one
                 continue
             if budget < 1:
-                break
+                self._left_out.add(r.request_id)
+                continue
             while not self.cache.reserve(r.request_id, 1):
                 victim = self._preempt_latest(exclude=r)
                 if victim is None:

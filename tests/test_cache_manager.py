@@ -121,3 +121,13 @@ def test_random_orders_of_requests_keep_every_page_accounted_for(seed):
         m.free_sequence(sid)
     m.check_invariants()
     assert all(g.pool.num_free == g.pool.num_pages for g in m.groups) and m.slots.num_free == 5
+
+
+def test_state_arrays_count_in_the_pool_sizing():
+    """When the pool is sized from free memory, the fixed-size state of every request slot is paid first."""
+    import torch
+    from inferrs_amd.cache import CacheManager, CacheStorage
+    from inferrs_amd.parts import FixedState, PagedKV
+    manager = CacheManager({0: PagedKV(2, 16), 1: FixedState((1000,), torch.float32), 2: PagedKV(2, 16, None, 24)}, 8, 0, 5)
+    assert CacheStorage.state_bytes(manager) == 5 * 1000 * 4
+    assert CacheStorage.page_bytes(manager, torch.bfloat16) == (2 * 8 * 32 + 2 * 8 * 40) * 2

@@ -144,6 +144,23 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert word in text
 
 
+def test_unread_tensors_are_a_note_unless_strict(tmp_path):
+    """A checkpoint with a tensor that the model does not read loads (the reference reads what it asks for,
+    candle-nn/src/var_builder.rs:501-529); the name is handed back, and `strict` makes it the one error."""
+    spec = Qwen3Config.from_dict(TINY_A).to_spec()
+    expected, optional = model_tensors(spec)
+    tensors = random_tensors(generated_tensors(spec), 1, torch.bfloat16)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    os.makedirs(tmp_path / "m")
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), tensors)
+    unused = []
+    got = load_weights(str(tmp_path / "m"), expected, optional, unused=unused)
+    assert unused == ["model.layers.0.self_attn.rotary_emb.inv_freq"] and set(got) == set(generated_tensors(spec))
+    with pytest.raises(WeightError, match=r"unexpected tensors \(1\): model.layers.0.self_attn.rotary_emb.inv_freq") as e:
+        load_weights(str(tmp_path / "m"), expected, optional, strict=True)
+    assert not e.value.missing and not e.value.wrong_shape
+
+
 def test_truncated_and_malformed_files(tmp_path):
     folder = tmp_path / "m"
     os.makedirs(folder)
@@ -187,3 +204,65 @@ def test_write_random_model_writes_a_loadable_folder(tmp_path):
     assert sorted(os.listdir(folder)) == ["config.json", "model.safetensors"]
     raw = json.load(open(os.path.join(folder, "config.json")))
     assert raw["architectures"] == ["Qwen3ForCausalLM"] and raw["head_dim"] == 16
+
+
+def test_block_arrangements_and_model_ends_are_registered_parts():
+    """The tensors of a model follow from its spec through the registered parts: a block of another arrangement
+    with its own number of norms, no final norm, and an unknown arrangement named in the error."""
+    from dataclasses import replace
+    from inferrs_amd.parts import BlockBase, register_block
+    from inferrs_amd.parts.block import part_tensors
+
+    @register_block("test_three_norms")
+    class ThreeNorms(BlockBase):
+        @classmethod
+        def tensors(cls, spec):
+            return part_tensors(spec, 3)
+
+    spec = Qwen3Config.from_dict(TINY_A).to_spec()
+    base, _ = model_tensors(spec)
+    layer0 = spec.layers[0]
+    wide = replace(layer0, norms=layer0.norms + (layer0.norms[0],), norm_names=layer0.norm_names + ("extra.weight",),
+                   arrangement="test_three_norms")
+    other = replace(spec, layers=(wide,) + spec.layers[1:], final_norm=None, final_norm_name=None)
+    other.validate()
+    names, _ = model_tensors(other)
+    assert set(names) == (set(base) | {"extra.weight"}) - {"model.norm.weight"}
+    from inferrs_amd.config import SpecError
+    with pytest.raises(SpecError, match="3 norms"):
+        model_tensors(replace(spec, layers=(replace(layer0, arrangement="test_three_norms"),)))
+    with pytest.raises(KeyError, match="no block is registered for the arrangement 'sideways'.*pre_norm"):
+        model_tensors(replace(spec, layers=(replace(layer0, arrangement="sideways"),)))
+    with pytest.raises(SpecError, match="come together"):
+        replace(spec, final_norm=None).validate()
+
+
+def test_stop_ids_of_a_folder(tmp_path):
+    """config.json's ids first, then generation_config.json's, the tokenizer's EOS and the well-known end
+    markers that the vocabulary holds (inferrs/src/tokenizer.rs:337-353), without repeats."""
+    from inferrs_amd.config import folder_stop_ids
+    folder = tmp_path / "m"
+    os.makedirs(folder)
+    assert folder_stop_ids(str(folder), (7,)) == (7,)
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": [151645, 151643, 7]}))
+    assert folder_stop_ids(str(folder), (7,)) == (7, 151645, 151643)
+    (folder / "tokenizer_config.json").write_text(json.dumps({"eos_token": {"content": "<eos>"}}))
+    (folder / "tokenizer.json").write_text(json.dumps({
+        "model": {"vocab": {"a": 0, "<|end|>": 5, "<eos>": 9}},
+        "added_tokens": [{"id": 151643, "content": "<|endoftext|>"}, {"id": 11, "content": "<|im_end|>"}, {"id": 3, "content": "x"}]}))
+    assert folder_stop_ids(str(folder), ()) == (151645, 151643, 7, 9, 11, 5)
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": "two"}))
+    with pytest.raises(ConfigError, match="generation_config.json"):
+        folder_stop_ids(str(folder), ())
+
+
+def test_chat_template_comes_from_the_folder_or_the_architecture(tmp_path):
+    from inferrs_amd import chat
+    folder = tmp_path / "m"
+    os.makedirs(folder)
+    assert chat.detect_template(str(folder), Qwen3Config) == "chatml" and chat.detect_template(str(folder)) == "plain"
+    (folder / "tokenizer_config.json").write_text(json.dumps({"chat_template": "{% for m in messages %}<|im_start|>..."}))
+    assert chat.detect_template(str(folder)) == "chatml"
+    assert chat.render("chatml", "hi", "be brief") == ("<|im_start|>system\nbe brief<|im_end|>\n<|im_start|>user\nhi<|im_end|>\n"
+                                                      "<|im_start|>assistant\n")
+    assert chat.render("plain", "hi") == "hi"

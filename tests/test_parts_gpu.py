@@ -241,8 +241,8 @@ def register_toy():
 
             def layer(i, mixer):
                 p = f"blocks.{i}."
-                return LayerSpec(mixer=mixer, ffn=ffn, norm_mixer=norm, norm_ffn=norm, mixer_prefix=p + "mixer.",
-                                 ffn_prefix=p + "ffn.", norm_mixer_name=p + "norm1.weight", norm_ffn_name=p + "norm2.weight")
+                return LayerSpec(mixer=mixer, ffn=ffn, norms=(norm, norm), norm_names=(p + "norm1.weight", p + "norm2.weight"),
+                                 mixer_prefix=p + "mixer.", ffn_prefix=p + "ffn.")
             layers = (layer(0, attn), layer(1, CumMeanSpec(h)), layer(2, attn))
             # layer 0 runs twice (two caches), layer 2 reads the cache that stop 0 wrote
             schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_of=0), ScheduleEntry(0))
@@ -334,6 +334,33 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype, page)
         elif dtype == "float32":
             cross = max(float(np.abs(got[r][i] - first[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
             assert cross < 2e-6, f"{mode} against whole: {cross:.3e}"
+
+
+def test_pages_that_a_window_has_passed_may_hold_anything(tmp_path):
+    """bfloat16, a window of 23 keys over pages of 16: the matrix-core kernel starts its walk at a multiple of
+    32 keys, which may lie in a page that the request has given back.  Every page starts out as NaN here, free
+    pages and the one that released table entries name included, and nothing of it reaches the logits."""
+    from inferrs_amd.engine import Engine, run_trace
+    from inferrs_amd.weights import write_random_model
+    ToyConfig = register_toy()
+    raw = dict(hidden_size=48, heads=4, kv_heads=2, head_dim=16, intermediate=80, vocab=101, eps=1e-5, window=23)
+    folder = write_random_model(str(tmp_path / "toy"), ToyConfig(raw), seed=4)
+    from safetensors.torch import load_file
+    p = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    reqs = {f"r{i}": random_tokens(n, 101, 130 + i) for i, n in enumerate([61, 40, 150, 97])}
+    ref = {r: toy_plain(p, raw, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for mode, trace in (("tail", tm.prefix_then_single(reqs, 40)), ("portions", tm.portions(reqs, [5, 2, 31, 3, 48])),
+                        ("mixed", tm.mixed(reqs, seed=6, max_live=3, decode_tail=30))):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=-(-trace.max_tokens // 16) + 2, max_seqs=4)
+        for layer in eng.storage.layers.values():
+            if layer.k is not None:
+                layer.k.fill_(float("nan"))
+                layer.v.fill_(float("nan"))
+        run_trace(eng, trace.lines, str(tmp_path / mode), io.StringIO())
+        got = trace.read(str(tmp_path / mode), 101)
+        err = float(np.max([np.abs(got[r][i] - ref[r][i]).max() for r in reqs for i in range(len(reqs[r]))])) / scale
+        assert err < 3e-2, f"{mode}: {err:.3e}"             # (numpy's maximum keeps a NaN, and a NaN compares false)
 
 
 # ---- a second toy architecture: a feed-forward with routing, another position encoding ----------
@@ -435,8 +462,8 @@ def register_toy_routed():
 
             def layer(i):
                 p = f"blocks.{i}."
-                return LayerSpec(mixer=attn, ffn=ffn, norm_mixer=norm, norm_ffn=norm, mixer_prefix=p + "mixer.",
-                                 ffn_prefix=p + "ffn.", norm_mixer_name=p + "norm1.weight", norm_ffn_name=p + "norm2.weight")
+                return LayerSpec(mixer=attn, ffn=ffn, norms=(norm, norm), norm_names=(p + "norm1.weight", p + "norm2.weight"),
+                                 mixer_prefix=p + "mixer.", ffn_prefix=p + "ffn.")
             layers = tuple(layer(i) for i in range(r["layers"]))
             return ModelSpec(architecture=self.architecture, vocab_size=r["vocab"], hidden=h, layers=layers,
                              schedule=tuple(ScheduleEntry(i) for i in range(r["layers"])), final_norm=norm,
@@ -550,3 +577,203 @@ def test_steps_of_a_few_rows_with_and_without_the_products_taking_the_norms(tmp_
         first = outs[most][0].cpu()
         for j, (r, t) in enumerate(prompts.items()):
             assert float((first[j] - want[r][3]).abs().max()) <= 3e-2 * scale, (most, r)
+
+
+# ---- a third toy architecture: other ends, another arrangement, values wider than keys -------------
+
+@dataclass(frozen=True)
+class WideValueSpec:
+    """One-head causal attention without position encoding whose values (dv) are wider than its keys (dk)."""
+    hidden: int
+    dk: int
+    dv: int
+    kind: str = "toy_wide_value"
+
+
+@dataclass(frozen=True)
+class ScaledEmbeddingSpec:
+    vocab_size: int
+    hidden: int
+    name: str
+    scale: float
+    kind: str = "toy_scaled_embedding"
+
+
+@dataclass(frozen=True)
+class CappedHeadSpec:
+    vocab_size: int
+    hidden: int
+    cap: float
+    kind: str = "toy_capped_head"
+
+
+def register_toy_ends():
+    from inferrs_amd import ops
+    from inferrs_amd.config import GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, ScheduleEntry
+    from inferrs_amd.config.registry import register_architecture
+    from inferrs_amd.parts import (BlockBase, Embedding, Head, Mixer, PagedKV, register_block, register_embedding,
+                                   register_head, register_mixer)
+    from inferrs_amd.parts.block import build_parts, normed, part_tensors
+    from inferrs_amd.weights import TensorSpec
+
+    @register_mixer("toy_wide_value")
+    class WideValue(Mixer):
+        @classmethod
+        def tensors(cls, spec):
+            return {"q.weight": TensorSpec((spec.dk, spec.hidden)), "k.weight": TensorSpec((spec.dk, spec.hidden)),
+                    "v.weight": TensorSpec((spec.dv, spec.hidden)), "o.weight": TensorSpec((spec.hidden, spec.dv))}
+
+        @classmethod
+        def cache_need(cls, spec):
+            return PagedKV(1, spec.dk, None, v_head_dim=spec.dv)
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.spec = spec
+            self.w = {n: tensors[n + ".weight"].to(device=device, dtype=dtype).contiguous() for n in "qkvo"}
+
+        def forward(self, ctx, h, cache):
+            s = self.spec
+            q, k, v = (ops.linear(h, self.w[n]) for n in "qkv")
+            group = ctx.groups[cache.group]
+            ps = group.page_size
+            assert tuple(cache.k.shape[1:]) == (1, ps, s.dk) and tuple(cache.v.shape[1:]) == (1, s.dv, ps)
+            slots = group.slots.long()
+            cache.k[slots // ps, 0, slots % ps] = k
+            cache.v[slots // ps, 0, :, slots % ps] = v
+            out = torch.empty((h.shape[0], s.dv), dtype=h.dtype, device=h.device)
+            off = 0
+            for row, (n, start) in enumerate(zip(ctx.q_lens, ctx.kv_starts)):      # a toy: one request at a time
+                total = start + n
+                pages = group.block_table[row, :-(-total // ps)].long()
+                keys = cache.k[pages, 0].reshape(-1, s.dk)[:total].float()
+                values = cache.v[pages, 0].permute(0, 2, 1).reshape(-1, s.dv)[:total].float()
+                scores = q[off:off + n].float() @ keys.T / s.dk ** 0.5
+                seen = torch.arange(total, device=h.device)[None, :] <= (start + torch.arange(n, device=h.device))[:, None]
+                out[off:off + n] = (torch.softmax(scores.masked_fill(~seen, float("-inf")), -1) @ values).to(h.dtype)
+                off += n
+            return ops.linear(out, self.w["o"])
+
+    @register_block("toy_sandwich")
+    class Sandwich(BlockBase):
+        """x += post_1(mixer(pre_1(x)));  x += post_2(ffn(pre_2(x))): four norms."""
+
+        @classmethod
+        def tensors(cls, spec):
+            return part_tensors(spec, 4)
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.mixer, self.ffn, self.norms = build_parts(spec, tensors, dtype, device)
+            self.first_norm = self.norms[0]
+
+        def parts(self):
+            return [self.mixer, self.ffn, *self.norms]
+
+        def forward(self, ctx, x, pending, cache, next_norm=None):
+            ctx.stream = ctx.stream_norm = None
+            h = normed(self.norms[0], x, pending)
+            a = self.norms[1].forward(self.mixer.forward(ctx, h, cache))
+            h2 = self.norms[2].add_forward(x, a)
+            return x, self.norms[3].forward(self.ffn.forward(ctx, h2))
+
+    @register_embedding("toy_scaled_embedding")
+    class ScaledEmbedding(Embedding):
+        @classmethod
+        def tensors(cls, spec):
+            return {spec.name: TensorSpec((spec.vocab_size, spec.hidden))}
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.spec = spec
+            self.table = tensors[spec.name].to(device=device, dtype=dtype).contiguous()
+
+        def forward(self, ctx):
+            return (ops.embed_gather(self.table, ctx.token_ids).float() * self.spec.scale).to(self.table.dtype)
+
+    @register_head("toy_capped_head")
+    class CappedHead(Head):
+        def __init__(self, spec, tensors, dtype, device, embedding=None):
+            self.spec, self.table = spec, embedding.table
+
+        def forward(self, rows):
+            logits = ops.linear(rows, self.table, torch.float32)
+            return torch.tanh(logits / self.spec.cap) * self.spec.cap
+
+    class EndsConfig:
+        architecture = "ToyEndsForCausalLM"
+        model_type = "toy_ends"
+
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def to_dict(self):
+            return dict(self.raw, architectures=[self.architecture], model_type=self.model_type)
+
+        def to_spec(self):
+            r = self.raw
+            h = r["hidden_size"]
+            norm = NormSpec(size=h, eps=r["eps"])
+            mixer = WideValueSpec(h, r["dk"], r["dv"])
+            ffn = GatedMlpSpec(hidden=h, intermediate=r["intermediate"])
+
+            def layer(i):
+                p = f"blocks.{i}."
+                return LayerSpec(mixer=mixer, ffn=ffn, norms=(norm,) * 4,
+                                 norm_names=tuple(p + f"norm{j}.weight" for j in range(4)),
+                                 mixer_prefix=p + "mixer.", ffn_prefix=p + "ffn.", arrangement="toy_sandwich")
+            return ModelSpec(architecture=self.architecture, vocab_size=r["vocab"], hidden=h,
+                             layers=tuple(layer(i) for i in range(r["layers"])),
+                             schedule=tuple(ScheduleEntry(i) for i in range(r["layers"])),
+                             final_norm=None, final_norm_name=None, embed_name="embed.weight", head_name=None,
+                             max_position=512,
+                             embedding=ScaledEmbeddingSpec(r["vocab"], h, "embed.weight", r["embed_scale"]),
+                             head=CappedHeadSpec(r["vocab"], h, r["cap"]))
+
+    register_architecture(EndsConfig)
+    return EndsConfig
+
+
+def toy_ends_plain(p, raw, ids):
+    t = len(ids)
+    x = p["embed.weight"][torch.as_tensor(ids)] * raw["embed_scale"]
+    causal = torch.arange(t)[None, :] > torch.arange(t)[:, None]
+    for i in range(raw["layers"]):
+        pre = f"blocks.{i}."
+        norm = lambda j, v: pm.rms_norm(v, p[pre + f"norm{j}.weight"], raw["eps"])
+        h = norm(0, x)
+        q, k, v = (pm.linear(h, p[pre + f"mixer.{n}.weight"]) for n in "qkv")
+        s = (q @ k.T / raw["dk"] ** 0.5).masked_fill(causal, float("-inf"))
+        x = x + norm(1, pm.linear(pm.softmax_last(s) @ v, p[pre + "mixer.o.weight"]))
+        x = x + norm(3, pm.mlp(norm(2, x), p[pre + "ffn.gate_proj.weight"], p[pre + "ffn.up_proj.weight"],
+                               p[pre + "ffn.down_proj.weight"]))
+    return torch.tanh(pm.linear(x, p["embed.weight"]) / raw["cap"]) * raw["cap"]
+
+
+@pytest.mark.parametrize("dtype,page", [("float32", 4), ("bfloat16", 16)])
+def test_toy_ends_arrangement_and_unequal_key_and_value_widths(tmp_path, dtype, page):
+    """An embedding that scales, a head that caps its logits, no final norm, a block of another arrangement with
+    four norms, and a mixer whose cached values are wider than its keys: registered and run from this file."""
+    from inferrs_amd.engine import Engine, run_trace
+    from inferrs_amd.weights import write_random_model
+    EndsConfig = register_toy_ends()
+    raw = dict(hidden_size=40, dk=12, dv=28, intermediate=56, vocab=77, eps=1e-5, layers=2, embed_scale=40 ** 0.5, cap=3.0)
+    folder = write_random_model(str(tmp_path / "ends"), EndsConfig(raw), seed=6)
+    from safetensors.torch import load_file
+    loaded = load_file(os.path.join(folder, "model.safetensors"))
+    assert "norm.weight" not in loaded and sum(n.startswith("blocks.0.norm") for n in loaded) == 4
+    p = {k: v.double() for k, v in loaded.items()}
+    reqs = {f"r{i}": random_tokens(n, 77, 80 + i) for i, n in enumerate([3, 29, 70])}
+    ref = {r: toy_ends_plain(p, raw, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for mode, trace in (("whole", tm.whole(reqs)), ("portions", tm.portions(reqs, [5, 2, 17])),
+                        ("mixed", tm.mixed(reqs, seed=8, max_live=3, decode_tail=6))):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-trace.max_tokens // page) + 2, max_seqs=4)
+        need = eng.cache.groups[0].need
+        assert need.head_dim == 12 and need.value_dim == 28 and len(eng.storage.arrays) == 2
+        run_trace(eng, trace.lines, str(tmp_path / mode), io.StringIO())
+        got = trace.read(str(tmp_path / mode), 77)
+        err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
+        assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
+        eng.cache.check_invariants()

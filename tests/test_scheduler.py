@@ -207,3 +207,22 @@ def test_a_request_can_be_ended_from_outside():
     run(s, cache)
     assert a.finish_reason == "length" and len(a.output) == 10
     assert cache.groups[0].pool.num_free == 16 and not cache.names.names()
+
+
+def test_a_budget_below_the_number_of_decodes_starves_nobody():
+    """Five requests decode under a budget of two tokens a step: those left out of a step go first in
+    the next, so that every request advances at the same pace (two steps out of five)."""
+    cache, s = make(max_tokens_per_step=2, max_seqs=5)
+    reqs = [req(i, 2, max_tokens=6) for i in range(5)]
+    for r in reqs:
+        s.add(r)
+    trace = []
+    run(s, cache, trace=trace)
+    assert all(r.finish_reason == "length" and len(r.output) == 6 for r in reqs)
+    decodes = [[e.request.request_id for e in p.entries if len(e.tokens) == 1 and e.request.output] for p in trace]
+    served = {i: [k for k, ids in enumerate(decodes) if i in ids] for i in range(5)}
+    # nobody waits more than three steps between two of its decodes while all five are decoding
+    both = [k for k, ids in enumerate(decodes) if len(ids) == 2]
+    for i in range(5):
+        gaps = [b - a for a, b in zip(served[i], served[i][1:]) if a in both and b in both]
+        assert gaps and max(gaps) <= 3, (i, served[i])

@@ -1,0 +1,208 @@
+"""Schedules of the decode path that the replay traces do not reach: captured graphs across a context
+bucket's boundary, a staging buffer that grows after graphs were captured, more shapes than graphs are
+kept, preemption under seeded draws and in bfloat16, and a window whose passed pages hold NaN."""
+import io
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+import trace_modes as tm
+from tiny_configs import TINY, random_tokens, write_model
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tiny(tmp_path_factory):
+    out = {}
+    for name in ("A", "B", "D"):
+        folder = write_model(str(tmp_path_factory.mktemp(f"sched_{name}")), TINY[name], seed=33)
+        out[name] = (folder, *pm.read_model(folder, torch.float64))
+    return out
+
+
+def forced_decode(eng, prompts, tails):
+    """Prompts in one step each, then the given tokens one step at a time for all requests together; returns
+    the logits of every decode step [steps][requests, vocab] (copies) and the replay count after each."""
+    from inferrs_amd.engine import Entry
+    for rid, p in prompts.items():
+        eng.step([Entry(rid, p, [])])
+    rows, replays = [], []
+    steps = len(next(iter(tails.values())))
+    for i in range(steps):
+        rows.append(eng.step([Entry(rid, [tails[rid][i]], [0]) for rid in prompts]).clone())
+        replays.append(eng.graph_replays)
+    for rid in prompts:
+        eng.end_request(rid)
+    return rows, replays
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_across_a_bucket_boundary(tiny, dtype):
+    """Three requests whose lengths pass 1,024 tokens (the end of a captured graph's context bucket) at different
+    steps: every step's logits equal those of an engine without graphs, on both sides of the boundary, and
+    graphs were replayed on both sides."""
+    from inferrs_amd.engine import Engine
+    folder, cfg, params = tiny["D"]
+    vocab = TINY["D"]["vocab_size"]
+    lengths = {"a": 1000, "b": 1015, "c": 980}
+    steps = 60
+    seqs = {r: random_tokens(n + steps, vocab, 900 + n) for r, n in lengths.items()}
+    prompts = {r: seqs[r][:lengths[r]] for r in seqs}
+    tails = {r: seqs[r][lengths[r]:] for r in seqs}
+    pages = sum(-(-(n + steps) // 16) for n in lengths.values()) + 2
+    outs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=pages, max_seqs=4, use_graphs=graphs)
+        assert eng.use_graphs == graphs
+        outs[graphs] = forced_decode(eng, prompts, tails)
+        eng.cache.check_invariants()
+    rows_g, replays = outs[True]
+    rows_e, none = outs[False]
+    assert none[-1] == 0
+    crossing = 1024 - 1015                    # the step whose longest request reaches 1,025 tokens with its new one
+    assert replays[crossing - 1] >= crossing - 2 and replays[-1] - replays[crossing + 1] >= steps - crossing - 4
+    assert replays[crossing] == replays[crossing - 1]           # the first step of the new bucket runs eagerly
+    scale = max(float(r.abs().max()) for r in rows_e)
+    worst = max(float((g - e).abs().max()) for g, e in zip(rows_g, rows_e)) / scale
+    # 32-bit: the same sums in the same order.  bfloat16: a graph's step sees the bucket's width, an eager step the
+    # longest request, so the keys may be split between waves in another way: rounding only
+    assert worst <= (1e-6 if dtype == "float32" else 2e-2), worst
+    # and both are the plain model's logits
+    ref = pm.forward(cfg, params, seqs["b"])
+    got = torch.stack([r[1] for r in rows_g]).cpu().double()
+    err = float((got - ref[lengths["b"]:lengths["b"] + steps]).abs().max() / ref.abs().max())
+    assert err <= (1e-5 if dtype == "float32" else 3e-2), err
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_runs_of_decode_steps_across_a_bucket_boundary(tiny, dtype):
+    """The generation loop queues eight decode steps at a time; a run never straddles a bucket, and the tokens
+    are those of single steps (32-bit: of an engine without graphs)."""
+    from inferrs_amd.engine import Engine, GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["D"]
+    vocab = TINY["D"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 950 + n) for n in (1003, 990, 1011)]
+    results = {}
+    for mode, graphs, run in (("runs", True, 8), ("single", True, 1), ("eager", False, 1)):
+        if mode == "eager" and dtype != "float32":
+            continue
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=3 * 68 + 2, max_seqs=4, use_graphs=graphs)
+        loop = GenerationLoop(eng, decode_run=run, stop_token_ids=[])
+        reqs = [loop.add(p, SamplingParams.greedy(max_tokens=60)) for p in prompts]
+        loop.run()
+        results[mode] = [list(r.output) for r in reqs]
+        if mode == "runs":
+            assert eng.graph_replays > 40
+        eng.cache.check_invariants()
+        assert not eng.cache.sequences
+    assert results["runs"] == results["single"]
+    if dtype == "float32":
+        assert results["runs"] == results["eager"]
+    assert all(len(o) == 60 for o in results["runs"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_staging_buffer_that_grows_drops_the_captured_graphs(tiny, dtype):
+    """Graphs hold the address of the step's device buffer.  A later, longer prompt portion makes that buffer
+    grow and move: the graphs captured before are dropped, and decode steps afterwards still give the
+    logits of an engine without graphs."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["D"]
+    vocab = TINY["D"]["vocab_size"]
+    short, long_prompt = random_tokens(40, vocab, 1), random_tokens(1500, vocab, 2)
+    tail = random_tokens(12, vocab, 3)
+    outs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=120, max_seqs=4, use_graphs=graphs)
+        eng.step([Entry("s", short, [])])
+        rows = [eng.step([Entry("s", [t], [0])]).clone() for t in tail[:6]]
+        generation, replays = eng.builder.generation, eng.graph_replays
+        if graphs:
+            assert replays >= 4
+        eng.step([Entry("l", long_prompt, [])])                     # 1,500 tokens: more words than the buffer had
+        assert eng.builder.generation > generation
+        rows += [eng.step([Entry("s", [t], [0])]).clone() for t in tail[6:]]
+        if graphs:
+            assert eng.graph_replays >= replays + 4                 # captured again over the new buffer, and replayed
+        outs[graphs] = rows
+    scale = max(float(r.abs().max()) for r in outs[False])
+    worst = max(float((g - e).abs().max()) for g, e in zip(outs[True], outs[False])) / scale
+    assert worst <= (1e-6 if dtype == "float32" else 2e-2), worst
+
+
+def test_more_shapes_than_graphs_are_kept(tiny):
+    """A batch that shrinks request by request, with room for three graphs only: old ones are dropped, every
+    step still equals the eager one."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    seqs = {f"r{i}": random_tokens(20 + 3 * i + 40, vocab, 40 + i) for i in range(6)}
+    outs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=80, max_seqs=6, use_graphs=graphs)
+        eng.MAX_GRAPHS = 3
+        live = {r: 20 + 3 * i for i, r in enumerate(seqs)}
+        for r, n in live.items():
+            eng.step([Entry(r, seqs[r][:n], [])])
+        rows = []
+        for step in range(36):
+            if step and step % 6 == 0:                              # a request ends: another shape from here on
+                gone = sorted(live)[-1]
+                eng.end_request(gone)
+                del live[gone]
+            rows.append(eng.step([Entry(r, [seqs[r][n]], [0]) for r, n in live.items()]).clone())
+            live = {r: n + 1 for r, n in live.items()}
+            assert len(eng._graphs) <= 3
+        outs[graphs] = rows
+        if graphs:
+            assert eng.graph_replays >= 6 * 4
+    assert all(torch.equal(g, e) for g, e in zip(outs[True], outs[False]))
+
+
+def test_preemption_under_seeded_draws_gives_the_same_tokens(tiny):
+    """A pool so tight that requests are preempted and recomputed: with temperature and fixed seeds the tokens
+    are those of a roomy pool (a draw depends on the seed and the token's index, not on when it is made)."""
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 190 + n) for n in (20, 24, 28, 18)]
+    sp = [SamplingParams(temperature=0.8, top_k=0, top_p=0.95, repetition_penalty=1.1, seed=70 + i, max_tokens=24,
+                         bypass_stop_tokens=True) for i in range(4)]
+    roomy = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=256, max_seqs=4)
+    want = roomy.generate(prompts, sp)
+    tight = Engine.from_folder(folder, dtype="float32", page_size=4, num_pages=30, max_seqs=4)
+    got = tight.generate(prompts, sp)
+    assert sum(g.preemptions for g in got) > 0 and sum(g.preemptions for g in want) == 0
+    assert [g.tokens for g in got] == [g.tokens for g in want]
+    tight.cache.check_invariants()
+
+
+def test_preemption_in_bfloat16_stays_with_the_plain_model(tiny):
+    """bfloat16 under a tight pool: a recomputed request's keys come from a prompt portion's kernels instead of
+    decode steps', so its logits move by rounding; greedy tokens agree with the plain model's wherever its two
+    best logits are further apart than that."""
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 290 + n) for n in (20, 24, 28, 18)]
+    tight = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=8, max_seqs=4)     # 128 slots for ~186 tokens
+    got = tight.generate(prompts, SamplingParams.greedy(max_tokens=24, bypass_stop_tokens=True))
+    assert sum(g.preemptions for g in got) > 0 and all(g.finish_reason == "length" for g in got)
+    for prompt, out in zip(prompts, got):
+        toks = list(prompt)
+        for i, t in enumerate(out.tokens):
+            row = pm.forward(cfg, params, toks)[-1]
+            top = torch.topk(row, 2)
+            if t != int(top.indices[0]):
+                assert float(top.values[0] - top.values[1]) < 0.02, f"token {i}: {t} against {int(top.indices[0])}"
+                break
+            toks.append(t)
+    tight.cache.check_invariants()
+    assert not tight.cache.sequences

@@ -34,8 +34,15 @@ TINY_E = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size
               head_dim=16, rope_theta=777.0, rms_norm_eps=1e-4, tie_word_embeddings=True,
               max_position_embeddings=512, hidden_act="silu")
 
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16, "E": 16}
+# A head size that is no multiple of 16 (24) and another that is no multiple of 8 (20 would not be even in halves
+# of 8: 24 / 2 = 12 rotary pairs): the matrix-core kernels refuse it, the plain kernels run it in both precisions.
+TINY_F = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=203, hidden_size=56,
+              intermediate_size=88, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=24, rope_theta=50000.0, rms_norm_eps=1e-5, tie_word_embeddings=True,
+              max_position_embeddings=512, hidden_act="silu")
+
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16, "E": 16, "F": 8}
 
 
 def write_model(folder: str, raw: dict, seed: int, dtype=torch.bfloat16, sharpen: float = 1.0) -> str:
