@@ -118,11 +118,134 @@ def test_gqa_head_mapping():
 def test_silu_and_mlp():
     assert pm.silu(torch.tensor(0.0)).item() == 0.0
     assert abs(pm.silu(torch.tensor(30.0)).item() - 30.0) < 1e-5
-    x = torch.randn(3, 8)
-    g, u, d = torch.randn(12, 8), torch.randn(12, 8), torch.randn(8, 12)
-    want = torch.nn.functional.linear(torch.nn.functional.silu(torch.nn.functional.linear(x, g))
-                                      * torch.nn.functional.linear(x, u), d)
-    assert torch.allclose(pm.mlp(x, g, u, d), want, atol=1e-5)
+    z = torch.linspace(-6, 6, 25)
+    assert torch.allclose(pm.silu(z), torch.nn.functional.silu(z), atol=1e-6)        # the library's routine
+    torch.manual_seed(3)
+    x = torch.randn(3, 8, dtype=torch.float64)
+    g, u, d = (torch.randn(12, 8, dtype=torch.float64), torch.randn(12, 8, dtype=torch.float64),
+               torch.randn(8, 12, dtype=torch.float64))
+    base = pm.mlp(x, g, u, d)
+    # Which of the two projections goes through the activation (attention_utils.rs:112-117: the gate): the result is
+    # linear in the up projection and in the down projection, and not in the gate.  With the two swapped the first
+    # line fails and the third holds.
+    assert torch.allclose(pm.mlp(x, g, 3.0 * u, d), 3.0 * base, atol=1e-12)
+    assert torch.allclose(pm.mlp(x, g, u, -2.0 * d), -2.0 * base, atol=1e-12)
+    assert not torch.allclose(pm.mlp(x, 3.0 * g, u, d), 3.0 * base, atol=1e-3)
+    # a gate that is shut (a large negative product) closes the unit whatever the up projection holds
+    shut = pm.mlp(torch.ones(1, 8, dtype=torch.float64), -40.0 * torch.ones(12, 8, dtype=torch.float64), u, d)
+    assert float(shut.abs().max()) < 1e-9
+    # and a wide-open gate lets gate * up through: silu(z) -> z
+    x1 = torch.ones(1, 8, dtype=torch.float64)
+    g1 = 5.0 * torch.ones(12, 8, dtype=torch.float64)
+    assert torch.allclose(pm.mlp(x1, g1, u, d), pm.linear(pm.linear(x1, g1) * pm.linear(x1, u), d), rtol=1e-12)
+
+
+def _layer_parts(seed=0, nq=4, nkv=2, d=8, hidden=24, t=9, spread=0.5):
+    """Random weights of one attention layer with norm weights that differ within every rotary pair."""
+    g = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    cfg = dict(num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, rms_norm_eps=1e-6)
+    p = {"q_proj.weight": rn(nq * d, hidden), "k_proj.weight": rn(nkv * d, hidden), "v_proj.weight": rn(nkv * d, hidden),
+         "o_proj.weight": rn(hidden, nq * d), "q_norm.weight": 1.0 + spread * rn(d), "k_norm.weight": 1.0 + spread * rn(d)}
+    return cfg, p, rn(t, hidden)
+
+
+def _tables(positions, d):
+    cos, sin = pm.rope_tables(torch.as_tensor(positions), 10000.0, d)
+    return cos.double(), sin.double()
+
+
+def test_attention_layer_counts_distances_only():
+    """Rotary attention sees distances between positions, never positions themselves: shifting every position by
+    the same amount changes nothing.  That holds when the per-head norm comes BEFORE the rotation
+    (qwen3.rs:128-135).  Were the norm applied after it, its weights, which differ within a rotated pair, would
+    scale the two halves of a pair differently and the scores would depend on the positions themselves: the
+    variant below, with the two steps in the other order, fails the same check."""
+    cfg, p, x = _layer_parts()
+    d = cfg["head_dim"]
+    here = pm.attention_layer(x, p, "", cfg, *_tables(range(9), d))
+    there = pm.attention_layer(x, p, "", cfg, *_tables(range(1000, 1009), d))
+    # (the angles are formed in 32-bit, as the reference forms them: at position 1,000 they are rounded to 6e-5)
+    assert float((here - there).abs().max()) < 1e-5 * float(here.abs().max())
+
+    def norm_after_rotation(x, cos, sin):
+        t, nq, nkv = x.shape[0], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+        q = pm.linear(x, p["q_proj.weight"]).reshape(t, nq, d).transpose(0, 1)
+        k = pm.linear(x, p["k_proj.weight"]).reshape(t, nkv, d).transpose(0, 1)
+        v = pm.linear(x, p["v_proj.weight"]).reshape(t, nkv, d).transpose(0, 1)
+        q = pm.rms_norm(pm.rope_half(q, cos, sin), p["q_norm.weight"], 1e-6)
+        k = pm.rms_norm(pm.rope_half(k, cos, sin), p["k_norm.weight"], 1e-6)
+        return pm.linear(pm.attention_core(q, k, v).transpose(0, 1).reshape(t, nq * d), p["o_proj.weight"])
+    wrong_here = norm_after_rotation(x, *_tables(range(9), d))
+    wrong_there = norm_after_rotation(x, *_tables(range(1000, 1009), d))
+    assert float((wrong_here - wrong_there).abs().max()) > 1e-2 * float(wrong_here.abs().max())
+    assert float((wrong_here - here).abs().max()) > 1e-2 * float(here.abs().max())
+
+
+def test_attention_layer_norms_queries_and_keys_per_head_and_not_values():
+    """What the per-head norm covers (qwen3.rs:128-129, attention_utils.rs:52-58): queries and keys, each head on
+    its own, values not.  So the layer does not notice a rescaled query or key head (a norm over all heads
+    together would, and so would no norm), and it is linear in the value projection (a normed value would not be)."""
+    cfg, p, x = _layer_parts(seed=1)
+    cfg["rms_norm_eps"] = 1e-14                                 # (so that a head's scale drops out exactly)
+    d = cfg["head_dim"]
+    tables = _tables(range(9), d)
+    base = pm.attention_layer(x, p, "", cfg, *tables)
+    scaled = dict(p)
+    scaled["q_proj.weight"] = p["q_proj.weight"].clone()
+    scaled["q_proj.weight"][d:2 * d] *= 7.0                     # query head 1 alone
+    scaled["k_proj.weight"] = p["k_proj.weight"].clone()
+    scaled["k_proj.weight"][:d] *= 0.2                          # key head 0 alone
+    assert torch.allclose(pm.attention_layer(x, scaled, "", cfg, *tables), base, atol=1e-6)
+    wide = dict(p, **{"v_proj.weight": 3.0 * p["v_proj.weight"]})
+    assert torch.allclose(pm.attention_layer(x, wide, "", cfg, *tables), 3.0 * base, atol=1e-9)
+    # one weight vector of head_dim entries serves every head
+    assert p["q_norm.weight"].shape == (d,)
+    # and it matters: other norm weights, other result
+    other = dict(p, **{"q_norm.weight": p["q_norm.weight"].flip(0)})
+    assert float((pm.attention_layer(x, other, "", cfg, *tables) - base).abs().max()) > 1e-3 * float(base.abs().max())
+
+
+def test_decoder_layer_keeps_the_stream_beside_its_parts():
+    """Pre-norm residuals (qwen3.rs:284-300): the stream goes round both parts untouched, and the norms stand on the
+    parts' inputs.  With output projections of zero the layer is the identity (a norm on the stream itself, or after
+    the sum, would change x); and what a part adds is a function of the NORMED stream: scaling the stream by a
+    constant scales the layer's additions not at all."""
+    torch.manual_seed(5)
+    cfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=8, rms_norm_eps=1e-9, hidden_size=24)
+    rn = lambda *s: torch.randn(*s, dtype=torch.float64)
+    pre = "model.layers.0."
+    p = {pre + "self_attn.q_proj.weight": rn(32, 24), pre + "self_attn.k_proj.weight": rn(16, 24),
+         pre + "self_attn.v_proj.weight": rn(16, 24), pre + "self_attn.o_proj.weight": rn(24, 32),
+         pre + "self_attn.q_norm.weight": 1 + 0.3 * rn(8), pre + "self_attn.k_norm.weight": 1 + 0.3 * rn(8),
+         pre + "input_layernorm.weight": 1 + 0.3 * rn(24), pre + "post_attention_layernorm.weight": 1 + 0.3 * rn(24),
+         pre + "mlp.gate_proj.weight": rn(40, 24), pre + "mlp.up_proj.weight": rn(40, 24),
+         pre + "mlp.down_proj.weight": rn(24, 40)}
+    x = rn(7, 24)
+    tables = _tables(range(7), 8)
+    silent = dict(p)
+    silent[pre + "self_attn.o_proj.weight"] = torch.zeros(24, 32, dtype=torch.float64)
+    silent[pre + "mlp.down_proj.weight"] = torch.zeros(24, 40, dtype=torch.float64)
+    assert torch.equal(pm.decoder_layer(x, silent, 0, cfg, *tables), x)
+    # the attention part alone (the feed-forward silent): its addition does not change when the stream is scaled
+    quiet_ffn = dict(p)
+    quiet_ffn[pre + "mlp.down_proj.weight"] = torch.zeros(24, 40, dtype=torch.float64)
+    add1 = pm.decoder_layer(x, quiet_ffn, 0, cfg, *tables) - x
+    add5 = pm.decoder_layer(5.0 * x, quiet_ffn, 0, cfg, *tables) - 5.0 * x
+    assert torch.allclose(add1, add5, atol=1e-7)
+    # the feed-forward reads the stream AFTER the attention's addition: with the attention silent it sees norm(x),
+    # with it speaking something else
+    quiet_attn = dict(p)
+    quiet_attn[pre + "self_attn.o_proj.weight"] = torch.zeros(24, 32, dtype=torch.float64)
+    ffn_alone = pm.decoder_layer(x, quiet_attn, 0, cfg, *tables) - x
+    want = pm.mlp(pm.rms_norm(x, p[pre + "post_attention_layernorm.weight"], 1e-9), p[pre + "mlp.gate_proj.weight"],
+                  p[pre + "mlp.up_proj.weight"], p[pre + "mlp.down_proj.weight"])
+    assert torch.allclose(ffn_alone, want, atol=1e-9)
+    both = pm.decoder_layer(x, p, 0, cfg, *tables)
+    mid = x + add1
+    want_both = mid + pm.mlp(pm.rms_norm(mid, p[pre + "post_attention_layernorm.weight"], 1e-9),
+                             p[pre + "mlp.gate_proj.weight"], p[pre + "mlp.up_proj.weight"], p[pre + "mlp.down_proj.weight"])
+    assert torch.allclose(both, want_both, atol=1e-9)
 
 
 def test_rand_f32_matches_integer_transcription():
@@ -186,4 +309,8 @@ def test_whole_model_shift_and_prefix_invariants(tmp_path, name):
         assert "lm_head.weight" not in p
     else:
         assert p["lm_head.weight"].shape == (raw["vocab_size"], raw["hidden_size"])
-    assert pm.greedy(cfg, p, toks[:5], 3) == pm.greedy(cfg, p, toks[:5], 3)
+    # greedy continuation feeds its own tokens back: the arg max of the logits after each of them
+    out = pm.greedy(cfg, p, toks[:5], 3)
+    assert out[0] == int(torch.argmax(full[4])) or toks[5] != out[0]
+    assert out[1] == int(torch.argmax(pm.forward(cfg, p, toks[:5] + out[:1])[-1]))
+    assert out[2] == int(torch.argmax(pm.forward(cfg, p, toks[:5] + out[:2])[-1]))
