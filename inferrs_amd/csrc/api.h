@@ -64,6 +64,15 @@ int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N,
 
 long long ia_argmax_workspace(int rows, int vocab);
 int ia_argmax(int* out, const float* logits, void* workspace, int rows, int vocab, hipStream_t stream);
+// The arg max without any allocation.  It has no counterpart in the reference; it is for callers that cannot
+// allocate device memory: code under HIP graph capture, tight serving loops, harnesses that forbid it.  The
+// two-step kernels' candidates go to an array of ia_argmax_static_capacity() 32-bit words (64 KiB) that the
+// library holds in each GPU's memory until the process ends, instead of a workspace of the caller's; sizes for
+// which ia_argmax_workspace(rows, vocab) exceeds that are refused with an error (about 430 rows at a
+// vocabulary of 152 k).  No hipMalloc, hipFree or allocating library call happens inside.  All calls on one GPU
+// share that GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+long long ia_argmax_static_capacity(void);
+int ia_argmax_static(int* out, const float* logits, int rows, int vocab, hipStream_t stream);
 int ia_penalize(float* logits, int rows, int vocab, const int* window, int w, const float* rep,
                 const float* freq, const float* pres, const int* bias_ids, const float* bias_vals,
                 int nb, hipStream_t stream);

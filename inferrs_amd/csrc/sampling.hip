@@ -21,6 +21,8 @@
 // shorter way (sample_top_k): their first top_k tokens are picked out and sorted, and the
 // reference's steps run on that list as it runs them.  Rows without a top_k try that way with
 // the first 1,024 tokens of their list and take the long one when the list does not end there.
+#include <mutex>
+
 #include "common.h"
 #include "api.h"
 
@@ -115,6 +117,60 @@ extern "C" int ia_argmax(int* out, const float* logits, void* workspace, int row
     }
     argmax_kernel<<<rows, 1024, 0, stream>>>(out, logits, vocab);
     IA_LAUNCH_CHECK("argmax");
+    return 0;
+}
+
+// ---- greedy, for callers that cannot allocate -----------------------------------------------
+// The two-step arg max needs a place for the stretches' candidates.  ia_argmax takes it from the caller; this
+// entry point keeps one of a fixed size in the library's own device memory instead, so that nothing is
+// allocated on the way (declared in api.h with the reasons).  Each GPU holds its own copy of the array at its
+// own address: the address is asked for once per device, with that device current, and only that pointer
+// (never the array's name, which on the host is a stand-in and no device address) goes to the kernels.
+#define ARGMAX_STATIC_WORDS 16384                  // 64 KiB a GPU, held until the process ends
+#define ARGMAX_STATIC_DEVICES 64
+static __device__ __align__(256) int argmax_scratch[ARGMAX_STATIC_WORDS];
+static void* g_argmax_scratch_ptr[ARGMAX_STATIC_DEVICES];    // per device; written once, under the lock
+static std::mutex g_argmax_scratch_lock;
+
+extern "C" long long ia_argmax_static_capacity(void) { return ARGMAX_STATIC_WORDS; }
+
+extern "C" int ia_argmax_static(int* out, const float* logits, int rows, int vocab, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && vocab > 0, "argmax_static: bad sizes rows=%d vocab=%d", rows, vocab);
+    IA_CHECK(out != nullptr && logits != nullptr, "argmax_static: null operand");
+    if (rows == 0) return 0;
+    const long long words = ia_argmax_workspace(rows, vocab);
+    IA_CHECK(words <= ARGMAX_STATIC_WORDS, "argmax_static: %d rows of %d logits need %lld words of scratch, the "
+             "library's array holds %d (use ia_argmax with a workspace of your own)", rows, vocab, words, ARGMAX_STATIC_WORDS);
+    if (words == 0) {                              // short rows: one block a row, no scratch at all
+        argmax_kernel<<<rows, 1024, 0, stream>>>(out, logits, vocab);
+        IA_LAUNCH_CHECK("argmax_static");
+        return 0;
+    }
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    IA_CHECK(e == hipSuccess && device >= 0 && device < ARGMAX_STATIC_DEVICES,
+             "argmax_static: cannot tell the current device (%s, device %d)", hipGetErrorString(e), device);
+    void* scratch = nullptr;
+    {
+        std::lock_guard<std::mutex> hold(g_argmax_scratch_lock);
+        if (g_argmax_scratch_ptr[device] == nullptr) {
+            void* ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(argmax_scratch));
+            IA_CHECK(e == hipSuccess && ptr != nullptr, "argmax_static: no address for the scratch array on device %d: %s",
+                     device, hipGetErrorString(e));
+            g_argmax_scratch_ptr[device] = ptr;
+        }
+        scratch = g_argmax_scratch_ptr[device];
+    }
+    IA_CHECK(rows <= 65535, "argmax_static: %d rows exceed the grid", rows);
+    const int stretches = (vocab + ARGMAX_STRETCH - 1) / ARGMAX_STRETCH;
+    // (every candidate that the second kernel reads is written by the first in this call: nothing has to start at zero)
+    float* cand_v = (float*)scratch;
+    int* cand_i = (int*)scratch + (size_t)rows * stretches;
+    argmax_stretch_kernel<<<dim3(stretches, rows), 256, 0, stream>>>(cand_v, cand_i, logits, vocab);
+    IA_LAUNCH_CHECK("argmax_static");
+    argmax_pick_kernel<<<rows, IA_WAVE, 0, stream>>>(out, cand_v, cand_i, stretches);
+    IA_LAUNCH_CHECK("argmax_static");
     return 0;
 }
 
