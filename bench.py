@@ -69,15 +69,9 @@ def decode_bytes(c, batch: int, context: float, esize: int = 2) -> float:
     return float(weights * esize + kv * esize + batch * c["hidden_size"] * esize)
 
 
-def fill_context(engine, ids, context: int) -> None:
-    """Gives each request `context` cached tokens without running them: pages are reserved and
-    filled with random keys and values."""
+def fill_storage(engine) -> None:
+    """Random keys and values in every page of the cache (decode time does not depend on their content)."""
     import torch
-    for sid in ids:
-        engine.add_request(sid)
-        if not engine.cache.reserve(sid, context):
-            raise RuntimeError("the cache pool is too small for the benchmark's context")
-        engine.cache.commit(sid, context)
     gen = torch.Generator(device=engine.device).manual_seed(1)
     for arr in engine.storage.arrays:
         flat = arr.view(-1)
@@ -86,6 +80,16 @@ def fill_context(engine, ids, context: int) -> None:
             part = flat[i:i + step]
             part.copy_(torch.randn(part.numel(), generator=gen, device=engine.device, dtype=torch.float32)
                        .mul_(0.5).to(arr.dtype))
+
+
+def fill_context(engine, ids, context: int) -> None:
+    """Gives each request `context` cached tokens without running them: pages are reserved (they hold the
+    random keys and values of `fill_storage`)."""
+    for sid in ids:
+        engine.add_request(sid)
+        if not engine.cache.reserve(sid, context):
+            raise RuntimeError("the cache pool is too small for the benchmark's context")
+        engine.cache.commit(sid, context)
 
 
 def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decode_run: int = 8):
@@ -120,11 +124,12 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decod
 
 
 def time_prefill(engine, n_tokens: int, runs: int, vocab: int):
+    """Seconds of each of `runs` prefills of one prompt of `n_tokens` tokens (after one that is not counted)."""
     import torch
     from inferrs_amd.engine import Entry
     g = torch.Generator().manual_seed(2)
     prompt = torch.randint(0, vocab, (n_tokens,), generator=g).tolist()
-    best = None
+    times = []
     for r in range(runs + 1):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -133,8 +138,82 @@ def time_prefill(engine, n_tokens: int, runs: int, vocab: int):
         dt = time.perf_counter() - t0
         engine.end_request("p")
         if r > 0:
-            best = dt if best is None else min(best, dt)
-    return best
+            times.append(dt)
+    return times
+
+
+def mean_std(values):
+    m = sum(values) / len(values)
+    var = sum((v - m) ** 2 for v in values) / max(len(values) - 1, 1)
+    return m, var ** 0.5
+
+
+def measured_roofs(engine):
+    """(GB/s of a pure streaming read over at least 4 GB, TFLOP/s of a large bfloat16 product through the vendor's
+    GEMM): what this GPU gives in practice, beside the published peaks."""
+    import torch
+    from inferrs_amd import ops
+    src = max(engine.storage.arrays, key=lambda a: a.numel() * a.element_size()).view(-1)
+    want = 8 << 30
+    n = min(src.numel(), want // src.element_size()) // 64 * 64
+    if n * src.element_size() < (4 << 30):                  # a small cache: a buffer of its own
+        src = torch.empty(4 << 30, dtype=torch.uint8, device=engine.device).random_(0, 255)
+        n = src.numel()
+    part = src[:n]
+    best = None
+    for blocks in (2048, 4096, 8192):
+        for _ in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            ops.stream_read(part, blocks)
+            b.record()
+            torch.cuda.synchronize()
+            gbs = n * part.element_size() / (a.elapsed_time(b) * 1e-3) / 1e9
+            best = gbs if best is None else max(best, gbs)
+    m = 8192
+    x = torch.randn(m, m, device=engine.device, dtype=torch.bfloat16)
+    w = torch.randn(m, m, device=engine.device, dtype=torch.bfloat16)
+    torch.nn.functional.linear(x, w)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(10):
+        torch.nn.functional.linear(x, w)
+    b.record()
+    torch.cuda.synchronize()
+    tflops = 10 * 2.0 * m ** 3 / (a.elapsed_time(b) * 1e-3) / 1e12
+    return best, tflops
+
+
+def kernel_breakdown(engine, batch: int, context: int, prefill_tokens: int, vocab: int):
+    """Microseconds by kernel entry point for one decode step (batch, context) and one prefill, each kernel call
+    bracketed by events (eager steps, no graph; an event pair adds a few microseconds to a short kernel)."""
+    import torch
+    from inferrs_amd import ops
+    from inferrs_amd.engine import Entry
+    out = {}
+    ids = [f"k{i}" for i in range(batch)]
+    fill_context(engine, ids, context - 4)
+    graphs, engine.use_graphs = engine.use_graphs, False
+    try:
+        entries = [Entry(sid, [1 + i], [0]) for i, sid in enumerate(ids)]
+        engine.step(entries)                                   # once without the timer
+        with ops.KernelTimer() as timer:
+            engine.step(entries)
+        out["decode"] = timer.summary()
+        for sid in ids:
+            engine.end_request(sid)
+        g = torch.Generator().manual_seed(3)
+        prompt = torch.randint(0, vocab, (prefill_tokens,), generator=g).tolist()
+        engine.step([Entry("kp", prompt, [prefill_tokens - 1])])
+        engine.end_request("kp")
+        with ops.KernelTimer() as timer:
+            engine.step([Entry("kp", prompt, [prefill_tokens - 1])])
+        out["prefill"] = timer.summary()
+        engine.end_request("kp")
+    finally:
+        engine.use_graphs = graphs
+    return {phase: {name: {"calls": calls, "us": round(us, 1)} for name, (calls, us) in sorted(table.items(), key=lambda kv: -kv[1][1])}
+            for phase, table in out.items()}
 
 
 WORKLOADS = {
@@ -225,6 +304,10 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="length of the prompt of the prefill")
+    ap.add_argument("--runs", type=int, default=5, help="times the decode steps and the prefill are measured (mean and deviation)")
+    ap.add_argument("--no-extra-points", dest="extra_points", action="store_false",
+                    help="only batch 1 and 64 and the prefill beside the headline (no further batches and contexts, "
+                         "no per-kernel times, no 32-bit path)")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
     args = ap.parse_args()
@@ -265,19 +348,35 @@ def main() -> int:
     note(f"random weights of {args.layers} layers and a cache of {num_pages} pages")
     engine = Engine.from_random(config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=num_pages,
                                 max_seqs=biggest + 1)
-    note(f"decode at batch {args.batch}, context {args.context}: {args.warmup} + {args.steps} steps")
+    fill_storage(engine)
+    vocab = raw["vocab_size"]
+
+    def prefill_record(tokens: int, runs: int, roof_tflops=None):
+        times = time_prefill(engine, tokens, runs, vocab)
+        mean, std = mean_std(times)
+        flops = prefill_flops(raw, tokens)
+        rec = {"value": round(tokens / mean, 1), "tokens": tokens, "ms": round(mean * 1e3, 3),
+               "frac": round(flops / mean / PEAK_FLOPS[dtype_key], 4), "runs": len(times),
+               "ms_std": round(std * 1e3, 3), "ms_best": round(min(times) * 1e3, 3)}
+        if roof_tflops:
+            rec["measured_peak_tflops"] = round(roof_tflops, 1)
+            rec["frac_of_measured"] = round(flops / mean / (roof_tflops * 1e12), 4)
+        return rec
 
     if args.prefill_only:
-        t = time_prefill(engine, args.prefill_tokens, max(1, args.steps), raw["vocab_size"])
-        print(json.dumps({"prefill": {"value": round(args.prefill_tokens / t, 1), "tokens": args.prefill_tokens,
-                                      "ms": round(t * 1e3, 3),
-                                      "frac": round(prefill_flops(raw, args.prefill_tokens) / t / PEAK_FLOPS[dtype_key], 4)}}))
+        print(json.dumps({"prefill": prefill_record(args.prefill_tokens, max(1, args.steps))}))
         return 0
+    note(f"decode at batch {args.batch}, context {args.context}: {args.warmup} + {args.steps} steps, {args.runs} times")
     elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
     nbytes = decode_bytes(raw, args.batch, mean_ctx, esize)
     achieved = nbytes / (elapsed / args.steps) / 1e9
+    # the same K steps again, for the spread (the reference's bench: warm-up, then runs, mean and standard
+    # deviation, inferrs/src/bench.rs:159-173,226-248); the headline stays the first K steps
+    repeats = [ms_per_step] + [time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run)[0]
+                               / args.steps * 1e3 for _ in range(max(0, args.runs - 1))]
+    rep_mean, rep_std = mean_std(repeats)
 
     record = {
         "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-{args.shape})", "value": round(value, 2), "unit": "tok/s",
@@ -296,20 +395,78 @@ def main() -> int:
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "decode_runs": {"runs": len(repeats), "ms_per_step_mean": round(rep_mean, 4), "ms_per_step_std": round(rep_std, 4),
+                        "tok_s_mean": round(args.batch / rep_mean * 1e3, 2)},
     }
     if not args.no_points:
+        note("measured roofs: a streaming read and a large bfloat16 product")
+        read_gbs, gemm_tflops = measured_roofs(engine)
+        record["roofline"]["measured_peak"] = round(read_gbs, 1)
+        record["roofline"]["frac_of_measured"] = round(achieved / read_gbs, 4)
         points = {}
-        for b in points_batches:
+
+        def decode_point(name: str, b: int, context: int):
             steps = max(8, args.steps // 2)
-            note(f"decode at batch {b}: {steps} steps")
-            el, _ = time_decode(engine, b, args.context, steps, min(args.warmup, 4), args.decode_run)
-            points[f"decode_b{b}"] = round(b * steps / el, 2)
+            note(f"decode at batch {b}, context {context}: {steps} steps")
+            el, ctx_mean = time_decode(engine, b, context, steps, min(args.warmup, 4), args.decode_run)
+            points[name] = round(b * steps / el, 2)
+            fractions[name] = round(decode_bytes(raw, b, ctx_mean, esize) / (el / steps) / 1e9 / PEAK_HBM_GBS, 4)
+
+        fractions = {}
+        for b in points_batches:
+            decode_point(f"decode_b{b}", b, args.context)
+        if args.extra_points:
+            for b in (16, 32):
+                if b <= biggest:
+                    decode_point(f"decode_b{b}", b, args.context)
+            long_ctx = 4 * args.context
+            if args.batch * (long_ctx // PAGE + 1) + 8 <= num_pages and long_ctx <= raw["max_position_embeddings"]:
+                decode_point(f"decode_b{args.batch}_ctx{long_ctx}", args.batch, long_ctx)
         record["points"] = points
+        record["points_hbm_frac"] = fractions
         note(f"prefill of {args.prefill_tokens} tokens")
-        t = time_prefill(engine, args.prefill_tokens, 3, raw["vocab_size"])
-        flops = prefill_flops(raw, args.prefill_tokens)
-        record["prefill"] = {"value": round(args.prefill_tokens / t, 1), "tokens": args.prefill_tokens,
-                             "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS[dtype_key], 4)}
+        record["prefill"] = prefill_record(args.prefill_tokens, args.runs, gemm_tflops)
+        # the time to a request's first token through the serving loop (scheduler, step, choice, copy to the host)
+        from inferrs_amd.engine import GenerationLoop
+        from inferrs_amd.sampling import SamplingParams
+        g = torch.Generator().manual_seed(4)
+        prompt = torch.randint(0, vocab, (args.prefill_tokens,), generator=g).tolist()
+        firsts = []
+        for _ in range(3):
+            loop = GenerationLoop(engine, max_batch_size=1, max_tokens_per_step=args.prefill_tokens)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            loop.add(prompt, SamplingParams.greedy(max_tokens=1, bypass_stop_tokens=True))
+            loop.run()
+            firsts.append(time.perf_counter() - t0)
+        record["prefill"]["first_token_ms"] = round(min(firsts) * 1e3, 3)
+        if args.extra_points:
+            long_prompt = 4 * args.prefill_tokens
+            note(f"prefill of {long_prompt} tokens")
+            rec = prefill_record(long_prompt, 3)
+            points[f"prefill_{long_prompt}"] = rec["value"]
+            fractions[f"prefill_{long_prompt}_mfma"] = rec["frac"]
+            note("per-kernel times of one decode step and one prefill")
+            record["kernels"] = kernel_breakdown(engine, args.batch, args.context, args.prefill_tokens, vocab)
+            # the true 32-bit path at the same layer sizes, four layers of them
+            if args.dtype == "bfloat16":
+                f32_layers = min(4, args.layers)
+                note(f"the 32-bit path: {f32_layers} layers")
+                del loop
+                raw32 = dict(raw, num_hidden_layers=f32_layers)
+                eng32 = Engine.from_random(Qwen3Config.from_dict(raw32), seed=0, dtype="float32", page_size=PAGE,
+                                           num_pages=max(args.batch * (-(-args.context // PAGE) + 1),
+                                                         -(-args.prefill_tokens // PAGE)) + 8, max_seqs=args.batch + 1)
+                fill_storage(eng32)
+                el, ctx_mean = time_decode(eng32, args.batch, args.context, 8, 3, args.decode_run)
+                points[f"f32_decode_b{args.batch}_layers{f32_layers}"] = round(args.batch * 8 / el, 2)
+                fractions[f"f32_decode_b{args.batch}_layers{f32_layers}"] = round(
+                    decode_bytes(raw32, args.batch, ctx_mean, 4) / (el / 8) / 1e9 / PEAK_HBM_GBS, 4)
+                times = time_prefill(eng32, args.prefill_tokens, 2, vocab)
+                points[f"f32_prefill_{args.prefill_tokens}_layers{f32_layers}"] = round(args.prefill_tokens / min(times), 1)
+                fractions[f"f32_prefill_{args.prefill_tokens}_layers{f32_layers}_fma"] = round(
+                    prefill_flops(raw32, args.prefill_tokens) / min(times) / PEAK_FLOPS["fp32"], 4)
+                del eng32
     print(json.dumps(record))
     return 0
 

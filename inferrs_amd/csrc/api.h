@@ -27,6 +27,9 @@ int ia_fill_normal(void* out, long long n, unsigned long long seed, double mean,
                    int dtype, hipStream_t stream);
 int ia_widen_bf16(float* out, const void* x, long long n, hipStream_t stream);
 int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream);
+// A pure streaming read of `bytes` bytes by `blocks` blocks (one word of `out` a block): the measurement script's
+// measured memory roof.  Nothing of the engine calls it.
+int ia_stream_read(unsigned* out, const void* x, long long bytes, int blocks, hipStream_t stream);
 int ia_rope_table(float* cos_out, float* sin_out, const int* positions, const float* inv_freq,
                   int n, int half, hipStream_t stream);
 

@@ -365,3 +365,35 @@ extern "C" int ia_rope_table(float* cos_out, float* sin_out, const int* position
     IA_LAUNCH_CHECK("rope_table");
     return 0;
 }
+
+// ---- a pure streaming read: the measured roof of this GPU's memory for the measurement script ----------------
+// Every thread reads 16-byte pieces a whole grid apart, four under way at a time, and folds them into one word; a
+// block leaves one word, so that nothing of the read can be dropped.  Nothing of the engine calls it.
+__global__ __launch_bounds__(256) void stream_read_kernel(unsigned* __restrict__ out, const uint4* __restrict__ x, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned acc = 0;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const uint4 a = x[i], b = x[i + stride], c = x[i + 2 * stride], d = x[i + 3 * stride];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < n16; i += stride) {
+        const uint4 a = x[i];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
+#pragma unroll
+    for (int o = IA_WAVE / 2; o > 0; o >>= 1) acc ^= __shfl_xor(acc, o, IA_WAVE);
+    __shared__ unsigned part[4];
+    if ((threadIdx.x & (IA_WAVE - 1)) == 0) part[threadIdx.x / IA_WAVE] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) out[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
+}
+
+// out: `blocks` words; x: `bytes` bytes, 16-byte aligned, a multiple of 16.
+extern "C" int ia_stream_read(unsigned* out, const void* x, long long bytes, int blocks, hipStream_t stream) {
+    IA_CHECK(bytes >= 0 && bytes % 16 == 0 && blocks > 0 && blocks <= 1048576, "stream_read: bad sizes bytes=%lld blocks=%d", bytes, blocks);
+    IA_CHECK((((uintptr_t)x) & 15) == 0, "stream_read: x must be 16-byte aligned");
+    stream_read_kernel<<<blocks, 256, 0, stream>>>(out, (const uint4*)x, (size_t)bytes / 16);
+    IA_LAUNCH_CHECK("stream_read");
+    return 0;
+}

@@ -28,11 +28,64 @@ _LIBS: Dict[str, ctypes.CDLL] = {}
 _LIB_PATHS: Dict[str, str] = {}
 
 
-def library(target: str = "core") -> ctypes.CDLL:
+class KernelTimer:
+    """Times every kernel call of this module with a pair of events while it is active:
+
+        with ops.KernelTimer() as timer: ...steps...
+        timer.summary() -> {entry point: (calls, microseconds)}
+
+    For measurement only: each call is bracketed on the current stream, so launches are not overlapped."""
+    active: Optional["KernelTimer"] = None
+
+    def __init__(self):
+        self.records = []                 # (name, start event, end event)
+
+    def __enter__(self):
+        KernelTimer.active = self
+        return self
+
+    def __exit__(self, *exc):
+        KernelTimer.active = None
+
+    def call(self, name, fn, *args):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        out = fn(*args)
+        b.record()
+        self.records.append((name, a, b))
+        return out
+
+    def summary(self) -> Dict[str, Tuple[int, float]]:
+        torch.cuda.synchronize()
+        out: Dict[str, Tuple[int, float]] = {}
+        for name, a, b in self.records:
+            calls, us = out.get(name, (0, 0.0))
+            out[name] = (calls + 1, us + a.elapsed_time(b) * 1e3)
+        return out
+
+
+class _Timed:
+    """A kernel library whose entry points report to the active `KernelTimer`, if there is one."""
+    __slots__ = ("_lib", "_short")
+
+    def __init__(self, lib: ctypes.CDLL):
+        object.__setattr__(self, "_lib", lib)
+        object.__setattr__(self, "_short", {})
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        if KernelTimer.active is None or not name.startswith("ia_") or name.endswith(("_workspace", "_blocks", "_block_rows",
+                                                                                      "_error", "_version", "_capacity", "_top")):
+            return fn
+        timer = KernelTimer.active
+        return lambda *args: timer.call(name[3:], fn, *args)
+
+
+def library(target: str = "core"):
     """A compiled kernel library; compiled on first use when no built one is found."""
     lib = _LIBS.get(target)
     if lib is not None:
-        return lib
+        return lib if KernelTimer.active is None else _Timed(lib)
     path = _build.library_path(target)
     if path is None:
         path = _build.build(target, verbose=True)
@@ -479,6 +532,16 @@ def fill_normal(shape, seed: int, mean: float, std: float, dtype: torch.dtype, d
     return out
 
 
+def stream_read(x: torch.Tensor, blocks: int = 4096) -> torch.Tensor:
+    """Reads all of `x` once (a multiple of 16 bytes) and returns one word a block: the measurement script times it
+    for the memory's practical read rate."""
+    _dev(x)
+    nbytes = x.numel() * x.element_size()
+    out = torch.empty((blocks,), dtype=torch.int32, device=x.device)
+    _check(library().ia_stream_read(_p(out), _p(x), ctypes.c_longlong(nbytes), blocks, _stream()))
+    return out
+
+
 def widen(x: torch.Tensor) -> torch.Tensor:
     """bfloat16 -> float32, exactly."""
     _dev(x)
@@ -594,7 +657,12 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch
     _dev(x, w)
     if w.shape[1] != k or w.dtype != x.dtype:
         raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
-    y = gemm_mfma_bf16(x, w) if _own_large(x, w) else torch.nn.functional.linear(x, w)
+    if _own_large(x, w):
+        y = gemm_mfma_bf16(x, w)
+    elif KernelTimer.active is not None:
+        y = KernelTimer.active.call("vendor_gemm", torch.nn.functional.linear, x, w)
+    else:
+        y = torch.nn.functional.linear(x, w)
     return widen(y) if out_dtype == torch.float32 else y
 
 

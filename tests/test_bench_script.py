@@ -36,8 +36,24 @@ def test_decode_record_has_the_agreed_keys():
     assert config["layers"] == 2 and config["layers_of_model"] == 36 and config["global_batch"] == 2
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / 8000.0) < 1e-3
-    assert set(rec["points"]) == {"decode_b1", "decode_b64"}
+    assert {"decode_b1", "decode_b64", "decode_b16", "decode_b32", "decode_b2_ctx1024", "prefill_8192",
+            "f32_decode_b2_layers2", "f32_prefill_2048_layers2"} <= set(rec["points"])
+    assert all(isinstance(v, (int, float)) and v > 0 for v in rec["points"].values())
+    assert set(rec["points"]) <= set(rec["points_hbm_frac"]) | {"prefill_8192", "f32_prefill_2048_layers2"}
     assert rec["prefill"]["tokens"] == 2048 and rec["prefill"]["value"] > 0 and 0 < rec["prefill"]["frac"] < 1
+    # mean and deviation over five repetitions, for decode and prefill
+    assert rec["decode_runs"]["runs"] == 5 and rec["decode_runs"]["ms_per_step_mean"] > 0 and rec["decode_runs"]["ms_per_step_std"] >= 0
+    assert rec["prefill"]["runs"] == 5 and rec["prefill"]["ms_std"] >= 0 and rec["prefill"]["ms_best"] <= rec["prefill"]["ms"]
+    assert rec["prefill"]["first_token_ms"] > 0
+    # fractions of the measured roofs beside those of the published peaks
+    roof = rec["roofline"]
+    assert 1000 < roof["measured_peak"] < 8000.0 and abs(roof["frac_of_measured"] - roof["achieved"] / roof["measured_peak"]) < 1e-3
+    assert 100 < rec["prefill"]["measured_peak_tflops"] < 2500 and rec["prefill"]["frac_of_measured"] > rec["prefill"]["frac"]
+    # microseconds by kernel for one decode step and one prefill
+    for phase in ("decode", "prefill"):
+        table = rec["kernels"][phase]
+        assert table and all(v["calls"] > 0 and v["us"] > 0 for v in table.values())
+    assert "gemm_skinny_stream" in rec["kernels"]["decode"] and "attention_mfma" in rec["kernels"]["prefill"]
 
 
 @pytest.mark.gpu
