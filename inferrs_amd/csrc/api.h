@@ -65,6 +65,19 @@ int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N,
                           int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
                           int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream);
 
+// Products of 17 to 64 bfloat16 rows (gemm_mid.hip); K a multiple of 128.  out_mode 0: out [M, N] bfloat16; 1: float;
+// 2: out [ia_gemm_mid_splits(N, K)][M][N] float, the sums of each split of k, to be added up by the reader
+// (ia_sum_partials, ia_add_rmsnorm_partials).  dual: w = [gate; up], out = silu(x . gate^T) * (x . up^T), mode 0.
+int ia_gemm_mid_splits(int N, int K);
+// (k steps of a chunk: 4, 8 or 16; chunks in shared memory: 2 to 4; the default is (4, 3); results do not depend on it)
+void ia_gemm_mid_tune(int kc, int ns);
+int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
+                     hipStream_t stream);
+int ia_sum_partials(void* out, const float* part, int splits, int M, int N, hipStream_t stream);
+// x += (sum of the splits, rounded to bfloat16) in place, out = rmsnorm(x) * w; bfloat16 rows of up to 8192 features.
+int ia_add_rmsnorm_partials(void* out, void* x, const float* part, int splits, const float* w, float eps,
+                            int rows, int cols, int add_one, hipStream_t stream);
+
 long long ia_argmax_workspace(int rows, int vocab);
 int ia_argmax(int* out, const float* logits, void* workspace, int rows, int vocab, hipStream_t stream);
 // The arg max without any allocation.  It has no counterpart in the reference; it is for callers that cannot

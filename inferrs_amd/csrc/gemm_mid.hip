@@ -1,0 +1,424 @@
+// bfloat16 products for steps of 17 to 64 rows (decode steps of many requests, short prompt portions):
+// out[M, N] = x[M, K] . w[N, K]^T, bound by reading the weights once, like the skinny product, but with so
+// many rows that the activations can no longer be fetched by every wave for itself (at 64 rows they are as
+// large as a block's share of the weights).
+//
+// The reference hands these products to cuBLAS like all others (`candle-core/src/cuda_backend/mod.rs:2260-2305`).
+//
+// A block of four waves owns 64 rows of w and a range of k.  A wave streams one tile of 16 weight rows from
+// memory straight into MFMA A-operands (v_mfma_f32_16x16x32_bf16: lane l supplies row l % 16 with the eight k
+// values 8 * (l / 16) .. + 8), three chunks of 128 k ahead of their use; the rows of x of a chunk (up to 64 rows
+// of 256 bytes) are brought into shared memory once a block by all four waves together (global_load_lds, 16 bytes
+// a lane, no register on the way), three chunks ahead as well, and every wave reads its B-operands from there.
+// All row tiles of x share every weight load.  Piece c (16 bytes) of row r of a chunk lies at place c ^ (r % 16)
+// of the row's 256 bytes, so that the 16 rows which one operand read takes at the same k fall on 16 different
+// places; a load instruction fills 1 KiB (four rows) in lane order, and the lane picks the piece it fetches
+// accordingly.
+//
+// With few rows of w (the output projection, the feed-forward's second product) 64 rows a block leave too few
+// blocks to fill the chip, so k is split between blocks (gridDim.y) and every split leaves its sums in 32-bit:
+// [splits][M][N].  They are added up, in the order of the splits, by whoever reads them: the kernel that adds a
+// product to the residual stream and norms it (ia_add_rmsnorm_partials), or ia_sum_partials.  The split depends
+// on the weight's shape alone, never on the rows of the step.
+//
+// DUAL: w = [gate; up] (N rows each); a block owns 32 output features, waves 0 and 1 their gate rows, waves 2 and 3
+// their up rows, and the result is silu(gate . x) * (up . x), the first product rounded to bfloat16 before the
+// activation as the two-kernel path rounds it.  No split of k (the activation needs whole sums).
+#include <type_traits>
+
+#include "common.h"
+#include "api.h"
+
+typedef __bf16 gmid_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float gmid_f32x4 __attribute__((ext_vector_type(4)));
+
+#define MID_WAVES 4
+#define MID_CHUNK_MIN_K 128               // k is shared out in multiples of this
+
+// s_waitcnt that waits until at most n vector-memory operations of this wave are under way (gfx9 encoding:
+// vmcnt in bits 3:0 and 15:14; the other counters left alone).
+#define MID_VMCNT(n) (((n) & 15) | ((((n) >> 4) & 3) << 14) | (7 << 4) | (15 << 8))
+
+enum { MID_OUT_BF16 = 0, MID_OUT_F32 = 1, MID_OUT_PARTIAL = 2 };
+
+// KC: k steps of 32 in a chunk (a row of x in a chunk is KC * 64 bytes); NS: chunks of x in shared memory, this one and
+// NS - 1 on their way.
+template <int MT, bool DUAL, int KC, int NS>
+__global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
+    void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+    int M, int N, int K, int k_per_block) {
+    constexpr int CHUNK_K = KC * 32;
+    constexpr int ROW_BYTES = KC * 64;                      // bytes of a row of x in a chunk
+    constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;         // rows that one load instruction (1 KiB) fills
+    constexpr int PIECES = KC * 4;                          // 16-byte pieces of a row
+    constexpr int X_LOADS = MT * 16 / ROWS_PER_LOAD / MID_WAVES;   // load instructions of x a wave issues for a chunk
+    constexpr int STAGE_BYTES = MT * 16 * ROW_BYTES;
+    static_assert(NS >= 2 && NS <= 4 && (KC == 4 || KC == 8 || KC == 16), "pipeline shape");
+    static_assert(MT * 16 / ROWS_PER_LOAD % MID_WAVES == 0, "the rows of a chunk are shared out evenly between the waves");
+    // A stage [MT * 16 rows][ROW_BYTES] an array: the compiler then knows that loads on their way into one stage do
+    // not touch the others, and does not wait for them before it reads operands out of this one.
+    __shared__ __attribute__((aligned(1024))) char mid_s0[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char mid_s1[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char mid_s2[NS > 2 ? STAGE_BYTES : 16];
+    __shared__ __attribute__((aligned(1024))) char mid_s3[NS > 3 ? STAGE_BYTES : 16];
+    auto stage_of = [&](auto stage_c) -> char* {
+        constexpr int S = decltype(stage_c)::value;
+        if constexpr (S == 0) return mid_s0;
+        else if constexpr (S == 1) return mid_s1;
+        else if constexpr (S == 2) return mid_s2;
+        else return mid_s3;
+    };
+    const int lane = threadIdx.x & (IA_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / IA_WAVE);
+    const int r = lane & 15, g = lane >> 4;
+    const int split = blockIdx.y;
+    const int k_begin = split * k_per_block;
+    const int k_len = K - k_begin < k_per_block ? K - k_begin : k_per_block;
+    const int nchunks = k_len / CHUNK_K;
+
+    // ---- this wave's 16 rows of w --------------------------------------------------------------------------
+    // (rows beyond the matrix read its last row: their sums are never stored)
+    int n_first;                 // output feature of the tile's first row
+    const bf16_t* wrow;
+    if (DUAL) {
+        n_first = blockIdx.x * 32 + 16 * (wave & 1);
+        const int n = n_first + r < N ? n_first + r : N - 1;
+        wrow = w + ((size_t)(wave >> 1) * N + n) * K + k_begin + g * 8;
+    } else {
+        n_first = blockIdx.x * 64 + 16 * wave;
+        const int n = n_first + r < N ? n_first + r : N - 1;
+        wrow = w + (size_t)n * K + k_begin + g * 8;
+    }
+
+    // ---- what this lane fetches of a chunk of x: X_LOADS instructions, each ROWS_PER_LOAD whole rows ------------
+    // instruction i of wave v covers rows ROWS_PER_LOAD * (4 i + v) .. ; lane l writes place l % PIECES of row l / PIECES
+    // of them, and fetches the piece that belongs there: piece c of row r lies at place c ^ (r % 16)
+    const char* xsrc[X_LOADS];
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) {
+        const int row = ROWS_PER_LOAD * (MID_WAVES * i + wave) + lane / PIECES;
+        const int piece = (lane % PIECES) ^ (row & 15);
+        xsrc[i] = (const char*)(x + (size_t)(row < M ? row : 0) * K + k_begin) + piece * 16;
+    }
+    // and where it reads its B-operands: row 16 mt + r, piece 4 ks + g, at place (4 ks + g) ^ r
+    uint32_t b_at[KC];
+#pragma unroll
+    for (int ks = 0; ks < KC; ++ks) b_at[ks] = (uint32_t)(r * ROW_BYTES + (((4 * ks + g) ^ r) * 16));
+
+    gmid_f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
+    uint4 wreg[NS][KC];
+
+    auto issue = [&](auto stage_c, int c) {
+        constexpr int S = decltype(stage_c)::value;
+        // the weights first, then the rows of x: a wait for the rows of a chunk covers its weights too
+#pragma unroll
+        for (int ks = 0; ks < KC; ++ks) wreg[S][ks] = *(const uint4*)(wrow + (size_t)c * CHUNK_K + ks * 32);
+        char* stage = stage_of(stage_c);
+#pragma unroll
+        for (int i = 0; i < X_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)(xsrc[i] + (size_t)c * ROW_BYTES),
+                (void __attribute__((address_space(3)))*)(stage + (MID_WAVES * i + wave) * 1024), 16, 0, 0);
+    };
+    constexpr int PER_CHUNK = KC + X_LOADS;           // vector-memory instructions a wave issues for a chunk
+    auto multiply = [&](auto stage_c) {
+        constexpr int S = decltype(stage_c)::value;
+        const char* stage = stage_of(stage_c);
+#pragma unroll
+        for (int ks = 0; ks < KC; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint4 b = *(const uint4*)(stage + mt * (16 * ROW_BYTES) + b_at[ks]);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(gmid_bf16x8, wreg[S][ks]), __builtin_bit_cast(gmid_bf16x8, b), acc[mt], 0, 0, 0);
+            }
+    };
+    // Chunk c has arrived when no more than the chunks after it are under way (loads return in order).  The bare
+    // barrier: __syncthreads() would wait for every load under way first.  After it everybody's part of chunk c is
+    // there, and everybody is done with chunk c - 1, whose stage chunk c + NS - 1 goes into.
+    auto full_step = [&](auto stage_c, int c) {              // chunks c + 1 .. c + NS - 1 exist
+        constexpr int S = decltype(stage_c)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(MID_VMCNT((NS - 2) * PER_CHUNK));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue(std::integral_constant<int, (S + NS - 1) % NS>(), c + NS - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(stage_c);
+    };
+    auto last_step = [&](auto stage_c, int c) {              // the last NS - 1 chunks: nothing left to ask for
+        __builtin_amdgcn_sched_barrier(0);
+        if (NS > 3 && c + 2 < nchunks) __builtin_amdgcn_s_waitcnt(MID_VMCNT(2 * PER_CHUNK));
+        else if (NS > 2 && c + 1 < nchunks) __builtin_amdgcn_s_waitcnt(MID_VMCNT(PER_CHUNK));
+        else __builtin_amdgcn_s_waitcnt(MID_VMCNT(0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(stage_c);
+    };
+    auto ring = [&](auto fn, int c) {                        // fn on chunks c .. c + NS - 1, each in its stage
+        fn(std::integral_constant<int, 0>(), c);
+        fn(std::integral_constant<int, 1>(), c + 1);
+        if constexpr (NS > 2) fn(std::integral_constant<int, 2>(), c + 2);
+        if constexpr (NS > 3) fn(std::integral_constant<int, 3>(), c + 3);
+    };
+    int c = 0;
+    if (nchunks >= 2 * NS - 1) {
+        // (a path of its own without a condition between the first loads and the loop: what is under way at the loop's
+        // head is then the same from both sides, and the compiler adds no wait of its own)
+        issue(std::integral_constant<int, 0>(), 0);
+        if constexpr (NS > 2) issue(std::integral_constant<int, 1>(), 1);
+        if constexpr (NS > 3) issue(std::integral_constant<int, 2>(), 2);
+        for (; c + 2 * NS - 1 <= nchunks; c += NS) ring(full_step, c);         // chunks up to c + 2 NS - 2 exist
+    } else {
+        if (nchunks > 0) issue(std::integral_constant<int, 0>(), 0);
+        if constexpr (NS > 2) { if (nchunks > 1) issue(std::integral_constant<int, 1>(), 1); }
+        if constexpr (NS > 3) { if (nchunks > 2) issue(std::integral_constant<int, 2>(), 2); }
+    }
+    // (c is a multiple of the number of stages here: chunk c + i lies in stage i % NS)
+    auto tail_step = [&](auto stage_c, int cc) {
+        if (cc >= nchunks) return;
+        if (cc + NS - 1 < nchunks) full_step(stage_c, cc);
+        else last_step(stage_c, cc);
+    };
+    ring(tail_step, c);
+    ring(tail_step, c + NS);
+
+    // ---- results: lane (r, g) holds features n_first + 4 g + i of row 16 mt + r ---------------------------------
+    if (DUAL) {
+        // the up rows' sums go through shared memory to the waves that hold the gate rows' sums of the same features
+        __syncthreads();
+        gmid_f32x4* swap = (gmid_f32x4*)mid_s0;                           // [2 tiles][MT][64 lanes]
+        if (wave >= 2) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) swap[((wave - 2) * MT + mt) * IA_WAVE + lane] = acc[mt];
+        }
+        __syncthreads();
+        if (wave >= 2) return;
+        const int nb = n_first + 4 * g;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            if (m >= M) continue;
+            const gmid_f32x4 up = swap[(wave * MT + mt) * IA_WAVE + lane];
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gate = bf16_bits_to_f32(f32_to_bf16_bits(acc[mt][i]));
+                const float u = bf16_bits_to_f32(f32_to_bf16_bits(up[i]));
+                v[i] = gate / (1.0f + expf(-gate)) * u;
+            }
+            bf16_t* o = (bf16_t*)out + (size_t)m * N + nb;
+            if (nb + 3 < N && (N & 3) == 0) {
+                *(uint2*)o = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (nb + i < N) o[i].bits = f32_to_bf16_bits(v[i]);
+            }
+        }
+        return;
+    }
+    const int nb = n_first + 4 * g;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + r;
+        if (m >= M) continue;
+        if (out_mode == MID_OUT_BF16) {
+            bf16_t* o = (bf16_t*)out + (size_t)m * N + nb;
+            if (nb + 3 < N && (N & 3) == 0) {
+                *(uint2*)o = make_uint2(pack_bf16x2(acc[mt][0], acc[mt][1]), pack_bf16x2(acc[mt][2], acc[mt][3]));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (nb + i < N) o[i].bits = f32_to_bf16_bits(acc[mt][i]);
+            }
+        } else {
+            float* o = (float*)out + ((size_t)(out_mode == MID_OUT_PARTIAL ? split : 0) * M + m) * N + nb;
+            if (nb + 3 < N && (N & 3) == 0) {
+                *(gmid_f32x4*)o = acc[mt];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (nb + i < N) o[i] = acc[mt][i];
+            }
+        }
+    }
+}
+
+// How many ways k is split between blocks: a function of the weight's shape and the chip alone.  64 rows of w a
+// block; splits double until there are three blocks for every two compute units or a split would fall below 512 k.
+static int mid_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    return cus;
+}
+
+extern "C" int ia_gemm_mid_splits(int N, int K) {
+    if (N <= 0 || K <= 0 || K % MID_CHUNK_MIN_K) return 0;
+    const int blocks = (N + 63) / 64;
+    const int chunks = K / MID_CHUNK_MIN_K;
+    int splits = 1;
+    while (2 * blocks * splits < 3 * mid_cus() && splits < 16 && chunks % (2 * splits) == 0 && chunks / (2 * splits) >= 4)
+        splits *= 2;
+    return splits;
+}
+
+// Tuning: k steps of a chunk (4, 8 or 16) and chunks in shared memory (2 to 4).  Measured at the sizes of an 8 B and a
+// 32 B model, 32 and 64 rows: all within a tenth of each other; (4, 3) is the default (the smallest stages, so that most
+// blocks fit a compute unit).
+static int g_mid_kc = 4, g_mid_ns = 3;
+extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns; }
+
+template <int MT, bool DUAL, int KC, int NS>
+static void launch_mid_shape(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
+                             hipStream_t stream) {
+    const dim3 grid(DUAL ? (N + 31) / 32 : (N + 63) / 64, splits);
+    gemm_mid_kernel<MT, DUAL, KC, NS><<<grid, MID_WAVES * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, K / splits);
+}
+
+template <int MT, bool DUAL>
+static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
+                      hipStream_t stream) {
+    const int k_block = K / splits;
+    // (a chunk must divide a block's share of k, and a stage of MT * 16 rows must leave room in shared memory)
+    if (g_mid_kc == 16 && g_mid_ns == 2 && k_block % 512 == 0) launch_mid_shape<MT, DUAL, 16, 2>(out, out_mode, x, w, M, N, K, splits, stream);
+    else if (g_mid_kc == 8 && g_mid_ns == 3 && k_block % 256 == 0) launch_mid_shape<MT, DUAL, 8, 3>(out, out_mode, x, w, M, N, K, splits, stream);
+    else if (g_mid_kc == 8 && g_mid_ns == 2 && k_block % 256 == 0) launch_mid_shape<MT, DUAL, 8, 2>(out, out_mode, x, w, M, N, K, splits, stream);
+    else if (g_mid_kc == 4 && g_mid_ns == 4) launch_mid_shape<MT, DUAL, 4, 4>(out, out_mode, x, w, M, N, K, splits, stream);
+    else launch_mid_shape<MT, DUAL, 4, 3>(out, out_mode, x, w, M, N, K, splits, stream);
+    return 0;
+}
+
+// out_mode 0: out [M, N] bfloat16; 1: out [M, N] float; 2: out [splits][M][N] float with splits =
+// ia_gemm_mid_splits(N, K), to be added up by the reader.  dual: w = [gate; up] of N rows each, out = silu(x . gate^T)
+// * (x . up^T) in bfloat16 (mode 0 only).  M in 1..64, K a multiple of 128.
+extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
+                                hipStream_t stream) {
+    IA_CHECK(M >= 1 && M <= 64 && N > 0 && K > 0, "gemm_mid: takes 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
+    IA_CHECK(K % MID_CHUNK_MIN_K == 0, "gemm_mid: K=%d must be a multiple of %d (use another product)", K, MID_CHUNK_MIN_K);
+    IA_CHECK(out_mode >= 0 && out_mode <= 2 && (!dual || out_mode == MID_OUT_BF16), "gemm_mid: output mode %d%s", out_mode,
+             dual ? " does not go with the activation inside" : " is unknown");
+    IA_CHECK((((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0, "gemm_mid: operands must be 16-byte aligned");
+    const int splits = out_mode == MID_OUT_PARTIAL ? ia_gemm_mid_splits(N, K) : 1;
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)w;
+    const int mt = (M + 15) / 16;
+    if (dual) {
+        if (mt == 1) launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        else if (mt == 2) launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        else if (mt == 3) launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        else launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+    } else {
+        if (mt == 1) launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        else if (mt == 2) launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        else if (mt == 3) launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        else launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+    }
+    IA_LAUNCH_CHECK("gemm_mid");
+    return 0;
+}
+
+// ---- readers of the splits' sums ------------------------------------------------------------------------------
+// out[m][n] = sum over the splits, in their order, rounded once.
+__global__ __launch_bounds__(256) void sum_partials_kernel(bf16_t* __restrict__ out, const float* __restrict__ part,
+                                                           int splits, size_t mn) {
+    const size_t i4 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i4 >= mn) return;
+    if (i4 + 3 < mn) {
+        float4 s = *(const float4*)(part + i4);
+        for (int k = 1; k < splits; ++k) {
+            const float4 o = *(const float4*)(part + (size_t)k * mn + i4);
+            s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+        }
+        *(uint2*)(out + i4) = make_uint2(pack_bf16x2(s.x, s.y), pack_bf16x2(s.z, s.w));
+    } else {
+        for (size_t i = i4; i < mn; ++i) {
+            float s = part[i];
+            for (int k = 1; k < splits; ++k) s += part[(size_t)k * mn + i];
+            out[i].bits = f32_to_bf16_bits(s);
+        }
+    }
+}
+
+extern "C" int ia_sum_partials(void* out, const float* part, int splits, int M, int N, hipStream_t stream) {
+    IA_CHECK(splits >= 1 && M >= 0 && N > 0, "sum_partials: bad sizes splits=%d M=%d N=%d", splits, M, N);
+    IA_CHECK(((size_t)M * N) % 4 == 0 || splits >= 1, "sum_partials: bad sizes");
+    if (M == 0) return 0;
+    const size_t mn = (size_t)M * N;
+    IA_CHECK((mn & 3) == 0 && (((uintptr_t)out | (uintptr_t)part) & 15) == 0, "sum_partials: M * N must be a multiple of 4 "
+             "and the arrays 16-byte aligned");
+    sum_partials_kernel<<<(unsigned)((mn / 4 + 255) / 256), 256, 0, stream>>>((bf16_t*)out, part, splits, mn);
+    IA_LAUNCH_CHECK("sum_partials");
+    return 0;
+}
+
+// x[row] += the product (the splits' sums added up in their order and rounded to bfloat16, as a product that is stored
+// would be), the sum formed in 32-bit and rounded; out[row] = rmsnorm(x[row]) * w.  One block a row, the row kept in
+// registers between the two passes.  The same arithmetic as the add-and-norm kernel of elementwise.hip on a stored product.
+#define APN_THREADS 256
+#define APN_MAX_PER_THREAD 8             // rows of up to 256 * 4 * 8 = 8192 features
+__global__ __launch_bounds__(APN_THREADS) void add_rmsnorm_partials_kernel(
+    bf16_t* __restrict__ out, bf16_t* __restrict__ x, const float* __restrict__ part, int splits, size_t mn,
+    const float* __restrict__ w, float eps, int cols, int add_one) {
+    __shared__ float scratch[16];
+    const size_t row = blockIdx.x;
+    float h[APN_MAX_PER_THREAD][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < APN_MAX_PER_THREAD; ++j) {
+        const int c = (j * APN_THREADS + threadIdx.x) * 4;
+        if (c >= cols) break;
+        const size_t at = row * cols + c;
+        float4 s = *(const float4*)(part + at);
+        for (int k = 1; k < splits; ++k) {
+            const float4 o = *(const float4*)(part + (size_t)k * mn + at);
+            s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+        }
+        const uint2 old = *(const uint2*)(x + at);
+        const float sv[4] = {s.x, s.y, s.z, s.w};
+        const uint16_t ob[4] = {(uint16_t)old.x, (uint16_t)(old.x >> 16), (uint16_t)old.y, (uint16_t)(old.y >> 16)};
+        uint16_t nb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float product = bf16_bits_to_f32(f32_to_bf16_bits(sv[i]));
+            nb[i] = f32_to_bf16_bits(product + bf16_bits_to_f32(ob[i]));
+            h[j][i] = bf16_bits_to_f32(nb[i]);
+            ss += h[j][i] * h[j][i];
+        }
+        *(uint2*)(x + at) = make_uint2((uint32_t)nb[0] | ((uint32_t)nb[1] << 16), (uint32_t)nb[2] | ((uint32_t)nb[3] << 16));
+    }
+    const float total = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(total / (float)cols + eps);
+#pragma unroll
+    for (int j = 0; j < APN_MAX_PER_THREAD; ++j) {
+        const int c = (j * APN_THREADS + threadIdx.x) * 4;
+        if (c >= cols) break;
+        const float4 g4 = *(const float4*)(w + c);
+        const float gw[4] = {g4.x, g4.y, g4.z, g4.w};
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = h[j][i] * scale * (add_one ? 1.0f + gw[i] : gw[i]);
+        *(uint2*)(out + row * cols + c) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    }
+}
+
+extern "C" int ia_add_rmsnorm_partials(void* out, void* x, const float* part, int splits, const float* w, float eps,
+                                       int rows, int cols, int add_one, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && cols > 0 && splits >= 1, "add_rmsnorm_partials: bad sizes rows=%d cols=%d splits=%d", rows, cols, splits);
+    IA_CHECK(cols % 4 == 0 && cols <= APN_THREADS * 4 * APN_MAX_PER_THREAD,
+             "add_rmsnorm_partials: rows of %d features: takes multiples of 4 up to %d", cols, APN_THREADS * 4 * APN_MAX_PER_THREAD);
+    IA_CHECK((((uintptr_t)out | (uintptr_t)x | (uintptr_t)part | (uintptr_t)w) & 15) == 0,
+             "add_rmsnorm_partials: arrays must be 16-byte aligned");
+    if (rows == 0) return 0;
+    add_rmsnorm_partials_kernel<<<rows, APN_THREADS, 0, stream>>>((bf16_t*)out, (bf16_t*)x, part, splits, (size_t)rows * cols,
+                                                                  w, eps, cols, add_one);
+    IA_LAUNCH_CHECK("add_rmsnorm_partials");
+    return 0;
+}

@@ -50,6 +50,7 @@ class StepContext:
     max_kv_multi: int = 0        # and among the others
     stream: Optional[torch.Tensor] = None   # set by a block around a part that may add its output to it itself
     stream_norm: Any = None                 # and the norm part that will read the stream next
+    partial_sums: bool = False              # set by a block whose norms take a part's last product split along k
     _tables: Dict[Any, Any] = field(default_factory=dict)
 
     @property

@@ -83,6 +83,8 @@ class DecoderModel:
         n_want = ctx.want_rows.numel()
         if n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
+        if isinstance(pending, ops.Partials):        # the last product is still split along k
+            pending = pending.materialize()
         xs = ops.gather_rows(x, ctx.want_rows)
         added = pending is None or isinstance(pending, ops.Added)   # the last block has left nothing to add
         if self.final_norm is None:

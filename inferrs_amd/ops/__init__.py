@@ -634,6 +634,98 @@ def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=
     return sums, scaled
 
 
+# ---- products of 17 to 64 rows -------------------------------------------------------------------
+# Decode steps of many requests and short prompt portions: still bound by reading the weights once, which the vendor's
+# GEMM does at 3.4 TB/s and the kernel of gemm_mid.hip faster.  Weights with few rows (the output projection, the
+# feed-forward's second product) are split along k between blocks, and the splits' sums are added up by the reader:
+# `Partials` stands for a product in that state.
+
+MID_MAX_ROWS = 64             # rows up to which the products of gemm_mid.hip take over from the vendor's GEMM
+# [gate; up] weights beyond this many bytes go to the vendor's GEMM and the SiLU kernel also at 17 to 64 rows.  Measured at 32
+# rows (kernel after kernel, launch gaps included): 2 x 12,288 x 4,096 (201 MB) 49 us here against 49 + 5 us there,
+# 2 x 25,600 x 5,120 (524 MB) 125 us here against 96 + 5 us there; the plain products are faster here at every size
+# (5,120 x 25,600: 57 us against 147).
+MID_DUAL_MAX_BYTES = 256 << 20
+MID_PRODUCTS = os.environ.get("INFERRS_AMD_MID_PRODUCTS", "own")      # "own" or "library"
+
+
+class Partials:
+    """A product [rows, features] as the 32-bit sums of each split of k, `parts` [splits, rows, features]; whoever
+    needs it adds them up in the order of the splits (`materialize()`, or `add_rmsnorm_partials`)."""
+    __slots__ = ("parts",)
+
+    def __init__(self, parts: torch.Tensor):
+        self.parts = parts
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+    def materialize(self) -> torch.Tensor:
+        splits, m, n = self.parts.shape
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=self.parts.device)
+        _check(library().ia_sum_partials(_p(out), _p(self.parts), splits, m, n, _stream()))
+        return out
+
+
+def mid_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    if MID_PRODUCTS not in ("own", "library"):
+        raise KernelError(f"INFERRS_AMD_MID_PRODUCTS / ops.MID_PRODUCTS: 'own' or 'library', not {MID_PRODUCTS!r}")
+    return (MID_PRODUCTS == "own" and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and SKINNY_MAX_ROWS < x.shape[0] <= MID_MAX_ROWS and x.shape[1] % 128 == 0 and w.shape[1] == x.shape[1]
+            and x.is_contiguous() and w.is_contiguous() and (x.data_ptr() | w.data_ptr()) % 16 == 0)
+
+
+def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, dual: bool = False,
+                  partial: bool = False):
+    """x [m, k] . w[n, k]^T for 1 to 64 bfloat16 rows and k a multiple of 128 (gemm_mid.hip).  `dual`: w = [gate; up],
+    the result silu(x . gate^T) * (x . up^T).  `partial`: the result stays split along k, as `Partials` (a weight that
+    needs no split gives a plain tensor)."""
+    _dev(x, w)
+    m, k = x.shape
+    rows, k2 = w.shape
+    if (k2 != k or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or k % 128 or not (1 <= m <= MID_MAX_ROWS)
+            or (dual and (rows % 2 or partial or out_dtype != torch.bfloat16))):
+        raise KernelError(f"gemm_mid: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype} "
+                          f"(1 to {MID_MAX_ROWS} rows, k a multiple of 128)")
+    n = rows // 2 if dual else rows
+    lib = library()
+    if partial:
+        splits = lib.ia_gemm_mid_splits(n, k)
+        if splits > 1 and (m * n) % 4 == 0:
+            parts = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            _check(lib.ia_gemm_mid_bf16(_p(parts), _p(x), _p(w), m, n, k, 2, 0, _stream()))
+            return Partials(parts)
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _check(lib.ia_gemm_mid_bf16(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
+                                int(dual), _stream()))
+    return out
+
+
+def linear_partials(x: torch.Tensor, w: torch.Tensor):
+    """x . w^T for a reader that takes `Partials` (the norm that adds the product to the stream): split along k where the
+    weight has few rows.  None when the product of 17 to 64 rows does not take these operands."""
+    if isinstance(x, torch.Tensor) and mid_fits(x, w):
+        return gemm_mid_bf16(x, w, partial=True)
+    return None
+
+
+def add_rmsnorm_partials(x: torch.Tensor, delta: Partials, w: torch.Tensor, eps: float, add_one: bool = False) -> torch.Tensor:
+    """x += delta in place, delta's splits added up and rounded to bfloat16 first (as a stored product would be);
+    returns rmsnorm(x)."""
+    parts = delta.parts
+    _dev(x, parts, w); _f32(w, "norm weight")
+    splits, rows, cols = parts.shape
+    if x.dtype != torch.bfloat16 or tuple(x.shape) != (rows, cols) or w.numel() != cols:
+        raise KernelError(f"add_rmsnorm_partials: x {tuple(x.shape)} {x.dtype} does not fit the product {tuple(parts.shape)}")
+    if cols % 4 or cols > 8192:
+        return add_rmsnorm(x, delta.materialize(), w, eps, add_one)
+    out = torch.empty_like(x)
+    _check(library().ia_add_rmsnorm_partials(_p(out), _p(x), _p(parts), splits, _p(w), ctypes.c_float(eps), rows, cols,
+                                             int(add_one), _stream()))
+    return out
+
+
 def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
     skinny MFMA kernel for up to SKINNY_MAX_ROWS rows, the vendor's GEMM beyond that (the reference uses
@@ -654,6 +746,11 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch
         return gemm_tiled(x, w, out_dtype)
     if m <= SKINNY_MAX_ROWS:
         return gemm_skinny_bf16(x, w, out_dtype)
+    if mid_fits(x, w):
+        if out_dtype == torch.float32:
+            return gemm_mid_bf16(x, w, torch.float32)
+        y = gemm_mid_bf16(x, w, partial=True)
+        return y.materialize() if isinstance(y, Partials) else y
     _dev(x, w)
     if w.shape[1] != k or w.dtype != x.dtype:
         raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
@@ -761,6 +858,9 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
         x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
         return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True)
+    if (w_gate_up.shape[0] % 2 == 0 and mid_fits(x, w_gate_up)
+            and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES):
+        return gemm_mid_bf16(x, w_gate_up, dual=True)
     if w_gate_up.shape[0] % 2 == 0 and x.dtype == torch.bfloat16 and skinny_fits(x, w_gate_up) and _own_large(x, w_gate_up):
         return gemm_mfma_bf16(x, w_gate_up, dual=True)
     return silu_mul(linear(x, w_gate_up))

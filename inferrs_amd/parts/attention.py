@@ -78,6 +78,10 @@ class Attention(Mixer):
             added = ops.linear_add(a, self.o.weight, ctx.stream, norm)
             if added is not None:
                 return ops.Added(added[0], added[1], norm)
+        if getattr(ctx, "partial_sums", False):
+            split = ops.linear_partials(a, self.o.weight)
+            if split is not None:
+                return split
         return self.o(a)
 
     def forward(self, ctx, h, cache):

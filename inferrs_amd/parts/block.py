@@ -76,6 +76,9 @@ class Block(BlockBase):
         # and a part that says `takes_normed_rows` may get `ops.NormedRows` made of these, whose norm its
         # first product finishes.
         few = x.dtype == torch.bfloat16 and 0 < x.shape[0] <= ops.STREAM_MAX_ROWS
+        # Steps of 17 to 64 bfloat16 rows: a part's last product may stay split along k (`ops.Partials`); the norm
+        # that adds it to the stream adds the splits up on the way (`normed` below, or whoever reads `pending`).
+        ctx.partial_sums = x.dtype == torch.bfloat16 and ops.SKINNY_MAX_ROWS < x.shape[0] <= ops.MID_MAX_ROWS
         h = normed(self.norm_mixer, x, pending, few and getattr(self.mixer, "takes_normed_rows", False))
         ctx.stream = x if few and getattr(self.mixer, "adds_to_stream", False) else None
         ctx.stream_norm = self.norm_ffn if getattr(self.ffn, "takes_normed_rows", False) else None
@@ -85,22 +88,30 @@ class Block(BlockBase):
         ctx.stream_norm = next_norm
         out = self.ffn.forward(ctx, h2)
         ctx.stream = ctx.stream_norm = None
+        ctx.partial_sums = False
         return x, out
 
 
 def settle(x: torch.Tensor, pending) -> torch.Tensor:
     """The stream with `pending` added (in place): for arrangements and model ends that do not begin with a norm."""
+    if isinstance(pending, ops.Partials):
+        pending = pending.materialize()
     if pending is not None and not isinstance(pending, ops.Added):
         ops.add_inplace(x, pending)
     return x
 
 
 def normed(norm, x: torch.Tensor, pending, lazy: bool = False):
-    """norm(x + pending), the sum left in x; `pending` None: nothing to add; `ops.Added`: x holds the sum
+    """norm(x + pending), the sum left in x; `pending` None: nothing to add; `ops.Partials`: a product still split along k, added
+    up by the norm's kernel (or here, for a norm that has none for it); `ops.Added`: x holds the sum
     already, and with `lazy` the norm is left to the product that reads the rows, if the part that added
     them has prepared them for this norm."""
     if pending is None:
         return norm.forward(x)
+    if isinstance(pending, ops.Partials):
+        if hasattr(norm, "add_forward_partials"):
+            return norm.add_forward_partials(x, pending)
+        pending = pending.materialize()
     if isinstance(pending, ops.Added):
         if lazy and pending.scaled is not None and pending.norm is norm and hasattr(norm, "rows_for_product"):
             return norm.rows_for_product(x, pending)

@@ -41,4 +41,8 @@ class GatedMlp(FeedForward):
             added = ops.linear_add(act, self.down.weight, ctx.stream, norm)
             if added is not None:
                 return ops.Added(added[0], added[1], norm)
+        if getattr(ctx, "partial_sums", False):
+            split = ops.linear_partials(act, self.down.weight)
+            if split is not None:
+                return split
         return self.down(act)

@@ -33,6 +33,10 @@ class RMSNorm(Norm):
     def add_forward(self, x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, self.add_one)
 
+    def add_forward_partials(self, x: torch.Tensor, delta: "ops.Partials") -> torch.Tensor:
+        """`add_forward` for a product that is still split along k."""
+        return ops.add_rmsnorm_partials(x, delta, self.weight, self.eps, self.add_one)
+
     def rows_for_product(self, x: torch.Tensor, added: "ops.Added") -> ops.NormedRows:
         """The norm of a stream's rows left to the product that reads them: `added` holds the rows times
         this norm's weight and their sums of squares."""

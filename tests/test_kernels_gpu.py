@@ -644,3 +644,102 @@ def test_attention_decode_fused_is_the_three_kernels_in_one(nq, nkv, d, page, wi
             # keys: the same but for a last bit here and there (the sum of squares is added up in another order)
             dk = (k2.float() - k1.float()).abs()
             assert float(dk.max()) <= 2 ** -7 * float(k1.float().abs().max()) and float((dk > 0).float().mean()) < 1e-3
+
+
+# ---- products of 17 to 64 rows (gemm_mid.hip) -----------------------------------------------------------------
+
+@pytest.mark.parametrize("m", [1, 17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("n,k", [(64, 128), (80, 256), (200, 896), (4096, 1024), (6144, 4096), (77, 3 * 128)])
+def test_mid_product(m, n, k):
+    """Every number of rows up to 64 (row tiles that are partly empty), feature counts that are no multiple of the
+    block's 64 or of 4, k ranges of one chunk, of fewer chunks than the pipeline is deep and of many; plain, in 32-bit,
+    and split along k."""
+    from inferrs_amd import ops
+    x = randn(m, k, dtype=torch.bfloat16, seed=m)
+    w = randn(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.05)
+    want = x.float() @ w.float().t()
+    close(ops.gemm_mid_bf16(dev(x), dev(w)), want, 2 ** -8, "mid product")
+    close(ops.gemm_mid_bf16(dev(x), dev(w), torch.float32), want, 2e-6 * math.sqrt(k), "mid product, 32-bit result")
+    split = ops.gemm_mid_bf16(dev(x), dev(w), partial=True)
+    if isinstance(split, ops.Partials):
+        assert split.parts.shape[0] == ops.library().ia_gemm_mid_splits(n, k) > 1
+        close(split.parts.sum(0), want, 2e-6 * math.sqrt(k), "the splits' sums")
+        close(split.materialize(), want, 2 ** -8, "sum of the splits")
+    else:
+        assert ops.library().ia_gemm_mid_splits(n, k) == 1 or (m * n) % 4
+
+
+def test_mid_product_splits_depend_on_the_weight_alone():
+    from inferrs_amd import ops
+    lib = ops.library()
+    assert lib.ia_gemm_mid_splits(4096, 4096) > 1 and lib.ia_gemm_mid_splits(151936, 4096) == 1
+    assert lib.ia_gemm_mid_splits(4096, 100) == 0                    # k that is no multiple of 128 is not taken
+    for n, k in ((4096, 4096), (4096, 12288), (6144, 4096), (5120, 25600)):
+        s = lib.ia_gemm_mid_splits(n, k)
+        assert k % (128 * s) == 0 and k // s >= 512
+
+
+@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("n,k", [(32, 128), (50, 256), (1408, 1024)])
+def test_mid_product_with_the_activation_inside(m, n, k):
+    from inferrs_amd import ops
+    x = randn(m, k, dtype=torch.bfloat16, seed=3 * m)
+    w = randn(2 * n, k, dtype=torch.bfloat16, seed=n, scale=0.08)
+    gate = (x.float() @ w[:n].float().t()).bfloat16().float()
+    up = (x.float() @ w[n:].float().t()).bfloat16().float()
+    want = gate / (1 + torch.exp(-gate)) * up
+    close(ops.gemm_mid_bf16(dev(x), dev(w), dual=True), want, 2 ** -7, "mid product with SiLU")
+    close(ops.gated_silu_linear(dev(x), dev(w)), want, 2 ** -7, "gated_silu_linear")
+
+
+def test_mid_product_rows_do_not_depend_on_the_batch():
+    """A row's result is bit for bit the same whatever else is in the step: alone in a tile, among 64 rows, at another
+    place among them."""
+    from inferrs_amd import ops
+    k, n = 1024, 4096
+    x = randn(64, k, dtype=torch.bfloat16, seed=8)
+    w = dev(randn(n, k, dtype=torch.bfloat16, seed=9, scale=0.05))
+    whole = ops.gemm_mid_bf16(dev(x), w).cpu()
+    for rows in ([5], list(range(17)), [63, 0, 31, 32], list(range(20, 53))):
+        part = ops.gemm_mid_bf16(dev(x[rows].contiguous()), w).cpu()
+        assert torch.equal(part, whole[rows]), rows
+    split = ops.gemm_mid_bf16(dev(x), w, partial=True)
+    assert isinstance(split, ops.Partials)
+    again = ops.gemm_mid_bf16(dev(x[10:40].contiguous()), w, partial=True)
+    assert torch.equal(again.parts.cpu(), split.parts[:, 10:40].cpu())
+
+
+@pytest.mark.parametrize("cols,add_one", [(128, False), (4096, False), (5120, True), (8192, False)])
+def test_add_rmsnorm_of_a_split_product(cols, add_one):
+    """The norm kernel that adds up a product's splits equals the plain add-and-norm kernel on the stored product."""
+    from inferrs_amd import ops
+    rows, splits = 37, 4
+    x = randn(rows, cols, dtype=torch.bfloat16, seed=1, scale=2.0)
+    parts = randn(splits, rows, cols, dtype=torch.float32, seed=2)
+    w = randn(cols, dtype=torch.float32, seed=3)
+    stored = ops.Partials(dev(parts)).materialize()
+    assert torch.equal(stored.cpu(), parts.sum(0).bfloat16()) or float((stored.cpu().float() - parts.sum(0)).abs().max()) < 0.05
+    x1, x2 = dev(x.clone()), dev(x.clone())
+    want = ops.add_rmsnorm(x1, stored, dev(w), 1e-5, add_one)
+    got = ops.add_rmsnorm_partials(x2, ops.Partials(dev(parts)), dev(w), 1e-5, add_one)
+    assert torch.equal(x1.cpu(), x2.cpu())
+    close(got, want, 2 ** -8, "add_rmsnorm_partials")
+
+
+def test_mid_product_is_the_same_for_every_pipeline_shape():
+    """Chunks of 4, 8 or 16 k steps and 2 to 4 of them in shared memory change when a value arrives, never the order of a
+    sum: the results are bit for bit the same."""
+    from inferrs_amd import ops
+    lib = ops.library()
+    x = dev(randn(50, 2048, dtype=torch.bfloat16, seed=1))
+    w = dev(randn(200, 2048, dtype=torch.bfloat16, seed=2, scale=0.05))
+    wd = dev(randn(2 * 96, 2048, dtype=torch.bfloat16, seed=3, scale=0.05))
+    try:
+        outs = []
+        for kc, ns in ((4, 3), (4, 4), (8, 3), (8, 2), (16, 2)):
+            lib.ia_gemm_mid_tune(kc, ns)
+            outs.append((ops.gemm_mid_bf16(x, w).cpu(), ops.gemm_mid_bf16(x, wd, dual=True).cpu()))
+    finally:
+        lib.ia_gemm_mid_tune(4, 3)
+    assert all(torch.equal(a, outs[0][0]) and torch.equal(b, outs[0][1]) for a, b in outs[1:])
+    close(outs[0][0], x.float().cpu() @ w.float().cpu().t(), 2 ** -8, "mid product")

@@ -39,8 +39,8 @@ TOL_PLAIN_F32 = 1e-5
 TOL_CROSS_F32 = 1e-6
 SHARP = {"float32": 2.0, "bfloat16": 1.5}
 # (configuration, sharpened or not)
-CASES = [("A", False), ("B", False), ("C", False), ("D", False), ("E", False), ("F", False), ("A", True), ("B", True),
-         ("D", True)]
+CASES = [("A", False), ("B", False), ("C", False), ("D", False), ("E", False), ("F", False), ("G", False), ("A", True),
+         ("B", True), ("D", True), ("G", True)]
 
 
 @pytest.fixture(scope="module")

@@ -41,8 +41,15 @@ TINY_F = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size
               head_dim=24, rope_theta=50000.0, rms_norm_eps=1e-5, tie_word_embeddings=True,
               max_position_embeddings=512, hidden_act="silu")
 
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16, "E": 16, "F": 8}
+# Widths in steps of 128 (what the products of 17 to 64 rows take) at the serving head size: steps of that many
+# rows run those kernels, and the two products of 1,024 inputs are split along k and added up by the norm after them.
+TINY_G = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=300, hidden_size=256,
+              intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2,
+              head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+              max_position_embeddings=1024, hidden_act="silu")
+
+TINY = {"G": TINY_G, "A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
+PAGE_SIZE = {"G": 16, "A": 4, "B": 8, "C": 16, "D": 16, "E": 16, "F": 8}
 
 
 def write_model(folder: str, raw: dict, seed: int, dtype=torch.bfloat16, sharpen: float = 1.0) -> str:
