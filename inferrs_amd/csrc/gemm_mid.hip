@@ -248,7 +248,8 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
 }
 
 // How many ways k is split between blocks: a function of the weight's shape and the chip alone.  64 rows of w a
-// block; splits double until there are three blocks for every two compute units or a split would fall below 512 k.
+// block; splits double until there is a block for every compute unit or a split would fall below 512 k (with three blocks
+// for every two units a decode step of 32 requests took 2.71 ms where it takes 2.61 now: the splits' sums are traffic too).
 static int mid_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -260,12 +261,16 @@ static int mid_cus() {
     return cus;
 }
 
+// blocks wanted before k stops being split, in halves of the number of compute units
+static int g_mid_split_target = 2;
+extern "C" void ia_gemm_mid_split_target(int halves) { g_mid_split_target = halves; }
+
 extern "C" int ia_gemm_mid_splits(int N, int K) {
     if (N <= 0 || K <= 0 || K % MID_CHUNK_MIN_K) return 0;
     const int blocks = (N + 63) / 64;
     const int chunks = K / MID_CHUNK_MIN_K;
     int splits = 1;
-    while (2 * blocks * splits < 3 * mid_cus() && splits < 16 && chunks % (2 * splits) == 0 && chunks / (2 * splits) >= 4)
+    while (2 * blocks * splits < g_mid_split_target * mid_cus() && splits < 16 && chunks % (2 * splits) == 0 && chunks / (2 * splits) >= 4)
         splits *= 2;
     return splits;
 }
@@ -360,11 +365,13 @@ extern "C" int ia_sum_partials(void* out, const float* part, int splits, int M, 
 }
 
 // x[row] += the product (the splits' sums added up in their order and rounded to bfloat16, as a product that is stored
-// would be), the sum formed in 32-bit and rounded; out[row] = rmsnorm(x[row]) * w.  One block a row, the row kept in
-// registers between the two passes.  The same arithmetic as the add-and-norm kernel of elementwise.hip on a stored product.
-#define APN_THREADS 256
-#define APN_MAX_PER_THREAD 8             // rows of up to 256 * 4 * 8 = 8192 features
-__global__ __launch_bounds__(APN_THREADS) void add_rmsnorm_partials_kernel(
+// would be), the sum formed in 32-bit and rounded; out[row] = rmsnorm(x[row]) * w.  One block a row, a thread four
+// neighbouring features at a time, all its splits' loads under way together; the row stays in registers between the
+// two passes.  The same arithmetic as the add-and-norm kernel of elementwise.hip on a stored product.
+#define APN_MAX_THREADS 1024
+#define APN_MAX_PER_THREAD 2             // rows of up to 1024 * 4 * 2 = 8192 features
+template <int SPLITS>                    // 0: any number, walked one by one
+__global__ __launch_bounds__(APN_MAX_THREADS) void add_rmsnorm_partials_kernel(
     bf16_t* __restrict__ out, bf16_t* __restrict__ x, const float* __restrict__ part, int splits, size_t mn,
     const float* __restrict__ w, float eps, int cols, int add_one) {
     __shared__ float scratch[16];
@@ -373,13 +380,23 @@ __global__ __launch_bounds__(APN_THREADS) void add_rmsnorm_partials_kernel(
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < APN_MAX_PER_THREAD; ++j) {
-        const int c = (j * APN_THREADS + threadIdx.x) * 4;
+        const int c = (j * (int)blockDim.x + (int)threadIdx.x) * 4;
         if (c >= cols) break;
         const size_t at = row * cols + c;
-        float4 s = *(const float4*)(part + at);
-        for (int k = 1; k < splits; ++k) {
-            const float4 o = *(const float4*)(part + (size_t)k * mn + at);
-            s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+        float4 s;
+        if constexpr (SPLITS > 0) {
+            float4 p[SPLITS];
+#pragma unroll
+            for (int k = 0; k < SPLITS; ++k) p[k] = *(const float4*)(part + (size_t)k * mn + at);
+            s = p[0];
+#pragma unroll
+            for (int k = 1; k < SPLITS; ++k) { s.x += p[k].x; s.y += p[k].y; s.z += p[k].z; s.w += p[k].w; }
+        } else {
+            s = *(const float4*)(part + at);
+            for (int k = 1; k < splits; ++k) {
+                const float4 o = *(const float4*)(part + (size_t)k * mn + at);
+                s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+            }
         }
         const uint2 old = *(const uint2*)(x + at);
         const float sv[4] = {s.x, s.y, s.z, s.w};
@@ -398,7 +415,7 @@ __global__ __launch_bounds__(APN_THREADS) void add_rmsnorm_partials_kernel(
     const float scale = 1.0f / sqrtf(total / (float)cols + eps);
 #pragma unroll
     for (int j = 0; j < APN_MAX_PER_THREAD; ++j) {
-        const int c = (j * APN_THREADS + threadIdx.x) * 4;
+        const int c = (j * (int)blockDim.x + (int)threadIdx.x) * 4;
         if (c >= cols) break;
         const float4 g4 = *(const float4*)(w + c);
         const float gw[4] = {g4.x, g4.y, g4.z, g4.w};
@@ -412,13 +429,23 @@ __global__ __launch_bounds__(APN_THREADS) void add_rmsnorm_partials_kernel(
 extern "C" int ia_add_rmsnorm_partials(void* out, void* x, const float* part, int splits, const float* w, float eps,
                                        int rows, int cols, int add_one, hipStream_t stream) {
     IA_CHECK(rows >= 0 && cols > 0 && splits >= 1, "add_rmsnorm_partials: bad sizes rows=%d cols=%d splits=%d", rows, cols, splits);
-    IA_CHECK(cols % 4 == 0 && cols <= APN_THREADS * 4 * APN_MAX_PER_THREAD,
-             "add_rmsnorm_partials: rows of %d features: takes multiples of 4 up to %d", cols, APN_THREADS * 4 * APN_MAX_PER_THREAD);
+    IA_CHECK(cols % 4 == 0 && cols <= APN_MAX_THREADS * 4 * APN_MAX_PER_THREAD,
+             "add_rmsnorm_partials: rows of %d features: takes multiples of 4 up to %d", cols, APN_MAX_THREADS * 4 * APN_MAX_PER_THREAD);
     IA_CHECK((((uintptr_t)out | (uintptr_t)x | (uintptr_t)part | (uintptr_t)w) & 15) == 0,
              "add_rmsnorm_partials: arrays must be 16-byte aligned");
     if (rows == 0) return 0;
-    add_rmsnorm_partials_kernel<<<rows, APN_THREADS, 0, stream>>>((bf16_t*)out, (bf16_t*)x, part, splits, (size_t)rows * cols,
-                                                                  w, eps, cols, add_one);
+    // as many threads as the row has groups of four features, in whole waves, up to 1,024
+    int threads = ((cols / 4 + IA_WAVE - 1) / IA_WAVE) * IA_WAVE;
+    threads = threads > APN_MAX_THREADS ? APN_MAX_THREADS : threads;
+    bf16_t* o = (bf16_t*)out;
+    bf16_t* xs = (bf16_t*)x;
+    const size_t mn = (size_t)rows * cols;
+#define APN_LAUNCH(S) add_rmsnorm_partials_kernel<S><<<rows, threads, 0, stream>>>(o, xs, part, splits, mn, w, eps, cols, add_one)
+    if (splits == 2) APN_LAUNCH(2);
+    else if (splits == 4) APN_LAUNCH(4);
+    else if (splits == 8) APN_LAUNCH(8);
+    else APN_LAUNCH(0);
+#undef APN_LAUNCH
     IA_LAUNCH_CHECK("add_rmsnorm_partials");
     return 0;
 }

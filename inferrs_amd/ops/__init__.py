@@ -75,7 +75,8 @@ class _Timed:
     def __getattr__(self, name):
         fn = getattr(self._lib, name)
         if KernelTimer.active is None or not name.startswith("ia_") or name.endswith(("_workspace", "_blocks", "_block_rows",
-                                                                                      "_error", "_version", "_capacity", "_top")):
+                                                                                      "_error", "_version", "_capacity", "_top",
+                                                                                      "_splits", "_tune", "_target")):
             return fn
         timer = KernelTimer.active
         return lambda *args: timer.call(name[3:], fn, *args)
