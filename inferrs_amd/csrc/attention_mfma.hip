@@ -26,6 +26,8 @@
 // 32-key step assign key k0 + 8G + 4t + i to row 4G+i of tile t, so that lane (col, G) ends
 // up holding the probabilities of keys k0+8G .. k0+8G+7 in order: exactly the B operand of the
 // second product.
+#include <type_traits>
+
 #include "common.h"
 #include "api.h"
 
@@ -534,15 +536,23 @@ __device__ __forceinline__ float column_sum(float x) {
 // loads costs nothing (they have arrived).  Two waves a SIMD leave the phases of a step (operands from
 // shared memory, first product, softmax, second product) mostly one after the other.
 #define TILE_WAVES 4
-#define TILE_COLS (TILE_WAVES * 32)
 #define TILE_STAGE 64
 #define TILE_K_BYTES (TILE_STAGE * HD * 2)
 #define TILE_BUF_BYTES (2 * TILE_K_BYTES)
 
+// Two column tiles of 16 a wave, two blocks a compute unit, two waves a SIMD.  (Four tiles a wave, so that every key and
+// value read out of shared memory serves twice as many products, take the registers of a whole SIMD; with the softmax of
+// one tile laid beside the products of the others in the instruction stream that ran at 530 TFLOP/s on a prompt of
+// 8,192 tokens where two waves a SIMD run at 730, and the rescaling of accumulators that live in the matrix cores' own
+// registers cost as much again.)
+#define TILE_NBW 2
 template <bool ENABLED = (HD == 128)>
 __global__ __launch_bounds__(TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_tile_kernel(const AttnParams p) {
     if constexpr (ENABLED) {
+        constexpr int NBW = TILE_NBW;
+        constexpr int WAVE_COLS = 16 * NBW;
+        constexpr int TILE_COLS = TILE_WAVES * WAVE_COLS;
         // Two stages, as two arrays: the compiler then knows that the loads on their way into one do not
         // touch the other, and does not wait for them before it reads an operand.
         __shared__ __align__(16) char stage_a[TILE_BUF_BYTES];
@@ -580,12 +590,12 @@ void attn_tile_kernel(const AttnParams p) {
         const int stages = hi > lo ? (hi - lo + TILE_STAGE - 1) / TILE_STAGE : 0;
 
         // this wave's columns (a wave without any still brings its share of the stages)
-        const int col0 = bcol0 + wave * 32;
+        const int col0 = bcol0 + wave * WAVE_COLS;
         const bool has_cols = col0 < n_cols;
-        int tq[2], head[2], pos[2];
-        bool cvalid[2];
+        int tq[NBW], head[NBW], pos[NBW];
+        bool cvalid[NBW];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NBW; ++nb) {
             const int c = col0 + nb * 16 + r;
             cvalid[nb] = c < n_cols;
             const int cc = cvalid[nb] ? c : n_cols - 1;
@@ -593,21 +603,21 @@ void attn_tile_kernel(const AttnParams p) {
             head[nb] = kvh * g + (cc - tq[nb] * g);
             pos[nb] = kv_start + tq[nb];
         }
-        const int wlast = (col0 + 32 <= n_cols ? col0 + 32 : n_cols) - 1;
+        const int wlast = (col0 + WAVE_COLS <= n_cols ? col0 + WAVE_COLS : n_cols) - 1;
         const int pmin = kv_start + (has_cols ? col0 : 0) / g, pmax = has_cols ? kv_start + wlast / g : -1;
         const int wlo = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;
 
-        uint4 qreg[2][KS];
+        uint4 qreg[NBW][KS];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NBW; ++nb) {
             const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) qreg[nb][ks] = cvalid[nb] ? *(const uint4*)(qrow + ks * 32 + G * 8) : zero4();
         }
-        f32x4 acc[2][DB];
-        float m[2], l[2];
+        f32x4 acc[NBW][DB];
+        float m[NBW], l[NBW];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NBW; ++nb) {
             m[nb] = -INFINITY;
             l[nb] = 0.f;
 #pragma unroll
@@ -711,82 +721,121 @@ void attn_tile_kernel(const AttnParams p) {
             };
             if (live[0]) read_keys(0);
             else if (live[1]) read_keys(1);
+            // A step of 32 keys.  The wave's two column tiles take turns so that the softmax of one (vector
+            // arithmetic) has matrix products of the other beside it in the same stretch of code: the scores of
+            // tile 1 beside the softmax of tile 0, the second product of tile 0 beside the softmax of tile 1.  The
+            // order of every sum is as before.  EDGE: some key of the step is masked for some column.
+            auto scores = [&](int nb, f32x4 (&sacc)[2]) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, kop[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), sacc[t], 0, 0, 0);
+                }
+            };
+            auto softmax = [&](auto edge_c, int nb, int k0, const f32x4 (&sacc)[2], uint4& pb, float& alpha) {
+                constexpr bool EDGE = decltype(edge_c)::value;
+                float sc[8];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sc[4 * t + i] = sacc[t][i];
+                if constexpr (EDGE) {
+                    const int kbase_idx = k0 + 8 * G;
+                    const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int key = kbase_idx + j;
+                        if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
+                    }
+                }
+                float mx = max2(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], max3(sc[5], sc[6], sc[7])));
+                mx = column_max(mx);
+                // The exponents' reference point moves only when the step's maximum has passed it by 2^8
+                // (probabilities then reach 2^8 at most, which 32-bit sums and bfloat16 operands hold as
+                // well as 1): the accumulators are rescaled a few times a walk instead of at most steps.
+                const float cand = mx * p.scale_log2;
+                const bool rise = cand > m[nb] + 8.0f;              // also the first finite maximum after -inf
+                const float m_new = rise ? cand : m[nb];
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                alpha = rise ? __builtin_amdgcn_exp2f(m[nb] - m_use) : 1.0f;
+                float pr[8], psum = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], p.scale_log2, -m_use));
+                    psum += pr[j];
+                }
+                l[nb] = l[nb] * alpha + psum;
+                m[nb] = m_new;
+                pb.x = pack_bf16x2(pr[0], pr[1]);
+                pb.y = pack_bf16x2(pr[2], pr[3]);
+                pb.z = pack_bf16x2(pr[4], pr[5]);
+                pb.w = pack_bf16x2(pr[6], pr[7]);
+            };
+            auto rescale = [&](int nb, float alpha) {
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        acc[nb][db][0] *= alpha; acc[nb][db][1] *= alpha;
+                        acc[nb][db][2] *= alpha; acc[nb][db][3] *= alpha;
+                    }
+                }
+            };
+            auto weighted = [&](int nb, const uint4 (&vop)[DB], const uint4& pb) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, vop[db]), __builtin_bit_cast(bf16x8, pb), acc[nb][db], 0, 0, 0);
+            };
+            // eight matrix products with a share of the vector instructions after each
+            auto beside = [&]() {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix product
+                    __builtin_amdgcn_sched_group_barrier(0x002, 9, 0);      // nine vector instructions
+                }
+            };
+            auto pin = [&](uint4& pb, float& alpha) {
+                // (pins the probabilities to the stretch of code they are formed in: left alone, the compiler moves
+                // their arithmetic behind the branch of the rescaling, next to the product that uses them)
+                asm volatile("" : "+v"(pb.x), "+v"(pb.y), "+v"(pb.z), "+v"(pb.w), "+v"(alpha));
+            };
+            auto step = [&](auto edge_c, int u) {
+                const int k0 = kb + 32 * u;
+                uint4 vop[DB];
+                f32x4 s0[2], s1[2];
+                uint4 pb0, pb1;
+                float alpha0, alpha1;
+                scores(0, s0);
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HD * 2) + db * 512 + v_at);
+                __builtin_amdgcn_sched_barrier(0);
+                scores(1, s1);
+                softmax(edge_c, 0, k0, s0, pb0, alpha0);
+                pin(pb0, alpha0);
+                beside();
+                __builtin_amdgcn_sched_barrier(0);
+                if (u == 0) read_keys(1);               // (a step that this wave skips: read all the same, used by nobody)
+                rescale(0, alpha0);
+                __builtin_amdgcn_sched_barrier(0);
+                weighted(0, vop, pb0);
+                softmax(edge_c, 1, k0, s1, pb1, alpha1);
+                pin(pb1, alpha1);
+                beside();
+                __builtin_amdgcn_sched_barrier(0);
+                rescale(1, alpha1);
+                weighted(1, vop, pb1);
+            };
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 if (!live[u]) continue;
                 const int k0 = kb + 32 * u;
                 const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
-                f32x4 sacc[2][2];
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        sacc[nb][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int ks = 0; ks < KS; ++ks)
-                            sacc[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                                __builtin_bit_cast(bf16x8, kop[t][ks]), __builtin_bit_cast(bf16x8, qreg[nb][ks]), sacc[nb][t], 0, 0, 0);
-                    }
-                uint4 vop[DB];
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HD * 2) + db * 512 + v_at);
-                __builtin_amdgcn_sched_barrier(0);
-                uint4 pb[2];
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
-                    float sc[8];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) sc[4 * t + i] = sacc[nb][t][i];
-                    if (edge) {
-                        const int kbase_idx = k0 + 8 * G;
-                        const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const int key = kbase_idx + j;
-                            if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
-                        }
-                    }
-                    float mx = max2(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], max3(sc[5], sc[6], sc[7])));
-                    mx = column_max(mx);
-                    // The exponents' reference point moves only when the step's maximum has passed it by 2^8
-                    // (probabilities then reach 2^8 at most, which 32-bit sums and bfloat16 operands hold as
-                    // well as 1): the accumulators are rescaled a few times a walk instead of at most steps.
-                    const float cand = mx * p.scale_log2;
-                    const bool rise = cand > m[nb] + 8.0f;              // also the first finite maximum after -inf
-                    const float m_new = rise ? cand : m[nb];
-                    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                    const float alpha = rise ? __builtin_amdgcn_exp2f(m[nb] - m_use) : 1.0f;
-                    float pr[8], psum = 0.f;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], p.scale_log2, -m_use));
-                        psum += pr[j];
-                    }
-                    l[nb] = l[nb] * alpha + psum;
-                    m[nb] = m_new;
-                    pb[nb].x = pack_bf16x2(pr[0], pr[1]);
-                    pb[nb].y = pack_bf16x2(pr[2], pr[3]);
-                    pb[nb].z = pack_bf16x2(pr[4], pr[5]);
-                    pb[nb].w = pack_bf16x2(pr[6], pr[7]);
-                    if (__any(alpha != 1.0f)) {
-#pragma unroll
-                        for (int db = 0; db < DB; ++db) {
-                            acc[nb][db][0] *= alpha; acc[nb][db][1] *= alpha;
-                            acc[nb][db][2] *= alpha; acc[nb][db][3] *= alpha;
-                        }
-                    }
-                }
-                if (u == 0 && live[1]) read_keys(1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-#pragma unroll
-                    for (int nb = 0; nb < 2; ++nb)
-                        acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8, vop[db]), __builtin_bit_cast(bf16x8, pb[nb]), acc[nb][db], 0, 0, 0);
+                if (edge) step(std::true_type(), u);
+                else step(std::false_type(), u);
             }
         };
         if (stages > 0) {
@@ -799,7 +848,7 @@ void attn_tile_kernel(const AttnParams p) {
             if (s + 1 < stages) stage(s + 1, stage_b, stage_a);
         }
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NBW; ++nb) {
             const float lt = column_sum(l[nb]);
             if (!cvalid[nb]) continue;
             const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
@@ -1012,9 +1061,10 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         // 16 columns a wave, whatever the number of query heads of a key/value head
         const dim3 fgrid((unsigned)((cols + 15) / 16), nkv * splits, n_seqs);
         attn_mfma_fused_kernel<><<<fgrid, IA_WAVE, 0, stream>>>(p);
-    } else if (HD == 128 && g_tiles && cols >= TILE_COLS && (splits == 1 || chunk % TILE_STAGE == 0)) {
+    } else if (HD == 128 && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
-        const dim3 tgrid((unsigned)((cols + TILE_COLS - 1) / TILE_COLS), nkv * splits, n_seqs);
+        const int tile_cols = 16 * TILE_NBW * TILE_WAVES;
+        const dim3 tgrid((unsigned)((cols + tile_cols - 1) / tile_cols), nkv * splits, n_seqs);
         static int cus = 0;
         if (cus == 0) {
             int dev = 0;

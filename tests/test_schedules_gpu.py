@@ -100,10 +100,23 @@ def test_runs_of_decode_steps_across_a_bucket_boundary(tiny, dtype):
             assert eng.graph_replays > 40
         eng.cache.check_invariants()
         assert not eng.cache.sequences
-    assert results["runs"] == results["single"]
-    if dtype == "float32":
-        assert results["runs"] == results["eager"]
     assert all(len(o) == 60 for o in results["runs"])
+    if dtype == "float32":
+        assert results["runs"] == results["single"] == results["eager"]
+        return
+    # bfloat16: a run that would end beyond the boundary is not queued, so near the boundary the two ways take the
+    # old bucket's graph for different steps, and a graph of a wider bucket may split the keys between waves in
+    # another way: rounding.  Where the tokens part, the two choices' logits are as close as that (in 32-bit).
+    from inferrs_amd.engine import Entry
+    exact = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=70, max_seqs=1, use_graphs=False)
+    for prompt, a, b in zip(prompts, results["runs"], results["single"]):
+        if a == b:
+            continue
+        i = next(j for j in range(60) if a[j] != b[j])
+        row = exact.step([Entry("x", prompt + a[:i], [len(prompt) + i - 1])])[0]
+        exact.end_request("x")
+        assert abs(float(row[a[i]] - row[b[i]])) < 0.02, f"token {i}: {a[i]} against {b[i]}, logits {float(row[a[i]])} and {float(row[b[i]])}"
+        assert float(row.max() - max(row[a[i]], row[b[i]])) < 0.02
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
