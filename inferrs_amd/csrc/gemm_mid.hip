@@ -42,8 +42,10 @@ typedef float gmid_f32x4 __attribute__((ext_vector_type(4)));
 enum { MID_OUT_BF16 = 0, MID_OUT_F32 = 1, MID_OUT_PARTIAL = 2 };
 
 // KC: k steps of 32 in a chunk (a row of x in a chunk is KC * 64 bytes); NS: chunks of x in shared memory, this one and
-// NS - 1 on their way.
-template <int MT, bool DUAL, int KC, int NS>
+// NS - 1 on their way.  KH: the waves of a block share k between them KH ways (1 or 2): with 2 a block owns half as many
+// rows of w (two tiles of 16, each walked by two waves over one half of k, their sums added through shared memory in a
+// fixed order), which makes twice as many blocks for the chip to balance.
+template <int MT, bool DUAL, int KC, int NS, int KH>
 __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
     void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     int M, int N, int K, int k_per_block) {
@@ -51,11 +53,13 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
     constexpr int ROW_BYTES = KC * 64;                      // bytes of a row of x in a chunk
     constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;         // rows that one load instruction (1 KiB) fills
     constexpr int PIECES = KC * 4;                          // 16-byte pieces of a row
-    constexpr int X_LOADS = MT * 16 / ROWS_PER_LOAD / MID_WAVES;   // load instructions of x a wave issues for a chunk
-    constexpr int STAGE_BYTES = MT * 16 * ROW_BYTES;
-    static_assert(NS >= 2 && NS <= 4 && (KC == 4 || KC == 8 || KC == 16), "pipeline shape");
-    static_assert(MT * 16 / ROWS_PER_LOAD % MID_WAVES == 0, "the rows of a chunk are shared out evenly between the waves");
-    // A stage [MT * 16 rows][ROW_BYTES] an array: the compiler then knows that loads on their way into one stage do
+    constexpr int TILES = MID_WAVES / KH;                   // tiles of 16 rows of w a block
+    constexpr int X_LOADS = MT * 16 / ROWS_PER_LOAD / TILES;       // load instructions of x a wave issues for a chunk
+    constexpr int HALF_BYTES = MT * 16 * ROW_BYTES;         // a chunk's rows of x for one share of k
+    constexpr int STAGE_BYTES = KH * HALF_BYTES;
+    static_assert(NS >= 2 && NS <= 4 && (KC == 4 || KC == 8 || KC == 16) && (KH == 1 || KH == 2), "pipeline shape");
+    static_assert(MT * 16 / ROWS_PER_LOAD % TILES == 0, "the rows of a chunk are shared out evenly between the waves");
+    // A stage [KH][MT * 16 rows][ROW_BYTES] an array: the compiler then knows that loads on their way into one stage do
     // not touch the others, and does not wait for them before it reads operands out of this one.
     __shared__ __attribute__((aligned(1024))) char mid_s0[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char mid_s1[STAGE_BYTES];
@@ -71,39 +75,42 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
     const int lane = threadIdx.x & (IA_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / IA_WAVE);
     const int r = lane & 15, g = lane >> 4;
+    const int tile = wave % TILES, kh = wave / TILES;
     const int split = blockIdx.y;
-    const int k_begin = split * k_per_block;
-    const int k_len = K - k_begin < k_per_block ? K - k_begin : k_per_block;
+    // the block's range of k, and this wave's share of it (whole chunks; the launcher sees to it that they divide)
+    const int kb_begin = split * k_per_block;
+    const int kb_len = K - kb_begin < k_per_block ? K - kb_begin : k_per_block;
+    const int k_len = kb_len / KH;
+    const int k_begin = kb_begin + kh * k_len;
     const int nchunks = k_len / CHUNK_K;
 
     // ---- this wave's 16 rows of w --------------------------------------------------------------------------
     // (rows beyond the matrix read its last row: their sums are never stored)
-    int n_first;                 // output feature of the tile's first row
+    // DUAL: half of a block's tiles are gate rows, the other half the up rows of the same features
+    constexpr int FEATURE_TILES = DUAL ? TILES / 2 : TILES;
+    const int part = DUAL ? tile / FEATURE_TILES : 0;                  // 0: gate (or a plain weight), 1: up
+    const int n_first = blockIdx.x * (16 * FEATURE_TILES) + 16 * (tile % FEATURE_TILES);   // output feature of the tile's first row
     const bf16_t* wrow;
-    if (DUAL) {
-        n_first = blockIdx.x * 32 + 16 * (wave & 1);
+    {
         const int n = n_first + r < N ? n_first + r : N - 1;
-        wrow = w + ((size_t)(wave >> 1) * N + n) * K + k_begin + g * 8;
-    } else {
-        n_first = blockIdx.x * 64 + 16 * wave;
-        const int n = n_first + r < N ? n_first + r : N - 1;
-        wrow = w + (size_t)n * K + k_begin + g * 8;
+        wrow = w + ((size_t)part * N + n) * K + k_begin + g * 8;
     }
 
     // ---- what this lane fetches of a chunk of x: X_LOADS instructions, each ROWS_PER_LOAD whole rows ------------
-    // instruction i of wave v covers rows ROWS_PER_LOAD * (4 i + v) .. ; lane l writes place l % PIECES of row l / PIECES
-    // of them, and fetches the piece that belongs there: piece c of row r lies at place c ^ (r % 16)
+    // The waves that share a range of k bring its rows together: instruction i of tile t covers rows ROWS_PER_LOAD *
+    // (TILES i + t) .. ; lane l writes place l % PIECES of row l / PIECES of them, and fetches the piece that belongs
+    // there: piece c of row r lies at place c ^ (r % 16)
     const char* xsrc[X_LOADS];
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i) {
-        const int row = ROWS_PER_LOAD * (MID_WAVES * i + wave) + lane / PIECES;
+        const int row = ROWS_PER_LOAD * (TILES * i + tile) + lane / PIECES;
         const int piece = (lane % PIECES) ^ (row & 15);
         xsrc[i] = (const char*)(x + (size_t)(row < M ? row : 0) * K + k_begin) + piece * 16;
     }
     // and where it reads its B-operands: row 16 mt + r, piece 4 ks + g, at place (4 ks + g) ^ r
     uint32_t b_at[KC];
 #pragma unroll
-    for (int ks = 0; ks < KC; ++ks) b_at[ks] = (uint32_t)(r * ROW_BYTES + (((4 * ks + g) ^ r) * 16));
+    for (int ks = 0; ks < KC; ++ks) b_at[ks] = (uint32_t)(kh * HALF_BYTES + r * ROW_BYTES + (((4 * ks + g) ^ r) * 16));
 
     gmid_f32x4 acc[MT];
 #pragma unroll
@@ -115,12 +122,12 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
         // the weights first, then the rows of x: a wait for the rows of a chunk covers its weights too
 #pragma unroll
         for (int ks = 0; ks < KC; ++ks) wreg[S][ks] = *(const uint4*)(wrow + (size_t)c * CHUNK_K + ks * 32);
-        char* stage = stage_of(stage_c);
+        char* stage = stage_of(stage_c) + kh * HALF_BYTES;
 #pragma unroll
         for (int i = 0; i < X_LOADS; ++i)
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)(xsrc[i] + (size_t)c * ROW_BYTES),
-                (void __attribute__((address_space(3)))*)(stage + (MID_WAVES * i + wave) * 1024), 16, 0, 0);
+                (void __attribute__((address_space(3)))*)(stage + (TILES * i + tile) * 1024), 16, 0, 0);
     };
     constexpr int PER_CHUNK = KC + X_LOADS;           // vector-memory instructions a wave issues for a chunk
     auto multiply = [&](auto stage_c) {
@@ -186,22 +193,39 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
     ring(tail_step, c + NS);
 
     // ---- results: lane (r, g) holds features n_first + 4 g + i of row 16 mt + r ---------------------------------
-    if (DUAL) {
-        // the up rows' sums go through shared memory to the waves that hold the gate rows' sums of the same features
-        __syncthreads();
-        gmid_f32x4* swap = (gmid_f32x4*)mid_s0;                           // [2 tiles][MT][64 lanes]
-        if (wave >= 2) {
+    // Sums meet in shared memory, in the stages' place: first the second share of k is added to the first, then (DUAL)
+    // the up rows' sums go to the waves that hold the gate rows' sums of the same features.
+    gmid_f32x4* swap_k = (gmid_f32x4*)mid_s0;                             // [TILES][MT][64 lanes]
+    gmid_f32x4* swap_up = (gmid_f32x4*)mid_s1;                            // [FEATURE_TILES][MT][64 lanes]
+    static_assert(TILES * MT * IA_WAVE * sizeof(gmid_f32x4) <= STAGE_BYTES, "the sums fit a stage");
+    if (KH == 2 || DUAL) __syncthreads();                                 // everybody is done with the stages
+    if constexpr (KH == 2) {
+        if (kh == 1) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) swap[((wave - 2) * MT + mt) * IA_WAVE + lane] = acc[mt];
+            for (int mt = 0; mt < MT; ++mt) swap_k[(tile * MT + mt) * IA_WAVE + lane] = acc[mt];
         }
         __syncthreads();
-        if (wave >= 2) return;
+        if (kh == 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const gmid_f32x4 o = swap_k[(tile * MT + mt) * IA_WAVE + lane];
+                acc[mt][0] += o[0]; acc[mt][1] += o[1]; acc[mt][2] += o[2]; acc[mt][3] += o[3];
+            }
+        }
+    }
+    if (DUAL) {
+        if (kh == 0 && part == 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) swap_up[((tile % FEATURE_TILES) * MT + mt) * IA_WAVE + lane] = acc[mt];
+        }
+        __syncthreads();
+        if (kh != 0 || part != 0) return;
         const int nb = n_first + 4 * g;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r;
             if (m >= M) continue;
-            const gmid_f32x4 up = swap[(wave * MT + mt) * IA_WAVE + lane];
+            const gmid_f32x4 up = swap_up[(tile * MT + mt) * IA_WAVE + lane];
             float v[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -220,6 +244,7 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
         }
         return;
     }
+    if (kh != 0) return;
     const int nb = n_first + 4 * g;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -275,29 +300,37 @@ extern "C" int ia_gemm_mid_splits(int N, int K) {
     return splits;
 }
 
-// Tuning: k steps of a chunk (4, 8 or 16) and chunks in shared memory (2 to 4).  Measured at the sizes of an 8 B and a
-// 32 B model, 32 and 64 rows: all within a tenth of each other; (4, 3) is the default (the smallest stages, so that most
-// blocks fit a compute unit).
-static int g_mid_kc = 4, g_mid_ns = 3;
-extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns; }
+// Tuning: k steps of a chunk (4 or 8), chunks in shared memory (2 to 4), and the share of k among a block's waves for
+// weights with the activation inside (1 or 2).  Measured at the sizes of an 8 B and a 32 B model, 32 and 64 rows: the
+// chunk shapes are within a tenth of each other; (4, 3) is the default (the smallest stages, so that most blocks fit a
+// compute unit).
+static int g_mid_kc = 4, g_mid_ns = 3, g_mid_dual_kh = 2;
+extern "C" void ia_gemm_mid_tune(int kc, int ns, int dual_kh) { g_mid_kc = kc; g_mid_ns = ns; g_mid_dual_kh = dual_kh; }
 
-template <int MT, bool DUAL, int KC, int NS>
+template <int MT, bool DUAL, int KC, int NS, int KH>
 static void launch_mid_shape(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
                              hipStream_t stream) {
-    const dim3 grid(DUAL ? (N + 31) / 32 : (N + 63) / 64, splits);
-    gemm_mid_kernel<MT, DUAL, KC, NS><<<grid, MID_WAVES * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, K / splits);
+    constexpr int FEATURES = 16 * (MID_WAVES / KH) / (DUAL ? 2 : 1);        // output features of a block
+    const dim3 grid((N + FEATURES - 1) / FEATURES, splits);
+    gemm_mid_kernel<MT, DUAL, KC, NS, KH><<<grid, MID_WAVES * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, K / splits);
 }
 
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
                       hipStream_t stream) {
     const int k_block = K / splits;
-    // (a chunk must divide a block's share of k, and a stage of MT * 16 rows must leave room in shared memory)
-    if (g_mid_kc == 16 && g_mid_ns == 2 && k_block % 512 == 0) launch_mid_shape<MT, DUAL, 16, 2>(out, out_mode, x, w, M, N, K, splits, stream);
-    else if (g_mid_kc == 8 && g_mid_ns == 3 && k_block % 256 == 0) launch_mid_shape<MT, DUAL, 8, 3>(out, out_mode, x, w, M, N, K, splits, stream);
-    else if (g_mid_kc == 8 && g_mid_ns == 2 && k_block % 256 == 0) launch_mid_shape<MT, DUAL, 8, 2>(out, out_mode, x, w, M, N, K, splits, stream);
-    else if (g_mid_kc == 4 && g_mid_ns == 4) launch_mid_shape<MT, DUAL, 4, 4>(out, out_mode, x, w, M, N, K, splits, stream);
-    else launch_mid_shape<MT, DUAL, 4, 3>(out, out_mode, x, w, M, N, K, splits, stream);
+    // (a chunk must divide a wave's share of k, and a stage of MT * 16 rows must leave room in shared memory)
+    if constexpr (DUAL) {
+        // (two ways up to 32 rows: 2 x 12,288 x 4,096 at 20 rows 48.9 -> 42.4 us, at 32 rows 48.5 -> 46.6; beyond, twice as
+        // many blocks fetching all the rows of x cost more than the balance gains: 64 rows 56 -> 67 us)
+        if (g_mid_dual_kh == 2 && MT <= 2 && k_block % 256 == 0) {
+            launch_mid_shape<MT, true, 4, 3, 2>(out, out_mode, x, w, M, N, K, splits, stream);
+            return 0;
+        }
+    }
+    if (g_mid_kc == 8 && g_mid_ns == 2 && k_block % 256 == 0) launch_mid_shape<MT, DUAL, 8, 2, 1>(out, out_mode, x, w, M, N, K, splits, stream);
+    else if (g_mid_kc == 4 && g_mid_ns == 4) launch_mid_shape<MT, DUAL, 4, 4, 1>(out, out_mode, x, w, M, N, K, splits, stream);
+    else launch_mid_shape<MT, DUAL, 4, 3, 1>(out, out_mode, x, w, M, N, K, splits, stream);
     return 0;
 }
 
