@@ -367,33 +367,33 @@ extern "C" int ia_rope_table(float* cos_out, float* sin_out, const int* position
 }
 
 // ---- a pure streaming read: the measured roof of this GPU's memory for the measurement script ----------------
-// Every thread reads 16-byte pieces a whole grid apart, four under way at a time, and folds them into one word; a
-// block leaves one word, so that nothing of the read can be dropped.  Nothing of the engine calls it.
-__global__ __launch_bounds__(256) void stream_read_kernel(unsigned* __restrict__ out, const uint4* __restrict__ x, size_t n16) {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+// A block owns a contiguous range; its threads read 16-byte pieces a block's width apart, four under way at a time, and
+// fold them into one word (kept by a condition that the data never meets, so that nothing of the read can be dropped).
+// Nothing of the engine calls it.  (Measured over 8 GB: 6.3 to 6.5 TB/s with 16 k to 64 k blocks; pieces a whole grid
+// apart: 5.5 to 6.3.)
+__global__ __launch_bounds__(512) void stream_read_kernel(unsigned* __restrict__ out, const uint4* __restrict__ x, size_t n16) {
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t begin = per * blockIdx.x;
+    const size_t end = begin + per < n16 ? begin + per : n16;
     unsigned acc = 0;
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        const uint4 a = x[i], b = x[i + stride], c = x[i + 2 * stride], d = x[i + 3 * stride];
+    size_t i = begin + threadIdx.x;
+    for (; i + 3 * (size_t)blockDim.x < end; i += 4 * (size_t)blockDim.x) {
+        const uint4 a = x[i], b = x[i + blockDim.x], c = x[i + 2 * (size_t)blockDim.x], d = x[i + 3 * (size_t)blockDim.x];
         acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
     }
-    for (; i < n16; i += stride) {
+    for (; i < end; i += blockDim.x) {
         const uint4 a = x[i];
         acc ^= a.x ^ a.y ^ a.z ^ a.w;
     }
-#pragma unroll
-    for (int o = IA_WAVE / 2; o > 0; o >>= 1) acc ^= __shfl_xor(acc, o, IA_WAVE);
-    __shared__ unsigned part[4];
-    if ((threadIdx.x & (IA_WAVE - 1)) == 0) part[threadIdx.x / IA_WAVE] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) out[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
+    if (acc == 0x9e3779b9u) out[blockIdx.x] = acc;
 }
 
-// out: `blocks` words; x: `bytes` bytes, 16-byte aligned, a multiple of 16.
+// out: `blocks` words (written only where a block's fold happens to equal a constant); x: `bytes` bytes, 16-byte aligned,
+// a multiple of 16.
 extern "C" int ia_stream_read(unsigned* out, const void* x, long long bytes, int blocks, hipStream_t stream) {
     IA_CHECK(bytes >= 0 && bytes % 16 == 0 && blocks > 0 && blocks <= 1048576, "stream_read: bad sizes bytes=%lld blocks=%d", bytes, blocks);
     IA_CHECK((((uintptr_t)x) & 15) == 0, "stream_read: x must be 16-byte aligned");
-    stream_read_kernel<<<blocks, 256, 0, stream>>>(out, (const uint4*)x, (size_t)bytes / 16);
+    stream_read_kernel<<<blocks, 512, 0, stream>>>(out, (const uint4*)x, (size_t)bytes / 16);
     IA_LAUNCH_CHECK("stream_read");
     return 0;
 }

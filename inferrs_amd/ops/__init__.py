@@ -534,11 +534,11 @@ def fill_normal(shape, seed: int, mean: float, std: float, dtype: torch.dtype, d
 
 
 def stream_read(x: torch.Tensor, blocks: int = 4096) -> torch.Tensor:
-    """Reads all of `x` once (a multiple of 16 bytes) and returns one word a block: the measurement script times it
-    for the memory's practical read rate."""
+    """Reads all of `x` once (a multiple of 16 bytes), a contiguous range a block: the measurement script times it for
+    the memory's practical read rate.  (The returned words are scratch.)"""
     _dev(x)
     nbytes = x.numel() * x.element_size()
-    out = torch.empty((blocks,), dtype=torch.int32, device=x.device)
+    out = torch.zeros((blocks,), dtype=torch.int32, device=x.device)
     _check(library().ia_stream_read(_p(out), _p(x), ctypes.c_longlong(nbytes), blocks, _stream()))
     return out
 
