@@ -110,6 +110,21 @@ int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_
                       int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                       int nq, int nkv, int d, int page_size, int window, float scale,
                       int splits, int chunk, hipStream_t stream);
+// Decode steps (one token a request, head sizes in steps of 64): per-head norm, rotation, cache write, attention
+// and the merge of the key splits in one kernel.  `workspace` holds ia_attention_decode_workspace() floats;
+// `counters` holds at least ia_attention_decode_counters() 32-bit words that are zero before the call and zero
+// again after it (calls that share them must not overlap).
+int ia_attention_mfma_has_fused(void);
+long long ia_attention_decode_workspace(int n, int nq, int nkv, int splits);
+long long ia_attention_decode_counters(int n, int nq, int nkv, int splits);
+int ia_attention_mfma_decode_fused(void* out, float* workspace, const void* qkv, void* k_cache,
+                                   void* v_cache, const int* block_table, const int* cu_tokens,
+                                   const int* positions, const int* slots, const float* q_norm_w,
+                                   const float* k_norm_w, const float* cos_t, const float* sin_t,
+                                   float eps, int add_one, int n, int seq_begin, int n_seqs,
+                                   int token_begin, int n_tokens, int max_kv_len, int max_pages,
+                                   int nq, int nkv, int d, int page_size, int window, float scale,
+                                   int splits, int chunk, int* counters, int n_counters, hipStream_t stream);
 
 #ifdef __cplusplus
 }

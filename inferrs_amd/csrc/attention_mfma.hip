@@ -2,11 +2,12 @@
 // (IA_HEAD_DIM, a multiple of 16 up to 256).  One kernel serves prefill and decode: a wave
 // owns up to 16 * NB columns, a column being one (query token, query head) pair of one
 // request and one key/value head, and walks that request's keys 32 at a time straight from
-// the cache pages into MFMA operands.  Decode batches (one token a request) have few
-// columns and long key ranges, so the keys are split between waves and the partial results
-// are merged by a second kernel.  At head size 128, steps with 128 columns or more of a request
-// (portions of prompts) go to a second kernel, blocks of four waves that share keys and values
-// through shared memory (attn_tile_kernel).
+// the cache pages into MFMA operands.  Where a step has few columns and long key ranges, the
+// keys are split between waves and the partial results are merged by a second kernel.  Decode
+// steps (one token a request) at head sizes in steps of 64 have a kernel of their own with the
+// per-head norm, the rotation, the cache write and that merge inside (attn_decode_kernel).  At
+// head size 128, steps with 128 columns or more of a request (portions of prompts) go to blocks
+// of four waves that share keys and values through shared memory (attn_tile_kernel).
 //
 // Formula as in the reference: S = (q . k) * scale after the product, keys j <= position
 // (inferrs-models/src/models/attention_utils.rs:61-85), softmax over keys, O = P v
@@ -56,8 +57,9 @@ struct AttnParams {
     const int* cu_tokens;       // [seqs + 1]  request s owns tokens cu[s]..cu[s+1]
     const int* positions;       // [n]         absolute position of each token
     int max_pages, nq, nkv, page, window, splits, chunk, pair, seq_begin;   // pair: see the kernels
+    int token_begin;            // decode kernel: request seq_begin + i owns token token_begin + i
     float scale_log2;           // scale * log2(e)
-    // Decode steps with the per-head norm, the rotation and the cache write inside (FUSE): q is not
+    // The decode kernel, with the per-head norm, the rotation and the cache write inside: q is not
     // read from `q` but formed from the projections' output, and the wave that walks a request's
     // newest key forms that key and value, uses them and writes them to the cache.
     const bf16_t* qkv;          // [n, (nq + 2 nkv) * d]: q heads, then k heads, then v heads
@@ -73,9 +75,8 @@ struct AttnParams {
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
 // One column block (16 * NB columns) of one request and key/value head, over one split of the keys.
-template <int NB, bool FUSE = false>
+template <int NB>
 __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, int kvh, int split, int seq) {
-    static_assert(!FUSE || (NB == 1 && HD % 64 == 0), "the fused form is for single tokens and head sizes in steps of 64");
     const int lane = threadIdx.x;
     const int r = lane & 15, G = lane >> 4;
     const int g = p.nq / p.nkv;
@@ -102,74 +103,15 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
     const int last_col = (col0 + 16 * NB <= n_cols ? col0 + 16 * NB : n_cols) - 1;
     const int pmin = kv_start + col0 / g, pmax = kv_start + last_col / g;
 
-    // FUSE: one head's row of the projections' output, normed and rotated as the separate kernel does
-    // it (32-bit throughout, one rounding at the end): lane (., G) holds the features ks * 32 + G * 8 ..
-    // + 8 of the row, and a feature's rotation partner, HD / 2 further on, lies in the same lane.
-    const int qkv_row = (p.nq + 2 * p.nkv) * HD;
-    auto normed_rotated = [&](const bf16_t* row, const float* norm_w, uint4 (&packed)[KS]) {
-        float f[KS][8];
-        float ss = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const uint4 raw = *(const uint4*)(row + ks * 32 + G * 8);
-            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                f[ks][2 * j] = __uint_as_float(w[j] << 16);
-                f[ks][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) ss += f[ks][j] * f[ks][j];
-        }
-        if (norm_w != nullptr) {
-            ss += __shfl_xor(ss, 16, IA_WAVE);
-            ss += __shfl_xor(ss, 32, IA_WAVE);
-            const float scale = 1.0f / sqrtf(ss / (float)HD + p.norm_eps);
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const float4 g0 = *(const float4*)(norm_w + ks * 32 + G * 8), g1 = *(const float4*)(norm_w + ks * 32 + G * 8 + 4);
-                const float gw[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) f[ks][j] = scale * f[ks][j] * (p.norm_add_one ? 1.0f + gw[j] : gw[j]);
-            }
-        }
-        if (p.cos_t != nullptr) {
-#pragma unroll
-            for (int ks = 0; ks < KS / 2; ++ks) {
-                // this token's angles for the lane's features of the first half
-                const size_t at = (size_t)t0 * (HD / 2) + ks * 32 + G * 8;
-                const float4 c0 = *(const float4*)(p.cos_t + at), c1 = *(const float4*)(p.cos_t + at + 4);
-                const float4 s0 = *(const float4*)(p.sin_t + at), s1 = *(const float4*)(p.sin_t + at + 4);
-                const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-                const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float a = f[ks][j], b = f[ks + KS / 2][j];
-                    f[ks][j] = a * c[j] - b * sn[j];
-                    f[ks + KS / 2][j] = a * sn[j] + b * c[j];
-                }
-            }
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-            packed[ks] = make_uint4(pack_bf16x2(f[ks][0], f[ks][1]), pack_bf16x2(f[ks][2], f[ks][3]),
-                                    pack_bf16x2(f[ks][4], f[ks][5]), pack_bf16x2(f[ks][6], f[ks][7]));
-    };
-
     // Q^T operands stay in registers for the whole walk.
     uint4 qreg[NB][KS];
-    if constexpr (FUSE) {
-        // every lane forms a row (invalid columns their request's last head: never stored)
-        normed_rotated(p.qkv + (size_t)t0 * qkv_row + (size_t)head[0] * HD, p.q_norm_w, qreg[0]);
-    } else {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
+    for (int nb = 0; nb < NB; ++nb) {
+        const bf16_t* qrow = p.q + ((size_t)(t0 + tq[nb]) * p.nq + head[nb]) * HD;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int dim = ks * 32 + G * 8;
-                qreg[nb][ks] = (cvalid[nb] && dim < HD) ? *(const uint4*)(qrow + dim) : zero4();
-            }
+        for (int ks = 0; ks < KS; ++ks) {
+            const int dim = ks * 32 + G * 8;
+            qreg[nb][ks] = (cvalid[nb] && dim < HD) ? *(const uint4*)(qrow + dim) : zero4();
         }
     }
 
@@ -372,50 +314,10 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
     //   v_permlane swaps instead of shared memory, late and early column blocks as separate waves
     //   instead of one after the other in a wave: within 1 % each.
     // - Addresses without a division in the step (above): 1 % at 2,048 tokens.
-    // - Decode steps, fused form: the first step's keys and values asked for before the query rows are normed and
-    //   rotated (the waves all start together and the memory stands idle meanwhile) needs both sets of registers at
-    //   once: 256 and spills, a batch-8 step 5.5 -> 6.3 ms.
     Place at = {lo / p.page, lo % p.page};
     for (int k0 = lo; k0 < hi; k0 += 32) {
         Operands op;
         load_step(op, k0, at);
-        if constexpr (FUSE) {
-            // The step that holds the request's newest key (position kv_total - 1, this step's token): its
-            // slot of the cache is not written yet.  The key and value are formed here, put into the
-            // operands in place of what the loads brought, and written to the cache for the steps to come.
-            const int kk = kv_total - 1 - k0;
-            if (p.slots != nullptr && kk >= 0 && kk < 32) {
-                const int slot = p.slots[t0];
-                const int page = slot / p.page, off = slot - page * p.page;
-                uint4 knew[KS];
-                normed_rotated(p.qkv + (size_t)t0 * qkv_row + (size_t)(p.nq + kvh) * HD, p.k_norm_w, knew);
-                const int r_new = ((kk >> 3) << 2) | (kk & 3), t_new = (kk >> 2) & 1;
-                if (r == r_new) {
-                    bf16_t* krow = p.k_cache_w + (((size_t)page * p.nkv + kvh) * p.page + off) * HD + G * 8;
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-                        if (t_new == 0) op.k[0][ks] = knew[ks]; else op.k[1][ks] = knew[ks];
-                        *(uint4*)(krow + ks * 32) = knew[ks];
-                    }
-                }
-                if (G == (kk >> 3)) {
-                    const bf16_t* vrow = p.qkv + (size_t)t0 * qkv_row + (size_t)(p.nq + p.nkv + kvh) * HD + r;
-                    bf16_t* vdst = p.v_cache_w + (((size_t)page * p.nkv + kvh) * HD + r) * p.page + off;
-                    const int j = kk & 7;
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) {
-                        const uint32_t bits = vrow[db * 16].bits;
-                        vdst[(size_t)db * 16 * p.page].bits = (uint16_t)bits;
-                        uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
-                        const uint32_t keep = (j & 1) ? 0x0000ffffu : 0xffff0000u;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (e == (j >> 1)) w[e] = (w[e] & keep) | ((j & 1) ? bits << 16 : bits);
-                        op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
-                    }
-                }
-            }
-        }
         compute_step(op, k0);
         advance(at, 32);
     }
@@ -473,17 +375,6 @@ void attn_mfma_kernel(const AttnParams p) {
     if (early != late) attn_column_block<NB>(p, early, kvh, split, seq);
 }
 
-// Decode steps (one token a request) with the per-head norm, the rotation and the cache write inside.
-template <bool ENABLED = (HD % 64 == 0)>
-__global__ __launch_bounds__(IA_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1, HD > 64 ? 2 : 8)))
-void attn_mfma_fused_kernel(const AttnParams p) {
-    if constexpr (ENABLED) {
-        const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
-        if ((int)blockIdx.x < (p.nq / p.nkv + 15) / 16)
-            attn_column_block<1, true>(p, (int)blockIdx.x, kvh, split, p.seq_begin + blockIdx.z);
-    }
-}
-
 // The maximum / the sum over the four lanes that hold a column's values (lanes l, l ^ 16, l ^ 32, l ^ 48), in all
 // of them, by swaps between rows of 16 lanes and between the halves of the wave: no trip through shared memory.
 // (the maximum instructions themselves, which return the other operand when one is a NaN: fmaxf() puts
@@ -513,6 +404,517 @@ __device__ __forceinline__ float column_sum(float x) {
     const uint32_t w = __float_as_uint(x);
     auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// ---- decode steps: one token a request, with the norm, the rotation, the cache write and the merge inside ------
+// A wave owns up to 16 query heads of one request and key/value head and one split of that request's keys, as
+// in the kernel above, but a decode step is short and every microsecond of it is latency, so the walk is laid
+// out for that:
+//  * the first step's keys and values are asked for before anything else: the query row is normed and rotated,
+//    and the request's new key and value are formed and written to the cache, while they are on their way;
+//  * a step's operands are asked for one step ahead (two sets of registers: a decode wave holds 16 columns and
+//    has the room), so a wave waits for the memory once, not once a step;
+//  * the waves of a block (`team`: 1, 2 or 4 neighbouring splits) add their results up in shared memory and
+//    leave one partial result a block; the block that finishes last for its (request, key/value head), known by
+//    a counter in memory, merges the blocks' partial results and writes the output.  No second kernel, and no
+//    wave reads another compute unit's results before they are there: every thread fences its stores before
+//    the block's one atomic increment, and the last block fences again before it reads.  The counters are zero
+//    between calls (the last block puts its counter back), so calls that share them must not overlap.
+// The sum over the splits runs in the order of the splits whoever comes last: the result is the same every time.
+// Measured (head size 128, 32 query and 8 key/value heads, context 8,192, time stamps inside the kernel): a wave
+// knows its token's position 0.8 us after it starts, has asked for the rows and the first keys at 2.5, has its rows
+// formed at 4.6 and its two steps done at 6.6 (batch 1, 64 keys a wave); the block's waves have met at 7.0, the
+// partial result is out at 7.5, the count back at 9.3 and the last block has merged at 13 to 16 us.  A fence of
+// device scope in place of the write-through stores cost 100 us a layer at batch 8 (it writes back and empties
+// the whole L2 of the die, once a block).  The kernel needs a SIMD's whole register file for a wave (two sets of
+// operands, and more in the rows' forming), so a compute unit holds one block: the step's split keeps its waves
+// within one round of the chip.  Against the kernel above with a merge kernel behind it, a layer, each at its
+// best split: batch 8 52.4 against 56.5 us, batch 3 26.0 against 29.0, batch 16 98.8 against 103, batch 32 189
+// against 195, batch 64 358 against 366; batch 8 at a context of 2,048 20.9 against 24.4, batch 64 at 1,024 49.0
+// against 56.7; batch 1 17 to 18 us both ways.
+// Partial results that blocks on other compute units read within the same kernel: written through to memory and
+// read past the caches that are not coherent between the chip's dies (32-bit accesses of device scope, no order
+// of their own), so that no cache has to be written back or emptied as a whole.
+__device__ __forceinline__ void put_across(float* at, float v) {
+    __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float get_across(const float* at) {
+    return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct DecodeOperands {
+    uint4 k[2][KS];             // as Operands above
+    uint4 v[DB];
+};
+
+template <bool ENABLED = (HD % 64 == 0)>
+__global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnParams p, int* counters, int team) {
+    if constexpr (ENABLED) {
+        extern __shared__ __align__(16) float team_mem[];       // [team][columns][HD] partial outputs, then [team][columns][2]
+        __shared__ int s_last;
+        // (the wave's number through a scalar register: what follows from it, the split's range and the pages' numbers,
+        // is then the same for all lanes by construction, and the block table is read through the scalar cache)
+        const int lane = threadIdx.x & (IA_WAVE - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / IA_WAVE);
+        const int r = lane & 15, G = lane >> 4;
+        const int g = p.nq / p.nkv;
+        const int teams = p.splits / team;
+        const int kvh = blockIdx.y / teams, tm = blockIdx.y - kvh * teams;
+        const int split = tm * team + wave;
+        const int seq = p.seq_begin + blockIdx.z;
+        const int col0 = blockIdx.x * 16;
+        const int n_cols = g - col0 < 16 ? g - col0 : 16;       // this block's columns (the grid has no empty block)
+        // What a wave needs before it can ask for its first keys is a chain of small reads, each a trip to the
+        // memory: the token's position, then the pages' numbers.  A decode step's token is known without a read
+        // (request seq_begin + i owns token token_begin + i), and where no window moves the walk's start the first
+        // two steps' pages are read from the block table at the same time as the position (entries past the
+        // request's last page are read but not used).
+        const int t0 = p.token_begin + (int)blockIdx.z;
+        const int* bt = p.block_table + (size_t)seq * p.max_pages;
+        const int c_lo = p.splits > 1 ? split * p.chunk : 0;
+        int early[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int idx = (c_lo + 16 * i) / p.page;
+            early[i] = bt[idx < p.max_pages ? idx : p.max_pages - 1];
+        }
+        const int kv_start = p.positions[t0];
+        const int kv_total = kv_start + 1;
+        const bool cvalid = r < n_cols;
+        const int head = kvh * g + col0 + (cvalid ? r : n_cols - 1);
+
+        const int window_floor = p.window > 0 ? (kv_start - p.window + 1 > 0 ? kv_start - p.window + 1 : 0) : 0;
+        int lo = window_floor > c_lo ? window_floor : c_lo, hi = kv_total;
+        if (p.splits > 1 && hi > c_lo + p.chunk) hi = c_lo + p.chunk;
+        lo &= ~31;
+
+        // ---- loads, in the order in which their results are needed ------------------------------------
+        // The rows of the projections' output that this wave norms and rotates (its query heads' rows and the new
+        // key's: every wave asks for it, one wave uses it), the norms' weights and the angles, then the first
+        // step's keys and values: the rows are formed while those are on their way, and the second step's are asked
+        // for after that (a wave can have 63 loads outstanding: all at once would stall the issue of the last ones
+        // until the first come back).
+        const int qkv_row = (p.nq + 2 * p.nkv) * HD;
+        const bf16_t* token_row = p.qkv + (size_t)t0 * qkv_row;
+        uint4 qraw[KS], kraw[KS];
+        uint32_t vnew[DB];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qraw[ks] = *(const uint4*)(token_row + (size_t)head * HD + ks * 32 + G * 8);
+            kraw[ks] = *(const uint4*)(token_row + (size_t)(p.nq + kvh) * HD + ks * 32 + G * 8);
+        }
+        // the norms' weights and the token's angles for this lane's features (a feature's rotation partner, HD / 2
+        // further on, lies in the same lane)
+        constexpr int HK = KS / 2 > 0 ? KS / 2 : 1;      // (head sizes without this kernel still parse it)
+        float4 qw[KS][2], kw[KS][2], cs[HK][2], sn[HK][2];
+        if (p.q_norm_w != nullptr) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    qw[ks][h] = *(const float4*)(p.q_norm_w + ks * 32 + G * 8 + 4 * h);
+                    kw[ks][h] = *(const float4*)(p.k_norm_w + ks * 32 + G * 8 + 4 * h);
+                }
+        }
+        if (p.cos_t != nullptr) {
+#pragma unroll
+            for (int ks = 0; ks < KS / 2; ++ks)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const size_t a0 = (size_t)t0 * (HD / 2) + ks * 32 + G * 8 + 4 * h;
+                    cs[ks][h] = *(const float4*)(p.cos_t + a0);
+                    sn[ks][h] = *(const float4*)(p.sin_t + a0);
+                }
+        }
+
+
+        // A step's 32 keys are two groups of 16 slots, each inside one page (page sizes are multiples of 16).
+        // Slots past the request's length are read like any others as long as their page is the request's (their
+        // scores are masked and their values zeroed in the step); pages past its last are not asked for.
+        const int last_idx = (kv_total - 1) / p.page;
+        const bool k_second = r >= 8, v_second = G >= 2;
+        const uint32_t k_lane[2] = {(uint32_t)((((8 * (r >> 2) + (r & 3)) & 15) * HD + G * 8) * 2),
+                                    (uint32_t)((((8 * (r >> 2) + 4 + (r & 3)) & 15) * HD + G * 8) * 2)};
+        const uint32_t v_lane = (uint32_t)((r * p.page + 8 * (G & 1)) * 2);
+        const size_t v_stride = (size_t)16 * p.page * 2;
+        auto load_pages = [&](DecodeOperands& op, int k0, int page_a, int page_b) __attribute__((always_inline)) {
+            const int off_a = k0 % p.page, off_b = (k0 + 16) % p.page;
+            const char* ka = (const char*)(p.k_cache + (((size_t)page_a * p.nkv + kvh) * p.page + off_a) * HD);
+            const char* kb = (const char*)(p.k_cache + (((size_t)page_b * p.nkv + kvh) * p.page + off_b) * HD);
+            const char* va = (const char*)(p.v_cache + ((size_t)page_a * p.nkv + kvh) * HD * p.page + off_a);
+            const char* vb = (const char*)(p.v_cache + ((size_t)page_b * p.nkv + kvh) * HD * p.page + off_b);
+            const char* kbase = k_second ? kb : ka;
+            const char* vbase = (v_second ? vb : va) + v_lane;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) op.k[t][ks] = *(const uint4*)(kbase + k_lane[t] + ks * 64);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) op.v[db] = *(const uint4*)(vbase + db * v_stride);
+        };
+        auto load_step = [&](DecodeOperands& op, int k0) __attribute__((always_inline)) {
+            int idx_a = k0 / p.page, idx_b = (k0 + 16) / p.page;
+            idx_a = idx_a < last_idx ? idx_a : last_idx;
+            idx_b = idx_b < last_idx ? idx_b : last_idx;
+            load_pages(op, k0, bt[idx_a], bt[idx_b]);
+        };
+        // the first two steps, with the pages read ahead where the walk starts at the split's own start
+        auto load_early = [&](DecodeOperands& op, int k0, int i) __attribute__((always_inline)) {
+            if (lo == c_lo && (k0 + 16) / p.page <= last_idx) load_pages(op, k0, early[2 * i], early[2 * i + 1]);
+            else load_step(op, k0);
+        };
+        const int n_steps = lo < hi ? (hi - lo + 31) / 32 : 0;
+        DecodeOperands opa, opb;
+        load_early(opa, lo, 0);
+
+        // One head's row, normed and rotated as the separate kernel does it (32-bit throughout, one rounding at
+        // the end): lane (., G) holds the features ks * 32 + G * 8 .. + 8 of the row, and a feature's rotation
+        // partner, HD / 2 further on, lies in the same lane.
+        auto normed_rotated = [&](const uint4 (&raw)[KS], const float4 (&nw)[KS][2], uint4 (&packed)[KS]) __attribute__((always_inline)) {
+            float f[KS][8];
+            float ss = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint32_t w[4] = {raw[ks].x, raw[ks].y, raw[ks].z, raw[ks].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    f[ks][2 * j] = __uint_as_float(w[j] << 16);
+                    f[ks][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ss += f[ks][j] * f[ks][j];
+            }
+            if (p.q_norm_w != nullptr) {
+                ss += __shfl_xor(ss, 16, IA_WAVE);
+                ss += __shfl_xor(ss, 32, IA_WAVE);
+                const float scale = 1.0f / sqrtf(ss / (float)HD + p.norm_eps);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const float gw[8] = {nw[ks][0].x, nw[ks][0].y, nw[ks][0].z, nw[ks][0].w,
+                                         nw[ks][1].x, nw[ks][1].y, nw[ks][1].z, nw[ks][1].w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[ks][j] = scale * f[ks][j] * (p.norm_add_one ? 1.0f + gw[j] : gw[j]);
+                }
+            }
+            if (p.cos_t != nullptr) {
+#pragma unroll
+                for (int ks = 0; ks < KS / 2; ++ks) {
+                    const float c[8] = {cs[ks][0].x, cs[ks][0].y, cs[ks][0].z, cs[ks][0].w,
+                                        cs[ks][1].x, cs[ks][1].y, cs[ks][1].z, cs[ks][1].w};
+                    const float sv[8] = {sn[ks][0].x, sn[ks][0].y, sn[ks][0].z, sn[ks][0].w,
+                                         sn[ks][1].x, sn[ks][1].y, sn[ks][1].z, sn[ks][1].w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float a = f[ks][j], b = f[ks + KS / 2][j];
+                        f[ks][j] = a * c[j] - b * sv[j];
+                        f[ks + KS / 2][j] = a * sv[j] + b * c[j];
+                    }
+                }
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                packed[ks] = make_uint4(pack_bf16x2(f[ks][0], f[ks][1]), pack_bf16x2(f[ks][2], f[ks][3]),
+                                        pack_bf16x2(f[ks][4], f[ks][5]), pack_bf16x2(f[ks][6], f[ks][7]));
+        };
+        uint4 qreg[KS], knew[KS];
+        normed_rotated(qraw, qw, qreg);
+        normed_rotated(kraw, kw, knew);
+        if (n_steps >= 2) load_early(opb, lo + 32, 1);
+
+        const bool has_new = p.slots != nullptr && hi == kv_total && lo < hi;
+
+        f32x4 acc[DB];
+        float m = -INFINITY, l = 0.f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+        auto compute_step = [&](DecodeOperands& op, int k0) __attribute__((always_inline)) {
+            if (k0 + 32 > kv_total) {
+                // slots beyond the request's length hold anything at all: zero those values so that a probability
+                // of zero times their content stays zero
+                const int first_bad = kv_total - (k0 + 8 * G);
+                if (first_bad < 8) {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            if (j >= first_bad) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                        op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                }
+            }
+            if (p.window > 0 && k0 < window_floor) {
+                // keys below the window may lie in pages that the request has given back: as above
+                const int first_good = window_floor - (k0 + 8 * G);
+                if (first_good > 0) {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            if (j < first_good) w[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                        op.v[db] = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                }
+            }
+            if (has_new && k0 + 32 >= kv_total) {
+                // (values chosen, never addresses: the operands stay in registers)
+                const int kk = kv_total - 1 - k0;
+                const bool mine = r == (((kk >> 3) << 2) | (kk & 3));
+                const bool first = mine && ((kk >> 2) & 1) == 0, second = mine && ((kk >> 2) & 1) == 1;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    op.k[0][ks].x = first ? knew[ks].x : op.k[0][ks].x; op.k[0][ks].y = first ? knew[ks].y : op.k[0][ks].y;
+                    op.k[0][ks].z = first ? knew[ks].z : op.k[0][ks].z; op.k[0][ks].w = first ? knew[ks].w : op.k[0][ks].w;
+                    op.k[1][ks].x = second ? knew[ks].x : op.k[1][ks].x; op.k[1][ks].y = second ? knew[ks].y : op.k[1][ks].y;
+                    op.k[1][ks].z = second ? knew[ks].z : op.k[1][ks].z; op.k[1][ks].w = second ? knew[ks].w : op.k[1][ks].w;
+                }
+                const int j = kk & 7;
+                const bool vmine = G == (kk >> 3);
+                const uint32_t keep = (j & 1) ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const uint32_t put = (j & 1) ? vnew[db] << 16 : vnew[db];
+                    op.v[db].x = vmine && (j >> 1) == 0 ? (op.v[db].x & keep) | put : op.v[db].x;
+                    op.v[db].y = vmine && (j >> 1) == 1 ? (op.v[db].y & keep) | put : op.v[db].y;
+                    op.v[db].z = vmine && (j >> 1) == 2 ? (op.v[db].z & keep) | put : op.v[db].z;
+                    op.v[db].w = vmine && (j >> 1) == 3 ? (op.v[db].w & keep) | put : op.v[db].w;
+                }
+            }
+            f32x4 s[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                s[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, op.k[t][ks]), __builtin_bit_cast(bf16x8, qreg[ks]), s[t], 0, 0, 0);
+            }
+            float sc[8];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sc[4 * t + i] = s[t][i];
+            if (k0 + 31 > kv_start || (p.window > 0 && k0 < window_floor)) {
+                const int kbase_idx = k0 + 8 * G;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int key = kbase_idx + j;
+                    if (key > kv_start || key < window_floor) sc[j] = -INFINITY;
+                }
+            }
+            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            mx = fmaxf(mx, __shfl_xor(mx, 16, IA_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, IA_WAVE));
+            const float m_new = fmaxf(m, mx * p.scale_log2);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+            float pr[8], psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], p.scale_log2, -m_use));
+                psum += pr[j];
+            }
+            l = l * alpha + psum;
+            m = m_new;
+            uint4 pb;
+            pb.x = pack_bf16x2(pr[0], pr[1]);
+            pb.y = pack_bf16x2(pr[2], pr[3]);
+            pb.z = pack_bf16x2(pr[4], pr[5]);
+            pb.w = pack_bf16x2(pr[6], pr[7]);
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    acc[db][0] *= alpha; acc[db][1] *= alpha;
+                    acc[db][2] *= alpha; acc[db][3] *= alpha;
+                }
+            }
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, op.v[db]), __builtin_bit_cast(bf16x8, pb), acc[db], 0, 0, 0);
+        };
+
+        // The walk: two steps' operands are under way at any time.  Inside the loop every step has a step two
+        // further on, so its loads are unconditional (the compiler counts what is outstanding and waits for the
+        // older set only); the last one to three steps follow it.  opa holds step k0, opb step k0 + 32.
+        int k0 = lo, left = n_steps;
+        while (left > 3) {
+            compute_step(opa, k0);
+            load_step(opa, k0 + 64);
+            compute_step(opb, k0 + 32);
+            load_step(opb, k0 + 96);
+            k0 += 64;
+            left -= 2;
+        }
+        if (left == 3) {
+            compute_step(opa, k0);
+            load_step(opa, k0 + 64);
+            compute_step(opb, k0 + 32);
+            k0 += 64;
+            left = 1;
+        }
+        // (the new value's features, for the wave that ends with the new key: asked for here, where they are needed)
+        if (has_new) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) vnew[db] = token_row[(size_t)(p.nq + p.nkv + kvh) * HD + db * 16 + r].bits;
+        }
+        if (left == 2) {
+            compute_step(opa, k0);
+            compute_step(opb, k0 + 32);
+        } else if (left == 1) {
+            compute_step(opa, k0);
+        }
+
+        // The request's newest key (position kv_total - 1, this step's token) is in no page yet: the wave whose
+        // keys end with it has put it and its value into its last step's operands in place of what the loads
+        // brought, and now writes them to the cache for the steps to come.  (After the walk: with no store before
+        // them, the block table's reads go through the scalar cache.)
+        if (has_new) {
+            const int slot = p.slots[t0];
+            const int page = slot / p.page, off = slot - page * p.page;
+            const int kk = (kv_total - 1) & 31;
+            if (r == (((kk >> 3) << 2) | (kk & 3))) {
+                bf16_t* krow = p.k_cache_w + (((size_t)page * p.nkv + kvh) * p.page + off) * HD + G * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) *(uint4*)(krow + ks * 32) = knew[ks];
+            }
+            if (G == (kk >> 3)) {
+                bf16_t* vdst = p.v_cache_w + (((size_t)page * p.nkv + kvh) * HD + r) * p.page + off;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) vdst[(size_t)db * 16 * p.page].bits = (uint16_t)vnew[db];
+            }
+        }
+
+        float lt = l;
+        lt += __shfl_xor(lt, 16, IA_WAVE);
+        lt += __shfl_xor(lt, 32, IA_WAVE);
+        const size_t row0 = (size_t)t0 * p.nq + kvh * g + col0;        // the block's first (token, head) row
+        if (p.splits == 1) {
+            if (!cvalid) return;
+            const float inv = 1.0f / lt;
+            bf16_t* o = p.out + (row0 + r) * HD + 4 * G;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                uint2 w;
+                w.x = pack_bf16x2(acc[db][0] * inv, acc[db][1] * inv);
+                w.y = pack_bf16x2(acc[db][2] * inv, acc[db][3] * inv);
+                *(uint2*)(o + 16 * db) = w;
+            }
+            return;
+        }
+
+        // ---- the block's waves add up: lane (col, G) holds dims 16 db + 4 G + i of its column --------
+        float* team_o = team_mem;                                       // [team][n_cols][HD]
+        float* team_ml = team_mem + (size_t)team * n_cols * HD;         // [team][n_cols][2]
+        if (cvalid) {
+            float* o = team_o + ((size_t)wave * n_cols + r) * HD + 4 * G;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) *(f32x4*)(o + 16 * db) = acc[db];
+            if (G == 0) {
+                team_ml[(wave * n_cols + r) * 2] = m;
+                team_ml[(wave * n_cols + r) * 2 + 1] = lt;
+            }
+        }
+        __syncthreads();
+        const int pieces = n_cols * (HD / 4);                           // 16-byte pieces of the block's result
+        for (int e = threadIdx.x; e < pieces; e += blockDim.x) {
+            const int col = e / (HD / 4), piece = e - col * (HD / 4);
+            float mx = -INFINITY;
+            for (int w = 0; w < team; ++w) mx = fmaxf(mx, team_ml[(w * n_cols + col) * 2]);
+            f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
+            float total = 0.f;
+            for (int w = 0; w < team; ++w) {
+                const float mw = team_ml[(w * n_cols + col) * 2];
+                const float wt = mw == -INFINITY ? 0.f : exp2f(mw - mx);      // a split that held no key of this row
+                const f32x4 v = *(const f32x4*)(team_o + ((size_t)w * n_cols + col) * HD + piece * 4);
+                o[0] = fmaf(v[0], wt, o[0]); o[1] = fmaf(v[1], wt, o[1]);
+                o[2] = fmaf(v[2], wt, o[2]); o[3] = fmaf(v[3], wt, o[3]);
+                total = fmaf(team_ml[(w * n_cols + col) * 2 + 1], wt, total);
+            }
+            if (teams == 1) {
+                const float inv = 1.0f / total;
+                uint2 w;
+                w.x = pack_bf16x2(o[0] * inv, o[1] * inv);
+                w.y = pack_bf16x2(o[2] * inv, o[3] * inv);
+                *(uint2*)(p.out + (row0 + col) * HD + piece * 4) = w;
+            } else {
+                float* po = p.part_o + ((row0 + col) * teams + tm) * HD + piece * 4;
+                put_across(po, o[0]); put_across(po + 1, o[1]); put_across(po + 2, o[2]); put_across(po + 3, o[3]);
+                if (piece == 0) {
+                    float* ml = p.part_ml + ((row0 + col) * teams + tm) * 2;
+                    put_across(ml, mx);
+                    put_across(ml + 1, total);
+                }
+            }
+        }
+        if (teams == 1) return;
+
+        // ---- the last block of this (request, key/value head, column block) merges the blocks' results --------
+        int* counter = counters + ((size_t)blockIdx.z * p.nkv + kvh) * gridDim.x + blockIdx.x;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");          // this thread's stores have arrived ...
+        __syncthreads();                                                // ... and every thread's, before the count
+        if (threadIdx.x == 0)
+            s_last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == teams - 1 ? 1 : 0;
+        __syncthreads();
+        if (!s_last) return;
+        // Every thread takes part: the block's threads form as many groups as there are 16-byte pieces of the result
+        // in them, group i sums the blocks i, i + groups, ... in that order, and the groups' sums meet in shared
+        // memory and are added in the groups' order.
+        const int groups = pieces <= (int)blockDim.x ? (int)blockDim.x / pieces : 1;
+        float* red = team_mem;                                          // [groups][pieces][6]: maximum, sum, four outputs
+        for (int e0 = 0; e0 < pieces; e0 += blockDim.x) {
+            const int grp = groups > 1 ? (int)threadIdx.x / pieces : 0;
+            const int e = groups > 1 ? (int)threadIdx.x - grp * pieces : e0 + (int)threadIdx.x;
+            const bool active = grp < groups && e < pieces;
+            float mx = -INFINITY, total = 0.f;
+            f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const int col = active ? e / (HD / 4) : 0, piece = active ? e - col * (HD / 4) : 0;
+            if (active) {
+                const float* ml = p.part_ml + (row0 + col) * teams * 2;
+                const float* po = p.part_o + (row0 + col) * teams * HD + piece * 4;
+#pragma unroll 8
+                for (int t = grp; t < teams; t += groups) {
+                    const float2 mt = make_float2(get_across(ml + 2 * t), get_across(ml + 2 * t + 1));
+                    const float* pv = po + (size_t)t * HD;
+                    const f32x4 v = (f32x4){get_across(pv), get_across(pv + 1), get_across(pv + 2), get_across(pv + 3)};
+                    const float m_new = fmaxf(mx, mt.x);
+                    const float back = m_new == -INFINITY ? 0.f : exp2f(mx - m_new);        // rescales what is summed so far
+                    const float wt = mt.x == -INFINITY ? 0.f : exp2f(mt.x - m_new);
+                    o[0] = fmaf(v[0], wt, o[0] * back); o[1] = fmaf(v[1], wt, o[1] * back);
+                    o[2] = fmaf(v[2], wt, o[2] * back); o[3] = fmaf(v[3], wt, o[3] * back);
+                    total = fmaf(mt.y, wt, total * back);
+                    mx = m_new;
+                }
+            }
+            if (groups > 1) {
+                if (active) {                                           // (the waves' results in this memory were read before the count)
+                    float* mine = red + ((size_t)grp * pieces + e) * 6;
+                    mine[0] = mx; mine[1] = total; mine[2] = o[0]; mine[3] = o[1]; mine[4] = o[2]; mine[5] = o[3];
+                }
+                __syncthreads();
+                if (!active || grp != 0) continue;
+                for (int gi = 1; gi < groups; ++gi) {
+                    const float* other = red + ((size_t)gi * pieces + e) * 6;
+                    const float m_new = fmaxf(mx, other[0]);
+                    const float back = m_new == -INFINITY ? 0.f : exp2f(mx - m_new);
+                    const float wt = other[0] == -INFINITY ? 0.f : exp2f(other[0] - m_new);
+                    o[0] = fmaf(other[2], wt, o[0] * back); o[1] = fmaf(other[3], wt, o[1] * back);
+                    o[2] = fmaf(other[4], wt, o[2] * back); o[3] = fmaf(other[5], wt, o[3] * back);
+                    total = fmaf(other[1], wt, total * back);
+                    mx = m_new;
+                }
+            } else if (!active) {
+                continue;
+            }
+            const float inv = 1.0f / total;
+            uint2 w;
+            w.x = pack_bf16x2(o[0] * inv, o[1] * inv);
+            w.y = pack_bf16x2(o[2] * inv, o[3] * inv);
+            *(uint2*)(p.out + (row0 + col) * HD + piece * 4) = w;
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     // zero again for the next call
+    }
 }
 
 // ---- prompt portions, head size 128: blocks of four waves that share keys and values ----------
@@ -1004,7 +1406,32 @@ extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
 struct FusedArgs {
     const void* qkv; const float* q_norm_w; const float* k_norm_w; const float* cos_t; const float* sin_t;
     const int* slots; float eps; int add_one;
+    int* counters; int n_counters;
 };
+
+// Neighbouring splits that one block of the decode kernel takes (a wave each): four, or two where the waves'
+// results for g query heads of a key/value head would not fit 64 KiB of shared memory.
+static size_t decode_team_bytes(int team, int g) {
+    const size_t waves = (size_t)team * (g < 16 ? g : 16) * (HD + 2), groups = (size_t)team * IA_WAVE * 6;   // (see the kernel's end)
+    return (waves > groups ? waves : groups) * sizeof(float);
+}
+static int decode_team(int splits, int g) {
+    const int team = decode_team_bytes(4, g) <= 65536 ? 4 : 2;
+    return splits >= team ? team : splits;
+}
+
+// Floats of workspace that a decode step of `splits` key splits needs (one partial result a block), and the
+// zeroed 32-bit counters (one for each request, key/value head and block of 16 query heads).
+extern "C" long long ia_attention_decode_workspace(int n, int nq, int nkv, int splits) {
+    if (n <= 0 || nq <= 0 || nkv <= 0 || splits <= 0) return 0;
+    const int teams = splits / decode_team(splits, nq / nkv);
+    return teams > 1 ? (long long)n * nq * teams * (HD + 2) : 0;
+}
+extern "C" long long ia_attention_decode_counters(int n, int nq, int nkv, int splits) {
+    if (n <= 0 || nq <= 0 || nkv <= 0 || splits <= 0) return 0;
+    const int teams = splits / decode_team(splits, nq / nkv);
+    return teams > 1 ? (long long)n * nkv * ((nq / nkv + 15) / 16) : 0;
+}
 
 static int attention_launch(void* out, float* workspace, const void* q, const void* k_cache,
                             const void* v_cache, const int* block_table, const int* cu_tokens,
@@ -1020,7 +1447,8 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     IA_CHECK(page_size > 0 && page_size % 16 == 0, "attention_mfma: page size %d must be a multiple of 16", page_size);
     IA_CHECK(max_pages > 0 && window >= 0 && max_q_len >= 1, "attention_mfma: bad geometry max_pages=%d window=%d max_q_len=%d",
              max_pages, window, max_q_len);
-    IA_CHECK(splits >= 1 && splits <= 256 && (splits == 1 || (workspace != nullptr && chunk >= 32 && chunk % 32 == 0)),
+    IA_CHECK(splits >= 1 && splits <= 256 &&
+             (splits == 1 || ((workspace != nullptr || fused != nullptr) && chunk >= 32 && chunk % 32 == 0)),
              "attention_mfma: bad split of the keys (splits=%d chunk=%d)", splits, chunk);
     IA_CHECK((long long)nkv * splits <= 65535 && n_seqs <= 65535, "attention_mfma: grid too large (nkv*splits=%d seqs=%d)",
              nkv * splits, n_seqs);
@@ -1041,7 +1469,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     p.cu_tokens = cu_tokens;
     p.positions = positions;
     p.max_pages = max_pages; p.nq = nq; p.nkv = nkv; p.page = page_size; p.window = window;
-    p.splits = splits; p.chunk = chunk; p.seq_begin = seq_begin;
+    p.splits = splits; p.chunk = chunk; p.seq_begin = seq_begin; p.token_begin = token_begin;
     p.scale_log2 = scale * 1.4426950408889634f;
     const long long cols = (long long)max_q_len * g;
     // Columns a wave: 16 for decode, 32 for portions of prompts.  (64 keep every loaded key and
@@ -1059,8 +1487,21 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         p.cos_t = fused->cos_t; p.sin_t = fused->sin_t; p.slots = fused->slots;
         p.norm_eps = fused->eps; p.norm_add_one = fused->add_one;
         // 16 columns a wave, whatever the number of query heads of a key/value head
-        const dim3 fgrid((unsigned)((cols + 15) / 16), nkv * splits, n_seqs);
-        attn_mfma_fused_kernel<><<<fgrid, IA_WAVE, 0, stream>>>(p);
+        IA_CHECK(splits == 1 || (splits & (splits - 1)) == 0, "attention_mfma: the decode kernel splits the keys 2^k ways, not %d", splits);
+        const int team = decode_team(splits, g), teams = splits / team;
+        const int col_blocks = (g + 15) / 16;
+        IA_CHECK(teams == 1 || workspace != nullptr, "attention_mfma: the decode kernel needs a workspace for %d blocks a request "
+                 "and key/value head", teams);
+        IA_CHECK(teams == 1 || (fused->counters != nullptr && (long long)n_seqs * nkv * col_blocks <= fused->n_counters),
+                 "attention_mfma: the decode kernel needs %lld zeroed counters, got %d", (long long)n_seqs * nkv * col_blocks,
+                 fused->counters ? fused->n_counters : 0);
+        IA_CHECK((long long)nkv * teams <= 65535, "attention_mfma: grid too large (nkv*blocks=%d)", nkv * teams);
+        p.part_ml = workspace ? workspace + (size_t)n * nq * teams * HD : nullptr;
+        const dim3 fgrid((unsigned)col_blocks, nkv * teams, n_seqs);
+        const size_t shared = team > 1 ? decode_team_bytes(team, g) : 0;
+        attn_decode_kernel<><<<fgrid, team * IA_WAVE, shared, stream>>>(p, fused->counters, team);
+        IA_LAUNCH_CHECK("attention_decode");
+        return 0;
     } else if (HD == 128 && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
         const int tile_cols = 16 * TILE_NBW * TILE_WAVES;
@@ -1119,13 +1560,14 @@ extern "C" int ia_attention_mfma_decode_fused(void* out, float* workspace, const
                                               float eps, int add_one, int n, int seq_begin, int n_seqs,
                                               int token_begin, int n_tokens, int max_kv_len, int max_pages,
                                               int nq, int nkv, int d, int page_size, int window, float scale,
-                                              int splits, int chunk, hipStream_t stream) {
+                                              int splits, int chunk, int* counters, int n_counters,
+                                              hipStream_t stream) {
     IA_CHECK(qkv != nullptr && (q_norm_w == nullptr) == (k_norm_w == nullptr) && (cos_t == nullptr) == (sin_t == nullptr),
              "attention_mfma_decode_fused: qkv is needed; norm weights and angle tables come in pairs");
     IA_CHECK((((uintptr_t)qkv | (uintptr_t)q_norm_w | (uintptr_t)k_norm_w | (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0,
              "attention_mfma_decode_fused: arrays must be 16-byte aligned");
     IA_CHECK(n_seqs == n_tokens, "attention_mfma_decode_fused: one token a request (%d requests, %d tokens)", n_seqs, n_tokens);
-    const FusedArgs fused = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, slots, eps, add_one};
+    const FusedArgs fused = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, slots, eps, add_one, counters, n_counters};
     return attention_launch(out, workspace, nullptr, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
                             n_seqs, token_begin, n_tokens, 1, max_kv_len, max_pages, nq, nkv, d, page_size,
                             window, scale, splits, chunk, &fused, stream);

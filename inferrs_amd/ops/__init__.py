@@ -76,7 +76,7 @@ class _Timed:
         fn = getattr(self._lib, name)
         if KernelTimer.active is None or not name.startswith("ia_") or name.endswith(("_workspace", "_blocks", "_block_rows",
                                                                                       "_error", "_version", "_capacity", "_top",
-                                                                                      "_splits", "_tune", "_target")):
+                                                                                      "_splits", "_tune", "_target", "_counters")):
             return fn
         timer = KernelTimer.active
         return lambda *args: timer.call(name[3:], fn, *args)
@@ -96,6 +96,8 @@ def library(target: str = "core"):
         raise KernelError(f"{path}: unexpected ABI version {lib.ia_abi_version()}")
     if target.startswith("attn_d"):
         lib.ia_attention_mfma_workspace.restype = ctypes.c_longlong
+        lib.ia_attention_decode_workspace.restype = ctypes.c_longlong
+        lib.ia_attention_decode_counters.restype = ctypes.c_longlong
     else:
         lib.ia_sample_workspace.restype = ctypes.c_longlong
         lib.ia_argmax_workspace.restype = ctypes.c_longlong
@@ -333,6 +335,24 @@ def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: i
     return splits, chunk
 
 
+DECODE_WAVES = 1024            # the decode kernel holds a wave a SIMD: as many waves as the chip has SIMDs, no more
+DECODE_MIN_CHUNK = 128         # fewest keys a wave's share is worth (four steps of 32)
+
+
+def decode_split(n_seqs: int, nkv: int, g: int, max_kv_len: int) -> Tuple[int, int]:
+    """(splits, keys per split) for the decode kernel: the largest power of two that keeps the step's waves
+    (request x kv head x 16 query heads x split) within one round of the chip and a wave's share at 128 keys
+    or more.  Measured at head size 128, 32 query and 8 kv heads, context 8,192 (microseconds a layer): batch 1
+    18.0 with 64 splits against 20.0 with 128, batch 3 27.6 with 32 against 34.1 with 64, batch 8 52.4 with 16
+    against 55.5 with 32, batch 64 358 with 2 against 375 with 4."""
+    items = n_seqs * nkv * -(-g // 16)
+    splits = 1
+    while items * splits * 2 <= DECODE_WAVES and max_kv_len >= 2 * splits * DECODE_MIN_CHUNK and splits < 128:
+        splits *= 2
+    chunk = -(-max_kv_len // splits)
+    return splits, -(-chunk // 32) * 32
+
+
 def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
                    cu_tokens: torch.Tensor, block_table: torch.Tensor, *, max_q_len: int, max_kv_len: int,
                    window: Optional[int], scale: float, splits: Optional[int] = None,
@@ -379,6 +399,29 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         n, seq_begin, n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, block_table.shape[1], nq, nkv, d,
         page_size, int(window or 0), ctypes.c_float(scale), splits, chunk, _stream()), target)
     return out
+
+
+# The decode kernel's counters: zero between calls (the kernel puts them back).  One array a device: calls that
+# share it must follow each other (one stream, or a graph replayed on it), as an engine's steps do.
+_DECODE_COUNTERS: Dict[int, torch.Tensor] = {}
+_DECODE_COUNTERS_OUTGROWN: list = []                # captured graphs may still hold their addresses: never freed
+DECODE_COUNTERS_MIN = 1 << 16
+
+
+def _decode_counters(device: torch.device, needed: int) -> Optional[torch.Tensor]:
+    if needed <= 0:
+        return None
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    have = _DECODE_COUNTERS.get(key)
+    if have is None or have.numel() < needed:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("attention_decode_fused: the counters of the decode kernel cannot be allocated under "
+                              "graph capture; run a step of this size once before capturing it")
+        if have is not None:
+            _DECODE_COUNTERS_OUTGROWN.append(have)
+        have = torch.zeros((max(DECODE_COUNTERS_MIN, 2 * needed),), dtype=torch.int32, device=device)
+        _DECODE_COUNTERS[key] = have
+    return have
 
 
 def attention_decode_fused_fits(dtype: torch.dtype, d: int, page_size: int, rot: int, interleaved: bool,
@@ -433,18 +476,22 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     elif tuple(out.shape) != (n, nq, d) or out.dtype != qkv.dtype:
         raise KernelError("attention_decode_fused: `out` must be [n, nq, d] in the dtype of qkv")
     if splits is None:
-        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, 1, max_kv_len)
+        splits, chunk = decode_split(n_seqs, nkv, nq // nkv, max_kv_len)
     else:
         chunk = -(-(-(-max_kv_len // splits)) // 32) * 32
+    if splits & (splits - 1):
+        raise KernelError(f"attention_decode_fused: the keys are split 2^k ways, not {splits}")
     target = _build.attn_target(d)
     lib = library(target)
-    ws_floats = lib.ia_attention_mfma_workspace(n, nq, splits)
+    ws_floats = lib.ia_attention_decode_workspace(n, nq, nkv, splits)
     ws = torch.empty((ws_floats,), dtype=torch.float32, device=qkv.device) if ws_floats else None
+    counters = _decode_counters(qkv.device, lib.ia_attention_decode_counters(n, nq, nkv, splits))
     _check(lib.ia_attention_mfma_decode_fused(
         _p(out), _p(ws), _p(qkv), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions), _p(slots),
         _p(q_norm_w), _p(k_norm_w), _p(cos), _p(sin), ctypes.c_float(eps), int(add_one), n, seq_begin, n_seqs,
         seq_begin, n_seqs, max_kv_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
-        ctypes.c_float(scale), splits, chunk, _stream()), target)
+        ctypes.c_float(scale), splits, chunk, _p(counters), counters.numel() if counters is not None else 0,
+        _stream()), target)
     return out
 
 

@@ -628,7 +628,7 @@ def test_attention_decode_fused_is_the_three_kernels_in_one(nq, nkv, d, page, wi
     q1 = ops.qk_rope_kv(dev(qkv), nq, nkv, d, q_norm_w=dv(qw), k_norm_w=dv(kw), eps=1e-5, add_one=False, cos=dv(cos),
                         sin=dv(sin), rot=d if rope else 0, interleaved=False, k_cache=k1, v_cache=v1,
                         slots=dev(slots) if write else None, page_size=page)
-    for splits in (None, 1, 4):
+    for splits in (None, 1, 4, 8, 32):                      # one block a (request, kv head); two and eight, merged by the last
         want = ops.attention_mfma(q1, k1, v1, dev(positions), dev(cu), dev(table), max_q_len=1, max_kv_len=max(lens),
                                   window=window, scale=scale, splits=splits).float().cpu()
         k2, v2 = dev(kc), dev(vc)
@@ -644,6 +644,69 @@ def test_attention_decode_fused_is_the_three_kernels_in_one(nq, nkv, d, page, wi
             # keys: the same but for a last bit here and there (the sum of squares is added up in another order)
             dk = (k2.float() - k1.float()).abs()
             assert float(dk.max()) <= 2 ** -7 * float(k1.float().abs().max()) and float((dk > 0).float().mean()) < 1e-3
+        # the counters that tell the last block are zero again
+        counters = ops._DECODE_COUNTERS.get(torch.cuda.current_device())
+        assert counters is None or int(counters.abs().sum()) == 0
+
+
+def test_attention_decode_merge_is_the_same_every_time():
+    """The blocks of a (request, key/value head) finish in any order and the last one merges: the sum runs in the
+    order of the splits, so twenty calls give the same bits, and so does a call captured in a graph and replayed."""
+    from inferrs_amd import ops
+    nq, nkv, d, page = 8, 2, 128, 16
+    lens = [2000, 1500, 700]
+    q, kc, vc, positions, token_seq, table = attention_case(torch.bfloat16, nq, nkv, d, page, lens, [1] * len(lens), 29)
+    n = len(lens)
+    qkv = dev(randn(n, (nq + 2 * nkv) * d, dtype=torch.bfloat16, seed=3))
+    cu = dev(torch.arange(n + 1, dtype=torch.int32))
+    k, v, pos, tab = dev(kc), dev(vc), dev(positions), dev(table)
+    call = lambda: ops.attention_decode_fused(qkv, k, v, pos, cu, tab, nq=nq, nkv=nkv, d=d, slots=None, q_norm_w=None,
+                                              k_norm_w=None, eps=1e-6, add_one=False, cos=None, sin=None,
+                                              max_kv_len=max(lens), window=None, scale=d ** -0.5, splits=64)
+    first = call().clone()
+    for _ in range(20):
+        assert torch.equal(call(), first)
+    want = ops.attention_mfma(qkv[:, :nq * d].view(n, nq, d).contiguous(), k, v, pos, cu, tab, max_q_len=1,
+                              max_kv_len=max(lens), window=None, scale=d ** -0.5, splits=1)
+    close(first, want.float().cpu(), 2 ** -7, "64 splits against one")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = call()
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, first)
+        assert torch.equal(call(), first)                   # eager work between the replays
+
+
+def test_attention_decode_counters_are_not_made_under_capture():
+    """The counters are allocated at a first call outside a graph capture; a capture that would have to allocate
+    them says so instead of putting them into the graph's own memory."""
+    from inferrs_amd import ops
+    nq, nkv, d, page = 4, 1, 64, 16
+    lens = [600]
+    q, kc, vc, positions, token_seq, table = attention_case(torch.bfloat16, nq, nkv, d, page, lens, [1], 31)
+    qkv = dev(randn(1, (nq + 2 * nkv) * d, dtype=torch.bfloat16, seed=4))
+    args = (qkv, dev(kc), dev(vc), dev(positions), dev(torch.arange(2, dtype=torch.int32)), dev(table))
+    kw = dict(nq=nq, nkv=nkv, d=d, slots=None, q_norm_w=None, k_norm_w=None, eps=1e-6, add_one=False, cos=None, sin=None,
+              max_kv_len=600, window=None, scale=d ** -0.5, splits=16)
+    kept = dict(ops._DECODE_COUNTERS)
+    ops._DECODE_COUNTERS.clear()
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with pytest.raises(ops.KernelError, match="graph capture"):
+            with torch.cuda.graph(graph):
+                ops.attention_decode_fused(*args, **kw)
+        eager = ops.attention_decode_fused(*args, **kw)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = ops.attention_decode_fused(*args, **kw)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+    finally:
+        ops._DECODE_COUNTERS.update({k: v for k, v in kept.items() if k not in ops._DECODE_COUNTERS})
 
 
 # ---- products of 17 to 64 rows (gemm_mid.hip) -----------------------------------------------------------------
