@@ -1030,14 +1030,25 @@ void attn_tile_kernel(const AttnParams p) {
         // Groups of 16 keys past the request's length are read from the group of its last key instead
         // (their scores are masked and their values zeroed below): the pages behind may not exist.
         // Wave w brings the stage's w-th group of 16 keys and their values: one place in one page, the same
-        // for all its lanes, looked up a stage ahead of its use so that nobody waits for the block table.
+        // for all its lanes.  The pages' numbers come 64 at a time into a register, lane i with the entry
+        // pages_base + i of the block table, and a stage takes its number from there with a lane read: a read
+        // of the block table in every stage, through the scalar cache, kept each wave waiting for a trip to the
+        // memory before its first operand of the stage (the counter of those reads is the shared memory's too).
         // What a lane adds to that place does not change from stage to stage.
         const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+        const int last_idx = (kv_total - 1) / p.page;
+        int pages_base = 0, pages_reg = 0;
+        auto pages_load = [&](int base) {
+            pages_base = base;
+            const int idx = base + lane;
+            pages_reg = bt[idx < last_idx ? idx : last_idx];
+        };
         auto pages_for = [&](int s, int& page, int& off) {
             const int key0 = lo + s * TILE_STAGE + 16 * wave_s;
             const int k = key0 < kv_total ? key0 : (kv_total - 1) & ~15;
             const int idx = k / p.page;
-            page = bt[idx];
+            if (idx >= pages_base + IA_WAVE) pages_load(idx);
+            page = __builtin_amdgcn_readlane(pages_reg, idx - pages_base);
             off = k - idx * p.page;
         };
         uint32_t k_from[4];             // keys: chunk c is rows 4 c .. + 4 of the group, a lane's piece swizzled
@@ -1241,6 +1252,7 @@ void attn_tile_kernel(const AttnParams p) {
             }
         };
         if (stages > 0) {
+            pages_load((lo + 16 * wave_s < kv_total ? lo + 16 * wave_s : (kv_total - 1) & ~15) / p.page);
             pages_for(0, page_l, off_l);
             issue(stage_a, page_l, off_l);
             if (stages > 1) pages_for(1, page_l, off_l);
