@@ -917,10 +917,11 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
     }
 }
 
-// ---- prompt portions, head size 128: blocks of four waves that share keys and values ----------
-// A block owns 128 columns of one request and key/value head (32 columns a wave) and walks the keys in
-// stages of 64.  A stage's keys and values come from the cache pages straight into shared memory
-// (global_load_lds, 16 bytes a lane: no register holds them on the way), the next stage while this
+// ---- prompt portions, head size 128: blocks of eight waves that share keys and values ----------
+// A block owns 128 columns of one request and key/value head and walks the keys in stages of 64: four waves
+// (32 columns each) share a stage, and the block has two such groups, one on the even stages and one on the odd
+// ones, that add up at the end.  A stage's keys and values come from the cache pages straight into shared memory
+// (global_load_lds, 16 bytes a lane: no register holds them on the way), a group's next stage while this
 // one is multiplied, and every wave reads its MFMA operands from there: the L2 is asked for a key once
 // a block instead of once a wave.  A load instruction fills 1 KiB of shared memory in lane order, so
 // the lane picks the piece it fetches such that the layout comes out swizzled:
@@ -930,14 +931,29 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
 // bytes would all begin in the same one).  The counters show no bank conflict for either array
 // (SQ_LDS_BANK_CONFLICT = 0); values with their halves swapped in every other block of eight features, which
 // looked as good on paper, cost two extra cycles a read.
-// Measured against the kernel of single waves (one request, 32 query and 8 key/value heads): a prompt of
-// 2,048 tokens 118 -> 80 us, of 8,192 tokens 1.20 -> 0.74 ms (750 TFLOP/s of the causal half); a portion of
-// 512 tokens at 8,192 (keys split four ways) 181 -> 106 us.  Timing-only variants of the kernel show no
-// single bound: without the exponentials 6 % faster, without the barrier 7 %, without the column maxima
-// 8 %, without the second product 11 %, without the loads into shared memory 16 %; the wait for a stage's
-// loads costs nothing (they have arrived).  Two waves a SIMD leave the phases of a step (operands from
-// shared memory, first product, softmax, second product) mostly one after the other.
-#define TILE_WAVES 4
+// Measured (one request, 32 query and 8 key/value heads; the kernel of single waves, then blocks of four waves, two
+// a compute unit, then these): a prompt of 2,048 tokens 118 -> 77 -> 68 us, of 4,096 tokens 257 -> 201 us, of 8,192
+// tokens 1.20 -> 0.75 -> 0.77 ms; a portion of 512 tokens at 7,680 181 -> 99 -> 116 us (keys split between two
+// blocks).  Time stamps inside the kernel, 2,048 tokens: with blocks of four waves a compute unit held a long walk
+// and a short one, the short one was done at once and the long one ran alone, a wave a SIMD, so the prompt took as
+// long as its longest walk alone; and the blocks were handed out head by head (x was the tile), the longest walks of
+// the last heads starting when the first heads' were done: compute units were busy between 15 and 102 us.  With the
+// order of the kernel's comment and these blocks every unit runs two blocks and is busy 57 to 63 us; a block's
+// pass over two stages takes 2.9 us (29 % of the matrix pipes' time), its start 1.2 us, the groups' sum 0.6, its
+// end 2.4.  Timing-only variants of the blocks of four waves showed no single bound: without the exponentials 6 %
+// faster, without the barrier 7 %, without the column maxima 8 %, without the second product 11 %, without the loads
+// into shared memory 16 %.  Measured on a SIMD by itself: a matrix product takes 16 cycles and holds the issue for
+// about 8 of them, an exponential 8 to 10, a 16-byte read of shared memory 32 when all four SIMDs read (128 bytes a
+// cycle a compute unit: at 32 columns a wave the reads take as long as the products).
+// 16 bytes a lane from memory straight into shared memory, 1 KiB a wave in lane order from `lds_at` on (the same for
+// all lanes).  Written out so that the compiler does not count it among the loads it waits for: whoever reads the
+// shared memory it fills waits for it by hand (s_waitcnt vmcnt) and passes a barrier.
+__device__ __forceinline__ void lds_load16(const char* from, uint32_t lds_at) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(lds_at) : "memory");     // (m0 holds nothing of the compiler's across statements)
+}
+
+#define TILE_WAVES 4              // waves that share a stage: each with its own columns
+#define TILE_GROUPS 2             // groups of such waves in a block: each with its own stages (see the kernel)
 #define TILE_STAGE 64
 #define TILE_K_BYTES (TILE_STAGE * HD * 2)
 #define TILE_BUF_BYTES (2 * TILE_K_BYTES)
@@ -949,32 +965,40 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
 // registers cost as much again.)
 #define TILE_NBW 2
 template <bool ENABLED = (HD == 128)>
-__global__ __launch_bounds__(TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(TILE_GROUPS * TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_tile_kernel(const AttnParams p) {
     if constexpr (ENABLED) {
         constexpr int NBW = TILE_NBW;
         constexpr int WAVE_COLS = 16 * NBW;
         constexpr int TILE_COLS = TILE_WAVES * WAVE_COLS;
-        // Two stages, as two arrays: the compiler then knows that the loads on their way into one do not
-        // touch the other, and does not wait for them before it reads an operand.
-        __shared__ __align__(16) char stage_a[TILE_BUF_BYTES];
-        __shared__ __align__(16) char stage_b[TILE_BUF_BYTES];
-        const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+        // Two stages for each group.  The loads that fill them are written as instructions of their own below
+        // (lds_load16): the compiler then neither knows of them nor waits for them before it reads an operand of
+        // the other stage (it would, not knowing which stage a pointer chosen at run time names); the waits that
+        // are needed stand in the code, one at the start of a stage.
+        __shared__ __align__(16) char stage_mem[TILE_GROUPS * 2 * TILE_BUF_BYTES];
+        // Two groups of four waves walk the same 128 columns: group 0 takes the even stages of the keys, group 1
+        // the odd ones, each through its own two stages of shared memory, and at the end group 1 hands its sums
+        // to group 0 through that memory.  A compute unit holds one block, two waves a SIMD that walk equally
+        // far, and takes the next block when it is done.  (Two blocks of four waves, a long walk and a short
+        // one so that a unit's work came out even, left the long walk alone on its unit for most of its time, a
+        // wave a SIMD: a prompt of 2,048 tokens took as long as its longest walk took alone.)
+        const int lane = threadIdx.x & (IA_WAVE - 1), wave = (threadIdx.x / IA_WAVE) & (TILE_WAVES - 1);
+        const int kg = __builtin_amdgcn_readfirstlane(threadIdx.x / (IA_WAVE * TILE_WAVES));
         const int r = lane & 15, G = lane >> 4;
-        const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
-        const int seq = p.seq_begin + blockIdx.z;
+        // The blocks of a launch are handed out in the order of their numbers, x fastest, to the chip's eight dies in
+        // turn: x holds the key/value head, the split and the request, y the tile, longest walk first.  So the
+        // longest walks of all heads and requests start first and a compute unit that is done takes the longest
+        // that is left, and a head's tiles, which read the same keys, meet on one die and its L2 (eight heads).
+        const int heads_splits = p.nkv * p.splits;
+        const int seq_local = blockIdx.x / heads_splits, head_split = blockIdx.x - seq_local * heads_splits;
+        const int kvh = head_split / p.splits, split = head_split - kvh * p.splits;
+        const int seq = p.seq_begin + seq_local;
         const int g = p.nq / p.nkv;
         const int t0 = p.cu_tokens[seq], q_len = p.cu_tokens[seq + 1] - t0;
         const int n_cols = q_len * g;
         const int n_tiles = (n_cols + TILE_COLS - 1) / TILE_COLS;
-        if ((int)blockIdx.x >= n_tiles) return;
-        // Long walks first.  When all blocks fit on the chip at once (two a compute unit), the second half
-        // of them, which joins the first half on its compute units, brings short walks first: a compute
-        // unit's two blocks then end together (one prompt of 2,048 tokens: 103 -> 88 us).
-        // (the order is one for all tiles of a request, key/value head and split: each tile is walked once)
-        const unsigned first_of_row = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-        const bool second = p.pair > 0 && ((first_of_row / (unsigned)p.pair) & 1u) != 0;
-        const int bcol0 = (second ? (int)blockIdx.x : n_tiles - 1 - (int)blockIdx.x) * TILE_COLS;
+        if ((int)blockIdx.y >= n_tiles) return;
+        const int bcol0 = (n_tiles - 1 - (int)blockIdx.y) * TILE_COLS;
         const int kv_start = p.positions[t0];
         const int kv_total = kv_start + q_len;
         const int* bt = p.block_table + (size_t)seq * p.max_pages;
@@ -1064,16 +1088,12 @@ void attn_tile_kernel(const AttnParams p) {
         auto issue = [&](char* buf, int page, int off) {
             const char* krows = (const char*)(p.k_cache + (((size_t)page * p.nkv + kvh) * p.page + off) * HD);
             const char* vrows = (const char*)(p.v_cache + ((size_t)page * p.nkv + kvh) * HD * p.page + off);
+            const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)buf;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) lds_load16(krows + k_from[c], at + (16 * wave_s + 4 * c) * (HD * 2));
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(krows + k_from[c]),
-                    (void __attribute__((address_space(3)))*)(buf + (16 * wave_s + 4 * c) * (HD * 2)), 16, 0, 0);
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(vrows + (size_t)c * 32 * p.page * 2 + v_from),
-                    (void __attribute__((address_space(3)))*)(buf + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024), 16, 0, 0);
+                lds_load16(vrows + (size_t)c * 32 * p.page * 2 + v_from, at + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024);
         };
         // values of keys past the request's length may hold anything at all: a lane zeroes them in the
         // pieces that it brought itself, once they have arrived
@@ -1108,13 +1128,17 @@ void attn_tile_kernel(const AttnParams p) {
         // values: group of 16 keys (G >> 1 of the step's two), feature row of 32 bytes, half G & 1
         const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HD * 2) + r * 32 + (G & 1) * 16);
         int page_l, off_l;
-        auto stage = [&](int s, char* buf, char* other) {
+        auto stage = [&](int s, char* buf, char* other) __attribute__((always_inline)) {
+            if (s >= stages) {                             // the other group has a stage more: its barrier is kept
+                __syncthreads();
+                return;
+            }
             __builtin_amdgcn_s_waitcnt(0);                 // this wave's part of stage s has arrived
             zero_tail(s, buf);
-            __syncthreads();                               // everybody's has, and everybody is done with stage s - 1
-            if (s + 1 < stages) {
+            __syncthreads();                               // everybody's has, and everybody is done with the stage before
+            if (s + TILE_GROUPS < stages) {
                 issue(other, page_l, off_l);
-                if (s + 2 < stages) pages_for(s + 2, page_l, off_l);
+                if (s + 2 * TILE_GROUPS < stages) pages_for(s + 2 * TILE_GROUPS, page_l, off_l);
             }
             const int kb = lo + s * TILE_STAGE;
             // Steps of 32 keys.  A wave's operands are asked for a phase ahead of their use: the values of a
@@ -1164,6 +1188,11 @@ void attn_tile_kernel(const AttnParams p) {
                         if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
                     }
                 }
+                // The maxima below are instructions written out, which the compiler does not check against the matrix
+                // products that wrote the scores: a vector instruction must not read a product's result before 7 wait
+                // states have passed (it would read what the register held before: seen as a maximum that was a
+                // probability of the step before).  The wait is tied to the scores, so it stands behind their products.
+                asm volatile("s_nop 6" : "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5]), "+v"(sc[6]), "+v"(sc[7]));
                 float mx = max2(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], max3(sc[5], sc[6], sc[7])));
                 mx = column_max(mx);
                 // The exponents' reference point moves only when the step's maximum has passed it by 2^8
@@ -1251,15 +1280,57 @@ void attn_tile_kernel(const AttnParams p) {
                 else step(std::false_type(), u);
             }
         };
-        if (stages > 0) {
-            pages_load((lo + 16 * wave_s < kv_total ? lo + 16 * wave_s : (kv_total - 1) & ~15) / p.page);
-            pages_for(0, page_l, off_l);
-            issue(stage_a, page_l, off_l);
-            if (stages > 1) pages_for(1, page_l, off_l);
-        }
-        for (int s = 0; s < stages; s += 2) {
-            stage(s, stage_a, stage_b);
-            if (s + 1 < stages) stage(s + 1, stage_b, stage_a);
+        // A group's walk: its stages are kg, kg + 2, ...; both groups pass the same number of barriers.
+        auto walk = [&](char* first, char* second) __attribute__((always_inline)) {
+            if (kg < stages) {
+                const int key0 = lo + kg * TILE_STAGE + 16 * wave_s;
+                pages_load((key0 < kv_total ? key0 : (kv_total - 1) & ~15) / p.page);
+                pages_for(kg, page_l, off_l);
+                issue(first, page_l, off_l);
+                if (kg + TILE_GROUPS < stages) pages_for(kg + TILE_GROUPS, page_l, off_l);
+            }
+            for (int s = kg; s - kg < stages; s += 2 * TILE_GROUPS) {
+                stage(s, first, second);
+                if (s - kg + TILE_GROUPS < stages) stage(s + TILE_GROUPS, second, first);
+            }
+        };
+        walk(stage_mem + (2 * kg) * TILE_BUF_BYTES, stage_mem + (2 * kg + 1) * TILE_BUF_BYTES);
+
+        // ---- group 1 hands its sums to group 0: accumulators through its own two stages, maxima and sums through
+        // group 0's first ------------------------------------------------------------------------------------------
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        {
+            f32x4* xacc = (f32x4*)(stage_mem + 2 * TILE_BUF_BYTES + wave_s * (TILE_BUF_BYTES / 2));      // [nb][db][lane]
+            __shared__ float2 xml_mem[TILE_WAVES * NBW * IA_WAVE];
+            float2* xml = xml_mem + wave_s * NBW * IA_WAVE;                                             // [nb][lane]
+            if (kg == 1) {
+#pragma unroll
+                for (int nb = 0; nb < NBW; ++nb) {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) xacc[(nb * DB + db) * IA_WAVE + lane] = acc[nb][db];
+                    xml[nb * IA_WAVE + lane] = make_float2(m[nb], l[nb]);
+                }
+            }
+            __syncthreads();
+            if (kg == 1) return;
+#pragma unroll
+            for (int nb = 0; nb < NBW; ++nb) {
+                const float2 other = xml[nb * IA_WAVE + lane];
+                const float top = fmaxf(m[nb], other.x);
+                const float mine_w = m[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[nb] - top);
+                const float other_w = other.x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(other.x - top);
+                l[nb] = l[nb] * mine_w + other.y * other_w;
+                m[nb] = top;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const f32x4 o = xacc[(nb * DB + db) * IA_WAVE + lane];
+                    acc[nb][db][0] = acc[nb][db][0] * mine_w + o[0] * other_w;
+                    acc[nb][db][1] = acc[nb][db][1] * mine_w + o[1] * other_w;
+                    acc[nb][db][2] = acc[nb][db][2] * mine_w + o[2] * other_w;
+                    acc[nb][db][3] = acc[nb][db][3] * mine_w + o[3] * other_w;
+                }
+            }
         }
 #pragma unroll
         for (int nb = 0; nb < NBW; ++nb) {
@@ -1517,16 +1588,11 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     } else if (HD == 128 && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
         const int tile_cols = 16 * TILE_NBW * TILE_WAVES;
-        const dim3 tgrid((unsigned)((cols + tile_cols - 1) / tile_cols), nkv * splits, n_seqs);
-        static int cus = 0;
-        if (cus == 0) {
-            int dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-                cus = 256;
-        }
-        p.pair = (long long)tgrid.x * tgrid.y * tgrid.z <= 2LL * cus ? cus : 0;     // the tile kernel's use of the field
-        attn_tile_kernel<><<<tgrid, TILE_WAVES * IA_WAVE, 0, stream>>>(p);
+        const long long tiles = (cols + tile_cols - 1) / tile_cols;
+        IA_CHECK(tiles <= 65535, "attention_mfma: %lld tiles of columns in a request (at most 65535)", tiles);
+        const dim3 tgrid((unsigned)(nkv * splits * n_seqs), (unsigned)tiles, 1);
+        p.pair = 0;
+        attn_tile_kernel<><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
     } else if (nb == 1) {
         attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
     } else {

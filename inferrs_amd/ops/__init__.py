@@ -310,7 +310,7 @@ def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int) -> bool:
 
 
 ATTN_TILE_COLS = 128           # head size 128, prompt portions: columns a block of four waves
-ATTN_TILE_BLOCKS = 512         # blocks wanted (two a compute unit) before the keys stop being split
+ATTN_TILE_BLOCKS = 256         # blocks wanted (one a compute unit: eight waves) before the keys stop being split
 ATTN_TILE_MIN_CHUNK = 512      # fewest keys a block's share is worth (eight stages of 64)
 
 
