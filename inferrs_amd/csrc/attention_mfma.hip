@@ -377,25 +377,13 @@ void attn_mfma_kernel(const AttnParams p) {
 
 // The maximum / the sum over the four lanes that hold a column's values (lanes l, l ^ 16, l ^ 32, l ^ 48), in all
 // of them, by swaps between rows of 16 lanes and between the halves of the wave: no trip through shared memory.
-// (the maximum instructions themselves, which return the other operand when one is a NaN: fmaxf() puts
-// an instruction in front of each operand that turns a signalling NaN into a quiet one)
-__device__ __forceinline__ float max2(float a, float b) {
-    float r;
-    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return r;
-}
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
 __device__ __forceinline__ float column_max(float x) {
     const uint32_t u = __float_as_uint(x);
     auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    x = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
     const uint32_t w = __float_as_uint(x);
     auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
-    return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float column_sum(float x) {
     const uint32_t u = __float_as_uint(x);
@@ -1136,10 +1124,12 @@ void attn_tile_kernel(const AttnParams p) {
             __builtin_amdgcn_s_waitcnt(0);                 // this wave's part of stage s has arrived
             zero_tail(s, buf);
             __syncthreads();                               // everybody's has, and everybody is done with the stage before
-            if (s + TILE_GROUPS < stages) {
-                issue(other, page_l, off_l);
-                if (s + 2 * TILE_GROUPS < stages) pages_for(s + 2 * TILE_GROUPS, page_l, off_l);
-            }
+            // The loads of the group's next stage: group 0 asks for them here, group 1 between its two steps.  A load
+            // instruction holds its wave until the compute unit's one address unit takes it, 1 KiB in 16 cycles: with
+            // all eight waves asking at once after the barrier (64 KiB a pass) each waited some 1,100 to 1,700 cycles
+            // of a pass's 6,500, all at the same time (8,192 tokens 736 -> 655 us).
+            const bool more = s + TILE_GROUPS < stages;
+            if (more && kg == 0) issue(other, page_l, off_l);
             const int kb = lo + s * TILE_STAGE;
             // Steps of 32 keys.  A wave's operands are asked for a phase ahead of their use: the values of a
             // step before its softmax is worked out, the keys of the next step before this step's second
@@ -1188,12 +1178,11 @@ void attn_tile_kernel(const AttnParams p) {
                         if (key > pos[nb] || key < floor_key) sc[j] = -INFINITY;
                     }
                 }
-                // The maxima below are instructions written out, which the compiler does not check against the matrix
-                // products that wrote the scores: a vector instruction must not read a product's result before 7 wait
-                // states have passed (it would read what the register held before: seen as a maximum that was a
-                // probability of the step before).  The wait is tied to the scores, so it stands behind their products.
-                asm volatile("s_nop 6" : "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5]), "+v"(sc[6]), "+v"(sc[7]));
-                float mx = max2(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], max3(sc[5], sc[6], sc[7])));
+                // (the compiler's own maximum: written out as v_max3 instructions, which the compiler does not check
+                // against the matrix products that wrote the scores, the maxima could read a score's register before
+                // its product had written it, and took a probability of the step before for a score; with the wait
+                // that forbids that tied to the scores a prompt of 8,192 tokens took 823 us, so 728)
+                float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
                 mx = column_max(mx);
                 // The exponents' reference point moves only when the step's maximum has passed it by 2^8
                 // (probabilities then reach 2^8 at most, which 32-bit sums and bfloat16 operands hold as
@@ -1273,12 +1262,14 @@ void attn_tile_kernel(const AttnParams p) {
             };
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
+                if (u == 1 && more && kg != 0) issue(other, page_l, off_l);
                 if (!live[u]) continue;
                 const int k0 = kb + 32 * u;
                 const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
                 if (edge) step(std::true_type(), u);
                 else step(std::false_type(), u);
             }
+            if (s + 2 * TILE_GROUPS < stages) pages_for(s + 2 * TILE_GROUPS, page_l, off_l);
         };
         // A group's walk: its stages are kg, kg + 2, ...; both groups pass the same number of barriers.
         auto walk = [&](char* first, char* second) __attribute__((always_inline)) {
