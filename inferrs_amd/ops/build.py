@@ -35,6 +35,11 @@ FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}",
          "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 
 HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-Wall"]
+# Flags of single sources.  The attention kernels take the maximum of scores that come out of matrix products:
+# told that no NaN reaches an arithmetic instruction (masked scores are replaced, never computed with), the
+# compiler leaves out the instruction that would quiet a signalling NaN in front of every maximum (a prompt of
+# 8,192 tokens 650 -> 614 us a layer).
+SOURCE_FLAGS = {"attention_mfma.hip": ["-fno-honor-nans"]}
 
 PER_HEAD_DIM = ("attention_mfma.hip",)
 SHARED = ("error.hip",)
@@ -81,6 +86,8 @@ def _digest(target: str) -> str:
         with open(p, "rb") as f:
             h.update(f.read())
     h.update(" ".join((HOST_FLAGS if host else FLAGS) + defines).encode())
+    for p in srcs:
+        h.update(" ".join(SOURCE_FLAGS.get(os.path.basename(p), [])).encode())
     return h.hexdigest()[:12]
 
 
@@ -156,7 +163,7 @@ def build(target: str = "core", verbose: bool = True, workers: Optional[int] = N
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.splitext(os.path.basename(src))[0] + ".o")
-        r = subprocess.run([hipcc, *flags, *defines, "-I", CSRC, "-c", src, "-o", obj],
+        r = subprocess.run([hipcc, *flags, *SOURCE_FLAGS.get(os.path.basename(src), []), *defines, "-I", CSRC, "-c", src, "-o", obj],
                            capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"{os.path.basename(hipcc)} failed on {src}:\n{r.stdout}\n{r.stderr}")
