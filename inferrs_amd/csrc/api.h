@@ -39,10 +39,13 @@ int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const void* qkv,
                   int interleaved, int page_size, float eps, int add_one, int dtype,
                   hipStream_t stream);
 
+// workspace: null, or ia_attention_generic_workspace(...) floats when that is not 0 (steps of few tokens: a wave a
+// segment of keys and a merge kernel, the same bits as without); max_kv_len: an upper bound of positions + 1
 int ia_attention_generic(void* out, const void* q, const void* k_cache, const void* v_cache,
                          const int* positions, const int* token_seq, const int* block_table,
                          int n, int max_pages, int nq, int nkv, int d, int page_size, int window,
-                         float scale, int dtype, hipStream_t stream);
+                         float scale, int dtype, float* workspace, int max_kv_len, hipStream_t stream);
+long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int max_kv_len);
 
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
                   int out_dtype, hipStream_t stream);

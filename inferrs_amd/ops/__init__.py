@@ -100,6 +100,7 @@ def library(target: str = "core"):
         lib.ia_attention_decode_counters.restype = ctypes.c_longlong
     else:
         lib.ia_sample_workspace.restype = ctypes.c_longlong
+        lib.ia_attention_generic_workspace.restype = ctypes.c_longlong
         lib.ia_argmax_workspace.restype = ctypes.c_longlong
     _LIBS[target], _LIB_PATHS[target] = lib, path
     return lib
@@ -282,10 +283,13 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, page_si
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
-                      *, window: Optional[int], scale: float) -> torch.Tensor:
+                      *, window: Optional[int], scale: float, max_kv_len: Optional[int] = None,
+                      split: Optional[bool] = None) -> torch.Tensor:
     """q [n, nq, d] against the paged cache; token i sees the keys at positions <= positions[i]
     (and > positions[i] - window) of row token_seq[i] of the table.  Any head size up to 512, any
-    page size, 32-bit or bfloat16 storage, all arithmetic in 32-bit."""
+    page size, 32-bit or bfloat16 storage, all arithmetic in 32-bit.  `max_kv_len`: an upper bound of
+    positions + 1 (default: what the table can hold).  Steps of few tokens run a wave a segment of 512 keys
+    and a merge kernel (`split`; None: the kernel's own rule); the bits are the same either way."""
     _dev(q, k_cache, v_cache, positions, token_seq, block_table)
     _i32(positions, "positions"); _i32(token_seq, "token_seq"); _i32(block_table, "block_table")
     n, nq, d = q.shape
@@ -293,11 +297,18 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention")
     if positions.numel() != n or token_seq.numel() != n or block_table.dim() != 2:
         raise KernelError("attention: positions, token_seq and block_table do not fit the batch")
+    capacity = block_table.shape[1] * page_size
+    max_kv_len = capacity if max_kv_len is None else min(int(max_kv_len), capacity)
     out = torch.empty_like(q)
-    _check(library().ia_attention_generic(
+    lib = library()
+    ws_floats = lib.ia_attention_generic_workspace(n, nq, nkv, d, max_kv_len) if split is not False else 0
+    if split and not ws_floats:
+        raise KernelError("attention: a step of this many tokens, or of so few keys, is not split")
+    ws = torch.empty((ws_floats,), dtype=torch.float32, device=q.device) if ws_floats else None
+    _check(lib.ia_attention_generic(
         _p(out), _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_seq), _p(block_table), n,
         block_table.shape[1], nq, nkv, d, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
-        _stream()))
+        _p(ws), max_kv_len, _stream()))
     return out
 
 

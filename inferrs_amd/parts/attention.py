@@ -123,5 +123,5 @@ class Attention(Mixer):
                                        max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, **common)
         else:
             a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
-                                      window=s.window, scale=s.softmax_scale)
+                                      window=s.window, scale=s.softmax_scale, max_kv_len=ctx.max_kv_len)
         return self._project(ctx, a.view(a.shape[0], s.n_heads * s.head_dim))

@@ -280,6 +280,34 @@ def test_attention_generic(dtype, nq, nkv, d, page, window):
     close(ref_attention_dense(q, kc, vc, positions, token_seq, table, window, scale), want, 1e-5, "the two references")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,page,window", [
+    (8, 2, 128, 16, None), (3, 1, 72, 8, None), (5, 5, 24, 5, None), (10, 2, 64, 16, 700), (2, 1, 320, 32, None)])
+def test_attention_generic_in_segments_is_the_same_bits_as_in_one_walk(dtype, nq, nkv, d, page, window):
+    """Keys beyond one segment of 512: a wave a segment with the merge kernel behind it (steps of few tokens)
+    against one wave that walks all segments of its token (steps of many tokens), bit for bit, and both against
+    the reference; head sizes and page sizes that are no multiple of four take the loads of single elements.
+    What the pages hold beyond a request's keys is NaN."""
+    from inferrs_amd import ops
+    lens, q_lens = [1500, 513, 1024, 40], [2, 1, 3, 1]
+    q, kc, vc, positions, token_seq, table = attention_case(dtype, nq, nkv, d, page, lens, q_lens, 29, needle=True)
+    want = ref_attention_dense(q, kc, vc, positions, token_seq, table, window, 1.0 / math.sqrt(d))
+    for s, l in enumerate(lens):                     # the rest of every request's last page
+        if l % page:
+            kc[int(table[s, l // page]), :, l % page:] = float("nan")
+            vc[int(table[s, l // page]), :, :, l % page:] = float("nan")
+    args = (dev(q), dev(kc), dev(vc), dev(positions), dev(token_seq), dev(table))
+    scale = 1.0 / math.sqrt(d)
+    whole = ops.attention_generic(*args, window=window, scale=scale, split=False)
+    parts = ops.attention_generic(*args, window=window, scale=scale, split=True)
+    bound = ops.attention_generic(*args, window=window, scale=scale, split=True, max_kv_len=max(lens))
+    assert torch.equal(whole, parts) and torch.equal(whole, bound)
+    close(whole, want, tol(dtype, 5e-6, 2 ** -7), "attention in segments")
+    assert ops.library().ia_attention_generic_workspace(4096, nq, nkv, d, 2000) == 0          # tokens enough: no split
+    with pytest.raises(ops.KernelError):
+        ops.attention_generic(*args, window=window, scale=scale, split=True, max_kv_len=300)  # one segment: nothing to split
+
+
 @pytest.mark.parametrize("nq,nkv,d,page,window", [
     (4, 2, 16, 16, None), (5, 1, 48, 16, None), (8, 1, 128, 16, None), (32, 8, 128, 16, None),
     (6, 3, 32, 32, 37), (3, 3, 80, 16, None), (2, 2, 256, 64, 100), (40, 2, 64, 16, None), (7, 7, 112, 48, 5)])
