@@ -69,11 +69,182 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(TO* __restrict__ out, c
     }
 }
 
+__device__ __forceinline__ float4 gr_load4(const float* p) { return *(const float4*)p; }
+__device__ __forceinline__ float4 gr_load4(const bf16_t* p) {
+    const uint2 v = *(const uint2*)p;
+    return make_float4(bf16_bits_to_f32((uint16_t)v.x), bf16_bits_to_f32((uint16_t)(v.x >> 16)),
+                       bf16_bits_to_f32((uint16_t)v.y), bf16_bits_to_f32((uint16_t)(v.y >> 16)));
+}
+
+// The same sums in tiles of 128 x 128 for many rows (prompts of the 32-bit path): a thread owns 8 x 8 outputs (rows
+// 4 ty .. + 4 and 64 + 4 ty .. + 4, features likewise with tx), so that every value read from shared memory meets eight
+// fused multiply-adds instead of four; k ascending for every output as above, hence the same bits.  K a multiple of 4.
+#define GB 128
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void gemm_tiled128_kernel(TO* __restrict__ out, const TI* __restrict__ x,
+                                                            const TI* __restrict__ w, int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) float xs[GK][GB + 4];
+    __shared__ __attribute__((aligned(16))) float ws[GK][GB + 4];
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * GB, n0 = blockIdx.x * GB;
+    float acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+    // a tile is 128 rows x 16 k = 512 pieces of four k: two a thread, of rows lr and lr + 64
+    const int lr = tid >> 2, lk = (tid & 3) * 4;
+    const TI* xp[2];
+    const TI* wp[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int m = m0 + lr + 64 * h, n = n0 + lr + 64 * h;
+        xp[h] = x + (size_t)(m < M ? m : M - 1) * K + lk;       // (rows beyond the matrices: never stored)
+        wp[h] = w + (size_t)(n < N ? n : N - 1) * K + lk;
+    }
+    float4 xr[2], wr[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const bool in = k0 + lk < K;
+            xr[h] = in ? gr_load4(xp[h] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            wr[h] = in ? gr_load4(wp[h] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += GK) {
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int r = lr + 64 * h;
+            xs[lk][r] = xr[h].x; xs[lk + 1][r] = xr[h].y; xs[lk + 2][r] = xr[h].z; xs[lk + 3][r] = xr[h].w;
+            ws[lk][r] = wr[h].x; ws[lk + 1][r] = wr[h].y; ws[lk + 2][r] = wr[h].z; ws[lk + 3][r] = wr[h].w;
+        }
+        if (k0 + GK < K) fetch(k0 + GK);
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GK; ++kk) {
+            const float4 a0 = *(const float4*)(&xs[kk][4 * ty]), a1 = *(const float4*)(&xs[kk][64 + 4 * ty]);
+            const float4 b0 = *(const float4*)(&ws[kk][4 * tx]), b1 = *(const float4*)(&ws[kk][64 + 4 * tx]);
+            const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int m = m0 + (i < 4 ? 4 * ty + i : 64 + 4 * ty + i - 4);
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int n = n0 + (j < 4 ? 4 * tx + j : 64 + 4 * tx + j - 4);
+            if (n < N) st(out + (size_t)m * N + n, acc[i][j]);
+        }
+    }
+}
+
+// The same product for up to 16 rows (decode steps of the 32-bit path), bound by reading the weights: a wave owns 16
+// output features, so that a weight of 4,096 features still makes a block for every compute unit; lane (n, group of
+// four rows) adds up its four sums with k ascending, one chain of fused multiply-adds each, which gives the bits of the
+// tiled kernel.  Chunks of 256 k come into shared memory in whole rows, the next chunk on its way from memory while
+// this one is multiplied.  K a multiple of 4.
+#define GR_N 16
+#define GR_K 256
+#define GR_PITCH (GR_K + 4)             // floats between staged rows: 16-byte aligned, no two of 16 lanes on a bank
+#define GR_ROWS 16
+#define GR_LOADS (GR_N * GR_K / 4 / IA_WAVE)     // loads of four elements a lane brings of each operand
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(IA_WAVE) void gemm_rows_kernel(TO* __restrict__ out, const TI* __restrict__ x,
+                                                            const TI* __restrict__ w, int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) float ws[GR_N * GR_PITCH];
+    __shared__ __attribute__((aligned(16))) float xs[GR_ROWS * GR_PITCH];
+    const int lane = threadIdx.x;
+    const int nn = lane & 15, mg = lane >> 4;
+    const int n0 = blockIdx.x * GR_N;
+    // what this lane fetches: load i takes piece (lane % 64) of row i of the 16 (a row of a chunk is 64 pieces of four)
+    const int piece = lane * 4;
+    float4 wr[GR_LOADS], xr[GR_LOADS];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < GR_LOADS; ++i) {
+            const int k = k0 + piece;
+            const int n = n0 + i < N ? n0 + i : N - 1;         // (features beyond the matrix: never stored)
+            wr[i] = k < K ? gr_load4(w + (size_t)n * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+            xr[i] = (k < K && i < M) ? gr_load4(x + (size_t)i * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += GR_K) {
+        __syncthreads();                                        // everybody is done with the chunk before
+#pragma unroll
+        for (int i = 0; i < GR_LOADS; ++i) {
+            *(float4*)(ws + i * GR_PITCH + piece) = wr[i];
+            *(float4*)(xs + i * GR_PITCH + piece) = xr[i];
+        }
+        if (k0 + GR_K < K) fetch(k0 + GR_K);
+        __syncthreads();
+        const float* wmine = ws + nn * GR_PITCH;
+        const float* xmine = xs + mg * 4 * GR_PITCH;
+#pragma unroll 4
+        for (int k4 = 0; k4 < GR_K / 4; ++k4) {
+            const float4 wv = *(const float4*)(wmine + k4 * 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 xv = *(const float4*)(xmine + i * GR_PITCH + k4 * 4);
+                acc[i] = fmaf(xv.x, wv.x, acc[i]);
+                acc[i] = fmaf(xv.y, wv.y, acc[i]);
+                acc[i] = fmaf(xv.z, wv.z, acc[i]);
+                acc[i] = fmaf(xv.w, wv.w, acc[i]);
+            }
+        }
+    }
+    const int n = n0 + nn;
+    if (n < N)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (mg * 4 + i < M) st(out + (size_t)(mg * 4 + i) * N + n, acc[i]);
+}
+static_assert(GR_LOADS == GR_N && GR_LOADS == GR_ROWS, "a lane brings one piece of every staged row");
+
 // in_dtype: storage of x and w; out_dtype: storage of the result.
 extern "C" int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K,
                              int in_dtype, int out_dtype, hipStream_t stream) {
     IA_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     if (M == 0) return 0;
+    const size_t elem = in_dtype == IA_F32 ? 4 : 2;
+    if (M <= GR_ROWS && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) % (4 * elem)) == 0) {
+        const unsigned blocks = (unsigned)((N + GR_N - 1) / GR_N);
+        if (in_dtype == IA_F32 && out_dtype == IA_F32)
+            gemm_rows_kernel<float, float><<<blocks, IA_WAVE, 0, stream>>>((float*)out, (const float*)x, (const float*)w, M, N, K);
+        else if (in_dtype == IA_BF16 && out_dtype == IA_BF16)
+            gemm_rows_kernel<bf16_t, bf16_t><<<blocks, IA_WAVE, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else if (in_dtype == IA_BF16 && out_dtype == IA_F32)
+            gemm_rows_kernel<bf16_t, float><<<blocks, IA_WAVE, 0, stream>>>((float*)out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else
+            IA_CHECK(false, "gemm_tiled: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+        IA_LAUNCH_CHECK("gemm_rows");
+        return 0;
+    }
+    if (M > 2 * GT && N >= GB && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) % (4 * elem)) == 0) {
+        const dim3 grid((N + GB - 1) / GB, (M + GB - 1) / GB);
+        IA_CHECK(grid.y <= 65535, "gemm_tiled: %d rows exceed the grid", M);
+        if (in_dtype == IA_F32 && out_dtype == IA_F32)
+            gemm_tiled128_kernel<float, float><<<grid, 256, 0, stream>>>((float*)out, (const float*)x, (const float*)w, M, N, K);
+        else if (in_dtype == IA_BF16 && out_dtype == IA_BF16)
+            gemm_tiled128_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else if (in_dtype == IA_BF16 && out_dtype == IA_F32)
+            gemm_tiled128_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((float*)out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
+        else
+            IA_CHECK(false, "gemm_tiled: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+        IA_LAUNCH_CHECK("gemm_tiled128");
+        return 0;
+    }
     const dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT);
     IA_CHECK(grid.y <= 65535, "gemm_tiled: %d rows exceed the grid", M);
     if (in_dtype == IA_F32 && out_dtype == IA_F32)

@@ -404,16 +404,21 @@ def test_gemm_reference_products():
     assert ops.linear(dev(torch.tensor([[10., 100.]])), dev(w)).cpu().tolist() == [[210., 430., 650.]]
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 130, 40), (65, 64, 64), (17, 515, 136), (130, 72, 200), (2, 7, 1000)])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 130, 40), (65, 64, 64), (17, 515, 136), (130, 72, 200), (2, 7, 1000),
+                                   (200, 300, 136), (300, 1000, 520), (16, 100, 1000), (129, 128, 4), (140, 131, 42)])
 def test_gemm_tiled_float32_is_true_32_bit(m, n, k):
+    """Three kernels share this product: one for up to 16 rows, tiles of 64 x 64, and tiles of 128 x 128 for more than 128
+    rows (k a multiple of 4); each adds an output up with k ascending, so they give the same bits."""
     from inferrs_amd import ops
     x, w = randn(m, k, dtype=torch.float32, seed=1), randn(n, k, dtype=torch.float32, seed=2)
     want = (x.double() @ w.double().t())
-    got = ops.linear(dev(x), dev(w)).cpu().double()
+    whole = ops.linear(dev(x), dev(w)).cpu()
     # a reduced-precision matrix mode (tf32-like, 10 bits) would be off by about 1e-3
-    assert float((got - want).abs().max()) <= 4e-6 * max(1.0, float(want.abs().max()))
-    # rows do not depend on what else is in the batch
-    assert torch.equal(ops.linear(dev(x[:1]), dev(w)).cpu(), ops.linear(dev(x), dev(w)).cpu()[:1])
+    assert float((whole.double() - want).abs().max()) <= 4e-6 * max(1.0, float(want.abs().max()))
+    # rows do not depend on what else is in the batch: alone, among 16, among 40 and among all
+    for rows in (1, 16, 40):
+        rows = min(rows, m)
+        assert torch.equal(ops.linear(dev(x[m - rows:]), dev(w)).cpu(), whole[m - rows:])
 
 
 @pytest.mark.parametrize("m", [1, 2, 8, 12, 13, 16, 17, 33, 64, 65, 200])
