@@ -785,13 +785,14 @@ def add_rmsnorm_partials(x: torch.Tensor, delta: Partials, w: torch.Tensor, eps:
     return out
 
 
-def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, mid: bool = True) -> torch.Tensor:
     """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
     skinny MFMA kernel for up to SKINNY_MAX_ROWS rows, the vendor's GEMM beyond that (the reference uses
     cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
     the skinny kernel's accumulators for those few rows; beyond that it is the vendor's bfloat16
     result widened, which is what the reference does for every row (its logits are computed in
-    the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`)."""
+    the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`).  `mid=False`: steps of 17 to 64 rows
+    go to the vendor's GEMM as well."""
     out_dtype = out_dtype or x.dtype
     if isinstance(x, NormedRows):
         if _takes_normed_rows(x, w, w.shape[0]):
@@ -805,7 +806,7 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch
         return gemm_tiled(x, w, out_dtype)
     if m <= SKINNY_MAX_ROWS:
         return gemm_skinny_bf16(x, w, out_dtype)
-    if mid_fits(x, w):
+    if mid and mid_fits(x, w):
         if out_dtype == torch.float32:
             return gemm_mid_bf16(x, w, torch.float32)
         y = gemm_mid_bf16(x, w, partial=True)
@@ -922,4 +923,5 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
         return gemm_mid_bf16(x, w_gate_up, dual=True)
     if w_gate_up.shape[0] % 2 == 0 and x.dtype == torch.bfloat16 and skinny_fits(x, w_gate_up) and _own_large(x, w_gate_up):
         return gemm_mfma_bf16(x, w_gate_up, dual=True)
-    return silu_mul(linear(x, w_gate_up))
+    # (a [gate; up] beyond MID_DUAL_MAX_BYTES at 17 to 64 rows: the vendor's GEMM, not the plain product of gemm_mid.hip)
+    return silu_mul(linear(x, w_gate_up, mid=False))
