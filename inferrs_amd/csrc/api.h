@@ -72,9 +72,9 @@ int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N,
 // 2: out [ia_gemm_mid_splits(N, K)][M][N] float, the sums of each split of k, to be added up by the reader
 // (ia_sum_partials, ia_add_rmsnorm_partials).  dual: w = [gate; up], out = silu(x . gate^T) * (x . up^T), mode 0.
 int ia_gemm_mid_splits(int N, int K);
-// (k steps of a chunk: 4 or 8; chunks in shared memory: 2 to 4; ways a block's waves share k for [gate; up] weights: 1 or 2;
-// the default is (4, 3, 2); plain products do not depend on it bit for bit, those with the activation inside by rounding)
-void ia_gemm_mid_tune(int kc, int ns, int dual_kh);
+// (a fixed pipeline for measurements and tests: k steps of a chunk, 2 or 4, and stages, 2 to 4; (0, 0): the kernel's own
+// rule; no product depends on it bit for bit)
+void ia_gemm_mid_tune(int kc, int ns);
 int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                      hipStream_t stream);
 int ia_sum_partials(void* out, const float* part, int splits, int M, int N, hipStream_t stream);

@@ -5,15 +5,19 @@
 //
 // The reference hands these products to cuBLAS like all others (`candle-core/src/cuda_backend/mod.rs:2260-2305`).
 //
-// A block of four waves owns 64 rows of w and a range of k.  A wave streams one tile of 16 weight rows from
-// memory straight into MFMA A-operands (v_mfma_f32_16x16x32_bf16: lane l supplies row l % 16 with the eight k
-// values 8 * (l / 16) .. + 8), three chunks of 128 k ahead of their use; the rows of x of a chunk (up to 64 rows
-// of 256 bytes) are brought into shared memory once a block by all four waves together (global_load_lds, 16 bytes
-// a lane, no register on the way), three chunks ahead as well, and every wave reads its B-operands from there.
-// All row tiles of x share every weight load.  Piece c (16 bytes) of row r of a chunk lies at place c ^ (r % 16)
-// of the row's 256 bytes, so that the 16 rows which one operand read takes at the same k fall on 16 different
-// places; a load instruction fills 1 KiB (four rows) in lane order, and the lane picks the piece it fetches
-// accordingly.
+// A block of four waves owns 64 rows of w and a range of k, and walks it in chunks of 128.  A stage of shared memory
+// holds a chunk's rows of x (up to 64) and the block's 64 rows of w alike, 256 bytes a row, brought by all four waves
+// together straight from memory (global_load_lds: 16 bytes a lane, four whole rows an instruction, no register on the
+// way), one or two stages ahead of their use.  A wave multiplies its tile of 16 weight rows (the MFMA A-operand:
+// v_mfma_f32_16x16x32_bf16, lane l supplies row l % 16 with the eight k values 8 * (l / 16) .. + 8) with every row tile of
+// x, both read from the stage.  Piece c (16 bytes) of row r lies at place c ^ (r % 16) of the row's 256 bytes, so that the
+// 16 rows which one operand read takes at the same k fall on 16 different places; a load instruction fills 1 KiB (four
+// rows) in lane order, and the lane picks the piece it fetches accordingly.
+//
+// The weights went straight from memory into the A-operands before (a load of 16 rows x 64 bytes a lane group): such a
+// load holds the compute unit's address unit for about 86 cycles, a load of 1 KiB in whole rows for about 32, and by its
+// own clocks that kernel spent 40 % of a step issuing its loads at 64 rows.  Through shared memory: q|k|v of 6,144 x
+// 4,096 at 64 rows 17.1 -> 14.5 us, [gate; up] with the activation 56 -> 50, the 32B shape's 5,120 x 25,600 82 -> 69.
 //
 // With few rows of w (the output projection, the feed-forward's second product) 64 rows a block leave too few
 // blocks to fill the chip, so k is split between blocks (gridDim.y) and every split leaves its sums in 32-bit:
@@ -41,185 +45,20 @@ typedef float gmid_f32x4 __attribute__((ext_vector_type(4)));
 
 enum { MID_OUT_BF16 = 0, MID_OUT_F32 = 1, MID_OUT_PARTIAL = 2 };
 
-// KC: k steps of 32 in a chunk (a row of x in a chunk is KC * 64 bytes); NS: chunks of x in shared memory, this one and
-// NS - 1 on their way.  KH: the waves of a block share k between them KH ways (1 or 2): with 2 a block owns half as many
-// rows of w (two tiles of 16, each walked by two waves over one half of k, their sums added through shared memory in a
-// fixed order), which makes twice as many blocks for the chip to balance.
-template <int MT, bool DUAL, int KC, int NS, int KH>
-__global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
-    void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-    int M, int N, int K, int k_per_block) {
-    constexpr int CHUNK_K = KC * 32;
-    constexpr int ROW_BYTES = KC * 64;                      // bytes of a row of x in a chunk
-    constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;         // rows that one load instruction (1 KiB) fills
-    constexpr int PIECES = KC * 4;                          // 16-byte pieces of a row
-    constexpr int TILES = MID_WAVES / KH;                   // tiles of 16 rows of w a block
-    constexpr int X_LOADS = MT * 16 / ROWS_PER_LOAD / TILES;       // load instructions of x a wave issues for a chunk
-    constexpr int HALF_BYTES = MT * 16 * ROW_BYTES;         // a chunk's rows of x for one share of k
-    constexpr int STAGE_BYTES = KH * HALF_BYTES;
-    static_assert(NS >= 2 && NS <= 4 && (KC == 4 || KC == 8 || KC == 16) && (KH == 1 || KH == 2), "pipeline shape");
-    static_assert(MT * 16 / ROWS_PER_LOAD % TILES == 0, "the rows of a chunk are shared out evenly between the waves");
-    // A stage [KH][MT * 16 rows][ROW_BYTES] an array: the compiler then knows that loads on their way into one stage do
-    // not touch the others, and does not wait for them before it reads operands out of this one.
-    __shared__ __attribute__((aligned(1024))) char mid_s0[STAGE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char mid_s1[STAGE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char mid_s2[NS > 2 ? STAGE_BYTES : 16];
-    __shared__ __attribute__((aligned(1024))) char mid_s3[NS > 3 ? STAGE_BYTES : 16];
-    auto stage_of = [&](auto stage_c) -> char* {
-        constexpr int S = decltype(stage_c)::value;
-        if constexpr (S == 0) return mid_s0;
-        else if constexpr (S == 1) return mid_s1;
-        else if constexpr (S == 2) return mid_s2;
-        else return mid_s3;
-    };
-    const int lane = threadIdx.x & (IA_WAVE - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / IA_WAVE);
-    const int r = lane & 15, g = lane >> 4;
-    const int tile = wave % TILES, kh = wave / TILES;
-    const int split = blockIdx.y;
-    // the block's range of k, and this wave's share of it (whole chunks; the launcher sees to it that they divide)
-    const int kb_begin = split * k_per_block;
-    const int kb_len = K - kb_begin < k_per_block ? K - kb_begin : k_per_block;
-    const int k_len = kb_len / KH;
-    const int k_begin = kb_begin + kh * k_len;
-    const int nchunks = k_len / CHUNK_K;
-
-    // ---- this wave's 16 rows of w --------------------------------------------------------------------------
-    // (rows beyond the matrix read its last row: their sums are never stored)
-    // DUAL: half of a block's tiles are gate rows, the other half the up rows of the same features
+// The end of the kernel.  Lane (r, g) holds features n_first + 4 g + i of row 16 mt + r.  DUAL: the up rows' sums go through
+// shared memory (swap_up, in a stage's place) to the waves that hold the gate rows' sums of the same features.
+template <int MT, bool DUAL, int TILES>
+__device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* swap_up, void* out, int out_mode,
+                                           int M, int N, int lane, int r, int g, int tile, int part, int n_first, int split) {
     constexpr int FEATURE_TILES = DUAL ? TILES / 2 : TILES;
-    const int part = DUAL ? tile / FEATURE_TILES : 0;                  // 0: gate (or a plain weight), 1: up
-    const int n_first = blockIdx.x * (16 * FEATURE_TILES) + 16 * (tile % FEATURE_TILES);   // output feature of the tile's first row
-    const bf16_t* wrow;
-    {
-        const int n = n_first + r < N ? n_first + r : N - 1;
-        wrow = w + ((size_t)part * N + n) * K + k_begin + g * 8;
-    }
-
-    // ---- what this lane fetches of a chunk of x: X_LOADS instructions, each ROWS_PER_LOAD whole rows ------------
-    // The waves that share a range of k bring its rows together: instruction i of tile t covers rows ROWS_PER_LOAD *
-    // (TILES i + t) .. ; lane l writes place l % PIECES of row l / PIECES of them, and fetches the piece that belongs
-    // there: piece c of row r lies at place c ^ (r % 16)
-    const char* xsrc[X_LOADS];
-#pragma unroll
-    for (int i = 0; i < X_LOADS; ++i) {
-        const int row = ROWS_PER_LOAD * (TILES * i + tile) + lane / PIECES;
-        const int piece = (lane % PIECES) ^ (row & 15);
-        xsrc[i] = (const char*)(x + (size_t)(row < M ? row : 0) * K + k_begin) + piece * 16;
-    }
-    // and where it reads its B-operands: row 16 mt + r, piece 4 ks + g, at place (4 ks + g) ^ r
-    uint32_t b_at[KC];
-#pragma unroll
-    for (int ks = 0; ks < KC; ++ks) b_at[ks] = (uint32_t)(kh * HALF_BYTES + r * ROW_BYTES + (((4 * ks + g) ^ r) * 16));
-
-    gmid_f32x4 acc[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
-    uint4 wreg[NS][KC];
-
-    auto issue = [&](auto stage_c, int c) {
-        constexpr int S = decltype(stage_c)::value;
-        // the weights first, then the rows of x: a wait for the rows of a chunk covers its weights too
-#pragma unroll
-        for (int ks = 0; ks < KC; ++ks) wreg[S][ks] = *(const uint4*)(wrow + (size_t)c * CHUNK_K + ks * 32);
-        char* stage = stage_of(stage_c) + kh * HALF_BYTES;
-#pragma unroll
-        for (int i = 0; i < X_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds(
-                (const void __attribute__((address_space(1)))*)(xsrc[i] + (size_t)c * ROW_BYTES),
-                (void __attribute__((address_space(3)))*)(stage + (TILES * i + tile) * 1024), 16, 0, 0);
-    };
-    constexpr int PER_CHUNK = KC + X_LOADS;           // vector-memory instructions a wave issues for a chunk
-    auto multiply = [&](auto stage_c) {
-        constexpr int S = decltype(stage_c)::value;
-        const char* stage = stage_of(stage_c);
-#pragma unroll
-        for (int ks = 0; ks < KC; ++ks)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const uint4 b = *(const uint4*)(stage + mt * (16 * ROW_BYTES) + b_at[ks]);
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(gmid_bf16x8, wreg[S][ks]), __builtin_bit_cast(gmid_bf16x8, b), acc[mt], 0, 0, 0);
-            }
-    };
-    // Chunk c has arrived when no more than the chunks after it are under way (loads return in order).  The bare
-    // barrier: __syncthreads() would wait for every load under way first.  After it everybody's part of chunk c is
-    // there, and everybody is done with chunk c - 1, whose stage chunk c + NS - 1 goes into.
-    auto full_step = [&](auto stage_c, int c) {              // chunks c + 1 .. c + NS - 1 exist
-        constexpr int S = decltype(stage_c)::value;
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(MID_VMCNT((NS - 2) * PER_CHUNK));
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        issue(std::integral_constant<int, (S + NS - 1) % NS>(), c + NS - 1);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(stage_c);
-    };
-    auto last_step = [&](auto stage_c, int c) {              // the last NS - 1 chunks: nothing left to ask for
-        __builtin_amdgcn_sched_barrier(0);
-        if (NS > 3 && c + 2 < nchunks) __builtin_amdgcn_s_waitcnt(MID_VMCNT(2 * PER_CHUNK));
-        else if (NS > 2 && c + 1 < nchunks) __builtin_amdgcn_s_waitcnt(MID_VMCNT(PER_CHUNK));
-        else __builtin_amdgcn_s_waitcnt(MID_VMCNT(0));
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(stage_c);
-    };
-    auto ring = [&](auto fn, int c) {                        // fn on chunks c .. c + NS - 1, each in its stage
-        fn(std::integral_constant<int, 0>(), c);
-        fn(std::integral_constant<int, 1>(), c + 1);
-        if constexpr (NS > 2) fn(std::integral_constant<int, 2>(), c + 2);
-        if constexpr (NS > 3) fn(std::integral_constant<int, 3>(), c + 3);
-    };
-    int c = 0;
-    if (nchunks >= 2 * NS - 1) {
-        // (a path of its own without a condition between the first loads and the loop: what is under way at the loop's
-        // head is then the same from both sides, and the compiler adds no wait of its own)
-        issue(std::integral_constant<int, 0>(), 0);
-        if constexpr (NS > 2) issue(std::integral_constant<int, 1>(), 1);
-        if constexpr (NS > 3) issue(std::integral_constant<int, 2>(), 2);
-        for (; c + 2 * NS - 1 <= nchunks; c += NS) ring(full_step, c);         // chunks up to c + 2 NS - 2 exist
-    } else {
-        if (nchunks > 0) issue(std::integral_constant<int, 0>(), 0);
-        if constexpr (NS > 2) { if (nchunks > 1) issue(std::integral_constant<int, 1>(), 1); }
-        if constexpr (NS > 3) { if (nchunks > 2) issue(std::integral_constant<int, 2>(), 2); }
-    }
-    // (c is a multiple of the number of stages here: chunk c + i lies in stage i % NS)
-    auto tail_step = [&](auto stage_c, int cc) {
-        if (cc >= nchunks) return;
-        if (cc + NS - 1 < nchunks) full_step(stage_c, cc);
-        else last_step(stage_c, cc);
-    };
-    ring(tail_step, c);
-    ring(tail_step, c + NS);
-
-    // ---- results: lane (r, g) holds features n_first + 4 g + i of row 16 mt + r ---------------------------------
-    // Sums meet in shared memory, in the stages' place: first the second share of k is added to the first, then (DUAL)
-    // the up rows' sums go to the waves that hold the gate rows' sums of the same features.
-    gmid_f32x4* swap_k = (gmid_f32x4*)mid_s0;                             // [TILES][MT][64 lanes]
-    gmid_f32x4* swap_up = (gmid_f32x4*)mid_s1;                            // [FEATURE_TILES][MT][64 lanes]
-    static_assert(TILES * MT * IA_WAVE * sizeof(gmid_f32x4) <= STAGE_BYTES, "the sums fit a stage");
-    if (KH == 2 || DUAL) __syncthreads();                                 // everybody is done with the stages
-    if constexpr (KH == 2) {
-        if (kh == 1) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) swap_k[(tile * MT + mt) * IA_WAVE + lane] = acc[mt];
-        }
-        __syncthreads();
-        if (kh == 0) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const gmid_f32x4 o = swap_k[(tile * MT + mt) * IA_WAVE + lane];
-                acc[mt][0] += o[0]; acc[mt][1] += o[1]; acc[mt][2] += o[2]; acc[mt][3] += o[3];
-            }
-        }
-    }
+    if (DUAL) __syncthreads();                                            // everybody is done with the stages
     if (DUAL) {
-        if (kh == 0 && part == 1) {
+        if (part == 1) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) swap_up[((tile % FEATURE_TILES) * MT + mt) * IA_WAVE + lane] = acc[mt];
         }
         __syncthreads();
-        if (kh != 0 || part != 0) return;
+        if (part != 0) return;
         const int nb = n_first + 4 * g;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -244,7 +83,6 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
         }
         return;
     }
-    if (kh != 0) return;
     const int nb = n_first + 4 * g;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -270,6 +108,145 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
             }
         }
     }
+}
+
+// KC: k steps of 32 in a chunk (a staged row is KC * 64 bytes); NS: stages, this chunk's and NS - 1 on their way.
+template <int MT, bool DUAL, int KC, int NS>
+__global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
+    void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+    int M, int N, int K, int k_per_block) {
+    constexpr int CHUNK_K = KC * 32;
+    constexpr int ROW_BYTES = KC * 64;
+    constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;
+    constexpr int PIECES = KC * 4;
+    constexpr int TILES = MID_WAVES;
+    constexpr int X_TILES = (MT + 1) / 2 * 2;               // tiles of x that are staged: an even number, so that the
+    constexpr int X_ROWS = X_TILES * 16;                    // loads divide between the waves
+    constexpr int W_ROWS = TILES * 16;
+    constexpr int ROWS = X_ROWS + W_ROWS;
+    constexpr int LOADS = ROWS / ROWS_PER_LOAD / MID_WAVES; // load instructions a wave issues for a stage
+    constexpr int STAGE_BYTES = ROWS * ROW_BYTES;
+    static_assert(NS >= 2 && NS <= 4 && (KC == 2 || KC == 4), "pipeline shape");
+    static_assert(ROWS % (ROWS_PER_LOAD * MID_WAVES) == 0, "the rows of a stage are shared out evenly between the waves");
+    __shared__ __attribute__((aligned(1024))) char mid_s0[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char mid_s1[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char mid_s2[NS > 2 ? STAGE_BYTES : 16];
+    __shared__ __attribute__((aligned(1024))) char mid_s3[NS > 3 ? STAGE_BYTES : 16];
+    auto stage_of = [&](auto stage_c) -> char* {
+        constexpr int S = decltype(stage_c)::value;
+        if constexpr (S == 0) return mid_s0;
+        else if constexpr (S == 1) return mid_s1;
+        else if constexpr (S == 2) return mid_s2;
+        else return mid_s3;
+    };
+    const int lane = threadIdx.x & (IA_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / IA_WAVE);
+    const int r = lane & 15, g = lane >> 4;
+    const int tile = wave;
+    const int split = blockIdx.y;
+    const int k_begin = split * k_per_block;
+    const int k_len = K - k_begin < k_per_block ? K - k_begin : k_per_block;
+    const int nchunks = k_len / CHUNK_K;
+    constexpr int FEATURE_TILES = DUAL ? TILES / 2 : TILES;
+    const int part = DUAL ? tile / FEATURE_TILES : 0;
+    const int n_first = blockIdx.x * (16 * FEATURE_TILES) + 16 * (tile % FEATURE_TILES);
+    // rows 16 t + i of a stage's 256-byte (or 128-byte) rows collide on the same banks for every i: a row's pieces are
+    // exchanged so that 16 rows at the same k fall on different places
+    auto swizzle = [](int row) { return KC == 4 ? (row & 15) : ((row >> 1) & 7); };
+
+    // ---- what this lane fetches of a stage: load i covers rows ROWS_PER_LOAD * (MID_WAVES i + wave) .. of the stage ----
+    const char* src[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int row = ROWS_PER_LOAD * (MID_WAVES * i + wave) + lane / PIECES;      // row of the stage
+        const int piece = (lane % PIECES) ^ swizzle(row);
+        const bf16_t* base;
+        if (row < X_ROWS) {
+            base = x + (size_t)(row < M ? row : 0) * K;                   // (rows beyond the step read row 0: never stored)
+        } else {
+            const int wr = row - X_ROWS, t = wr / 16;                          // weight row of the block: tile t, row wr % 16
+            const int pt = DUAL ? t / FEATURE_TILES : 0;
+            const int n = blockIdx.x * (16 * FEATURE_TILES) + 16 * (t % FEATURE_TILES) + (wr & 15);
+            base = w + ((size_t)pt * N + (n < N ? n : N - 1)) * K;        // (rows beyond the matrix: never stored)
+        }
+        src[i] = (const char*)(base + k_begin) + piece * 16;
+    }
+    uint32_t a_at[KC], b_at[KC];
+#pragma unroll
+    for (int ks = 0; ks < KC; ++ks) {
+        b_at[ks] = (uint32_t)(r * ROW_BYTES + (((4 * ks + g) ^ swizzle(r)) * 16));
+        a_at[ks] = (uint32_t)((X_ROWS + 16 * tile) * ROW_BYTES) + b_at[ks];
+    }
+    gmid_f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
+
+    auto issue = [&](auto stage_c, int c) {
+        char* stage = stage_of(stage_c);
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i)
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)(src[i] + (size_t)c * ROW_BYTES),
+                (void __attribute__((address_space(3)))*)(stage + (MID_WAVES * i + wave) * 1024), 16, 0, 0);
+    };
+    auto multiply = [&](auto stage_c) {
+        const char* stage = stage_of(stage_c);
+#pragma unroll
+        for (int ks = 0; ks < KC; ++ks) {
+            const uint4 a = *(const uint4*)(stage + a_at[ks]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint4 b = *(const uint4*)(stage + mt * (16 * ROW_BYTES) + b_at[ks]);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(gmid_bf16x8, a), __builtin_bit_cast(gmid_bf16x8, b), acc[mt], 0, 0, 0);
+            }
+        }
+    };
+    auto full_step = [&](auto stage_c, int c) {              // chunks c + 1 .. c + NS - 1 exist
+        constexpr int S = decltype(stage_c)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(MID_VMCNT((NS - 2) * LOADS));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue(std::integral_constant<int, (S + NS - 1) % NS>(), c + NS - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(stage_c);
+    };
+    auto last_step = [&](auto stage_c, int c) {              // the last NS - 1 chunks: nothing left to ask for
+        __builtin_amdgcn_sched_barrier(0);
+        if (NS > 3 && c + 2 < nchunks) __builtin_amdgcn_s_waitcnt(MID_VMCNT(2 * LOADS));
+        else if (NS > 2 && c + 1 < nchunks) __builtin_amdgcn_s_waitcnt(MID_VMCNT(LOADS));
+        else __builtin_amdgcn_s_waitcnt(MID_VMCNT(0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(stage_c);
+    };
+    auto ring = [&](auto fn, int c) {
+        fn(std::integral_constant<int, 0>(), c);
+        fn(std::integral_constant<int, 1>(), c + 1);
+        if constexpr (NS > 2) fn(std::integral_constant<int, 2>(), c + 2);
+        if constexpr (NS > 3) fn(std::integral_constant<int, 3>(), c + 3);
+    };
+    int c = 0;
+    if (nchunks >= 2 * NS - 1) {
+        issue(std::integral_constant<int, 0>(), 0);
+        if constexpr (NS > 2) issue(std::integral_constant<int, 1>(), 1);
+        if constexpr (NS > 3) issue(std::integral_constant<int, 2>(), 2);
+        for (; c + 2 * NS - 1 <= nchunks; c += NS) ring(full_step, c);
+    } else {
+        if (nchunks > 0) issue(std::integral_constant<int, 0>(), 0);
+        if constexpr (NS > 2) { if (nchunks > 1) issue(std::integral_constant<int, 1>(), 1); }
+        if constexpr (NS > 3) { if (nchunks > 2) issue(std::integral_constant<int, 2>(), 2); }
+    }
+    auto tail_step = [&](auto stage_c, int cc) {
+        if (cc >= nchunks) return;
+        if (cc + NS - 1 < nchunks) full_step(stage_c, cc);
+        else last_step(stage_c, cc);
+    };
+    ring(tail_step, c);
+    ring(tail_step, c + NS);
+    static_assert(!DUAL || TILES * MT * IA_WAVE * sizeof(gmid_f32x4) <= STAGE_BYTES, "the sums fit a stage");
+    mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split);
 }
 
 // How many ways k is split between blocks: a function of the weight's shape and the chip alone.  64 rows of w a
@@ -300,37 +277,29 @@ extern "C" int ia_gemm_mid_splits(int N, int K) {
     return splits;
 }
 
-// Tuning: k steps of a chunk (4 or 8), chunks in shared memory (2 to 4), and the share of k among a block's waves for
-// weights with the activation inside (1 or 2).  Measured at the sizes of an 8 B and a 32 B model, 32 and 64 rows: the
-// chunk shapes are within a tenth of each other; (4, 3) is the default (the smallest stages, so that most blocks fit a
-// compute unit).
-static int g_mid_kc = 4, g_mid_ns = 3, g_mid_dual_kh = 2;
-extern "C" void ia_gemm_mid_tune(int kc, int ns, int dual_kh) { g_mid_kc = kc; g_mid_ns = ns; g_mid_dual_kh = dual_kh; }
-
-template <int MT, bool DUAL, int KC, int NS, int KH>
-static void launch_mid_shape(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
-                             hipStream_t stream) {
-    constexpr int FEATURES = 16 * (MID_WAVES / KH) / (DUAL ? 2 : 1);        // output features of a block
-    const dim3 grid((N + FEATURES - 1) / FEATURES, splits);
-    gemm_mid_kernel<MT, DUAL, KC, NS, KH><<<grid, MID_WAVES * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, K / splits);
-}
+// The pipeline's shape: chunks of 128 k two deep, or three deep where the chip gets no more blocks than it has compute units
+// (a block a unit then, and what a block has under way is all that hides the memory's latency there: 4,096 x 12,288 at 64
+// rows 26.5 -> 22.8 us; with more blocks a unit the deeper stages only take room: 6,144 x 4,096 14.5 -> 17.0 us).  Every
+// shape adds an output's products up in the same order, so the choice may depend on the step (tested bit for bit).
+// ia_gemm_mid_tune(kc, ns): a fixed shape for measurements and tests (0, 0: the rule above); kc 2 or 4, ns 2 to 4.
+static int g_mid_kc = 0, g_mid_ns = 0;
+extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns; }
 
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
                       hipStream_t stream) {
+    constexpr int FEATURES = 16 * MID_WAVES / (DUAL ? 2 : 1);          // output features of a block
+    const dim3 grid((N + FEATURES - 1) / FEATURES, splits);
     const int k_block = K / splits;
-    // (a chunk must divide a wave's share of k, and a stage of MT * 16 rows must leave room in shared memory)
-    if constexpr (DUAL) {
-        // (two ways up to 32 rows: 2 x 12,288 x 4,096 at 20 rows 48.9 -> 42.4 us, at 32 rows 48.5 -> 46.6; beyond, twice as
-        // many blocks fetching all the rows of x cost more than the balance gains: 64 rows 56 -> 67 us)
-        if (g_mid_dual_kh == 2 && MT <= 2 && k_block % 256 == 0) {
-            launch_mid_shape<MT, true, 4, 3, 2>(out, out_mode, x, w, M, N, K, splits, stream);
-            return 0;
-        }
-    }
-    if (g_mid_kc == 8 && g_mid_ns == 2 && k_block % 256 == 0) launch_mid_shape<MT, DUAL, 8, 2, 1>(out, out_mode, x, w, M, N, K, splits, stream);
-    else if (g_mid_kc == 4 && g_mid_ns == 4) launch_mid_shape<MT, DUAL, 4, 4, 1>(out, out_mode, x, w, M, N, K, splits, stream);
-    else launch_mid_shape<MT, DUAL, 4, 3, 1>(out, out_mode, x, w, M, N, K, splits, stream);
+    int kc = g_mid_kc, ns = g_mid_ns;
+    if (kc == 0) { kc = 4; ns = (long long)grid.x * grid.y <= mid_cus() ? 3 : 2; }
+#define MID_SHAPE(KC, NS) gemm_mid_kernel<MT, DUAL, KC, NS><<<grid, MID_WAVES * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block)
+    if (kc == 4 && ns == 2) MID_SHAPE(4, 2);
+    else if (kc == 4 && ns == 3) MID_SHAPE(4, 3);
+    else if (kc == 2 && ns == 3) MID_SHAPE(2, 3);
+    else if (kc == 2 && ns == 4) MID_SHAPE(2, 4);
+    else IA_CHECK(false, "gemm_mid: no pipeline of chunks of %d k steps %d deep", kc, ns);
+#undef MID_SHAPE
     return 0;
 }
 
@@ -348,17 +317,19 @@ extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, 
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
     const int mt = (M + 15) / 16;
+    int rc = 0;
     if (dual) {
-        if (mt == 1) launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
-        else if (mt == 2) launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
-        else if (mt == 3) launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
-        else launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        else rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
     } else {
-        if (mt == 1) launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
-        else if (mt == 2) launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
-        else if (mt == 3) launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
-        else launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        else rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
     }
+    if (rc != 0) return rc;
     IA_LAUNCH_CHECK("gemm_mid");
     return 0;
 }

@@ -103,7 +103,7 @@ def library(target: str = "core"):
         lib.ia_attention_generic_workspace.restype = ctypes.c_longlong
         lib.ia_argmax_workspace.restype = ctypes.c_longlong
     _LIBS[target], _LIB_PATHS[target] = lib, path
-    return lib
+    return lib if KernelTimer.active is None else _Timed(lib)
 
 
 def library_files() -> Dict[str, str]:

@@ -805,6 +805,27 @@ def test_mid_product_rows_do_not_depend_on_the_batch():
     assert torch.equal(again.parts.cpu(), split.parts[:, 10:40].cpu())
 
 
+def test_which_kernels_a_gated_product_of_17_to_64_rows_takes(monkeypatch):
+    """[gate; up] at 17 to 64 rows: the kernel with the activation inside up to `MID_DUAL_MAX_BYTES`, the vendor's GEMM
+    and the SiLU kernel beyond, never the plain product of 17 to 64 rows with the SiLU kernel behind it; the same
+    values either way."""
+    from inferrs_amd import ops
+    x = dev(randn(32, 512, dtype=torch.bfloat16, seed=1))
+    w = dev(randn(2 * 640, 512, dtype=torch.bfloat16, seed=2, scale=0.05))
+    def entry_points():
+        with ops.KernelTimer() as timer:
+            out = ops.gated_silu_linear(x, w)
+        return out, set(timer.summary())
+    inside, names = entry_points()
+    assert names == {"gemm_mid_bf16"}
+    monkeypatch.setattr(ops, "MID_DUAL_MAX_BYTES", w.numel() * 2 - 1)
+    outside, names = entry_points()
+    assert names == {"vendor_gemm", "silu_mul"}
+    want = torch.nn.functional.silu(x.float() @ w[:640].float().t()) * (x.float() @ w[640:].float().t())
+    close(inside, want.cpu(), 2 ** -6, "activation inside")
+    close(outside, want.cpu(), 2 ** -6, "vendor's product and the SiLU kernel")
+
+
 @pytest.mark.parametrize("cols,add_one", [(128, False), (4096, False), (5120, True), (8192, False)])
 def test_add_rmsnorm_of_a_split_product(cols, add_one):
     """The norm kernel that adds up a product's splits equals the plain add-and-norm kernel on the stored product."""
@@ -823,9 +844,9 @@ def test_add_rmsnorm_of_a_split_product(cols, add_one):
 
 
 def test_mid_product_is_the_same_for_every_pipeline_shape():
-    """Chunks of 4 or 8 k steps and 2 to 4 of them in shared memory change when a value arrives, never the order of a
-    sum: the results are bit for bit the same.  Two waves sharing k for a [gate; up] weight add their halves in a fixed
-    order: another rounding than one wave's walk, the same for every batch of up to 32 rows."""
+    """Chunks of 64 or 128 k and two to four stages of them in shared memory change when a value arrives, never the
+    order of a sum: the results are bit for bit the same, with the activation inside as well, and a row's result is the
+    same whatever stands beside it."""
     from inferrs_amd import ops
     lib = ops.library()
     x = dev(randn(50, 2048, dtype=torch.bfloat16, seed=1))
@@ -833,21 +854,19 @@ def test_mid_product_is_the_same_for_every_pipeline_shape():
     wd = dev(randn(2 * 96, 2048, dtype=torch.bfloat16, seed=3, scale=0.05))
     try:
         outs = {}
-        for kc, ns, kh in ((4, 3, 1), (4, 4, 1), (8, 2, 1), (4, 3, 2), (8, 2, 2)):
-            lib.ia_gemm_mid_tune(kc, ns, kh)
-            outs[(kc, ns, kh)] = (ops.gemm_mid_bf16(x, w).cpu(), ops.gemm_mid_bf16(x, wd, dual=True).cpu(),
-                                  ops.gemm_mid_bf16(x[7:30].contiguous(), wd, dual=True).cpu(),
-                                  ops.gemm_mid_bf16(x[:32].contiguous(), wd, dual=True).cpu())
+        for kc, ns in ((0, 0), (4, 2), (4, 3), (2, 3), (2, 4)):
+            lib.ia_gemm_mid_tune(kc, ns)
+            outs[(kc, ns)] = (ops.gemm_mid_bf16(x, w).cpu(), ops.gemm_mid_bf16(x, wd, dual=True).cpu(),
+                              ops.gemm_mid_bf16(x[7:30].contiguous(), wd, dual=True).cpu(),
+                              ops.gemm_mid_bf16(x[:32].contiguous(), wd, dual=True).cpu())
+        lib.ia_gemm_mid_tune(8, 2)
+        with pytest.raises(ops.KernelError, match="no pipeline"):
+            ops.gemm_mid_bf16(x, w)
     finally:
-        lib.ia_gemm_mid_tune(4, 3, 2)
-    first = outs[(4, 3, 1)]
-    assert all(torch.equal(o[0], first[0]) for o in outs.values())
-    assert all(torch.equal(o[1], first[1]) for k, o in outs.items() if k[2] == 1)
-    assert torch.equal(outs[(4, 3, 2)][1], outs[(8, 2, 2)][1])
-    # rows do not see each other: within the steps that share k between two waves (up to 32 rows) and within those that do
-    # not, a row's result is the same whatever stands beside it
-    assert all(torch.equal(o[2], o[3][7:30]) for o in outs.values())
-    assert all(torch.equal(o[2], o[1][7:30]) for k, o in outs.items() if k[2] == 1)
+        lib.ia_gemm_mid_tune(0, 0)
+    first = outs[(0, 0)]
+    assert all(torch.equal(o[0], first[0]) and torch.equal(o[1], first[1]) for o in outs.values())
+    assert all(torch.equal(o[2], o[3][7:30]) and torch.equal(o[2], o[1][7:30]) for o in outs.values())
     gate = (x.float().cpu() @ wd[:96].float().cpu().t()).bfloat16().float()
     up = (x.float().cpu() @ wd[96:].float().cpu().t()).bfloat16().float()
     for o in outs.values():
