@@ -36,7 +36,6 @@
 typedef __bf16 gmid_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float gmid_f32x4 __attribute__((ext_vector_type(4)));
 
-#define MID_WAVES 4
 #define MID_CHUNK_MIN_K 128               // k is shared out in multiples of this
 
 // s_waitcnt that waits until at most n vector-memory operations of this wave are under way (gfx9 encoding:
@@ -110,24 +109,25 @@ __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* sw
     }
 }
 
-// KC: k steps of 32 in a chunk (a staged row is KC * 64 bytes); NS: stages, this chunk's and NS - 1 on their way.
-template <int MT, bool DUAL, int KC, int NS>
-__global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
+// KC: k steps of 32 in a chunk (a staged row is KC * 64 bytes); NS: stages, this chunk's and NS - 1 on their way; W: waves of
+// a block, a tile of 16 weight rows each (DUAL: W / 2 of gate rows, then W / 2 of up rows).
+template <int MT, bool DUAL, int KC, int NS, int W>
+__global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     int M, int N, int K, int k_per_block) {
     constexpr int CHUNK_K = KC * 32;
     constexpr int ROW_BYTES = KC * 64;
     constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;
     constexpr int PIECES = KC * 4;
-    constexpr int TILES = MID_WAVES;
-    constexpr int X_TILES = (MT + 1) / 2 * 2;               // tiles of x that are staged: an even number, so that the
-    constexpr int X_ROWS = X_TILES * 16;                    // loads divide between the waves
+    constexpr int TILES = W;
+    constexpr int X_ROWS = MT * 16;
     constexpr int W_ROWS = TILES * 16;
     constexpr int ROWS = X_ROWS + W_ROWS;
-    constexpr int LOADS = ROWS / ROWS_PER_LOAD / MID_WAVES; // load instructions a wave issues for a stage
-    constexpr int STAGE_BYTES = ROWS * ROW_BYTES;
+    constexpr int ROW_LOADS = ROWS / ROWS_PER_LOAD;         // load instructions (1 KiB each) that a stage's rows take
+    constexpr int LOADS = (ROW_LOADS + W - 1) / W;          // load instructions a wave issues for a stage; where they do not
+    constexpr int STAGE_BYTES = LOADS * W * 1024;           // divide, the last ones fetch a row of x again into a place nobody reads
+    static_assert(!DUAL || W % 2 == 0, "gate and up rows: an even number of waves");
     static_assert(NS >= 2 && NS <= 4 && (KC == 2 || KC == 4), "pipeline shape");
-    static_assert(ROWS % (ROWS_PER_LOAD * MID_WAVES) == 0, "the rows of a stage are shared out evenly between the waves");
     __shared__ __attribute__((aligned(1024))) char mid_s0[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char mid_s1[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char mid_s2[NS > 2 ? STAGE_BYTES : 16];
@@ -154,14 +154,14 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
     // exchanged so that 16 rows at the same k fall on different places
     auto swizzle = [](int row) { return KC == 4 ? (row & 15) : ((row >> 1) & 7); };
 
-    // ---- what this lane fetches of a stage: load i covers rows ROWS_PER_LOAD * (MID_WAVES i + wave) .. of the stage ----
+    // ---- what this lane fetches of a stage: load i covers rows ROWS_PER_LOAD * (W i + wave) .. of the stage ----
     const char* src[LOADS];
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
-        const int row = ROWS_PER_LOAD * (MID_WAVES * i + wave) + lane / PIECES;      // row of the stage
+        const int row = ROWS_PER_LOAD * (W * i + wave) + lane / PIECES;              // row of the stage
         const int piece = (lane % PIECES) ^ swizzle(row);
         const bf16_t* base;
-        if (row < X_ROWS) {
+        if (row < X_ROWS || row >= ROWS) {
             base = x + (size_t)(row < M ? row : 0) * K;                   // (rows beyond the step read row 0: never stored)
         } else {
             const int wr = row - X_ROWS, t = wr / 16;                          // weight row of the block: tile t, row wr % 16
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
         for (int i = 0; i < LOADS; ++i)
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)(src[i] + (size_t)c * ROW_BYTES),
-                (void __attribute__((address_space(3)))*)(stage + (MID_WAVES * i + wave) * 1024), 16, 0, 0);
+                (void __attribute__((address_space(3)))*)(stage + (W * i + wave) * 1024), 16, 0, 0);
     };
     auto multiply = [&](auto stage_c) {
         const char* stage = stage_of(stage_c);
@@ -249,9 +249,15 @@ __global__ __launch_bounds__(MID_WAVES * IA_WAVE) void gemm_mid_kernel(
     mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split);
 }
 
-// How many ways k is split between blocks: a function of the weight's shape and the chip alone.  64 rows of w a
-// block; splits double until there is a block for every compute unit or a split would fall below 512 k (with three blocks
-// for every two units a decode step of 32 requests took 2.71 ms where it takes 2.61 now: the splits' sums are traffic too).
+// How a weight is shared out: a function of its shape and the chip alone, never of the rows of the step.
+//   waves  tiles of 16 weight rows a block (DUAL: half of them gate rows, half the up rows of the same features)
+//   splits ways k is split between blocks (gridDim.y); the splits' sums are added up by the reader
+//   stages of the pipeline
+// Wanted: a block for every compute unit and no more, three stages deep (a block a unit: what it has under way is all that
+// hides the memory's latency; two rounds of blocks would leave the second half empty).  Among the ways that fill nine
+// tenths of the chip, the one with the most waves a block wins (the rows of x are fetched once a block) as long as a block
+// keeps eight chunks of k.  A weight that no way fits (a logits head: thousands of blocks) takes four waves a block two stages
+// deep, several blocks a unit, k split until there is a block for every unit.
 static int mid_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -263,43 +269,93 @@ static int mid_cus() {
     return cus;
 }
 
-// blocks wanted before k stops being split, in halves of the number of compute units
-static int g_mid_split_target = 2;
-extern "C" void ia_gemm_mid_split_target(int halves) { g_mid_split_target = halves; }
+struct MidPlan { int waves, splits, stages; };
+// a plan for measurements and tests: waves (0: the rule), splits, stages
+static MidPlan g_mid_forced = {0, 0, 0};
+extern "C" void ia_gemm_mid_plan(int waves, int splits, int stages) { g_mid_forced = {waves, splits, stages}; }
+
+#define MID_MAX_WAVES 8
+static MidPlan mid_plan(int N, int K, bool dual) {
+    const int cus = mid_cus();
+    const int tiles = (N + 15) / 16;                       // of a part
+    const int chunks = K / MID_CHUNK_MIN_K;
+    if (g_mid_forced.waves > 0) return g_mid_forced;
+    MidPlan best = {0, 0, 0};
+    double best_fill = 0.0;
+    bool best_long = false;
+    for (int t = 1; t <= (dual ? MID_MAX_WAVES / 2 : MID_MAX_WAVES); ++t) {
+        if (!dual && t < 2) continue;
+        const int blocks = (tiles + t - 1) / t;
+        for (int splits = 1; splits <= (dual ? 1 : 16); splits *= 2) {
+            if (chunks % splits || chunks / splits < 4) break;
+            if ((long long)blocks * splits > cus) break;
+            // the share of the chip's compute units that get a block, times the share of a block's tiles that are real
+            const double fill = (double)blocks * splits / cus * ((double)tiles / ((double)blocks * t));
+            const bool is_long = chunks / splits >= 8;
+            const bool better = fill > best_fill + 0.02 || (fill > best_fill - 0.02 && (is_long || !best_long));
+            if (best.waves == 0 || better) {
+                best = {dual ? 2 * t : t, splits, 3};
+                best_fill = fill > best_fill ? fill : best_fill;
+                best_long = is_long;
+            }
+        }
+    }
+    if (best.waves != 0 && best_fill >= 0.9) return best;
+    MidPlan wide = {4, 1, 2};
+    if (!dual) {
+        const int blocks = (N + 63) / 64;
+        while (blocks * wide.splits < cus && wide.splits < 16 && chunks % (2 * wide.splits) == 0 && chunks / (2 * wide.splits) >= 4)
+            wide.splits *= 2;
+    }
+    return wide;
+}
 
 extern "C" int ia_gemm_mid_splits(int N, int K) {
     if (N <= 0 || K <= 0 || K % MID_CHUNK_MIN_K) return 0;
-    const int blocks = (N + 63) / 64;
-    const int chunks = K / MID_CHUNK_MIN_K;
-    int splits = 1;
-    while (2 * blocks * splits < g_mid_split_target * mid_cus() && splits < 16 && chunks % (2 * splits) == 0 && chunks / (2 * splits) >= 4)
-        splits *= 2;
-    return splits;
+    return mid_plan(N, K, false).splits;
 }
 
-// The pipeline's shape: chunks of 128 k two deep, or three deep where the chip gets no more blocks than it has compute units
-// (a block a unit then, and what a block has under way is all that hides the memory's latency there: 4,096 x 12,288 at 64
-// rows 26.5 -> 22.8 us; with more blocks a unit the deeper stages only take room: 6,144 x 4,096 14.5 -> 17.0 us).  Every
-// shape adds an output's products up in the same order, so the choice may depend on the step (tested bit for bit).
-// ia_gemm_mid_tune(kc, ns): a fixed shape for measurements and tests (0, 0: the rule above); kc 2 or 4, ns 2 to 4.
+// ia_gemm_mid_tune(kc, ns): a fixed pipeline of four waves a block for tests (chunks of kc k steps, 2 or 4, ns deep;
+// 0, 0: the plan's own).  Every pipeline and every plan of the same splits adds an output's products up in the same order.
 static int g_mid_kc = 0, g_mid_ns = 0;
 extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns; }
 
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
                       hipStream_t stream) {
-    constexpr int FEATURES = 16 * MID_WAVES / (DUAL ? 2 : 1);          // output features of a block
-    const dim3 grid((N + FEATURES - 1) / FEATURES, splits);
+    MidPlan plan = mid_plan(N, K, DUAL);
+    if (out_mode != MID_OUT_PARTIAL && !DUAL && plan.splits != 1) {
+        // a stored product cannot be split: four waves a block over all of k
+        plan = {4, 1, 2};
+    }
+    if (g_mid_kc != 0) plan = {4, DUAL || out_mode != MID_OUT_PARTIAL ? 1 : plan.splits, g_mid_ns};
+    const int kc = g_mid_kc != 0 ? g_mid_kc : 4;
+    IA_CHECK(plan.splits == splits, "gemm_mid: the plan's %d splits against the caller's %d", plan.splits, splits);
+    const int features = 16 * plan.waves / (DUAL ? 2 : 1);            // output features of a block
+    const dim3 grid((N + features - 1) / features, splits);
     const int k_block = K / splits;
-    int kc = g_mid_kc, ns = g_mid_ns;
-    if (kc == 0) { kc = 4; ns = (long long)grid.x * grid.y <= mid_cus() ? 3 : 2; }
-#define MID_SHAPE(KC, NS) gemm_mid_kernel<MT, DUAL, KC, NS><<<grid, MID_WAVES * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block)
-    if (kc == 4 && ns == 2) MID_SHAPE(4, 2);
-    else if (kc == 4 && ns == 3) MID_SHAPE(4, 3);
-    else if (kc == 2 && ns == 3) MID_SHAPE(2, 3);
-    else if (kc == 2 && ns == 4) MID_SHAPE(2, 4);
-    else IA_CHECK(false, "gemm_mid: no pipeline of chunks of %d k steps %d deep", kc, ns);
+#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block)
+    if (kc == 4 && plan.stages == 3) {
+        switch (plan.waves) {
+            case 2: MID_SHAPE(4, 3, 2); return 0;
+            case 4: MID_SHAPE(4, 3, 4); return 0;
+            case 6: MID_SHAPE(4, 3, 6); return 0;
+            case 8: MID_SHAPE(4, 3, 8); return 0;
+        }
+        if constexpr (!DUAL) {
+            switch (plan.waves) {
+                case 3: MID_SHAPE(4, 3, 3); return 0;
+                case 5: MID_SHAPE(4, 3, 5); return 0;
+                case 7: MID_SHAPE(4, 3, 7); return 0;
+            }
+        }
+    } else if (plan.waves == 4) {
+        if (kc == 4 && plan.stages == 2) { MID_SHAPE(4, 2, 4); return 0; }
+        if (kc == 2 && plan.stages == 3) { MID_SHAPE(2, 3, 4); return 0; }
+        if (kc == 2 && plan.stages == 4) { MID_SHAPE(2, 4, 4); return 0; }
+    }
 #undef MID_SHAPE
+    IA_CHECK(false, "gemm_mid: no pipeline of %d waves, chunks of %d k steps, %d deep", plan.waves, kc, plan.stages);
     return 0;
 }
 
@@ -313,7 +369,7 @@ extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, 
     IA_CHECK(out_mode >= 0 && out_mode <= 2 && (!dual || out_mode == MID_OUT_BF16), "gemm_mid: output mode %d%s", out_mode,
              dual ? " does not go with the activation inside" : " is unknown");
     IA_CHECK((((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0, "gemm_mid: operands must be 16-byte aligned");
-    const int splits = out_mode == MID_OUT_PARTIAL ? ia_gemm_mid_splits(N, K) : 1;
+    const int splits = out_mode == MID_OUT_PARTIAL && !dual ? mid_plan(N, K, false).splits : 1;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
     const int mt = (M + 15) / 16;
