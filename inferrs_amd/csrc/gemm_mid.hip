@@ -180,13 +180,20 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     gmid_f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
+    // Blocks start at different places of their range of k and wrap around: blocks that are started together and walk k in
+    // step ask the same few memory channels at any moment (rows are a power of two apart).  The order of a sum depends
+    // on the block, that is on the output feature, never on the step's rows.
+    // (in steps of 128 k whatever the chunk, so that every pipeline shape adds up in the same order)
+    const int rot = k_len >= MID_CHUNK_MIN_K
+        ? (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)(k_len / MID_CHUNK_MIN_K)) * (MID_CHUNK_MIN_K / CHUNK_K) : 0;
 
     auto issue = [&](auto stage_c, int c) {
         char* stage = stage_of(stage_c);
+        const int cc = c + rot < nchunks ? c + rot : c + rot - nchunks;
 #pragma unroll
         for (int i = 0; i < LOADS; ++i)
             __builtin_amdgcn_global_load_lds(
-                (const void __attribute__((address_space(1)))*)(src[i] + (size_t)c * ROW_BYTES),
+                (const void __attribute__((address_space(1)))*)(src[i] + (size_t)cc * ROW_BYTES),
                 (void __attribute__((address_space(3)))*)(stage + (W * i + wave) * 1024), 16, 0, 0);
     };
     auto multiply = [&](auto stage_c) {
@@ -316,7 +323,8 @@ extern "C" int ia_gemm_mid_splits(int N, int K) {
 }
 
 // ia_gemm_mid_tune(kc, ns): a fixed pipeline of four waves a block for tests (chunks of kc k steps, 2 or 4, ns deep;
-// 0, 0: the plan's own).  Every pipeline and every plan of the same splits adds an output's products up in the same order.
+// 0, 0: the plan's own).  Every pipeline adds an output's products up in the same order; plans differ in where a block
+// starts its walk of k.
 static int g_mid_kc = 0, g_mid_ns = 0;
 extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns; }
 
