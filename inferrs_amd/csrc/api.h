@@ -72,11 +72,17 @@ int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N,
 // 2: out [ia_gemm_mid_splits(N, K)][M][N] float, the sums of each split of k, to be added up by the reader
 // (ia_sum_partials, ia_add_rmsnorm_partials).  dual: w = [gate; up], out = silu(x . gate^T) * (x . up^T), mode 0.
 int ia_gemm_mid_splits(int N, int K);
+// whether the weight's blocks fill the chip evenly, one a compute unit (dual: [gate; up] of N features each)
+int ia_gemm_mid_fills(int N, int K, int dual);
 // (a fixed pipeline for measurements and tests: k steps of a chunk, 2 or 4, and stages, 2 to 4; (0, 0): the kernel's own
 // rule; no product depends on it bit for bit)
 void ia_gemm_mid_tune(int kc, int ns);
 int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                      hipStream_t stream);
+// the same for up to 16 rows that are a norm's input times its weight, with their sums of squares sums_in [M][n_sums]: every sum
+// of the product is multiplied by the row's rsqrt(sum of sums_in / K + eps); out_mode 0 or 1
+int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
+                            const float* sums_in, int n_sums, float eps, hipStream_t stream);
 int ia_sum_partials(void* out, const float* part, int splits, int M, int N, hipStream_t stream);
 // x += (sum of the splits, rounded to bfloat16) in place, out = rmsnorm(x) * w; bfloat16 rows of up to 8192 features.
 int ia_add_rmsnorm_partials(void* out, void* x, const float* part, int splits, const float* w, float eps,

@@ -114,7 +114,7 @@ __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* sw
 template <int MT, bool DUAL, int KC, int NS, int W>
 __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-    int M, int N, int K, int k_per_block) {
+    int M, int N, int K, int k_per_block, const float* __restrict__ sums_in, int n_sums, float eps) {
     constexpr int CHUNK_K = KC * 32;
     constexpr int ROW_BYTES = KC * 64;
     constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;
@@ -153,6 +153,30 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     // rows 16 t + i of a stage's 256-byte (or 128-byte) rows collide on the same banks for every i: a row's pieces are
     // exchanged so that 16 rows at the same k fall on different places
     auto swizzle = [](int row) { return KC == 4 ? (row & 15) : ((row >> 1) & 7); };
+
+    // ---- rows that come scaled by a norm's weight, with their sums of squares block by block (sums_in [M][n_sums]; one tile
+    // of rows): every sum of the product is multiplied by the row's rsqrt(mean of squares + eps) before it is rounded.  The
+    // sums of squares are asked for now, before any stage (loads return in order: they are there when the stages are),
+    // a row a wave, and added up at the end in the order of the skinny product (a lane's four neighbours, its second four,
+    // then across the lanes), so that a row gets the same scale from both kernels.
+    constexpr int SS_ROWS = (16 + W - 1) / W;
+    float4 ss_mine[MT == 1 ? SS_ROWS : 1][2];
+    const bool ss_wide = MT == 1 && sums_in != nullptr && (n_sums & 3) == 0 && n_sums <= 8 * IA_WAVE;
+    if constexpr (MT == 1) {
+        if (ss_wide) {
+#pragma unroll
+            for (int j = 0; j < SS_ROWS; ++j) {
+                const int m = wave + j * W;
+#pragma unroll
+                for (int v = 0; v < 2; ++v) {
+                    const int at = 4 * (lane + v * IA_WAVE);
+                    ss_mine[j][v] = (m < M && at < n_sums) ? *(const float4*)(sums_in + (size_t)m * n_sums + at)
+                                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        }
+    }
+    __shared__ float mid_ss[16];
 
     // ---- what this lane fetches of a stage: load i covers rows ROWS_PER_LOAD * (W i + wave) .. of the stage ----
     const char* src[LOADS];
@@ -253,6 +277,27 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     ring(tail_step, c);
     ring(tail_step, c + NS);
     static_assert(!DUAL || TILES * MT * IA_WAVE * sizeof(gmid_f32x4) <= STAGE_BYTES, "the sums fit a stage");
+    if constexpr (MT == 1) {
+        if (sums_in != nullptr) {
+#pragma unroll
+            for (int j = 0; j < SS_ROWS; ++j) {
+                const int m = wave + j * W;
+                if (m >= M) continue;
+                float ss = 0.f;
+                if (ss_wide) {
+                    ss = ((ss_mine[j][0].x + ss_mine[j][0].y) + ss_mine[j][0].z) + ss_mine[j][0].w;
+                    ss += ((ss_mine[j][1].x + ss_mine[j][1].y) + ss_mine[j][1].z) + ss_mine[j][1].w;
+                } else {
+                    for (int b = lane; b < n_sums; b += IA_WAVE) ss += sums_in[(size_t)m * n_sums + b];
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) mid_ss[m] = ss;
+            }
+            __syncthreads();
+            const float scale = 1.0f / sqrtf(mid_ss[r < M ? r : 0] / (float)K + eps);
+            acc[0][0] *= scale; acc[0][1] *= scale; acc[0][2] *= scale; acc[0][3] *= scale;
+        }
+    }
     mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split);
 }
 
@@ -317,6 +362,12 @@ static MidPlan mid_plan(int N, int K, bool dual) {
     return wide;
 }
 
+// Whether the weight's blocks fill the chip evenly, one a compute unit, three stages deep (dual: [gate; up] of N features).
+extern "C" int ia_gemm_mid_fills(int N, int K, int dual) {
+    if (N <= 0 || K <= 0 || K % MID_CHUNK_MIN_K) return 0;
+    return mid_plan(N, K, dual != 0).stages == 3;
+}
+
 extern "C" int ia_gemm_mid_splits(int N, int K) {
     if (N <= 0 || K <= 0 || K % MID_CHUNK_MIN_K) return 0;
     return mid_plan(N, K, false).splits;
@@ -330,7 +381,7 @@ extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns;
 
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
-                      hipStream_t stream) {
+                      const float* sums_in, int n_sums, float eps, hipStream_t stream) {
     MidPlan plan = mid_plan(N, K, DUAL);
     if (out_mode != MID_OUT_PARTIAL && !DUAL && plan.splits != 1) {
         // a stored product cannot be split: four waves a block over all of k
@@ -342,7 +393,7 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
     const int features = 16 * plan.waves / (DUAL ? 2 : 1);            // output features of a block
     const dim3 grid((N + features - 1) / features, splits);
     const int k_block = K / splits;
-#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block)
+#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps)
     if (kc == 4 && plan.stages == 3) {
         switch (plan.waves) {
             case 2: MID_SHAPE(4, 3, 2); return 0;
@@ -370,8 +421,12 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
 // out_mode 0: out [M, N] bfloat16; 1: out [M, N] float; 2: out [splits][M][N] float with splits =
 // ia_gemm_mid_splits(N, K), to be added up by the reader.  dual: w = [gate; up] of N rows each, out = silu(x . gate^T)
 // * (x . up^T) in bfloat16 (mode 0 only).  M in 1..64, K a multiple of 128.
-extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
-                                hipStream_t stream) {
+// sums_in [M][n_sums] (or null): the rows of x are a norm's input times its weight, and every sum of the product is multiplied by
+// the row's rsqrt(sum of its sums_in / K + eps); up to 16 rows, whole sums only (no split of k).
+extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
+                                       const float* sums_in, int n_sums, float eps, hipStream_t stream) {
+    IA_CHECK(sums_in == nullptr || (M <= 16 && n_sums > 0 && out_mode != MID_OUT_PARTIAL && (((uintptr_t)sums_in) & 15) == 0),
+             "gemm_mid: rows with their sums of squares: up to 16 rows, whole sums (M=%d, n_sums=%d, mode %d)", M, n_sums, out_mode);
     IA_CHECK(M >= 1 && M <= 64 && N > 0 && K > 0, "gemm_mid: takes 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
     IA_CHECK(K % MID_CHUNK_MIN_K == 0, "gemm_mid: K=%d must be a multiple of %d (use another product)", K, MID_CHUNK_MIN_K);
     IA_CHECK(out_mode >= 0 && out_mode <= 2 && (!dual || out_mode == MID_OUT_BF16), "gemm_mid: output mode %d%s", out_mode,
@@ -383,19 +438,24 @@ extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, 
     const int mt = (M + 15) / 16;
     int rc = 0;
     if (dual) {
-        if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
-        else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
-        else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
-        else rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, stream);
+        if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
+        else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
+        else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
+        else rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
     } else {
-        if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
-        else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
-        else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
-        else rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, stream);
+        if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
+        else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
+        else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
+        else rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
     }
     if (rc != 0) return rc;
     IA_LAUNCH_CHECK("gemm_mid");
     return 0;
+}
+
+extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
+                                hipStream_t stream) {
+    return ia_gemm_mid_bf16_scaled(out, x, w, M, N, K, out_mode, dual, nullptr, 0, 0.f, stream);
 }
 
 // ---- readers of the splits' sums ------------------------------------------------------------------------------

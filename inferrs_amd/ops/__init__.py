@@ -76,7 +76,7 @@ class _Timed:
         fn = getattr(self._lib, name)
         if KernelTimer.active is None or not name.startswith("ia_") or name.endswith(("_workspace", "_blocks", "_block_rows",
                                                                                       "_error", "_version", "_capacity", "_top",
-                                                                                      "_splits", "_tune", "_target", "_counters")):
+                                                                                      "_splits", "_tune", "_target", "_counters", "_fills", "_plan")):
             return fn
         timer = KernelTimer.active
         return lambda *args: timer.call(name[3:], fn, *args)
@@ -727,19 +727,21 @@ class Partials:
         return out
 
 
-def mid_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+def mid_fits(x: torch.Tensor, w: torch.Tensor, few_rows: bool = False) -> bool:
+    """Whether x . w^T goes to gemm_mid.hip: 17 to 64 rows (`few_rows`: 1 to 64)."""
     if MID_PRODUCTS not in ("own", "library"):
         raise KernelError(f"INFERRS_AMD_MID_PRODUCTS / ops.MID_PRODUCTS: 'own' or 'library', not {MID_PRODUCTS!r}")
     return (MID_PRODUCTS == "own" and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-            and SKINNY_MAX_ROWS < x.shape[0] <= MID_MAX_ROWS and x.shape[1] % 128 == 0 and w.shape[1] == x.shape[1]
+            and (0 if few_rows else SKINNY_MAX_ROWS) < x.shape[0] <= MID_MAX_ROWS and x.shape[1] % 128 == 0 and w.shape[1] == x.shape[1]
             and x.is_contiguous() and w.is_contiguous() and (x.data_ptr() | w.data_ptr()) % 16 == 0)
 
 
 def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, dual: bool = False,
-                  partial: bool = False):
+                  partial: bool = False, sums_in: Optional[torch.Tensor] = None, eps: float = 0.0):
     """x [m, k] . w[n, k]^T for 1 to 64 bfloat16 rows and k a multiple of 128 (gemm_mid.hip).  `dual`: w = [gate; up],
     the result silu(x . gate^T) * (x . up^T).  `partial`: the result stays split along k, as `Partials` (a weight that
-    needs no split gives a plain tensor)."""
+    needs no split gives a plain tensor).  `sums_in` [m, blocks] (up to 16 rows): the rows are a norm's input times its
+    weight and these their sums of squares; every sum is multiplied by the row's rsqrt(mean of squares + eps)."""
     _dev(x, w)
     m, k = x.shape
     rows, k2 = w.shape
@@ -756,6 +758,13 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = tor
             _check(lib.ia_gemm_mid_bf16(_p(parts), _p(x), _p(w), m, n, k, 2, 0, _stream()))
             return Partials(parts)
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if sums_in is not None:
+        _dev(sums_in); _f32(sums_in, "sums of squares")
+        if partial or m > 16 or sums_in.dim() != 2 or sums_in.shape[0] != m or not sums_in.is_contiguous():
+            raise KernelError(f"gemm_mid: sums of squares {tuple(sums_in.shape)} for {m} rows (up to 16, whole sums)")
+        _check(lib.ia_gemm_mid_bf16_scaled(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
+                                           int(dual), _p(sums_in), sums_in.shape[1], ctypes.c_float(eps), _stream()))
+        return out
     _check(lib.ia_gemm_mid_bf16(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
                                 int(dual), _stream()))
     return out
@@ -907,16 +916,29 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return out if n_top is None else (out, lp, ids)
 
 
+def _mid_dual_fits(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
+    """[gate; up] at up to 16 rows on gemm_mid.hip: where the weight makes a block for every compute unit."""
+    return (w_gate_up.shape[0] % 2 == 0 and mid_fits(x, w_gate_up, few_rows=True)
+            and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES
+            and bool(library().ia_gemm_mid_fills(w_gate_up.shape[0] // 2, w_gate_up.shape[1], 1)))
+
+
 def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(x . gate^T) * (x . up^T) for w_gate_up = [gate; up]: one fused kernel for few bfloat16
     rows, else the product followed by the element-wise kernel."""
+    # (few rows too go to gemm_mid.hip where its blocks fill the chip evenly: inside a decode step the pair of this product
+    # and the next takes 58.0 us against 60.6 at 8 rows and 60.4 against 67.2 at 16, sizes of an 8B model)
     if isinstance(x, NormedRows):
         if w_gate_up.shape[0] % 2 == 0 and _takes_normed_rows(x, w_gate_up, w_gate_up.shape[0] // 2):
             _dev(x.scaled, w_gate_up, x.sums)
+            if _mid_dual_fits(x.scaled, w_gate_up):
+                return gemm_mid_bf16(x.scaled, w_gate_up, dual=True, sums_in=x.sums, eps=x.eps)
             return _stream_product(x.scaled, w_gate_up, w_gate_up.shape[0] // 2, x.scaled.dtype, True,
                                    sums_in=x.sums, eps=x.eps)
         x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
+        if _mid_dual_fits(x, w_gate_up):
+            return gemm_mid_bf16(x, w_gate_up, dual=True)
         return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True)
     if (w_gate_up.shape[0] % 2 == 0 and mid_fits(x, w_gate_up)
             and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES):

@@ -533,6 +533,40 @@ def test_products_around_a_residual_stream(m, n, k, n2, add_one):
     assert only[1] is None and torch.equal(only[0], sums)
 
 
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("blocks", [32, 30])
+def test_gated_product_of_few_normed_rows_on_blocks_that_fill_the_chip(m, blocks, monkeypatch):
+    """A [gate; up] whose blocks fill the chip evenly (12,288 features: 256 blocks of 48) takes the kernel of 17 to 64
+    rows also for few rows, with the norm's end inside (the rows' sums of squares, in fours or one by one): against the
+    exact result, against the skinny product's way, and a row does not depend on its batch."""
+    from inferrs_amd import ops
+    k, n2 = 512, 12288
+    x = randn(m, k, dtype=torch.bfloat16, seed=41, scale=2.0)
+    gain = 1.0 + 0.1 * randn(k, dtype=torch.float32, seed=42)
+    w3 = dev(randn(2 * n2, k, dtype=torch.bfloat16, seed=43, scale=0.05))
+    scaled = (x.float() * gain).to(torch.bfloat16)
+    sums = x.float().pow(2).view(m, blocks, -1).sum(-1) if k % blocks == 0 else \
+        torch.cat([x.float().pow(2)[:, :17 * (blocks - 1)].reshape(m, blocks - 1, 17).sum(-1),
+                   x.float().pow(2)[:, 17 * (blocks - 1):].sum(-1, keepdim=True)], 1)
+    assert sums.shape == (m, blocks)
+    rows = ops.NormedRows(dev(x), dev(scaled), dev(sums.contiguous()), dev(gain), 1e-6, False)
+    assert ops.library().ia_gemm_mid_fills(n2, k, 1) == 1
+    with ops.KernelTimer() as timer:
+        got = ops.gated_silu_linear(rows, w3)
+    assert set(timer.summary()) == {"gemm_mid_bf16_scaled"}
+    part = ops.NormedRows(dev(x[m // 3:]), dev(scaled[m // 3:].contiguous()), dev(sums[m // 3:].contiguous()), dev(gain), 1e-6, False)
+    assert torch.equal(ops.gated_silu_linear(part, w3), got[m // 3:])
+    monkeypatch.setattr(ops, "MID_PRODUCTS", "library")
+    with ops.KernelTimer() as timer:
+        skinny = ops.gated_silu_linear(rows, w3)
+    assert set(timer.summary()) == {"gemm_skinny_stream"}
+    exact = scaled.double() / torch.sqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-6)
+    g = (exact @ w3[:n2].double().cpu().t()).to(torch.bfloat16).double()
+    want = g / (1 + torch.exp(-g)) * (exact @ w3[n2:].double().cpu().t()).to(torch.bfloat16).double()
+    close(got, want, 2 ** -6, "with the norm's end inside")
+    close(got, skinny, 2 ** -7, "against the skinny product")
+
+
 def test_products_leave_the_stream_alone_where_they_cannot_take_it():
     from inferrs_amd import ops
     # more rows than the skinny product takes, or a 32-bit stream: the product does not add itself
