@@ -8,6 +8,18 @@
 #include "common.h"
 #include "api.h"
 
+// A row copied by a block: 16 bytes a thread at a time where the row's size and both addresses allow it.
+template <typename T>
+__device__ __forceinline__ void copy_row(T* __restrict__ dst, const T* __restrict__ src, int n) {
+    const size_t bytes = (size_t)n * sizeof(T);
+    if ((bytes & 15) == 0 && (((uintptr_t)dst | (uintptr_t)src) & 15) == 0) {
+        const int pieces = (int)(bytes / 16);
+        for (int c = threadIdx.x; c < pieces; c += blockDim.x) ((uint4*)dst)[c] = ((const uint4*)src)[c];
+    } else {
+        for (int c = threadIdx.x; c < n; c += blockDim.x) dst[c] = src[c];
+    }
+}
+
 // ---- embedding ------------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_gather_kernel(T* __restrict__ out, const T* __restrict__ table,
@@ -17,10 +29,8 @@ __global__ void embed_gather_kernel(T* __restrict__ out, const T* __restrict__ t
     const bool ok = id >= 0 && id < vocab;
     const T* src = table + (size_t)(ok ? id : 0) * hidden;
     T* dst = out + (size_t)row * hidden;
-    for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-        if (ok) dst[c] = src[c];
-        else st(dst + c, 0.f);
-    }
+    if (ok) { copy_row(dst, src, hidden); return; }
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) st(dst + c, 0.f);
 }
 
 extern "C" int ia_embed_gather(void* out, const void* table, const int* ids, int n, int hidden,
@@ -42,9 +52,7 @@ extern "C" int ia_embed_gather(void* out, const void* table, const int* ids, int
 template <typename T>
 __global__ void gather_rows_kernel(T* __restrict__ out, const T* __restrict__ x,
                                    const int* __restrict__ rows, int cols) {
-    const T* src = x + (size_t)rows[blockIdx.x] * cols;
-    T* dst = out + (size_t)blockIdx.x * cols;
-    for (int c = threadIdx.x; c < cols; c += blockDim.x) dst[c] = src[c];
+    copy_row(out + (size_t)blockIdx.x * cols, x + (size_t)rows[blockIdx.x] * cols, cols);
 }
 
 extern "C" int ia_gather_rows(void* out, const void* x, const int* rows, int n, int cols,

@@ -27,13 +27,8 @@
 #include "api.h"
 
 // ---- greedy ---------------------------------------------------------------------------------
-__device__ __forceinline__ void argmax_row(const float* __restrict__ row, int vocab, float* sv, int* si, int* out) {
-    float best = -INFINITY;
-    int idx = 0x7fffffff;
-    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-        const float v = row[c];
-        if (v > best || (v == best && c < idx)) { best = v; idx = c; }
-    }
+// every thread's best (value, index; 0x7fffffff: none) -> the block's, the lowest index among equal maxima, in *out
+__device__ __forceinline__ void argmax_block(float best, int idx, float* sv, int* si, int* out) {
 #pragma unroll
     for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, IA_WAVE);
@@ -50,6 +45,16 @@ __device__ __forceinline__ void argmax_row(const float* __restrict__ row, int vo
             if (sv[w] > best || (sv[w] == best && si[w] < idx)) { best = sv[w]; idx = si[w]; }
         *out = idx == 0x7fffffff ? 0 : idx;       // a row of NaN or -inf
     }
+}
+
+__device__ __forceinline__ void argmax_row(const float* __restrict__ row, int vocab, float* sv, int* si, int* out) {
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+        const float v = row[c];
+        if (v > best || (v == best && c < idx)) { best = v; idx = c; }
+    }
+    argmax_block(best, idx, sv, si, out);
 }
 
 __global__ __launch_bounds__(1024) void argmax_kernel(int* __restrict__ out, const float* __restrict__ logits, int vocab) {
@@ -69,7 +74,31 @@ __global__ __launch_bounds__(256) void argmax_stretch_kernel(float* __restrict__
     const int lo = stretch * ARGMAX_STRETCH;
     const int len = vocab - lo < ARGMAX_STRETCH ? vocab - lo : ARGMAX_STRETCH;
     int idx;
-    argmax_row(logits + (size_t)row * vocab + lo, len, sv, si, &idx);
+    if ((vocab & 3) == 0 && ((uintptr_t)logits & 15) == 0) {
+        // four neighbours a load and all of a thread's loads under way together (one after the other, each waiting for
+        // its own, a stretch took 16 us)
+        constexpr int PER = ARGMAX_STRETCH / 4 / 256;
+        const float4* src = (const float4*)(logits + (size_t)row * vocab + lo);
+        float4 v[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int c = (j * 256 + (int)threadIdx.x) * 4;
+            v[j] = c < len ? src[c / 4] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        }
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int c = (j * 256 + (int)threadIdx.x) * 4;
+            const float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (c + i < len && (e[i] > best || (e[i] == best && c + i < at))) { best = e[i]; at = c + i; }
+        }
+        argmax_block(best, at, sv, si, &idx);
+    } else {
+        argmax_row(logits + (size_t)row * vocab + lo, len, sv, si, &idx);
+    }
     if (threadIdx.x == 0) {
         cand_i[(size_t)row * gridDim.x + stretch] = lo + idx;
         cand_v[(size_t)row * gridDim.x + stretch] = logits[(size_t)row * vocab + lo + idx];
