@@ -77,6 +77,9 @@ int ia_gemm_mid_fills(int N, int K, int dual);
 // (a fixed pipeline for measurements and tests: k steps of a chunk, 2 or 4, and stages, 2 to 4; (0, 0): the kernel's own
 // rule; no product depends on it bit for bit)
 void ia_gemm_mid_tune(int kc, int ns);
+// (a fixed shape of the blocks for measurements and tests: waves a block, 2 to 8 (0: the kernel's own rule), ways k is split
+// and stages, 2 or 3 (2: four waves only); the caller's partial sums must have as many splits)
+void ia_gemm_mid_plan(int waves, int splits, int stages);
 int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                      hipStream_t stream);
 // the same for up to 16 rows that are a norm's input times its weight, with their sums of squares sums_in [M][n_sums]: every sum

@@ -839,6 +839,38 @@ def test_mid_product_rows_do_not_depend_on_the_batch():
     assert torch.equal(again.parts.cpu(), split.parts[:, 10:40].cpu())
 
 
+@pytest.mark.parametrize("m", [5, 33, 64])
+def test_mid_product_with_every_shape_of_block(m):
+    """The rule picks the waves of a block and the split of k by the weight's shape; here every shape is forced on one
+    weight (features that fill no block, rows that fill no tile): plain with its sums split two ways, and with the
+    activation inside."""
+    from inferrs_amd import ops
+    lib = ops.library()
+    n, k = 300, 1024
+    x = dev(randn(m, k, dtype=torch.bfloat16, seed=1))
+    w = dev(randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05))
+    wd = dev(randn(2 * n, k, dtype=torch.bfloat16, seed=3, scale=0.05))
+    want = x.float().cpu() @ w.float().cpu().t()
+    gate = (x.float().cpu() @ wd[:n].float().cpu().t()).bfloat16().float()
+    up = (x.float().cpu() @ wd[n:].float().cpu().t()).bfloat16().float()
+    try:
+        for waves in range(2, 9):
+            lib.ia_gemm_mid_plan(waves, 2, 3)
+            assert lib.ia_gemm_mid_splits(n, k) == 2
+            parts = ops.gemm_mid_bf16(x, w, partial=True)
+            assert isinstance(parts, ops.Partials) and parts.parts.shape[0] == 2
+            close(parts.materialize(), want, 2 ** -8, f"{waves} waves a block")
+            if waves % 2 == 0:
+                lib.ia_gemm_mid_plan(waves, 1, 3)
+                close(ops.gemm_mid_bf16(x, wd, dual=True), gate / (1 + torch.exp(-gate)) * up, 2 ** -7,
+                      f"{waves} waves a block with SiLU")
+        lib.ia_gemm_mid_plan(9, 1, 3)
+        with pytest.raises(ops.KernelError, match="no pipeline"):
+            ops.gemm_mid_bf16(x, wd, dual=True)
+    finally:
+        lib.ia_gemm_mid_plan(0, 0, 0)
+
+
 def test_which_kernels_a_gated_product_of_17_to_64_rows_takes(monkeypatch):
     """[gate; up] at 17 to 64 rows: the kernel with the activation inside up to `MID_DUAL_MAX_BYTES`, the vendor's GEMM
     and the SiLU kernel beyond, never the plain product of 17 to 64 rows with the SiLU kernel behind it; the same
