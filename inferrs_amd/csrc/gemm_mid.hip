@@ -1,32 +1,38 @@
 // bfloat16 products for steps of 17 to 64 rows (decode steps of many requests, short prompt portions):
 // out[M, N] = x[M, K] . w[N, K]^T, bound by reading the weights once, like the skinny product, but with so
 // many rows that the activations can no longer be fetched by every wave for itself (at 64 rows they are as
-// large as a block's share of the weights).
+// large as a block's share of the weights).  A [gate; up] whose blocks fill the chip evenly comes here with fewer rows
+// too (ia_gemm_mid_bf16_scaled: rows of a residual stream whose norm the product finishes).
 //
 // The reference hands these products to cuBLAS like all others (`candle-core/src/cuda_backend/mod.rs:2260-2305`).
 //
-// A block of four waves owns 64 rows of w and a range of k, and walks it in chunks of 128.  A stage of shared memory
-// holds a chunk's rows of x (up to 64) and the block's 64 rows of w alike, 256 bytes a row, brought by all four waves
-// together straight from memory (global_load_lds: 16 bytes a lane, four whole rows an instruction, no register on the
-// way), one or two stages ahead of their use.  A wave multiplies its tile of 16 weight rows (the MFMA A-operand:
+// A block of W waves (2 to 8) owns 16 W rows of w and a range of k, and walks it in chunks of 128, each block from another
+// place of its range (blocks that are started together and walk in step ask the same few memory channels at any moment).
+// A stage of shared memory holds a chunk's rows of x (up to 64) and the block's rows of w alike, 256 bytes a row, brought by
+// all waves together straight from memory (global_load_lds: 16 bytes a lane, four whole rows an instruction, no register on
+// the way), one or two stages ahead of their use.  A wave multiplies its tile of 16 weight rows (the MFMA A-operand:
 // v_mfma_f32_16x16x32_bf16, lane l supplies row l % 16 with the eight k values 8 * (l / 16) .. + 8) with every row tile of
 // x, both read from the stage.  Piece c (16 bytes) of row r lies at place c ^ (r % 16) of the row's 256 bytes, so that the
 // 16 rows which one operand read takes at the same k fall on 16 different places; a load instruction fills 1 KiB (four
 // rows) in lane order, and the lane picks the piece it fetches accordingly.
+//
+// How many waves a block has and how k is split follow from the weight's shape (mid_plan below): the chip should get a block
+// for every compute unit and no more, three stages deep; a weight that no such shape fits takes four waves a block, two
+// stages and several blocks a unit.
 //
 // The weights went straight from memory into the A-operands before (a load of 16 rows x 64 bytes a lane group): such a
 // load holds the compute unit's address unit for about 86 cycles, a load of 1 KiB in whole rows for about 32, and by its
 // own clocks that kernel spent 40 % of a step issuing its loads at 64 rows.  Through shared memory: q|k|v of 6,144 x
 // 4,096 at 64 rows 17.1 -> 14.5 us, [gate; up] with the activation 56 -> 50, the 32B shape's 5,120 x 25,600 82 -> 69.
 //
-// With few rows of w (the output projection, the feed-forward's second product) 64 rows a block leave too few
+// With few rows of w (the output projection, the feed-forward's second product) whole columns of k leave too few
 // blocks to fill the chip, so k is split between blocks (gridDim.y) and every split leaves its sums in 32-bit:
 // [splits][M][N].  They are added up, in the order of the splits, by whoever reads them: the kernel that adds a
 // product to the residual stream and norms it (ia_add_rmsnorm_partials), or ia_sum_partials.  The split depends
 // on the weight's shape alone, never on the rows of the step.
 //
-// DUAL: w = [gate; up] (N rows each); a block owns 32 output features, waves 0 and 1 their gate rows, waves 2 and 3
-// their up rows, and the result is silu(gate . x) * (up . x), the first product rounded to bfloat16 before the
+// DUAL: w = [gate; up] (N rows each); a block owns 8 W output features, the first half of its waves their gate rows, the
+// second half their up rows, and the result is silu(gate . x) * (up . x), the first product rounded to bfloat16 before the
 // activation as the two-kernel path rounds it.  No split of k (the activation needs whole sums).
 #include <type_traits>
 
