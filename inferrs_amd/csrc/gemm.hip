@@ -218,16 +218,24 @@ extern "C" int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int
     IA_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     if (M == 0) return 0;
     const size_t elem = in_dtype == IA_F32 ? 4 : 2;
-    if (M <= GR_ROWS && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) % (4 * elem)) == 0) {
+    // up to 64 rows, 16 at a time, where the tiles of 64 x 64 would be few (the weights are read once for every 16 rows:
+    // at 32 rows of the 32-bit path a decode step of four layers at the sizes of an 8B model still takes a third of the time)
+    if (M <= 4 * GR_ROWS && (M <= GR_ROWS || N <= 4096 * 4) && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) % (4 * elem)) == 0) {
         const unsigned blocks = (unsigned)((N + GR_N - 1) / GR_N);
-        if (in_dtype == IA_F32 && out_dtype == IA_F32)
-            gemm_rows_kernel<float, float><<<blocks, IA_WAVE, 0, stream>>>((float*)out, (const float*)x, (const float*)w, M, N, K);
-        else if (in_dtype == IA_BF16 && out_dtype == IA_BF16)
-            gemm_rows_kernel<bf16_t, bf16_t><<<blocks, IA_WAVE, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
-        else if (in_dtype == IA_BF16 && out_dtype == IA_F32)
-            gemm_rows_kernel<bf16_t, float><<<blocks, IA_WAVE, 0, stream>>>((float*)out, (const bf16_t*)x, (const bf16_t*)w, M, N, K);
-        else
-            IA_CHECK(false, "gemm_tiled: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+        const size_t out_elem = out_dtype == IA_F32 ? 4 : 2;
+        for (int m0 = 0; m0 < M; m0 += GR_ROWS) {
+            const int rows = M - m0 < GR_ROWS ? M - m0 : GR_ROWS;
+            void* o = (char*)out + (size_t)m0 * N * out_elem;
+            const void* xi = (const char*)x + (size_t)m0 * K * elem;
+            if (in_dtype == IA_F32 && out_dtype == IA_F32)
+                gemm_rows_kernel<float, float><<<blocks, IA_WAVE, 0, stream>>>((float*)o, (const float*)xi, (const float*)w, rows, N, K);
+            else if (in_dtype == IA_BF16 && out_dtype == IA_BF16)
+                gemm_rows_kernel<bf16_t, bf16_t><<<blocks, IA_WAVE, 0, stream>>>((bf16_t*)o, (const bf16_t*)xi, (const bf16_t*)w, rows, N, K);
+            else if (in_dtype == IA_BF16 && out_dtype == IA_F32)
+                gemm_rows_kernel<bf16_t, float><<<blocks, IA_WAVE, 0, stream>>>((float*)o, (const bf16_t*)xi, (const bf16_t*)w, rows, N, K);
+            else
+                IA_CHECK(false, "gemm_tiled: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+        }
         IA_LAUNCH_CHECK("gemm_rows");
         return 0;
     }
