@@ -13,9 +13,9 @@
 // neighbouring features of one row of the result: an 8-byte store.  Blocks stay on their compute units and take
 // tile after tile.
 //
-// Shared memory: a row of 64 bytes holds four 16-byte pieces; piece c of row r lies at place c ^ ((r >> 2) & 3),
-// so that the 16 rows that lanes read at the same k fall into 16 different places of the 256 bytes that the banks
-// cover.  A load instruction fills 1 KiB (16 rows) in lane order: the lane picks the piece it fetches accordingly.
+// Shared memory: a row of 64 bytes holds four 16-byte pieces; piece c of row r lies at place c ^ ((r >> 1) & 3),
+// so that the eight rows that a read takes in one cycle (eight lanes, 128 bytes: the banks cover 128 bytes) fall on
+// eight different places of them (with (r >> 2) & 3 rows r and r + 2 met on the same banks: twice the cycles).  A load instruction fills 1 KiB (16 rows) in lane order: the lane picks the piece it fetches accordingly.
 //
 // Measured at 2,048 rows and the sizes of an 8 B model (TFLOP/s; the vendor's GEMM in brackets, for gate|up with its
 // SiLU kernel): gate|up 1,081 (1,240; with the SiLU kernel 382 against 332 + 30 us), qkv 1,041 (1,265: 192 tiles on
@@ -101,7 +101,7 @@ void gemm_mfma_kernel(const GemmMfmaParams p) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int row = ((i & 3) * 4 + wave) * 16 + (lane >> 2);       // row of the operand's tile
-        const int piece = (lane & 3) ^ ((row >> 2) & 3);
+        const int piece = (lane & 3) ^ ((row >> 1) & 3);
         if (i < 4) {
             int m = m0 + row;
             m = m < p.M ? m : p.M - 1;
@@ -129,10 +129,10 @@ void gemm_mfma_kernel(const GemmMfmaParams p) {
                   lds0 + (uint32_t)(slot & (GM_RING - 1)) * GM_STAGE + (i < 4 ? 0 : GM_TILE) + (uint32_t)((i & 3) * 4 + wave) * 1024);
     };
     // ---- the wave's share: rows wm * 128 .. of x, rows wn * 128 .. of w -------------------------------------
-    // Shared memory: a row of 64 bytes holds four 16-byte pieces; piece c of row r lies at place c ^ ((r >> 2) & 3), so
-    // that the 16 rows that lanes read at the same k fall into 16 different places of the 256 bytes the banks cover.
+    // Shared memory: a row of 64 bytes holds four 16-byte pieces; piece c of row r lies at place c ^ ((r >> 1) & 3), so
+    // that the eight rows which a read takes in one cycle fall on eight different places of the 128 bytes the banks cover.
     const int wm = wave & 1, wn = wave >> 1;
-    const uint32_t at = (uint32_t)(r * GM_ROW + ((g ^ ((r >> 2) & 3)) * 16));      // the lane's place in a 16-row tile
+    const uint32_t at = (uint32_t)(r * GM_ROW + ((g ^ ((r >> 1) & 3)) * 16));      // the lane's place in a 16-row tile
     const uint32_t x_at = (uint32_t)(wm * 128 * GM_ROW) + at, w_at = (uint32_t)(GM_TILE + wn * 128 * GM_ROW) + at;
 
     gm_f32x4 acc[8][8];                 // [tile of w rows][tile of x rows]
