@@ -43,6 +43,9 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--random-weights", action="store_true",
                    help="seeded random weights for the folder's config.json instead of its safetensors")
     p.add_argument("--seed", type=int, default=None, help="sampling seed (and weight seed with --random-weights)")
+    p.add_argument("--allow-ignored-keys", action="store_true",
+                   help="load a config.json that asks for what the architecture does not do (attention bias, scaled "
+                        "rotation, a sliding window, another activation) and ignore those keys, as the reference does")
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -85,8 +88,9 @@ def load_engine(args):
         options["memory_fraction"] = args.paged_attention
     print(f"inferrs-amd: loading {args.model} ({dtype})", file=sys.stderr, flush=True)
     if args.random_weights:
-        return Engine.from_random(load_config(args.model), seed=args.seed or 0, **options)
-    return Engine.from_folder(args.model, **options)
+        return Engine.from_random(load_config(args.model, allow_ignored_keys=args.allow_ignored_keys),
+                                  seed=args.seed or 0, **options)
+    return Engine.from_folder(args.model, allow_ignored_keys=args.allow_ignored_keys, **options)
 
 
 class TokenCodec:
@@ -158,94 +162,18 @@ def cmd_run(args) -> int:
     if args.prompt is not None:
         answer(args.prompt)
         return 0
-    return repl(args, params, answer)
+    return prompt_lines(answer)
 
 
-REPL_HELP = """Commands:
-  /bye, /exit, /quit          Exit the REPL
-  /clear                       Clear conversation history
-  /set system <text>           Set a system prompt
-  /set temperature <n>         Set sampling temperature
-  /set top_p <n>               Set nucleus sampling threshold
-  /set top_k <n>               Set top-k sampling
-  /set max_tokens <n>          Set max tokens per response
-  /show history                Print conversation history
-  /show params                 Print sampling parameters
-  /help, /?                    Show this help
-
-Multiline input:
-  Start a message with \"\"\" to enter multi-line mode.
-  End with \"\"\" on its own line to send."""
-
-
-def repl(args, params, answer) -> int:
-    """The read-eval loop of the reference's `run` without a prompt (`inferrs/src/run.rs:882-983`):
-    the same commands with the same wording.  Each prompt is answered on its own: this engine keeps
-    no chat template, so the history is a record, not a context."""
-    history: List[str] = []
-    print('inferrs-amd: enter a prompt per line ("/help" lists the commands)', file=sys.stderr, flush=True)
-    lines = iter(sys.stdin)
-    for line in lines:
-        line = line.rstrip("\n")
-        if line.strip().startswith('"""'):
-            body = [line.strip()[3:]]
-            for more in lines:
-                more = more.rstrip("\n")
-                if more.strip().endswith('"""'):
-                    body.append(more.strip()[:-3])
-                    break
-                body.append(more)
-            line = "\n".join(body).strip()
+def prompt_lines(answer) -> int:
+    """Without a prompt on the command line: one prompt a line from standard input until it ends, each
+    answered on its own (nothing of an earlier answer is context for the next).  Blank lines are skipped."""
+    print("inferrs-amd: one prompt a line; end of input ends the run", file=sys.stderr, flush=True)
+    for line in sys.stdin:
         line = line.strip()
-        if not line:
-            continue
-        if not line.startswith("/"):
-            history.append(line)
+        if line:
             answer(line)
-            continue
-        parts = line.split(None, 2)
-        cmd = parts[0]
-        if cmd in ("/bye", "/exit", "/quit"):
-            break
-        elif cmd == "/clear":
-            history.clear()
-            print("Conversation cleared.")
-        elif cmd == "/set" and len(parts) >= 3:
-            name, value = parts[1], parts[2]
-            try:
-                if name == "system":
-                    args.system = value
-                    print("System prompt set.")
-                elif name == "temperature":
-                    params.temperature = float(value)
-                    print(f"temperature set to {params.temperature}")
-                elif name == "top_p":
-                    params.top_p = float(value)
-                    print(f"top_p set to {params.top_p}")
-                elif name == "top_k":
-                    params.top_k = int(value)
-                    print(f"top_k set to {params.top_k}")
-                elif name in ("num_predict", "max_tokens"):
-                    params.max_tokens = int(value)
-                    print(f"max_tokens set to {params.max_tokens}")
-                else:
-                    print(f"Unknown /set option: {name}")
-            except ValueError:
-                print(f"Invalid value: {value}")
-        elif cmd == "/show" and len(parts) >= 2:
-            if parts[1] == "history":
-                for i, text in enumerate(history):
-                    print(f"[{i}] user: {text}")
-            elif parts[1] == "params":
-                print(f"temperature={params.temperature} top_p={params.top_p} top_k={params.top_k} "
-                      f"max_tokens={params.max_tokens}")
-            else:
-                print(f"Unknown /show option: {parts[1]}")
-        elif cmd in ("/help", "/?"):
-            print(REPL_HELP)
-        else:
-            print(f"Unknown command: {line}")
-        sys.stdout.flush()
+            sys.stdout.flush()
     return 0
 
 

@@ -5,11 +5,17 @@ Keys and defaults follow the reference's `to_qwen3_config`
 `hidden_size / num_attention_heads`, `rms_norm_eps` to 1e-6, `rope_theta` to
 1e6, `tie_word_embeddings` to true, `max_position_embeddings` to 40960
 (`config.rs:728`).  Unlike the reference, the sizes themselves have no default
-here: a config.json without them is an error that names the key.  As in the
-reference, `sliding_window`, `max_window_layers`, `layer_types`,
-`rope_scaling` and `hidden_act` do not change the model (`qwen3.rs:28-45`
-holds none of them): every layer attends to all earlier positions and the
-activation is SiLU.
+here: a config.json without them is an error that names the key.
+
+The reference's model holds no bias, no scaling of the rotation, no window and no
+activation but SiLU (`qwen3.rs:28-45`; `hidden_act` is parsed and not used,
+`config.rs:291-292`), and it loads a config.json that asks for any of these without
+a word, as another model.  Here such a value is an error that names key and value:
+`attention_bias` true, a `rope_scaling` that is not null, a `hidden_act` other than
+"silu", `use_sliding_window` true, a `layer_types` entry other than "full_attention".
+`allow_ignored_keys=True` gives the reference's silence back (the keys are then
+ignored as it ignores them).  `sliding_window` and `max_window_layers` alone change
+nothing while `use_sliding_window` is false, there and here.
 """
 from __future__ import annotations
 
@@ -40,8 +46,32 @@ class Qwen3Config:
     model_type = "qwen3"
     chat_template = "chatml"        # the family's prompts (`inferrs_amd.chat`), when the folder does not say
 
+    @staticmethod
+    def unhonoured_keys(raw: Dict[str, Any]) -> Dict[str, Any]:
+        """The keys of `raw` that ask for what this model does not do, with their values."""
+        found: Dict[str, Any] = {}
+        if raw.get("attention_bias") not in (None, False):
+            found["attention_bias"] = raw["attention_bias"]
+        if raw.get("rope_scaling") is not None:
+            found["rope_scaling"] = raw["rope_scaling"]
+        if raw.get("hidden_act") not in (None, "silu"):
+            found["hidden_act"] = raw["hidden_act"]
+        if raw.get("use_sliding_window") not in (None, False):
+            found["use_sliding_window"] = raw["use_sliding_window"]
+        types = raw.get("layer_types")
+        if types is not None and (not isinstance(types, list) or any(t != "full_attention" for t in types)):
+            found["layer_types"] = types
+        return found
+
     @classmethod
-    def from_dict(cls, raw: Dict[str, Any]) -> "Qwen3Config":
+    def from_dict(cls, raw: Dict[str, Any], allow_ignored_keys: bool = False) -> "Qwen3Config":
+        unhonoured = cls.unhonoured_keys(raw)
+        if unhonoured and not allow_ignored_keys:
+            what = ", ".join(f"'{k}' = {v!r}" for k, v in unhonoured.items())
+            raise ConfigError(
+                f"config.json: {what}: {cls.architecture} as built here has no attention bias, no scaled rotation, no "
+                "sliding window and no activation but 'silu', and would compute another model's logits "
+                "(allow_ignored_keys=True, --allow-ignored-keys on the command line, ignores such keys as the reference does)")
         hidden = _require_int(raw, "hidden_size")
         heads = _require_int(raw, "num_attention_heads")
         kv_heads = raw.get("num_key_value_heads")

@@ -52,10 +52,13 @@ def resolve_architecture(raw: Dict[str, Any]) -> Type:
         f"registered: {registered_architectures()}")
 
 
-def load_config(model_dir: str):
-    """config.json of `model_dir` -> typed configuration of its registered architecture."""
+def load_config(model_dir: str, allow_ignored_keys: bool = False):
+    """config.json of `model_dir` -> typed configuration of its registered architecture.
+    `allow_ignored_keys`: handed to the architecture's `from_dict` when set (an architecture that refuses
+    values it does not honour then ignores them instead)."""
     raw = read_config_json(model_dir)
-    return resolve_architecture(raw).from_dict(raw)
+    config_cls = resolve_architecture(raw)
+    return config_cls.from_dict(raw, allow_ignored_keys=True) if allow_ignored_keys else config_cls.from_dict(raw)
 
 
 def load_spec(model_dir: str) -> ModelSpec:

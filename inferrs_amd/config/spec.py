@@ -57,6 +57,8 @@ class AttentionSpec:
     qk_norm: Optional[NormSpec] = None     # per-head norm of q and k before rotation
     window: Optional[int] = None           # keys kept: the last `window` positions; None = all
     scale: Optional[float] = None          # None = 1/sqrt(head_dim)
+    qkv_bias: bool = False                 # q_proj.bias, k_proj.bias, v_proj.bias are added to the projections
+    o_bias: bool = False                   # o_proj.bias is added to the output projection
     kind: str = "attention"
 
     @property
@@ -66,10 +68,12 @@ class AttentionSpec:
 
 @dataclass(frozen=True)
 class GatedMlpSpec:
-    """down( act(gate(x)) * up(x) ), no biases."""
+    """down( act(gate(x)) * up(x) ).  `activation`: "silu", or "gelu_tanh" (GELU in its tanh form); `bias`: every
+    projection has a bias vector beside its weight."""
     hidden: int
     intermediate: int
     activation: str = "silu"
+    bias: bool = False
     kind: str = "gated_mlp"
 
 

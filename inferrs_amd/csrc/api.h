@@ -26,7 +26,11 @@ int ia_add_inplace(void* x, const void* delta, long long n, int dtype, hipStream
 int ia_fill_normal(void* out, long long n, unsigned long long seed, double mean, double std,
                    int dtype, hipStream_t stream);
 int ia_widen_bf16(float* out, const void* x, long long n, hipStream_t stream);
-int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream);
+// rows of [gate | up] -> act(gate) * up; act: 1 SiLU, 2 GELU in its tanh form (the same numbers name the activation
+// in the `dual` argument of the products below, where 0 means a plain product)
+int ia_gate_mul(void* out, const void* gu, int rows, int inter, int act, int dtype, hipStream_t stream);
+// x[row][c] += bias[c] in place (x and bias in the same precision)
+int ia_add_bias(void* x, const void* bias, int rows, int cols, int dtype, hipStream_t stream);
 // A pure streaming read of `bytes` bytes by `blocks` blocks (one word of `out` a block): the measurement script's
 // measured memory roof.  Nothing of the engine calls it.
 int ia_stream_read(unsigned* out, const void* x, long long bytes, int blocks, hipStream_t stream);
@@ -49,10 +53,11 @@ long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int max_
 
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
                   int out_dtype, hipStream_t stream);
-int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
+// bias: bfloat16 [N] ([2 N] with dual), or null
+int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, const void* bias, int M, int N, int K,
                         int out_dtype, int dual, hipStream_t stream);
 // Large bfloat16 products in tiles of 256 x 256 (gemm_mfma.hip); K a multiple of 64; with `dual` w is [gate; up]
-// and out = silu(x . gate^T) * (x . up^T).
+// and out = act(x . gate^T) * (x . up^T).
 int ia_gemm_mfma_bf16(void* out, const void* x, const void* w, int M, int N, int K, int dual, hipStream_t stream);
 // Tuning knobs of the skinny product (tests switch the staged variants off with stage = 0); the defaults are
 // (2048, 8, 5, 8, 1).
@@ -64,22 +69,23 @@ void ia_gemm_skinny_tune(int target_waves, int min_ksteps, int rot_mul, int min_
 // neighbouring features each, a choice that depends on N and on the chip's number of compute units)
 int ia_gemm_skinny_blocks(int N);
 int ia_gemm_skinny_block_rows(int N);
-int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype,
+int ia_gemm_skinny_stream(void* out, const void* x, const void* w, const void* bias, int M, int N, int K, int out_dtype,
                           int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
                           int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream);
 
 // Products of 17 to 64 bfloat16 rows (gemm_mid.hip); K a multiple of 128.  out_mode 0: out [M, N] bfloat16; 1: float;
 // 2: out [ia_gemm_mid_splits(N, K)][M][N] float, the sums of each split of k, to be added up by the reader
-// (ia_sum_partials, ia_add_rmsnorm_partials).  dual: w = [gate; up], out = silu(x . gate^T) * (x . up^T), mode 0.
+// (ia_sum_partials, ia_add_rmsnorm_partials).  dual: w = [gate; up], out = act(x . gate^T) * (x . up^T), mode 0.
 int ia_gemm_mid_splits(int N, int K);
 // whether the weight's blocks fill the chip evenly, one a compute unit (dual: [gate; up] of N features each)
 int ia_gemm_mid_fills(int N, int K, int dual);
 // (a fixed pipeline for measurements and tests: k steps of a chunk, 2 or 4, and stages, 2 to 4; (0, 0): the kernel's own
-// rule; no product depends on it bit for bit)
-void ia_gemm_mid_tune(int kc, int ns);
+// rule; no product depends on it bit for bit); anything else is an error and changes nothing
+int ia_gemm_mid_tune(int kc, int ns);
 // (a fixed shape of the blocks for measurements and tests: waves a block, 2 to 8 (0: the kernel's own rule), ways k is split
-// and stages, 2 or 3 (2: four waves only); the caller's partial sums must have as many splits)
-void ia_gemm_mid_plan(int waves, int splits, int stages);
+// and stages, 2 or 3 (2: four waves only); the caller's partial sums must have as many splits); a shape that has no
+// kernel is an error and changes nothing
+int ia_gemm_mid_plan(int waves, int splits, int stages);
 int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                      hipStream_t stream);
 // the same for up to 16 rows that are a norm's input times its weight, with their sums of squares sums_in [M][n_sums]: every sum

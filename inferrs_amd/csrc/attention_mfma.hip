@@ -405,8 +405,9 @@ __device__ __forceinline__ float column_sum(float x) {
 //  * the waves of a block (`team`: 1, 2 or 4 neighbouring splits) add their results up in shared memory and
 //    leave one partial result a block; the block that finishes last for its (request, key/value head), known by
 //    a counter in memory, merges the blocks' partial results and writes the output.  No second kernel, and no
-//    wave reads another compute unit's results before they are there: every thread fences its stores before
-//    the block's one atomic increment, and the last block fences again before it reads.  The counters are zero
+//    wave reads another compute unit's results before they are there: every wave waits until the memory has taken
+//    its stores (`s_waitcnt vmcnt(0)`) before the barrier that precedes the block's one atomic increment, and the
+//    last block reads past the caches after it has seen the full count.  The counters are zero
 //    between calls (the last block puts its counter back), so calls that share them must not overlap.
 // The sum over the splits runs in the order of the splits whoever comes last: the result is the same every time.
 // Measured (head size 128, 32 query and 8 key/value heads, context 8,192, time stamps inside the kernel): a wave
@@ -840,12 +841,22 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
 
         // ---- the last block of this (request, key/value head, column block) merges the blocks' results --------
         int* counter = counters + ((size_t)blockIdx.z * p.nkv + kvh) * gridDim.x + blockIdx.x;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");          // this thread's stores have arrived ...
-        __syncthreads();                                                // ... and every thread's, before the count
+        // The hand-over.  Writer: a wave's vector-memory counter counts a store down when the memory has taken it
+        // (the stores above are written through, so that is the point where every die reads it), and
+        // `s_waitcnt vmcnt(0)` holds the wave until all of its stores are there; then the barrier, so that this
+        // holds for every wave of the block; only then the count.  (A release fence of workgroup scope does not wait
+        // for stores that leave the compute unit, and one of device scope writes the die's L2 back.)  The compiler
+        // moves no store across the wait (the asm names memory).
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
         if (threadIdx.x == 0)
             s_last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == teams - 1 ? 1 : 0;
         __syncthreads();
         if (!s_last) return;
+        // Reader: thread 0 has the counter's old value in a register before it can write s_last, so the increment
+        // that made it teams - 1, and with it every other block's stores, is in memory before any thread passes the
+        // barrier above; the loads below are issued after it, and they read past the caches (device scope), so they
+        // cannot meet a line that was fetched before the stores arrived.
         // Every thread takes part: the block's threads form as many groups as there are 16-byte pieces of the result
         // in them, group i sums the blocks i, i + groups, ... in that order, and the groups' sums meet in shared
         // memory and are added in the groups' order.

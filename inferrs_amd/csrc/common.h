@@ -44,6 +44,17 @@ __device__ __forceinline__ float round_to(const bf16_t*, float v) {
     return bf16_bits_to_f32(f32_to_bf16_bits(v));
 }
 
+// ---- the activation of a gated feed-forward ---------------------------------------------------
+// act(gate) * up, in 32-bit.  The entry points' `dual` / `act` argument names the activation: 1 SiLU,
+// gate / (1 + exp(-gate)); 2 GELU in its tanh form, gate / 2 * (1 + tanh(sqrt(2 / pi) * (gate + 0.044715 gate^3))).
+// The choice is the same for all lanes of a launch.
+enum { IA_ACT_NONE = 0, IA_ACT_SILU = 1, IA_ACT_GELU_TANH = 2, IA_ACT_LAST = IA_ACT_GELU_TANH };
+
+__device__ __forceinline__ float gate_act(float g, int act) {
+    if (act == IA_ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 // ---- reductions -----------------------------------------------------------------------------
 // Butterfly over the 64 lanes: every lane ends with the same value, and the order of the
 // additions is fixed by the lane numbers alone.

@@ -238,21 +238,46 @@ extern "C" int ia_add_inplace(void* x, const void* delta, long long n, int dtype
     return 0;
 }
 
-// ---- SiLU(gate) * up ------------------------------------------------------------------------
+// ---- x[row][c] += bias[c] -------------------------------------------------------------------
+// For products whose kernel has no place for a bias; the sum is formed in 32-bit and rounded once.
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const T* __restrict__ bias, int cols, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+        st(x + i, ld(x + i) + ld(bias + (i % cols)));
+}
+
+extern "C" int ia_add_bias(void* x, const void* bias, int rows, int cols, int dtype, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && cols > 0, "add_bias: bad sizes rows=%d cols=%d", rows, cols);
+    if (rows == 0) return 0;
+    const size_t total = (size_t)rows * cols;
+    const size_t want = (total + 255) / 256;
+    const int grid = (int)(want < 65535 ? want : 65535);
+    if (dtype == IA_F32)
+        add_bias_kernel<float><<<grid, 256, 0, stream>>>((float*)x, (const float*)bias, cols, total);
+    else if (dtype == IA_BF16)
+        add_bias_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)x, (const bf16_t*)bias, cols, total);
+    else
+        IA_CHECK(false, "add_bias: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("add_bias");
+    return 0;
+}
+
+// ---- act(gate) * up -------------------------------------------------------------------------
 // `gu` holds rows of [gate(0..inter) | up(0..inter)]; the product is formed in 32-bit.
 template <typename T>
-__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, size_t total) {
+__global__ void gate_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, size_t total, int act) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t row = i / inter;
         const int c = (int)(i - row * inter);
         const float g = ld(gu + row * 2 * inter + c);
         const float u = ld(gu + row * 2 * inter + inter + c);
-        st(out + i, g / (1.0f + expf(-g)) * u);
+        st(out + i, gate_act(g, act) * u);
     }
 }
 
 // bfloat16 rows whose half length is a multiple of 8: eight products a thread, 16-byte accesses.
-__global__ void silu_mul_bf16_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gu, int inter, size_t total_vecs) {
+__global__ void gate_mul_bf16_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gu, int inter, size_t total_vecs,
+                                         int act) {
     const int vecs_per_row = inter / 8;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total_vecs; i += (size_t)gridDim.x * blockDim.x) {
         const size_t row = i / vecs_per_row;
@@ -265,34 +290,35 @@ __global__ void silu_mul_bf16_vec_kernel(bf16_t* __restrict__ out, const bf16_t*
         for (int j = 0; j < 4; ++j) {
             const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
             const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-            o[j] = pack_bf16x2(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+            o[j] = pack_bf16x2(gate_act(g0, act) * u0, gate_act(g1, act) * u1);
         }
         *(uint4*)(out + row * inter + c) = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 
-extern "C" int ia_silu_mul(void* out, const void* gu, int rows, int inter, int dtype, hipStream_t stream) {
-    IA_CHECK(rows >= 0 && inter > 0, "silu_mul: bad sizes rows=%d inter=%d", rows, inter);
+extern "C" int ia_gate_mul(void* out, const void* gu, int rows, int inter, int act, int dtype, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && inter > 0, "gate_mul: bad sizes rows=%d inter=%d", rows, inter);
+    IA_CHECK(act >= IA_ACT_SILU && act <= IA_ACT_LAST, "gate_mul: unknown activation %d", act);
     if (rows == 0) return 0;
     const size_t total = (size_t)rows * inter;
     const int block = 256;
     if (dtype == IA_BF16 && inter % 8 == 0 && ((((uintptr_t)out) | ((uintptr_t)gu)) & 15) == 0) {
         const size_t vecs = total / 8;
         const size_t want = (vecs + block - 1) / block;
-        silu_mul_bf16_vec_kernel<<<(unsigned)(want < 65535 * 8 ? want : 65535 * 8), block, 0, stream>>>(
-            (bf16_t*)out, (const bf16_t*)gu, inter, vecs);
-        IA_LAUNCH_CHECK("silu_mul");
+        gate_mul_bf16_vec_kernel<<<(unsigned)(want < 65535 * 8 ? want : 65535 * 8), block, 0, stream>>>(
+            (bf16_t*)out, (const bf16_t*)gu, inter, vecs, act);
+        IA_LAUNCH_CHECK("gate_mul");
         return 0;
     }
     const size_t want = (total + block - 1) / block;
     const int grid = (int)(want < 65535 ? want : 65535);
     if (dtype == IA_F32)
-        silu_mul_kernel<float><<<grid, block, 0, stream>>>((float*)out, (const float*)gu, inter, total);
+        gate_mul_kernel<float><<<grid, block, 0, stream>>>((float*)out, (const float*)gu, inter, total, act);
     else if (dtype == IA_BF16)
-        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, inter, total);
+        gate_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, inter, total, act);
     else
-        IA_CHECK(false, "silu_mul: unknown dtype %d", dtype);
-    IA_LAUNCH_CHECK("silu_mul");
+        IA_CHECK(false, "gate_mul: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("gate_mul");
     return 0;
 }
 

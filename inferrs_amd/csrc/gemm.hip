@@ -304,6 +304,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 //     sums_out[row][block] and the new values times next_w (or 1 + next_w) to scaled_out [M, N].
 //   sums_in: x holds such scaled rows, and sums_in[row][0 .. n_sums) their sums of squares: every sum of
 //     the product is multiplied by rsqrt(sum of the row's sums_in / K + eps) before it is rounded.
+//   bias: a vector that is added to every row of the product (after the scale, before the activation, the
+//     rounding and the sum into the stream).
 // One rounding of the normed value, as in the norm kernel, at another place (before the scale instead of
 // after it); the sum of squares is added up in another order than there.
 struct SkinnyStream {
@@ -315,6 +317,8 @@ struct SkinnyStream {
     int n_sums;
     float eps;
     int add_one;
+    int act;                    // DUAL: the gate's activation (IA_ACT_*)
+    const bf16_t* bias;         // [N] ([2 N] with DUAL), added to every row's sums before anything is rounded; or null
 };
 
 // STAGE: 0, or the k steps of a staged chunk (8 or 16).
@@ -584,6 +588,14 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                     for (int q = 0; q < NA; ++q) { s[q][0] *= scale; s[q][1] *= scale; s[q][2] *= scale; s[q][3] *= scale; }
                 }
             }
+            if (st.bias != nullptr) {
+                const int fb = n0 + t * 16 + 4 * g;
+#pragma unroll
+                for (int q = 0; q < NA; ++q)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (fb + i < N) s[q][i] += bf16_bits_to_f32(st.bias[(size_t)q * N + fb + i].bits);
+            }
             if constexpr (!DUAL && RT == 1 && MT == 1) {
                 if (st.resid != nullptr) {
                     // (all lanes of the wave stay for the sums; rows and features outside add nothing)
@@ -639,7 +651,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * IA_WAVE) void gemm_skinny_kernel(
                     // activation, as the two-kernel path rounds it
                     const float gate = bf16_bits_to_f32(f32_to_bf16_bits(s[0][i]));
                     const float up = bf16_bits_to_f32(f32_to_bf16_bits(s[NA - 1][i]));
-                    v[i] = gate / (1.0f + expf(-gate)) * up;
+                    v[i] = gate_act(gate, st.act) * up;
                 } else {
                     v[i] = s[0][i];
                 }
@@ -814,8 +826,10 @@ static int launch_skinny(void* out, int out_f32, const bf16_t* x, const bf16_t* 
 }
 
 static int skinny_product(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype, int dual,
-                          const SkinnyStream& st, hipStream_t stream) {
+                          SkinnyStream st, hipStream_t stream) {
     IA_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+    IA_CHECK(dual >= 0 && dual <= IA_ACT_LAST, "gemm_skinny: unknown activation %d", dual);
+    st.act = dual;
     IA_CHECK(K % 8 == 0, "gemm_skinny: K=%d must be a multiple of 8 (use the tiled product)", K);
     IA_CHECK(out_dtype == IA_F32 || out_dtype == IA_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
     IA_CHECK((((uintptr_t)x | (uintptr_t)w) & 15) == 0, "gemm_skinny: x and w must be 16-byte aligned");
@@ -829,6 +843,7 @@ static int skinny_product(void* out, const void* x, const void* w, int M, int N,
     IA_CHECK(st.sums_in == nullptr || st.n_sums > 0, "gemm_skinny: scaled rows come with their sums of squares");
     IA_CHECK((((uintptr_t)st.resid | (uintptr_t)st.scaled_out | (uintptr_t)st.next_w) & 15) == 0,
              "gemm_skinny: the stream's arrays must be 16-byte aligned");
+    IA_CHECK((((uintptr_t)st.bias) & 1) == 0, "gemm_skinny: the bias must be 2-byte aligned");
     if (M == 0) return 0;
     const int out_f32 = out_dtype == IA_F32;
     const bf16_t* xb = (const bf16_t*)x;
@@ -854,10 +869,11 @@ static int skinny_product(void* out, const void* x, const void* w, int M, int N,
     return 0;
 }
 
-// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` out[M, N] = silu(x . w[0:N]^T) * (x . w[N:2N]^T).
-extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, int M, int N, int K,
+// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` (an activation, IA_ACT_*) out[M, N] = act(x . w[0:N]^T) * (x . w[N:2N]^T);
+// bias [N] ([2 N] with dual) in bfloat16, or null: added to every row of the product(s).
+extern "C" int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, const void* bias, int M, int N, int K,
                                    int out_dtype, int dual, hipStream_t stream) {
-    const SkinnyStream none = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0};
+    const SkinnyStream none = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0, 0, (const bf16_t*)bias};
     return skinny_product(out, x, w, M, N, K, out_dtype, dual, none, stream);
 }
 
@@ -876,10 +892,11 @@ extern "C" int ia_gemm_skinny_blocks(int N) {
 //     scaled_out[M, N] (may be null, with next_w) the new rows times next_w [N] (1 + next_w with add_one).
 //   sums_in != null: x [M, K] holds such scaled rows and sums_in[M][n_sums] their sums of squares; the
 //     product's sums are multiplied by rsqrt(sum / K + eps) before anything else happens to them.
-extern "C" int ia_gemm_skinny_stream(void* out, const void* x, const void* w, int M, int N, int K, int out_dtype,
+extern "C" int ia_gemm_skinny_stream(void* out, const void* x, const void* w, const void* bias, int M, int N, int K, int out_dtype,
                                      int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
                                      int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream) {
-    const SkinnyStream st = {(bf16_t*)resid, sums_out, (bf16_t*)scaled_out, next_w, sums_in, n_sums, eps, add_one};
+    const SkinnyStream st = {(bf16_t*)resid, sums_out, (bf16_t*)scaled_out, next_w, sums_in, n_sums, eps, add_one, 0,
+                             (const bf16_t*)bias};
     IA_CHECK(out != nullptr || resid != nullptr, "gemm_skinny: no place for the result");
     return skinny_product(out, x, w, M, N, K, out_dtype, dual, st, stream);
 }

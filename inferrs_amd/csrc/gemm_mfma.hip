@@ -58,6 +58,7 @@ struct GemmMfmaParams {
     const bf16_t* x;
     const bf16_t* w;
     int M, N, K;            // N: output features (with the activation inside, w has 2 N rows)
+    int act;                // DUAL: the gate's activation (IA_ACT_*)
     int tiles_m, tiles_n;
 };
 
@@ -264,7 +265,7 @@ void gemm_mfma_kernel(const GemmMfmaParams p) {
                     // two-kernel way rounds them
                     const float gate = bf16_bits_to_f32(f32_to_bf16_bits(acc[a][b][i]));
                     const float up = bf16_bits_to_f32(f32_to_bf16_bits(acc[a + 4][b][i]));
-                    v[i] = gate / (1.0f + expf(-gate)) * up;
+                    v[i] = gate_act(gate, p.act) * up;
                 }
             } else {
                 n = n0 + wn * 128 + a * 16 + 4 * g;
@@ -300,16 +301,18 @@ static int gemm_mfma_launch(const GemmMfmaParams& p, hipStream_t stream) {
     return 0;
 }
 
-// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` out[M, N] = silu(x . w[0:N]^T) * (x . w[N:2N]^T); bfloat16,
+// out[M, N] = x[M, K] . w[N, K]^T, or with `dual` (an activation, IA_ACT_*) out[M, N] = act(x . w[0:N]^T) * (x . w[N:2N]^T); bfloat16,
 // K a multiple of 64.
 extern "C" int ia_gemm_mfma_bf16(void* out, const void* x, const void* w, int M, int N, int K, int dual,
                                  hipStream_t stream) {
     IA_CHECK(M > 0 && N > 0 && K > 0, "gemm_mfma: bad sizes M=%d N=%d K=%d", M, N, K);
+    IA_CHECK(dual >= 0 && dual <= IA_ACT_LAST, "gemm_mfma: unknown activation %d", dual);
     IA_CHECK(K % (2 * GM_BK) == 0, "gemm_mfma: K=%d must be a multiple of %d", K, 2 * GM_BK);
     IA_CHECK((((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0, "gemm_mfma: operands must be 16-byte aligned");
     GemmMfmaParams p;
     p.out = (bf16_t*)out; p.x = (const bf16_t*)x; p.w = (const bf16_t*)w;
     p.M = M; p.N = N; p.K = K;
+    p.act = dual;
     p.tiles_m = (M + GM_BM - 1) / GM_BM;
     p.tiles_n = dual ? (N + GM_BN / 2 - 1) / (GM_BN / 2) : (N + GM_BN - 1) / GM_BN;
     IA_CHECK((long long)p.tiles_m * p.tiles_n < (1LL << 31), "gemm_mfma: too many tiles");

@@ -54,7 +54,8 @@ enum { MID_OUT_BF16 = 0, MID_OUT_F32 = 1, MID_OUT_PARTIAL = 2 };
 // shared memory (swap_up, in a stage's place) to the waves that hold the gate rows' sums of the same features.
 template <int MT, bool DUAL, int TILES>
 __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* swap_up, void* out, int out_mode,
-                                           int M, int N, int lane, int r, int g, int tile, int part, int n_first, int split) {
+                                           int M, int N, int lane, int r, int g, int tile, int part, int n_first, int split,
+                                           int act) {
     constexpr int FEATURE_TILES = DUAL ? TILES / 2 : TILES;
     if (DUAL) __syncthreads();                                            // everybody is done with the stages
     if (DUAL) {
@@ -75,7 +76,7 @@ __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* sw
             for (int i = 0; i < 4; ++i) {
                 const float gate = bf16_bits_to_f32(f32_to_bf16_bits(acc[mt][i]));
                 const float u = bf16_bits_to_f32(f32_to_bf16_bits(up[i]));
-                v[i] = gate / (1.0f + expf(-gate)) * u;
+                v[i] = gate_act(gate, act) * u;
             }
             bf16_t* o = (bf16_t*)out + (size_t)m * N + nb;
             if (nb + 3 < N && (N & 3) == 0) {
@@ -120,7 +121,7 @@ __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* sw
 template <int MT, bool DUAL, int KC, int NS, int W>
 __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-    int M, int N, int K, int k_per_block, const float* __restrict__ sums_in, int n_sums, float eps) {
+    int M, int N, int K, int k_per_block, const float* __restrict__ sums_in, int n_sums, float eps, int act) {
     constexpr int CHUNK_K = KC * 32;
     constexpr int ROW_BYTES = KC * 64;
     constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
             acc[0][0] *= scale; acc[0][1] *= scale; acc[0][2] *= scale; acc[0][3] *= scale;
         }
     }
-    mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split);
+    mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split, act);
 }
 
 // How a weight is shared out: a function of its shape and the chip alone, never of the rows of the step.
@@ -330,9 +331,16 @@ static int mid_cus() {
 struct MidPlan { int waves, splits, stages; };
 // a plan for measurements and tests: waves (0: the rule), splits, stages
 static MidPlan g_mid_forced = {0, 0, 0};
-extern "C" void ia_gemm_mid_plan(int waves, int splits, int stages) { g_mid_forced = {waves, splits, stages}; }
-
 #define MID_MAX_WAVES 8
+extern "C" int ia_gemm_mid_plan(int waves, int splits, int stages) {
+    IA_CHECK(waves == 0 || (waves >= 2 && waves <= MID_MAX_WAVES && splits >= 1 && splits <= 16 && (splits & (splits - 1)) == 0
+                            && (stages == 3 || (waves == 4 && stages == 2))),
+             "gemm_mid_plan: no block of %d waves with %d splits of k, %d stages deep (2 to 8 waves, 2^k splits up to 16, "
+             "3 stages, or 4 waves with 2; 0 waves: the plan's own)", waves, splits, stages);
+    g_mid_forced = {waves, splits, stages};
+    return 0;
+}
+
 static MidPlan mid_plan(int N, int K, bool dual) {
     const int cus = mid_cus();
     const int tiles = (N + 15) / 16;                       // of a part
@@ -383,11 +391,17 @@ extern "C" int ia_gemm_mid_splits(int N, int K) {
 // 0, 0: the plan's own).  Every pipeline adds an output's products up in the same order; plans differ in where a block
 // starts its walk of k.
 static int g_mid_kc = 0, g_mid_ns = 0;
-extern "C" void ia_gemm_mid_tune(int kc, int ns) { g_mid_kc = kc; g_mid_ns = ns; }
+extern "C" int ia_gemm_mid_tune(int kc, int ns) {
+    IA_CHECK((kc == 0 && ns == 0) || (kc == 4 && ns == 2) || (kc == 2 && (ns == 3 || ns == 4)),
+             "gemm_mid_tune: no pipeline of chunks of %d k steps, %d deep (4 x 2, 2 x 3, 2 x 4, or 0, 0 for the plan's own)", kc, ns);
+    g_mid_kc = kc;
+    g_mid_ns = ns;
+    return 0;
+}
 
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
-                      const float* sums_in, int n_sums, float eps, hipStream_t stream) {
+                      const float* sums_in, int n_sums, float eps, int act, hipStream_t stream) {
     MidPlan plan = mid_plan(N, K, DUAL);
     if (out_mode != MID_OUT_PARTIAL && !DUAL && plan.splits != 1) {
         // a stored product cannot be split: four waves a block over all of k
@@ -398,8 +412,12 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
     IA_CHECK(plan.splits == splits, "gemm_mid: the plan's %d splits against the caller's %d", plan.splits, splits);
     const int features = 16 * plan.waves / (DUAL ? 2 : 1);            // output features of a block
     const dim3 grid((N + features - 1) / features, splits);
+    // every block's share of k is whole chunks (a share that is not would lose its tail and start off the loads' alignment)
+    IA_CHECK(splits >= 1 && K % (splits * MID_CHUNK_MIN_K) == 0, "gemm_mid: K=%d does not split %d ways in multiples of %d",
+             K, splits, MID_CHUNK_MIN_K);
+    IA_CHECK(plan.waves >= 2 && plan.waves <= MID_MAX_WAVES, "gemm_mid: a block of %d waves", plan.waves);
     const int k_block = K / splits;
-#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps)
+#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps, act)
     if (kc == 4 && plan.stages == 3) {
         switch (plan.waves) {
             case 2: MID_SHAPE(4, 3, 2); return 0;
@@ -425,7 +443,7 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
 }
 
 // out_mode 0: out [M, N] bfloat16; 1: out [M, N] float; 2: out [splits][M][N] float with splits =
-// ia_gemm_mid_splits(N, K), to be added up by the reader.  dual: w = [gate; up] of N rows each, out = silu(x . gate^T)
+// ia_gemm_mid_splits(N, K), to be added up by the reader.  dual (an activation, IA_ACT_*): w = [gate; up] of N rows each, out = act(x . gate^T)
 // * (x . up^T) in bfloat16 (mode 0 only).  M in 1..64, K a multiple of 128.
 // sums_in [M][n_sums] (or null): the rows of x are a norm's input times its weight, and every sum of the product is multiplied by
 // the row's rsqrt(sum of its sums_in / K + eps); up to 16 rows, whole sums only (no split of k).
@@ -437,6 +455,7 @@ extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, 
     IA_CHECK(K % MID_CHUNK_MIN_K == 0, "gemm_mid: K=%d must be a multiple of %d (use another product)", K, MID_CHUNK_MIN_K);
     IA_CHECK(out_mode >= 0 && out_mode <= 2 && (!dual || out_mode == MID_OUT_BF16), "gemm_mid: output mode %d%s", out_mode,
              dual ? " does not go with the activation inside" : " is unknown");
+    IA_CHECK(dual >= 0 && dual <= IA_ACT_LAST, "gemm_mid: unknown activation %d", dual);
     IA_CHECK((((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0, "gemm_mid: operands must be 16-byte aligned");
     const int splits = out_mode == MID_OUT_PARTIAL && !dual ? mid_plan(N, K, false).splits : 1;
     const bf16_t* xb = (const bf16_t*)x;
@@ -444,15 +463,15 @@ extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, 
     const int mt = (M + 15) / 16;
     int rc = 0;
     if (dual) {
-        if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
-        else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
-        else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
-        else rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, stream);
+        if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
     } else {
-        if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
-        else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
-        else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
-        else rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, stream);
+        if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
     }
     if (rc != 0) return rc;
     IA_LAUNCH_CHECK("gemm_mid");

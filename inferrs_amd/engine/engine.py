@@ -76,21 +76,28 @@ class Engine:
         self.use_graphs = use_graphs and model.graph_safe
         self.unused_tensors: List[str] = []
         self.stop_token_ids: Tuple[int, ...] = tuple(model.spec.eos_token_ids)
+        # a part that will run off its fast path says so once, here, and not at every step
+        self.load_notes: List[str] = model.load_notes(page_size)
+        for note in self.load_notes:
+            log.warning("%s", note)
         self._graphs: Dict[Tuple[int, int, int], object] = {}
         self._graphs_generation = self.builder.generation    # the staging buffer the graphs were captured over
         self.graph_replays = 0
 
     # ---- construction -----------------------------------------------------------------------
     @classmethod
-    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", strict: bool = False, **kw) -> "Engine":
-        """`strict`: tensors of the folder that the model does not read are an error instead of a note."""
-        config = load_config(model_dir)
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", strict: bool = False,
+                    allow_ignored_keys: bool = False, **kw) -> "Engine":
+        """`strict`: tensors of the folder that the model does not read are an error instead of a warning.
+        `allow_ignored_keys`: config.json values that the architecture does not honour are ignored, as the
+        reference ignores them, instead of refused."""
+        config = load_config(model_dir, allow_ignored_keys=allow_ignored_keys)
         spec = config.to_spec()
         expected, optional = model_tensors(spec)
         unused: List[str] = []
         tensors = load_weights(model_dir, expected, optional, strict=strict, unused=unused)
         if unused:
-            log.info("%s: %d tensors are not read by %s: %s", model_dir, len(unused), spec.architecture,
+            log.warning("%s: %d tensors are not read by %s: %s", model_dir, len(unused), spec.architecture,
                      ", ".join(unused[:8]) + (" ..." if len(unused) > 8 else ""))
         model = DecoderModel(spec, tensors, parse_dtype(dtype), device)
         eng = cls(model, **kw)
@@ -137,7 +144,11 @@ class Engine:
         """Run one batch; returns float32 logits `[wanted, vocab]` on the device, in the order
         of the entries and of each entry's `want`.  Pages that the entries need beyond what is
         reserved for them are reserved here.  With `commit` the requests' cached lengths advance;
-        a caller that passes False (the scheduler) does that itself."""
+        a caller that passes False (the scheduler) does that itself.
+
+        The tensor that a decode step (one token a request) returns under `use_graphs` is the captured
+        graph's own output buffer: it holds this step's logits until the next step of the same shape
+        overwrites them.  Read or `.clone()` it before stepping again."""
         if not entries:
             raise StepError("a step needs at least one entry")
         vocab = self.spec.vocab_size

@@ -59,6 +59,22 @@ class DecoderModel:
             parts += list(b.parts())
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
+    def all_parts(self):
+        parts = [self.embedding, self.head, self.final_norm]
+        for b in self.blocks:
+            parts += list(b.parts())
+        return [p for p in parts if p is not None]
+
+    def load_notes(self, page_size: int):
+        """What the parts have to say once about how they will run (a part may offer `load_notes(page_size)`):
+        every different note once, in the order of the parts."""
+        notes = []
+        for p in self.all_parts():
+            for note in (p.load_notes(page_size) if hasattr(p, "load_notes") else []):
+                if note not in notes:
+                    notes.append(note)
+        return notes
+
     def cache_needs(self) -> Dict[int, object]:
         """Schedule stop that owns a cache -> what its mixer keeps per request."""
         needs: Dict[int, object] = {}
@@ -112,4 +128,5 @@ class DecoderModel:
                     add(v)
                 elif isinstance(v, Linear):
                     add(v.weight)
+                    add(v.bias)
         return total

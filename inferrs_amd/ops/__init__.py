@@ -212,16 +212,43 @@ def add_inplace(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return x
 
 
-def silu_mul(gu: torch.Tensor) -> torch.Tensor:
-    """rows of [gate | up] -> silu(gate) * up."""
+# The activations a gated feed-forward may name, and their numbers in the kernels' `dual` / `act` argument
+# (0 there: a plain product).  "gelu_tanh" is GELU in its tanh form, x / 2 * (1 + tanh(sqrt(2 / pi) * (x + 0.044715 x^3))).
+ACTIVATIONS: Dict[str, int] = {"silu": 1, "gelu_tanh": 2}
+
+
+def activation_code(activation: str) -> int:
+    try:
+        return ACTIVATIONS[activation]
+    except KeyError:
+        raise KernelError(f"no kernel has the activation {activation!r}; known: {sorted(ACTIVATIONS)}") from None
+
+
+def gate_mul(gu: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """rows of [gate | up] -> act(gate) * up."""
     _dev(gu)
     if gu.shape[-1] % 2:
-        raise KernelError(f"silu_mul: last dimension {gu.shape[-1]} must be even")
+        raise KernelError(f"gate_mul: last dimension {gu.shape[-1]} must be even")
     inter = gu.shape[-1] // 2
     rows = gu.numel() // (2 * inter)
     out = torch.empty((*gu.shape[:-1], inter), dtype=gu.dtype, device=gu.device)
-    _check(library().ia_silu_mul(_p(out), _p(gu), rows, inter, _dt(gu), _stream()))
+    _check(library().ia_gate_mul(_p(out), _p(gu), rows, inter, activation_code(activation), _dt(gu), _stream()))
     return out
+
+
+def silu_mul(gu: torch.Tensor) -> torch.Tensor:
+    """rows of [gate | up] -> silu(gate) * up."""
+    return gate_mul(gu, "silu")
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """x[row] += bias in place, for products whose kernel has no place for a bias."""
+    _dev(x, bias)
+    cols = x.shape[-1]
+    if bias.numel() != cols or bias.dtype != x.dtype:
+        raise KernelError(f"add_bias: a bias of {bias.numel()} {bias.dtype} entries for rows of {cols} {x.dtype}")
+    _check(library().ia_add_bias(_p(x), _p(bias), x.numel() // cols, cols, _dt(x), _stream()))
+    return x
 
 
 # ---- position encoding ----------------------------------------------------------------------
@@ -530,9 +557,9 @@ def _own_large(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.is_contiguous() and w.is_contiguous())
 
 
-def gemm_mfma_bf16(x: torch.Tensor, w: torch.Tensor, dual: bool = False) -> torch.Tensor:
+def gemm_mfma_bf16(x: torch.Tensor, w: torch.Tensor, dual: bool = False, activation: str = "silu") -> torch.Tensor:
     """x [m, k] . w[n, k]^T in bfloat16 by the tiled matrix-core kernel (k a multiple of 64); with `dual`
-    w is [gate; up] and the result silu(x . gate^T) * (x . up^T)."""
+    w is [gate; up] and the result act(x . gate^T) * (x . up^T)."""
     _dev(x, w)
     m, k = x.shape
     rows, k2 = w.shape
@@ -543,7 +570,8 @@ def gemm_mfma_bf16(x: torch.Tensor, w: torch.Tensor, dual: bool = False) -> torc
     n = rows // 2 if dual else rows
     out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     if m:
-        _check(library().ia_gemm_mfma_bf16(_p(out), _p(x), _p(w), m, n, k, int(dual), _stream()))
+        _check(library().ia_gemm_mfma_bf16(_p(out), _p(x), _p(w), m, n, k, activation_code(activation) if dual else 0,
+                                           _stream()))
     return out
 
 
@@ -559,11 +587,18 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     return out
 
 
+def _skinny_bias(bias: Optional[torch.Tensor], rows: int) -> None:
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != rows or not bias.is_cuda
+                             or not bias.is_contiguous()):
+        raise KernelError(f"gemm_skinny: the bias must be a contiguous bfloat16 vector of {rows} entries on the GPU")
+
+
 def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                     dual: bool = False) -> torch.Tensor:
-    """x [m, k] . w[n, k]^T on the matrix cores, made for few rows.  `dual`: w is [gate; up]
-    stacked along its rows and the result is silu(x . gate^T) * (x . up^T)."""
+                     dual: bool = False, activation: str = "silu", bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [m, k] . w[n, k]^T (+ bias) on the matrix cores, made for few rows.  `dual`: w is [gate; up]
+    stacked along its rows and the result is act(x . gate^T + bias[:n]) * (x . up^T + bias[n:])."""
     _dev(x, w)
+    _skinny_bias(bias, w.shape[0])
     m, k = x.shape
     n, k2 = w.shape
     if k != k2 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
@@ -573,7 +608,8 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = 
             raise KernelError(f"gemm_skinny: a stacked [gate; up] weight needs an even row count, got {n}")
         n //= 2
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    _check(library().ia_gemm_skinny_bf16(_p(out), _p(x), _p(w), m, n, k, _DT[out_dtype], int(dual), _stream()))
+    _check(library().ia_gemm_skinny_bf16(_p(out), _p(x), _p(w), _p(bias), m, n, k, _DT[out_dtype],
+                                         activation_code(activation) if dual else 0, _stream()))
     return out
 
 
@@ -654,11 +690,14 @@ class NormedRows:
 
 
 def _stream_product(x: torch.Tensor, w: torch.Tensor, n: int, out_dtype, dual: bool, resid=None, sums_out=None,
-                    scaled_out=None, next_w=None, add_one: bool = False, sums_in=None, eps: float = 0.0):
+                    scaled_out=None, next_w=None, add_one: bool = False, sums_in=None, eps: float = 0.0,
+                    activation: str = "silu", bias: Optional[torch.Tensor] = None):
     m, k = x.shape
+    _skinny_bias(bias, w.shape[0])
     out = None if resid is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
     _check(library().ia_gemm_skinny_stream(
-        _p(out), _p(x), _p(w), m, n, k, _DT[out_dtype], int(dual), _p(resid), _p(sums_out), _p(scaled_out), _p(next_w),
+        _p(out), _p(x), _p(w), _p(bias), m, n, k, _DT[out_dtype], activation_code(activation) if dual else 0, _p(resid),
+        _p(sums_out), _p(scaled_out), _p(next_w),
         int(add_one), _p(sums_in), sums_in.shape[1] if sums_in is not None else 0, ctypes.c_float(eps), _stream()))
     return out
 
@@ -670,8 +709,9 @@ def _takes_normed_rows(x: NormedRows, w: torch.Tensor, n: int) -> bool:
             and x.sums.is_contiguous() and x.scaled.is_contiguous())
 
 
-def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=None):
-    """resid += x . w^T in place, as `add_rmsnorm` would add the product (rounded, then summed in 32-bit
+def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=None,
+               bias: Optional[torch.Tensor] = None):
+    """resid += x . w^T (+ bias) in place, as `add_rmsnorm` would add the product (rounded, then summed in 32-bit
     and rounded), by the skinny kernel itself.  Returns (sums, scaled): the partial sums of squares of the
     new rows [rows, blocks], and the new rows times the weight of `next_norm` (a norm part with `weight`
     and `add_one`; None: no such rows); or None when this product cannot (the caller then forms it and
@@ -680,7 +720,7 @@ def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=
     n = w.shape[0]
     if (m > SKINNY_MAX_ROWS or m == 0 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k
             or not skinny_fits(x, w) or n >= 65536 or resid.dtype != torch.bfloat16 or tuple(resid.shape) != (m, n)
-            or not resid.is_contiguous()):
+            or not resid.is_contiguous() or (bias is not None and bias.dtype != torch.bfloat16)):
         return None
     next_w = getattr(next_norm, "weight", None)
     if next_w is not None and (next_w.dtype != torch.float32 or next_w.numel() != n):
@@ -689,7 +729,7 @@ def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=
     sums = torch.empty((m, library().ia_gemm_skinny_blocks(n)), dtype=torch.float32, device=x.device)
     scaled = torch.empty_like(resid) if next_w is not None else None
     _stream_product(x, w, n, torch.bfloat16, False, resid=resid, sums_out=sums, scaled_out=scaled, next_w=next_w,
-                    add_one=bool(getattr(next_norm, "add_one", False)))
+                    add_one=bool(getattr(next_norm, "add_one", False)), bias=bias)
     return sums, scaled
 
 
@@ -737,9 +777,10 @@ def mid_fits(x: torch.Tensor, w: torch.Tensor, few_rows: bool = False) -> bool:
 
 
 def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, dual: bool = False,
-                  partial: bool = False, sums_in: Optional[torch.Tensor] = None, eps: float = 0.0):
+                  partial: bool = False, sums_in: Optional[torch.Tensor] = None, eps: float = 0.0,
+                  activation: str = "silu"):
     """x [m, k] . w[n, k]^T for 1 to 64 bfloat16 rows and k a multiple of 128 (gemm_mid.hip).  `dual`: w = [gate; up],
-    the result silu(x . gate^T) * (x . up^T).  `partial`: the result stays split along k, as `Partials` (a weight that
+    the result act(x . gate^T) * (x . up^T).  `partial`: the result stays split along k, as `Partials` (a weight that
     needs no split gives a plain tensor).  `sums_in` [m, blocks] (up to 16 rows): the rows are a norm's input times its
     weight and these their sums of squares; every sum is multiplied by the row's rsqrt(mean of squares + eps)."""
     _dev(x, w)
@@ -751,6 +792,7 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = tor
                           f"(1 to {MID_MAX_ROWS} rows, k a multiple of 128)")
     n = rows // 2 if dual else rows
     lib = library()
+    act = activation_code(activation) if dual else 0
     if partial:
         splits = lib.ia_gemm_mid_splits(n, k)
         if splits > 1 and (m * n) % 4 == 0:
@@ -763,17 +805,18 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = tor
         if partial or m > 16 or sums_in.dim() != 2 or sums_in.shape[0] != m or not sums_in.is_contiguous():
             raise KernelError(f"gemm_mid: sums of squares {tuple(sums_in.shape)} for {m} rows (up to 16, whole sums)")
         _check(lib.ia_gemm_mid_bf16_scaled(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
-                                           int(dual), _p(sums_in), sums_in.shape[1], ctypes.c_float(eps), _stream()))
+                                           act, _p(sums_in), sums_in.shape[1], ctypes.c_float(eps), _stream()))
         return out
     _check(lib.ia_gemm_mid_bf16(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
-                                int(dual), _stream()))
+                                act, _stream()))
     return out
 
 
-def linear_partials(x: torch.Tensor, w: torch.Tensor):
+def linear_partials(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None):
     """x . w^T for a reader that takes `Partials` (the norm that adds the product to the stream): split along k where the
-    weight has few rows.  None when the product of 17 to 64 rows does not take these operands."""
-    if isinstance(x, torch.Tensor) and mid_fits(x, w):
+    weight has few rows.  None when the product of 17 to 64 rows does not take these operands (a bias among them: the
+    caller then forms the whole product, and `linear` adds the bias)."""
+    if bias is None and isinstance(x, torch.Tensor) and mid_fits(x, w):
         return gemm_mid_bf16(x, w, partial=True)
     return None
 
@@ -794,27 +837,40 @@ def add_rmsnorm_partials(x: torch.Tensor, delta: Partials, w: torch.Tensor, eps:
     return out
 
 
-def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, mid: bool = True) -> torch.Tensor:
-    """x [m, k] . w[n, k]^T.  32-bit: the tiled kernel (true 32-bit, fixed order).  bfloat16: the
-    skinny MFMA kernel for up to SKINNY_MAX_ROWS rows, the vendor's GEMM beyond that (the reference uses
-    cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
+def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, mid: bool = True,
+           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [m, k] . w[n, k]^T (+ bias [n], in the precision of w).  32-bit: the tiled kernel (true 32-bit, fixed
+    order).  bfloat16: the skinny MFMA kernel for up to SKINNY_MAX_ROWS rows, the vendor's GEMM beyond that (the
+    reference uses cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
     the skinny kernel's accumulators for those few rows; beyond that it is the vendor's bfloat16
     result widened, which is what the reference does for every row (its logits are computed in
     the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`).  `mid=False`: steps of 17 to 64 rows
-    go to the vendor's GEMM as well."""
+    go to the vendor's GEMM as well.  The skinny kernel adds a bias to its sums before it rounds them; behind every
+    other product a kernel of its own adds it to the stored rows."""
     out_dtype = out_dtype or x.dtype
+    if bias is not None and (bias.dtype != w.dtype or bias.numel() != w.shape[0]):
+        raise KernelError(f"linear: a bias of {bias.numel()} {bias.dtype} entries for a weight {tuple(w.shape)} {w.dtype}")
     if isinstance(x, NormedRows):
         if _takes_normed_rows(x, w, w.shape[0]):
             _dev(x.scaled, w, x.sums)
-            return _stream_product(x.scaled, w, w.shape[0], out_dtype, False, sums_in=x.sums, eps=x.eps)
+            return _stream_product(x.scaled, w, w.shape[0], out_dtype, False, sums_in=x.sums, eps=x.eps, bias=bias)
         x = x.materialize()
+    if x.dtype == torch.bfloat16 and skinny_fits(x, w) and x.shape[0] <= SKINNY_MAX_ROWS:
+        return gemm_skinny_bf16(x, w, out_dtype, bias=bias)
+    y = _linear_no_bias(x, w, out_dtype if bias is None else x.dtype, mid)
+    if bias is None:
+        return y
+    add_bias(y, bias)
+    return widen(y) if out_dtype == torch.float32 and y.dtype != torch.float32 else y
+
+
+def _linear_no_bias(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, mid: bool) -> torch.Tensor:
+    """The products of `linear` beyond the skinny kernel's rows."""
     if x.dtype == torch.float32:
         return gemm_tiled(x, w, out_dtype)
     m, k = x.shape
     if not skinny_fits(x, w):
         return gemm_tiled(x, w, out_dtype)
-    if m <= SKINNY_MAX_ROWS:
-        return gemm_skinny_bf16(x, w, out_dtype)
     if mid and mid_fits(x, w):
         if out_dtype == torch.float32:
             return gemm_mid_bf16(x, w, torch.float32)
@@ -923,27 +979,37 @@ def _mid_dual_fits(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
             and bool(library().ia_gemm_mid_fills(w_gate_up.shape[0] // 2, w_gate_up.shape[1], 1)))
 
 
-def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(x . gate^T) * (x . up^T) for w_gate_up = [gate; up]: one fused kernel for few bfloat16
-    rows, else the product followed by the element-wise kernel."""
+def gated_linear(x, w_gate_up: torch.Tensor, activation: str = "silu",
+                 bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """act(x . gate^T) * (x . up^T) for w_gate_up = [gate; up] (`activation`: a name of `ACTIVATIONS`; `bias`
+    [2 n]: added to both products before the activation): one fused kernel for few bfloat16 rows, else the
+    product followed by the element-wise kernel."""
     # (few rows too go to gemm_mid.hip where its blocks fill the chip evenly: inside a decode step the pair of this product
     # and the next takes 58.0 us against 60.6 at 8 rows and 60.4 against 67.2 at 16, sizes of an 8B model)
+    activation_code(activation)
+    even = w_gate_up.shape[0] % 2 == 0
     if isinstance(x, NormedRows):
-        if w_gate_up.shape[0] % 2 == 0 and _takes_normed_rows(x, w_gate_up, w_gate_up.shape[0] // 2):
+        if even and _takes_normed_rows(x, w_gate_up, w_gate_up.shape[0] // 2):
             _dev(x.scaled, w_gate_up, x.sums)
-            if _mid_dual_fits(x.scaled, w_gate_up):
-                return gemm_mid_bf16(x.scaled, w_gate_up, dual=True, sums_in=x.sums, eps=x.eps)
+            if bias is None and _mid_dual_fits(x.scaled, w_gate_up):
+                return gemm_mid_bf16(x.scaled, w_gate_up, dual=True, sums_in=x.sums, eps=x.eps, activation=activation)
             return _stream_product(x.scaled, w_gate_up, w_gate_up.shape[0] // 2, x.scaled.dtype, True,
-                                   sums_in=x.sums, eps=x.eps)
+                                   sums_in=x.sums, eps=x.eps, activation=activation, bias=bias)
         x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
-        if _mid_dual_fits(x, w_gate_up):
-            return gemm_mid_bf16(x, w_gate_up, dual=True)
-        return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True)
-    if (w_gate_up.shape[0] % 2 == 0 and mid_fits(x, w_gate_up)
-            and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES):
-        return gemm_mid_bf16(x, w_gate_up, dual=True)
-    if w_gate_up.shape[0] % 2 == 0 and x.dtype == torch.bfloat16 and skinny_fits(x, w_gate_up) and _own_large(x, w_gate_up):
-        return gemm_mfma_bf16(x, w_gate_up, dual=True)
+        if bias is None and _mid_dual_fits(x, w_gate_up):
+            return gemm_mid_bf16(x, w_gate_up, dual=True, activation=activation)
+        return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True, activation=activation, bias=bias)
+    if bias is None:
+        if (even and mid_fits(x, w_gate_up)
+                and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES):
+            return gemm_mid_bf16(x, w_gate_up, dual=True, activation=activation)
+        if even and x.dtype == torch.bfloat16 and skinny_fits(x, w_gate_up) and _own_large(x, w_gate_up):
+            return gemm_mfma_bf16(x, w_gate_up, dual=True, activation=activation)
     # (a [gate; up] beyond MID_DUAL_MAX_BYTES at 17 to 64 rows: the vendor's GEMM, not the plain product of gemm_mid.hip)
-    return silu_mul(linear(x, w_gate_up, mid=False))
+    return gate_mul(linear(x, w_gate_up, mid=bias is not None, bias=bias), activation)
+
+
+def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """`gated_linear` with SiLU and no bias."""
+    return gated_linear(x, w_gate_up, "silu")

@@ -38,6 +38,12 @@ class Attention(Mixer):
         if spec.qk_norm is not None:
             t["q_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
             t["k_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
+        if spec.qkv_bias:
+            t["q_proj.bias"] = TensorSpec((q_out,))
+            t["k_proj.bias"] = TensorSpec((kv_out,))
+            t["v_proj.bias"] = TensorSpec((kv_out,))
+        if spec.o_bias:
+            t["o_proj.bias"] = TensorSpec((spec.hidden,))
         return t
 
     @classmethod
@@ -59,9 +65,9 @@ class Attention(Mixer):
         if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
             raise SpecError("attention: qk_norm must span head_dim")
         self.spec = spec
-        self.qkv = Linear([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]],
-                          dtype, device)
-        self.o = Linear([tensors["o_proj.weight"]], dtype, device)
+        self.qkv = Linear([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dtype, device,
+                          [tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]] if spec.qkv_bias else None)
+        self.o = Linear([tensors["o_proj.weight"]], dtype, device, [tensors["o_proj.bias"]] if spec.o_bias else None)
         if spec.qk_norm is not None:
             self.q_norm_w = tensors["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
             self.k_norm_w = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
@@ -71,15 +77,30 @@ class Attention(Mixer):
             self.norm_eps, self.norm_add_one = 0.0, False
         self.position = part_class("position", spec.position)(spec.position, {}, dtype, device)
 
+    def load_notes(self, page_size: int):
+        """What the log should say once when a model with this part is set up: a decode step that cannot take the
+        fused kernel still runs, three kernels where one would do."""
+        dtype = self.qkv.weight.dtype
+        has_rotation = self.position.rot_dim > 0
+        if dtype != torch.bfloat16 or ops.attention_decode_fused_fits(dtype, self.spec.head_dim, page_size,
+                                                                      self.position.rot_dim, self.position.interleaved,
+                                                                      has_rotation):
+            return []
+        s = self.spec
+        return [f"attention with head size {s.head_dim}, page size {page_size}, rotation of {self.position.rot_dim} features "
+                f"({'interleaved' if self.position.interleaved else 'halves'}): decode steps do not take the fused kernel "
+                "(head sizes in steps of 64, page sizes in steps of 16, whole heads rotated in halves); norm and "
+                "rotation, the cache write and the attention run as kernels of their own"]
+
     def _project(self, ctx, a: torch.Tensor):
         """The output projection: added to the step's stream by the product itself where that can be."""
         if getattr(ctx, "stream", None) is not None:
             norm = getattr(ctx, "stream_norm", None)
-            added = ops.linear_add(a, self.o.weight, ctx.stream, norm)
+            added = ops.linear_add(a, self.o.weight, ctx.stream, norm, self.o.bias)
             if added is not None:
                 return ops.Added(added[0], added[1], norm)
         if getattr(ctx, "partial_sums", False):
-            split = ops.linear_partials(a, self.o.weight)
+            split = ops.linear_partials(a, self.o.weight, self.o.bias)
             if split is not None:
                 return split
         return self.o(a)

@@ -19,7 +19,7 @@ finds the stream in `ctx.stream` (and in `ctx.stream_norm` the norm part that re
 add its output to it itself, returning `ops.Added` (the new rows' partial sums of squares, and the
 rows times that norm's weight) instead of the output; one with `takes_normed_rows = True` may be
 handed `ops.NormedRows` instead of normed rows, whose norm its first product finishes (`ops.linear`
-and `ops.gated_silu_linear` take them; `.materialize()` gives plain rows).  A norm takes part if it
+and `ops.gated_linear` take them; `.materialize()` gives plain rows).  A norm takes part if it
 offers `rows_for_product(x, added)`.  Parts without these attributes are run as ever.
 """
 from __future__ import annotations

@@ -266,3 +266,35 @@ def test_chat_template_comes_from_the_folder_or_the_architecture(tmp_path):
     assert chat.render("chatml", "hi", "be brief") == ("<|im_start|>system\nbe brief<|im_end|>\n<|im_start|>user\nhi<|im_end|>\n"
                                                       "<|im_start|>assistant\n")
     assert chat.render("plain", "hi") == "hi"
+
+
+@pytest.mark.parametrize("key,value", [("attention_bias", True), ("rope_scaling", {"rope_type": "yarn", "factor": 4.0}),
+                                       ("hidden_act", "gelu"), ("use_sliding_window", True),
+                                       ("layer_types", ["full_attention", "sliding_attention"])])
+def test_values_that_the_model_does_not_honour_are_refused(tmp_path, key, value):
+    """The reference reads these keys and ignores them (`inferrs-models/src/config.rs:291-292`, `qwen3.rs:28-45`): a
+    folder that asks for biases, a scaled rotation, a window or another activation would be computed as another model.
+    Here the load fails and names key and value; `allow_ignored_keys` gives the reference's silence back."""
+    raw = dict(TINY_A, **{key: value})
+    with pytest.raises(ConfigError) as err:
+        Qwen3Config.from_dict(raw)
+    assert f"'{key}'" in str(err.value) and repr(value) in str(err.value)
+    assert Qwen3Config.from_dict(raw, allow_ignored_keys=True) == Qwen3Config.from_dict(TINY_A)
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    with pytest.raises(ConfigError, match=key):
+        load_config(str(tmp_path))
+    assert load_config(str(tmp_path), allow_ignored_keys=True) == Qwen3Config.from_dict(TINY_A)
+
+
+def test_values_that_change_nothing_are_accepted():
+    """What real folders of this architecture hold: the keys are there, with the values that the model has anyway."""
+    raw = dict(TINY_A, attention_bias=False, rope_scaling=None, hidden_act="silu", use_sliding_window=False,
+               sliding_window=4096, max_window_layers=2, layer_types=["full_attention", "full_attention"],
+               attention_dropout=0.0, torch_dtype="bfloat16")
+    assert Qwen3Config.from_dict(raw) == Qwen3Config.from_dict(TINY_A)
+
+
+def test_several_unhonoured_values_are_named_together():
+    with pytest.raises(ConfigError) as err:
+        Qwen3Config.from_dict(dict(TINY_A, attention_bias=True, hidden_act="gelu_pytorch_tanh"))
+    assert "'attention_bias' = True" in str(err.value) and "'hidden_act' = 'gelu_pytorch_tanh'" in str(err.value)

@@ -133,17 +133,16 @@ def test_command_line_run_and_bench(tiny):
     assert proc.returncode == 0, proc.stderr[-2000:]
     rec = json.loads(proc.stdout.strip().splitlines()[-1])
     assert rec["prefill_tok_s"] > 0 and rec["decode_tok_s"] > 0
-    # without a prompt: the read-eval loop with the reference's commands
-    script = "/set temperature 0\n/set max_tokens 5\n/show params\n/nonsense\n" + " ".join(map(str, prompt)) + "\n/bye\n"
-    proc = subprocess.run(exe + ["run", folder, "--dtype", "f32", "--repetition-penalty", "1.0", "--block-size", "4",
-                                 "--max-blocks", "32", "--max-batch-size", "2"], input=script,
-                          capture_output=True, text=True, timeout=300)
+    # without a prompt: one prompt a line from standard input, each answered on its own
+    other = random_tokens(4, TINY["A"]["vocab_size"], 8)
+    want_other, _ = plain_greedy_with_margins(cfg, params, other, 5)
+    script = " ".join(map(str, prompt)) + "\n\n" + ",".join(map(str, other)) + "\n"
+    proc = subprocess.run(exe + ["run", folder, "--dtype", "f32", "--temperature", "0", "--repetition-penalty", "1.0",
+                                 "--max-tokens", "5", "--block-size", "4", "--max-blocks", "32", "--max-batch-size", "2"],
+                          input=script, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     out = proc.stdout.splitlines()
-    assert out[0] == "temperature set to 0.0" and out[1] == "max_tokens set to 5"
-    assert out[2].startswith("temperature=0.0 ") and "max_tokens=5" in out[2]
-    assert out[3] == "Unknown command: /nonsense"
-    assert [int(t) for t in out[4].split()] == want
+    assert [[int(t) for t in line.split()] for line in out] == [want, want_other]
     proc = subprocess.run(exe + ["serve", folder], capture_output=True, text=True, timeout=60)
     assert proc.returncode == 2 and "not part of this engine" in proc.stderr
 

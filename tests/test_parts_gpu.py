@@ -777,3 +777,127 @@ def test_toy_ends_arrangement_and_unequal_key_and_value_widths(tmp_path, dtype, 
         err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
         assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
         eng.cache.check_invariants()
+
+
+# ---- a fourth toy architecture: biases on every projection, another activation in the gate -------------
+
+def register_toy_biased():
+    from inferrs_amd.config import AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec, ScheduleEntry
+    from inferrs_amd.config.registry import register_architecture
+
+    class BiasedConfig:
+        architecture = "ToyBiasedForCausalLM"
+        model_type = "toy_biased"
+
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def to_dict(self):
+            return dict(self.raw, architectures=[self.architecture], model_type=self.model_type)
+
+        def to_spec(self):
+            r = self.raw
+            h, d = r["hidden_size"], r["head_dim"]
+            norm = NormSpec(size=h, eps=r["eps"])
+            attn = AttentionSpec(hidden=h, n_heads=r["heads"], n_kv_heads=r["kv_heads"], head_dim=d,
+                                 position=PositionSpec(kind="rope", head_dim=d, rot_dim=d, theta=1e4),
+                                 qk_norm=NormSpec(size=d, eps=r["eps"]), qkv_bias=True, o_bias=True)
+            ffn = GatedMlpSpec(hidden=h, intermediate=r["intermediate"], activation="gelu_tanh", bias=True)
+
+            def layer(i):
+                p = f"blocks.{i}."
+                return LayerSpec(mixer=attn, ffn=ffn, norms=(norm, norm), norm_names=(p + "norm1.weight", p + "norm2.weight"),
+                                 mixer_prefix=p + "mixer.", ffn_prefix=p + "ffn.")
+            return ModelSpec(architecture=self.architecture, vocab_size=r["vocab"], hidden=h,
+                             layers=tuple(layer(i) for i in range(r["layers"])),
+                             schedule=tuple(ScheduleEntry(i) for i in range(r["layers"])), final_norm=norm,
+                             final_norm_name="norm.weight", embed_name="embed.weight", head_name=None, max_position=512)
+
+    register_architecture(BiasedConfig)
+    return BiasedConfig
+
+
+def gelu_tanh(x):
+    return 0.5 * x * (1.0 + torch.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
+
+
+def toy_biased_plain(p, raw, ids):
+    t = len(ids)
+    x = p["embed.weight"][torch.as_tensor(ids)]
+    d, nq, nkv = raw["head_dim"], raw["heads"], raw["kv_heads"]
+    cos, sin = pm.rope_tables(torch.arange(t), 1e4, d)
+    cos, sin = cos.double(), sin.double()
+    causal = torch.arange(t)[None, :] > torch.arange(t)[:, None]
+    for i in range(raw["layers"]):
+        pre = f"blocks.{i}."
+        lin = lambda v, name: pm.linear(v, p[pre + name + ".weight"]) + p[pre + name + ".bias"]
+        h = pm.rms_norm(x, p[pre + "norm1.weight"], raw["eps"])
+        q = lin(h, "mixer.q_proj").reshape(t, nq, d).transpose(0, 1)
+        k = lin(h, "mixer.k_proj").reshape(t, nkv, d).transpose(0, 1)
+        v = lin(h, "mixer.v_proj").reshape(t, nkv, d).transpose(0, 1)
+        q = pm.rope_half(pm.rms_norm(q, p[pre + "mixer.q_norm.weight"], raw["eps"]), cos, sin)
+        k = pm.rope_half(pm.rms_norm(k, p[pre + "mixer.k_norm.weight"], raw["eps"]), cos, sin)
+        k, v = pm.repeat_kv(k, nq // nkv), pm.repeat_kv(v, nq // nkv)
+        s = (torch.matmul(q, k.transpose(1, 2)) / d ** 0.5).masked_fill(causal, float("-inf"))
+        x = x + lin(torch.matmul(pm.softmax_last(s), v).transpose(0, 1).reshape(t, nq * d), "mixer.o_proj")
+        h = pm.rms_norm(x, p[pre + "norm2.weight"], raw["eps"])
+        x = x + lin(gelu_tanh(lin(h, "ffn.gate_proj")) * lin(h, "ffn.up_proj"), "ffn.down_proj")
+    return pm.linear(pm.rms_norm(x, p["norm.weight"], raw["eps"]), p["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype,page,sizes", [("float32", 4, (48, 4, 2, 16, 80)), ("bfloat16", 16, (48, 4, 2, 16, 80)),
+                                              ("bfloat16", 16, (128, 4, 2, 64, 256))])
+def test_toy_biases_and_another_gate_activation(tmp_path, dtype, page, sizes):
+    """Attention whose four projections have biases and a gated feed-forward with biases and GELU (tanh form) in the
+    gate, from the framework's own parts by their specs alone.  The second bfloat16 case has widths in steps of 128 and
+    head size 64: decode steps keep the fused attention kernel and the products that take over the stream's sums and
+    norms (the bias goes into their sums), and its steps of 17 to 64 rows run the products made for them with the
+    bias added behind."""
+    from call_counter import CallCounter
+    from inferrs_amd.engine import Engine, run_trace
+    from inferrs_amd.weights import write_random_model
+    BiasedConfig = register_toy_biased()
+    hidden, heads, kv_heads, head_dim, inter = sizes
+    raw = dict(hidden_size=hidden, heads=heads, kv_heads=kv_heads, head_dim=head_dim, intermediate=inter, vocab=97,
+               eps=1e-5, layers=2)
+    folder = write_random_model(str(tmp_path / "biased"), BiasedConfig(raw), seed=12)
+    from safetensors.torch import load_file, save_file
+    loaded = load_file(os.path.join(folder, "model.safetensors"))
+    assert loaded["blocks.1.mixer.k_proj.bias"].shape == (kv_heads * head_dim,) and "blocks.0.ffn.down_proj.bias" in loaded
+    # biases as large as the products they are added to, so that a lost or misplaced one shows
+    for name in loaded:
+        if name.endswith(".bias"):
+            loaded[name] = (loaded[name].float() * 20).to(loaded[name].dtype)
+    save_file(loaded, os.path.join(folder, "model.safetensors"))
+    p = {k: v.double() for k, v in loaded.items()}
+    reqs = {f"r{i}": random_tokens(n, 97, 90 + i) for i, n in enumerate([3, 21, 45, 70])}
+    ref = {r: toy_biased_plain(p, raw, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for mode, trace in (("whole", tm.whole(reqs)), ("tail", tm.prefix_then_single(reqs, 12)),
+                        ("portions", tm.portions(reqs, [5, 2, 19, 33])), ("mixed", tm.mixed(reqs, seed=3, max_live=4, decode_tail=9))):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-trace.max_tokens // page) + 2, max_seqs=4)
+        assert eng.model.graph_safe
+        assert bool(eng.load_notes) == (dtype == "bfloat16" and head_dim % 64 != 0)     # off the fused decode kernel: said once
+        with CallCounter("attention_decode_fused", "_stream_product", "add_bias") as counted:
+            run_trace(eng, trace.lines, str(tmp_path / mode), io.StringIO())
+        if dtype == "bfloat16" and head_dim == 64 and mode == "tail":
+            assert counted.calls["attention_decode_fused"] > 0 and counted.calls["_stream_product"] > 0, counted.calls
+            assert eng.graph_replays > 0
+        if dtype == "float32" or mode == "portions":
+            assert counted.calls["add_bias"] > 0
+        got = trace.read(str(tmp_path / mode), 97)
+        err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
+        assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
+        eng.cache.check_invariants()
+
+
+def test_an_activation_without_a_kernel_is_refused_by_name():
+    from inferrs_amd.config import GatedMlpSpec, SpecError
+    from inferrs_amd.parts import part_class
+    spec = GatedMlpSpec(hidden=8, intermediate=8, activation="relu")
+    with pytest.raises(SpecError, match="relu.*gelu_tanh.*silu"):
+        part_class("ffn", spec)(spec, {}, torch.float32, DEV)

@@ -311,6 +311,49 @@ def test_whole_model_shift_and_prefix_invariants(tmp_path, name):
         assert p["lm_head.weight"].shape == (raw["vocab_size"], raw["hidden_size"])
     # greedy continuation feeds its own tokens back: the arg max of the logits after each of them
     out = pm.greedy(cfg, p, toks[:5], 3)
-    assert out[0] == int(torch.argmax(full[4])) or toks[5] != out[0]
+    assert out[0] == int(torch.argmax(full[4]))            # (causality: position 4 does not see what follows it)
     assert out[1] == int(torch.argmax(pm.forward(cfg, p, toks[:5] + out[:1])[-1]))
     assert out[2] == int(torch.argmax(pm.forward(cfg, p, toks[:5] + out[:2])[-1]))
+
+
+def _two_ends_model(tmp_path, **changes):
+    """Tiny configuration B (its head is a matrix of its own) in 64-bit, with `changes` to its config."""
+    folder = write_model(str(tmp_path / "ends"), TINY["B"], seed=6)
+    cfg, p = pm.read_model(folder, torch.float64)
+    assert "lm_head.weight" in p and not TINY["B"]["tie_word_embeddings"]
+    return dict(cfg, **changes), p
+
+
+def test_final_norm_stands_before_the_head(tmp_path):
+    """`x = norm(x)` before the logits (qwen3.rs:398-405, attention_utils.rs:382-395).  Scale the embedding table and
+    every output projection (o_proj, down_proj) by c: every part reads the normed stream, so each addition and the
+    stream itself become c times what they were, and a norm in front of the head takes the factor out again: the
+    logits do not change.  Without the final norm they would be c times as large; with a norm applied to something
+    else than the final stream (only the last layer's addition, say) the factor would survive as well."""
+    cfg, p = _two_ends_model(tmp_path, rms_norm_eps=1e-14)            # (so that a scale drops out exactly)
+    toks = random_tokens(19, TINY["B"]["vocab_size"], 3)
+    base = pm.forward(cfg, p, toks)
+    c = 7.0
+    scaled = {k: (c * v if k == "model.embed_tokens.weight" or k.endswith(("o_proj.weight", "down_proj.weight")) else v)
+              for k, v in p.items()}
+    assert float((pm.forward(cfg, scaled, toks) - base).abs().max()) < 1e-9 * float(base.abs().max())
+    # the check can fail: scale the head instead and the logits follow
+    louder = dict(p, **{"lm_head.weight": c * p["lm_head.weight"]})
+    assert torch.allclose(pm.forward(cfg, louder, toks), c * base, rtol=1e-12)
+
+
+def test_embedding_enters_the_stream_unscaled(tmp_path):
+    """`x = embed(ids)` and nothing else (qwen3.rs:398-400: no sqrt(hidden) factor as other families have).  With
+    output projections of zero the stream is the embedding row itself, and with an eps so large that the norm's
+    divisor is sqrt(eps) the logits are (E[id] * w_final) . W_head^T / sqrt(eps) in plain arithmetic: a factor on the
+    embedding would show one to one."""
+    eps = 1e6
+    cfg, p = _two_ends_model(tmp_path, rms_norm_eps=eps)
+    silent = {k: (torch.zeros_like(v) if k.endswith(("o_proj.weight", "down_proj.weight")) else v) for k, v in p.items()}
+    toks = random_tokens(13, TINY["B"]["vocab_size"], 4)
+    got = pm.forward(cfg, silent, toks)
+    rows = p["model.embed_tokens.weight"][torch.as_tensor(toks)]
+    want = (rows * p["model.norm.weight"]) @ p["lm_head.weight"].T / eps ** 0.5
+    assert float((got - want).abs().max()) < 1e-6 * float(want.abs().max())
+    hidden = TINY["B"]["hidden_size"]
+    assert float((got - want * hidden ** 0.5).abs().max()) > 0.5 * float(want.abs().max())     # what a scaled embedding would give

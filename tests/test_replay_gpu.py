@@ -29,6 +29,7 @@ import torch
 
 import plain_model as pm
 import trace_modes as tm
+from call_counter import CallCounter
 from tiny_configs import PAGE_SIZE, TINY, random_tokens, write_model
 
 pytestmark = pytest.mark.gpu
@@ -394,3 +395,108 @@ def test_real_layer_sizes_long_prompt_in_portions(tmp_path):
         assert err <= 2e-2, f"{mode}: {err:.3e} at {where}"
         del eng
         torch.cuda.empty_cache()
+
+
+@pytest.fixture(scope="module")
+def many_requests(models):
+    """64 requests of different lengths on configuration G (widths in steps of 128, head size 128: the products of 17 to
+    64 rows run on the kernels made for them, the two of 1,024 inputs split along k), each a prompt and 12 tokens that
+    are fed one by one whatever the model would choose; the plain implementation's logits at the fed places, and the
+    bfloat16 bound measured on these very sequences."""
+    folder, raw, _, _ = models[("G", 1.0)]
+    n_steps = 12
+    prompts = [random_tokens(3 + (7 * i) % 61 + i, raw["vocab_size"], 900 + i) for i in range(64)]
+    feeds = [random_tokens(n_steps, raw["vocab_size"], 1900 + i) for i in range(64)]
+    cfg, params = pm.read_model(folder, torch.float64)
+    cfg_b, params_b = pm.read_model(folder, torch.bfloat16)
+    ref, err = [], 0.0
+    for p, f in zip(prompts, feeds):
+        exact = pm.forward(cfg, params, p + f).numpy()[len(p):]
+        rounded = pm.forward(cfg_b, params_b, p + f).float().numpy()[len(p):]
+        ref.append(exact.astype(np.float32))
+        err = max(err, float(np.abs(rounded - exact).max()))
+    scale = max(float(np.abs(r).max()) for r in ref)
+    return folder, raw, prompts, feeds, ref, scale, err / scale
+
+
+@pytest.mark.parametrize("n_req", [24, 40, 64])
+def test_decode_steps_of_17_to_64_requests(many_requests, n_req):
+    """24, 40 and 64 requests decode 12 steps side by side: eagerly and through captured graphs, every step's logits
+    against each other and against the plain implementation.  The products must have run on the kernels of 17 to 64
+    rows, the split ones added up by the norm that follows them."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, raw, prompts, feeds, ref, scale, limit = many_requests
+    n_steps = len(feeds[0])
+    outs = {}
+    for graphs in (False, True):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=n_req * 8, max_seqs=n_req + 1,
+                                 use_graphs=graphs)
+        for i in range(n_req):
+            eng.step([Entry(i, prompts[i], [])])
+        with CallCounter("gemm_mid_bf16", "add_rmsnorm_partials") as counted:
+            rows = []
+            for s in range(n_steps):
+                logits = eng.step([Entry(i, [feeds[i][s]], [0]) for i in range(n_req)])
+                rows.append(logits.cpu().numpy().copy())
+                if s % 5 == 2:                   # an eager step of another shape between the replays
+                    eng.step([Entry("extra", random_tokens(19, raw["vocab_size"], s), [18])])
+                    eng.end_request("extra")
+        outs[graphs] = rows
+        assert (eng.graph_replays >= n_steps - 2) == graphs
+        layers = raw["num_hidden_layers"]
+        # q|k|v, o, [gate; up] and down of every layer in every step that was not a replay; o and down leave splits
+        eager_steps = n_steps if not graphs else 2
+        assert counted.calls["gemm_mid_bf16"] >= 4 * layers * eager_steps, counted.calls
+        assert counted.calls["add_rmsnorm_partials"] >= (2 * layers - 1) * eager_steps, counted.calls
+        eng.cache.check_invariants()
+    for graphs in (False, True):
+        for s in range(n_steps):
+            want = np.stack([ref[i][s] for i in range(n_req)])
+            err = float(np.abs(outs[graphs][s] - want).max()) / scale
+            assert err <= limit, f"graphs={graphs} step {s}: {err:.3e} of the scale against the plain implementation ({limit:.3e})"
+    # eager step and replay run the same kernels; the padded block tables may split the keys differently
+    errs = [float(np.abs(outs[True][s] - outs[False][s]).max()) / scale for s in range(n_steps)]
+    assert max(errs) <= limit / 2, f"replays differ from eager steps: {errs}"
+
+
+@pytest.mark.parametrize("n_req", [24, 64])
+def test_runs_of_decode_steps_of_many_requests(many_requests, n_req):
+    """The generation loop queues eight decode steps of 24 or 64 requests at once; the tokens are those of single
+    steps (greedy; both runs replay the same graphs, so the bits are the same)."""
+    from inferrs_amd.engine import Engine, GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    folder, raw, prompts, *_ = many_requests
+    results = {}
+    for run in (1, 8):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=n_req * 8, max_seqs=n_req)
+        loop = GenerationLoop(eng, decode_run=run, max_batch_size=n_req, stop_token_ids=[])
+        reqs = [loop.add(prompts[i], SamplingParams.greedy(max_tokens=21)) for i in range(n_req)]
+        with CallCounter("gemm_mid_bf16") as counted:
+            loop.run()
+        results[run] = [list(r.output) for r in reqs]
+        assert counted.calls["gemm_mid_bf16"] > 0
+        assert eng.graph_replays >= 12
+        eng.cache.check_invariants()
+        assert not eng.cache.sequences
+    assert results[8] == results[1]
+    assert all(len(o) == 21 for o in results[8])
+
+
+def test_twenty_decodes_beside_a_prompt_portion(many_requests):
+    """One step of 20 decoded tokens and a 30-token portion of another request's prompt (50 rows: the products of 17 to
+    64 rows, the attention launched apart for the two kinds), against the plain implementation."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, raw, prompts, feeds, ref, scale, limit = many_requests
+    eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=200, max_seqs=22)
+    for i in range(20):
+        eng.step([Entry(i, prompts[i], [])])
+    long = prompts[63] + feeds[63]
+    cut = len(prompts[63]) - 25
+    eng.step([Entry("p", long[:cut], [])])
+    with CallCounter("gemm_mid_bf16") as counted:
+        got = eng.step([Entry(i, [feeds[i][0]], [0]) for i in range(20)]
+                       + [Entry("p", long[cut:cut + 30], [25, 29])]).cpu().numpy()
+    assert counted.calls["gemm_mid_bf16"] >= 4 * raw["num_hidden_layers"]
+    want = np.stack([ref[i][0] for i in range(20)] + [ref[63][0], ref[63][4]])
+    err = float(np.abs(got - want).max()) / scale
+    assert err <= limit, f"{err:.3e} of the scale against the plain implementation ({limit:.3e})"

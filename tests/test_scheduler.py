@@ -226,3 +226,44 @@ def test_a_budget_below_the_number_of_decodes_starves_nobody():
     for i in range(5):
         gaps = [b - a for a, b in zip(served[i], served[i][1:]) if a in both and b in both]
         assert gaps and max(gaps) <= 3, (i, served[i])
+
+
+def test_make_trace_program_and_modes(tmp_path):
+    """`bin/make_trace` and `make_trace`: every mode feeds every token of every request exactly once and in order,
+    asks for every position's logits once, ends every request, and states the pool that the replay needs."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from inferrs_amd.engine.trace import MODES, make_trace
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    requests = {"a": list(range(3)), "b": list(range(100, 170)), "c": list(range(200, 333)), "d": [7]}
+    for mode in MODES:
+        trace = make_trace(requests, mode, tail=9, sizes=[5, 2, 31], seed=3, max_live=3)
+        fed = {r: [] for r in requests}
+        wanted = {r: [] for r in requests}
+        ended = []
+        for i, line in enumerate(trace.lines):
+            rec = json.loads(line)
+            assert rec["step"] == i
+            for e in rec["entries"]:
+                assert e["id"] not in ended
+                start = len(fed[e["id"]])
+                fed[e["id"]] += e["tokens"]
+                wanted[e["id"]] += [start + w for w in e["want"]]
+            ended += rec["end"]
+        assert fed == requests and sorted(ended) == sorted(requests), mode
+        assert all(wanted[r] == list(range(len(t))) for r, t in requests.items()), mode
+        assert trace.max_live <= (3 if mode == "mixed" else 1)
+        assert trace.max_tokens >= 192 and trace.max_tokens % 64 == 0
+    with pytest.raises(ValueError, match="unknown mode"):
+        make_trace(requests, "sideways")
+    manifest = tmp_path / "m.json"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "make_trace"), "--mode", "mixed", "--lengths", "5,37,70",
+                           "--vocab", "50", "--seed", "4", "--manifest", str(manifest)], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    info = json.loads(manifest.read_text())
+    lines = proc.stdout.splitlines()
+    assert sorted(len(t) for t in info["requests"].values()) == [5, 37, 70] and info["max_tokens"] % 64 == 0
+    assert sum(len(rows) for rows in info["rows"].values()) == 112 and len(lines) > 10
+    assert all(0 <= t < 50 for line in lines for e in json.loads(line)["entries"] for t in e["tokens"])
