@@ -216,6 +216,53 @@ def kernel_breakdown(engine, batch: int, context: int, prefill_tokens: int, voca
             for phase, table in out.items()}
 
 
+def host_gap(engine, entries_of, repeats: int = 3):
+    """One eager step as the host sees it: (wall milliseconds from the call to the synchronised end, milliseconds of
+    the same step's kernels replayed from a captured graph, kernel calls of the step).  What is between the two is the
+    host: Python between the kernel calls, where the GPU waits for the next launch.  `entries_of()` sets the step's
+    requests up and returns (entries, clean-up)."""
+    import torch
+    from inferrs_amd import ops
+    graphs, engine.use_graphs = engine.use_graphs, False
+    try:
+        walls = []
+        for _ in range(repeats + 1):
+            entries, cleanup = entries_of()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.step(entries)
+            torch.cuda.synchronize()
+            walls.append(time.perf_counter() - t0)
+            cleanup()
+        # the same step's kernels without the host between them: captured once, replayed
+        entries, cleanup = entries_of()
+        for e in entries:
+            if not engine.has_request(e.seq_id):
+                engine.add_request(e.seq_id)
+        if not engine.cache.ensure_reserved([(e.seq_id, len(e.tokens)) for e in entries]):
+            raise RuntimeError("the cache pool is too small for this step")
+        ctx = engine.builder.build([(e.seq_id, e.tokens, e.want) for e in entries])
+        with ops.KernelTimer() as timer:
+            engine.model.forward(ctx, engine.storage)
+        n_calls = sum(calls for calls, _us in timer.summary().values())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            engine.model.forward(ctx, engine.storage)
+        replays = []
+        for _ in range(repeats + 1):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            torch.cuda.synchronize()
+            replays.append(a.elapsed_time(b))
+        del graph
+        cleanup()
+    finally:
+        engine.use_graphs = graphs
+    return min(walls[1:]) * 1e3, min(replays[1:]), n_calls
+
+
 WORKLOADS = {
     # name: (shape, requests, shortest prompt, longest prompt, portion, decode tokens)
     "mixed16": ("14B", 16, 128, 4096, 512, 128),
@@ -441,6 +488,45 @@ def main() -> int:
             firsts.append(time.perf_counter() - t0)
         record["prefill"]["first_token_ms"] = round(min(firsts) * 1e3, 3)
         if args.extra_points:
+            # shorter contexts and prompts, where a step is short and the host's share of it largest: the reference's
+            # own bench times a prompt of 128 tokens (inferrs/src/bench.rs:35-37)
+            for context in (512, 2048):
+                if context < args.context:
+                    for b in sorted(set([1, args.batch] + ([64] if 64 in points_batches else []))):
+                        decode_point(f"decode_b{b}_ctx{context}", b, context)
+            for tokens in (128, 512):
+                if tokens < args.prefill_tokens:
+                    rec = prefill_record(tokens, 3)
+                    points[f"prefill_{tokens}"] = rec["value"]
+                    fractions[f"prefill_{tokens}_mfma"] = rec["frac"]
+            # eager steps as the host sees them: wall time against the sum of the kernels' own times
+            from inferrs_amd.engine import Entry
+            note("eager steps: wall time against the kernels' times")
+            gp = torch.Generator().manual_seed(5)
+            portion = torch.randint(0, vocab, (512,), generator=gp).tolist()
+            mixed_context = min(2048, args.context)
+
+            def mixed_step():
+                ids = [f"m{i}" for i in range(args.batch)]
+                fill_context(engine, ids, mixed_context - 1)
+                def cleanup():
+                    for sid in ids + ["mp"]:
+                        if engine.has_request(sid):
+                            engine.end_request(sid)
+                return [Entry(sid, [1 + i], [0]) for i, sid in enumerate(ids)] + [Entry("mp", portion, [511])], cleanup
+
+            def short_prompt(tokens):
+                def setup():
+                    return [Entry("hp", portion[:tokens], [tokens - 1])], lambda: engine.end_request("hp")
+                return setup
+
+            host = {}
+            for name, setup in ((f"mixed_{args.batch}_decodes_and_512", mixed_step), ("prefill_128", short_prompt(128)),
+                                ("prefill_512", short_prompt(512))):
+                wall, kernels, calls = host_gap(engine, setup)
+                host[name] = {"wall_ms": round(wall, 3), "graph_ms": round(kernels, 3), "kernel_calls": calls,
+                              "host_frac": round(max(0.0, 1.0 - kernels / wall), 4)}
+            record["eager_steps"] = host
             long_prompt = 4 * args.prefill_tokens
             note(f"prefill of {long_prompt} tokens")
             rec = prefill_record(long_prompt, 3)

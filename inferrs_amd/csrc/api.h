@@ -73,7 +73,7 @@ int ia_gemm_skinny_stream(void* out, const void* x, const void* w, const void* b
                           int dual, void* resid, float* sums_out, void* scaled_out, const float* next_w,
                           int add_one, const float* sums_in, int n_sums, float eps, hipStream_t stream);
 
-// Products of 17 to 64 bfloat16 rows (gemm_mid.hip); K a multiple of 128.  out_mode 0: out [M, N] bfloat16; 1: float;
+// Products of 17 to 128 bfloat16 rows (gemm_mid.hip); K a multiple of 128.  out_mode 0: out [M, N] bfloat16; 1: float;
 // 2: out [ia_gemm_mid_splits(N, K)][M][N] float, the sums of each split of k, to be added up by the reader
 // (ia_sum_partials, ia_add_rmsnorm_partials).  dual: w = [gate; up], out = act(x . gate^T) * (x . up^T), mode 0.
 int ia_gemm_mid_splits(int N, int K);

@@ -1,7 +1,9 @@
-// bfloat16 products for steps of 17 to 64 rows (decode steps of many requests, short prompt portions):
+// bfloat16 products for steps of 17 to 128 rows (decode steps of many requests, short prompt portions):
 // out[M, N] = x[M, K] . w[N, K]^T, bound by reading the weights once, like the skinny product, but with so
 // many rows that the activations can no longer be fetched by every wave for itself (at 64 rows they are as
-// large as a block's share of the weights).  A [gate; up] whose blocks fill the chip evenly comes here with fewer rows
+// large as a block's share of the weights).  65 to 128 rows (six or eight tiles of rows) walk k in chunks of 64, four
+// stages deep, so that the stages still fit a compute unit's shared memory; a wave then reads nine operands from
+// shared memory for eight matrix products, which is about what the memory delivers of weights meanwhile.  A [gate; up] whose blocks fill the chip evenly comes here with fewer rows
 // too (ia_gemm_mid_bf16_scaled: rows of a residual stream whose norm the product finishes).
 //
 // The reference hands these products to cuBLAS like all others (`candle-core/src/cuda_backend/mod.rs:2260-2305`).
@@ -283,7 +285,8 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     };
     ring(tail_step, c);
     ring(tail_step, c + NS);
-    static_assert(!DUAL || TILES * MT * IA_WAVE * sizeof(gmid_f32x4) <= STAGE_BYTES, "the sums fit a stage");
+    static_assert(!DUAL || FEATURE_TILES * MT * IA_WAVE * sizeof(gmid_f32x4) <= STAGE_BYTES, "the up rows' sums fit a stage");
+    static_assert(NS * STAGE_BYTES <= 160 * 1024, "the stages fit a compute unit's shared memory");
     if constexpr (MT == 1) {
         if (sums_in != nullptr) {
 #pragma unroll
@@ -407,7 +410,7 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
         // a stored product cannot be split: four waves a block over all of k
         plan = {4, 1, 2};
     }
-    if (g_mid_kc != 0) plan = {4, DUAL || out_mode != MID_OUT_PARTIAL ? 1 : plan.splits, g_mid_ns};
+    if (g_mid_kc != 0 && MT <= 4) plan = {4, DUAL || out_mode != MID_OUT_PARTIAL ? 1 : plan.splits, g_mid_ns};
     const int kc = g_mid_kc != 0 ? g_mid_kc : 4;
     IA_CHECK(plan.splits == splits, "gemm_mid: the plan's %d splits against the caller's %d", plan.splits, splits);
     const int features = 16 * plan.waves / (DUAL ? 2 : 1);            // output features of a block
@@ -418,7 +421,22 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
     IA_CHECK(plan.waves >= 2 && plan.waves <= MID_MAX_WAVES, "gemm_mid: a block of %d waves", plan.waves);
     const int k_block = K / splits;
 #define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps, act)
-    if (kc == 4 && plan.stages == 3) {
+    if constexpr (MT > 4) {
+        // more than 64 rows: chunks of 64 k, four stages deep, whatever the plan's depth
+        switch (plan.waves) {
+            case 2: MID_SHAPE(2, 4, 2); return 0;
+            case 4: MID_SHAPE(2, 4, 4); return 0;
+            case 6: MID_SHAPE(2, 4, 6); return 0;
+            case 8: MID_SHAPE(2, 4, 8); return 0;
+        }
+        if constexpr (!DUAL) {
+            switch (plan.waves) {
+                case 3: MID_SHAPE(2, 4, 3); return 0;
+                case 5: MID_SHAPE(2, 4, 5); return 0;
+                case 7: MID_SHAPE(2, 4, 7); return 0;
+            }
+        }
+    } else if (kc == 4 && plan.stages == 3) {
         switch (plan.waves) {
             case 2: MID_SHAPE(4, 3, 2); return 0;
             case 4: MID_SHAPE(4, 3, 4); return 0;
@@ -444,14 +462,14 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
 
 // out_mode 0: out [M, N] bfloat16; 1: out [M, N] float; 2: out [splits][M][N] float with splits =
 // ia_gemm_mid_splits(N, K), to be added up by the reader.  dual (an activation, IA_ACT_*): w = [gate; up] of N rows each, out = act(x . gate^T)
-// * (x . up^T) in bfloat16 (mode 0 only).  M in 1..64, K a multiple of 128.
+// * (x . up^T) in bfloat16 (mode 0 only).  M in 1..128, K a multiple of 128.
 // sums_in [M][n_sums] (or null): the rows of x are a norm's input times its weight, and every sum of the product is multiplied by
 // the row's rsqrt(sum of its sums_in / K + eps); up to 16 rows, whole sums only (no split of k).
 extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                                        const float* sums_in, int n_sums, float eps, hipStream_t stream) {
     IA_CHECK(sums_in == nullptr || (M <= 16 && n_sums > 0 && out_mode != MID_OUT_PARTIAL && (((uintptr_t)sums_in) & 15) == 0),
              "gemm_mid: rows with their sums of squares: up to 16 rows, whole sums (M=%d, n_sums=%d, mode %d)", M, n_sums, out_mode);
-    IA_CHECK(M >= 1 && M <= 64 && N > 0 && K > 0, "gemm_mid: takes 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
+    IA_CHECK(M >= 1 && M <= 128 && N > 0 && K > 0, "gemm_mid: takes 1 to 128 rows, got M=%d N=%d K=%d", M, N, K);
     IA_CHECK(K % MID_CHUNK_MIN_K == 0, "gemm_mid: K=%d must be a multiple of %d (use another product)", K, MID_CHUNK_MIN_K);
     IA_CHECK(out_mode >= 0 && out_mode <= 2 && (!dual || out_mode == MID_OUT_BF16), "gemm_mid: output mode %d%s", out_mode,
              dual ? " does not go with the activation inside" : " is unknown");
@@ -466,12 +484,16 @@ extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, 
         if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
         else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
         else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
-        else rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 4) rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt <= 6) rc = launch_mid<6, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else rc = launch_mid<8, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
     } else {
         if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
         else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
         else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
-        else rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 4) rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt <= 6) rc = launch_mid<6, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else rc = launch_mid<8, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
     }
     if (rc != 0) return rc;
     IA_LAUNCH_CHECK("gemm_mid");

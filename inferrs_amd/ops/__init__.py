@@ -733,13 +733,14 @@ def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=
     return sums, scaled
 
 
-# ---- products of 17 to 64 rows -------------------------------------------------------------------
+# ---- products of 17 to 128 rows ------------------------------------------------------------------
 # Decode steps of many requests and short prompt portions: still bound by reading the weights once, which the vendor's
-# GEMM does at 3.4 TB/s and the kernel of gemm_mid.hip faster.  Weights with few rows (the output projection, the
+# GEMM does at 2 to 3.4 TB/s and the kernel of gemm_mid.hip faster.  (Sizes of an 8B model, a prompt of 128 tokens, the four
+# products of a layer inside the model: 129 us against 174 through the vendor's GEMM; of 65 tokens: 108 against 182.)  Weights with few rows (the output projection, the
 # feed-forward's second product) are split along k between blocks, and the splits' sums are added up by the reader:
 # `Partials` stands for a product in that state.
 
-MID_MAX_ROWS = 64             # rows up to which the products of gemm_mid.hip take over from the vendor's GEMM
+MID_MAX_ROWS = 128            # rows up to which the products of gemm_mid.hip take over from the vendor's GEMM
 # [gate; up] weights beyond this many bytes go to the vendor's GEMM and the SiLU kernel also at 17 to 64 rows.  Measured at 32
 # rows (kernel after kernel, launch gaps included): 2 x 12,288 x 4,096 (201 MB) 49 us here against 49 + 5 us there,
 # 2 x 25,600 x 5,120 (524 MB) 125 us here against 96 + 5 us there; the plain products are faster here at every size
@@ -768,7 +769,7 @@ class Partials:
 
 
 def mid_fits(x: torch.Tensor, w: torch.Tensor, few_rows: bool = False) -> bool:
-    """Whether x . w^T goes to gemm_mid.hip: 17 to 64 rows (`few_rows`: 1 to 64)."""
+    """Whether x . w^T goes to gemm_mid.hip: 17 to `MID_MAX_ROWS` rows (`few_rows`: from 1 row on)."""
     if MID_PRODUCTS not in ("own", "library"):
         raise KernelError(f"INFERRS_AMD_MID_PRODUCTS / ops.MID_PRODUCTS: 'own' or 'library', not {MID_PRODUCTS!r}")
     return (MID_PRODUCTS == "own" and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
@@ -779,7 +780,7 @@ def mid_fits(x: torch.Tensor, w: torch.Tensor, few_rows: bool = False) -> bool:
 def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, dual: bool = False,
                   partial: bool = False, sums_in: Optional[torch.Tensor] = None, eps: float = 0.0,
                   activation: str = "silu"):
-    """x [m, k] . w[n, k]^T for 1 to 64 bfloat16 rows and k a multiple of 128 (gemm_mid.hip).  `dual`: w = [gate; up],
+    """x [m, k] . w[n, k]^T for 1 to 128 bfloat16 rows and k a multiple of 128 (gemm_mid.hip).  `dual`: w = [gate; up],
     the result act(x . gate^T) * (x . up^T).  `partial`: the result stays split along k, as `Partials` (a weight that
     needs no split gives a plain tensor).  `sums_in` [m, blocks] (up to 16 rows): the rows are a norm's input times its
     weight and these their sums of squares; every sum is multiplied by the row's rsqrt(mean of squares + eps)."""

@@ -76,7 +76,7 @@ class Block(BlockBase):
         # and a part that says `takes_normed_rows` may get `ops.NormedRows` made of these, whose norm its
         # first product finishes.
         few = x.dtype == torch.bfloat16 and 0 < x.shape[0] <= ops.STREAM_MAX_ROWS
-        # Steps of 17 to 64 bfloat16 rows: a part's last product may stay split along k (`ops.Partials`); the norm
+        # Steps of 17 to `ops.MID_MAX_ROWS` bfloat16 rows: a part's last product may stay split along k (`ops.Partials`); the norm
         # that adds it to the stream adds the splits up on the way (`normed` below, or whoever reads `pending`).
         ctx.partial_sums = x.dtype == torch.bfloat16 and ops.SKINNY_MAX_ROWS < x.shape[0] <= ops.MID_MAX_ROWS
         h = normed(self.norm_mixer, x, pending, few and getattr(self.mixer, "takes_normed_rows", False))

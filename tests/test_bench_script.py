@@ -36,10 +36,13 @@ def test_decode_record_has_the_agreed_keys():
     assert config["layers"] == 2 and config["layers_of_model"] == 36 and config["global_batch"] == 2
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / 8000.0) < 1e-3
-    assert {"decode_b1", "decode_b64", "decode_b16", "decode_b32", "decode_b2_ctx1024", "prefill_8192",
-            "f32_decode_b2_layers2", "f32_prefill_2048_layers2"} <= set(rec["points"])
+    assert {"decode_b1", "decode_b64", "decode_b16", "decode_b32", "decode_b2_ctx1024", "prefill_8192", "prefill_128",
+            "prefill_512", "f32_decode_b2_layers2", "f32_prefill_2048_layers2"} <= set(rec["points"])
+    # eager steps: the wall time beside the kernels' own
+    for step in rec["eager_steps"].values():
+        assert step["wall_ms"] > 0 and step["graph_ms"] > 0 and step["kernel_calls"] > 0 and 0 <= step["host_frac"] < 1
     assert all(isinstance(v, (int, float)) and v > 0 for v in rec["points"].values())
-    assert set(rec["points"]) <= set(rec["points_hbm_frac"]) | {"prefill_8192", "f32_prefill_2048_layers2"}
+    assert set(rec["points"]) <= set(rec["points_hbm_frac"]) | {"prefill_8192", "prefill_128", "prefill_512", "f32_prefill_2048_layers2"}
     assert rec["prefill"]["tokens"] == 2048 and rec["prefill"]["value"] > 0 and 0 < rec["prefill"]["frac"] < 1
     # mean and deviation over five repetitions, for decode and prefill
     assert rec["decode_runs"]["runs"] == 5 and rec["decode_runs"]["ms_per_step_mean"] > 0 and rec["decode_runs"]["ms_per_step_std"] >= 0

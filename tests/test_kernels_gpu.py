@@ -776,12 +776,12 @@ def test_attention_decode_counters_are_not_made_under_capture():
         ops._DECODE_COUNTERS.update({k: v for k, v in kept.items() if k not in ops._DECODE_COUNTERS})
 
 
-# ---- products of 17 to 64 rows (gemm_mid.hip) -----------------------------------------------------------------
+# ---- products of 17 to 128 rows (gemm_mid.hip) ----------------------------------------------------------------
 
-@pytest.mark.parametrize("m", [1, 17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("m", [1, 17, 31, 32, 33, 48, 64, 65, 90, 96, 97, 128])
 @pytest.mark.parametrize("n,k", [(64, 128), (80, 256), (200, 896), (4096, 1024), (6144, 4096), (77, 3 * 128)])
 def test_mid_product(m, n, k):
-    """Every number of rows up to 64 (row tiles that are partly empty), feature counts that are no multiple of the
+    """Every number of rows up to 128 (row tiles that are partly empty; beyond 64 rows another pipeline), feature counts that are no multiple of the
     block's 64 or of 4, k ranges of one chunk, of fewer chunks than the pipeline is deep and of many; plain, in 32-bit,
     and split along k."""
     from inferrs_amd import ops
@@ -809,7 +809,7 @@ def test_mid_product_splits_depend_on_the_weight_alone():
         assert k % (128 * s) == 0 and k // s >= 512
 
 
-@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("m", [17, 40, 64, 70, 128])
 @pytest.mark.parametrize("n,k", [(32, 128), (50, 256), (1408, 1024)])
 def test_mid_product_with_the_activation_inside(m, n, k):
     from inferrs_amd import ops
@@ -823,14 +823,17 @@ def test_mid_product_with_the_activation_inside(m, n, k):
 
 
 def test_mid_product_rows_do_not_depend_on_the_batch():
-    """A row's result is bit for bit the same whatever else is in the step: alone in a tile, among 64 rows, at another
-    place among them."""
+    """A row's result is bit for bit the same whatever else is in the step: alone in a tile, among 64 or 128 rows (which
+    walk k in other chunks, four stages deep), at another place among them."""
     from inferrs_amd import ops
     k, n = 1024, 4096
-    x = randn(64, k, dtype=torch.bfloat16, seed=8)
+    x = randn(128, k, dtype=torch.bfloat16, seed=8)
     w = dev(randn(n, k, dtype=torch.bfloat16, seed=9, scale=0.05))
     whole = ops.gemm_mid_bf16(dev(x), w).cpu()
-    for rows in ([5], list(range(17)), [63, 0, 31, 32], list(range(20, 53))):
+    wd = dev(randn(2 * 1408, k, dtype=torch.bfloat16, seed=10, scale=0.05))
+    whole_gated = ops.gemm_mid_bf16(dev(x), wd, dual=True).cpu()
+    for rows in ([5], list(range(17)), [63, 0, 31, 32], list(range(20, 53)), list(range(64)), list(range(30, 110)), [127, 64, 3]):
+        assert torch.equal(ops.gemm_mid_bf16(dev(x[rows].contiguous()), wd, dual=True).cpu(), whole_gated[rows]), rows
         part = ops.gemm_mid_bf16(dev(x[rows].contiguous()), w).cpu()
         assert torch.equal(part, whole[rows]), rows
     split = ops.gemm_mid_bf16(dev(x), w, partial=True)
@@ -839,7 +842,7 @@ def test_mid_product_rows_do_not_depend_on_the_batch():
     assert torch.equal(again.parts.cpu(), split.parts[:, 10:40].cpu())
 
 
-@pytest.mark.parametrize("m", [5, 33, 64])
+@pytest.mark.parametrize("m", [5, 33, 64, 83, 128])
 def test_mid_product_with_every_shape_of_block(m):
     """The rule picks the waves of a block and the split of k by the weight's shape; here every shape is forced on one
     weight (features that fill no block, rows that fill no tile): plain with its sums split two ways, and with the

@@ -399,14 +399,14 @@ def test_real_layer_sizes_long_prompt_in_portions(tmp_path):
 
 @pytest.fixture(scope="module")
 def many_requests(models):
-    """64 requests of different lengths on configuration G (widths in steps of 128, head size 128: the products of 17 to
-    64 rows run on the kernels made for them, the two of 1,024 inputs split along k), each a prompt and 12 tokens that
+    """100 requests of different lengths on configuration G (widths in steps of 128, head size 128: the products of 17 to
+    128 rows run on the kernels made for them, the two of 1,024 inputs split along k), each a prompt and 12 tokens that
     are fed one by one whatever the model would choose; the plain implementation's logits at the fed places, and the
     bfloat16 bound measured on these very sequences."""
     folder, raw, _, _ = models[("G", 1.0)]
     n_steps = 12
-    prompts = [random_tokens(3 + (7 * i) % 61 + i, raw["vocab_size"], 900 + i) for i in range(64)]
-    feeds = [random_tokens(n_steps, raw["vocab_size"], 1900 + i) for i in range(64)]
+    prompts = [random_tokens(3 + (7 * i) % 61 + i % 64, raw["vocab_size"], 900 + i) for i in range(100)]
+    feeds = [random_tokens(n_steps, raw["vocab_size"], 1900 + i) for i in range(100)]
     cfg, params = pm.read_model(folder, torch.float64)
     cfg_b, params_b = pm.read_model(folder, torch.bfloat16)
     ref, err = [], 0.0
@@ -419,10 +419,10 @@ def many_requests(models):
     return folder, raw, prompts, feeds, ref, scale, err / scale
 
 
-@pytest.mark.parametrize("n_req", [24, 40, 64])
-def test_decode_steps_of_17_to_64_requests(many_requests, n_req):
-    """24, 40 and 64 requests decode 12 steps side by side: eagerly and through captured graphs, every step's logits
-    against each other and against the plain implementation.  The products must have run on the kernels of 17 to 64
+@pytest.mark.parametrize("n_req", [24, 40, 64, 100])
+def test_decode_steps_of_17_to_128_requests(many_requests, n_req):
+    """24, 40, 64 and 100 requests decode 12 steps side by side: eagerly and through captured graphs, every step's logits
+    against each other and against the plain implementation.  The products must have run on the kernels of 17 to 128
     rows, the split ones added up by the norm that follows them."""
     from inferrs_amd.engine import Engine, Entry
     folder, raw, prompts, feeds, ref, scale, limit = many_requests
