@@ -270,13 +270,14 @@ WORKLOADS = {
 }
 
 
-def run_workload(engine, lengths, portion: int, decode_tokens: int, budget: int, vocab: int, seed: int):
+def run_workload(engine, lengths, portion: int, decode_tokens: int, budget: int, vocab: int, seed: int, row_multiple: int = 256):
     """All requests arrive at once and run to their last token.  Returns (seconds, seconds to each
     request's first token, loop steps, seconds until the last prompt was through)."""
     import torch
     from inferrs_amd.engine import GenerationLoop
     from inferrs_amd.sampling import SamplingParams
-    loop = GenerationLoop(engine, max_batch_size=len(lengths), max_tokens_per_step=budget, prefill_chunk=portion)
+    loop = GenerationLoop(engine, max_batch_size=len(lengths), max_tokens_per_step=budget, prefill_chunk=portion,
+                          row_multiple=row_multiple)
     g = torch.Generator().manual_seed(seed)
     params = SamplingParams.greedy(max_tokens=decode_tokens, bypass_stop_tokens=True)
     requests = [loop.add(torch.randint(0, vocab, (n,), generator=g).tolist(), params) for n in lengths]
@@ -306,8 +307,8 @@ def workload_main(args, raw, engine_factory) -> int:
     pages = sum(-(-(n + decode_tokens + 1) // PAGE) + 1 for n in lengths) + 8
     note(f"{args.workload}: {n_req} requests, {sum(lengths)} prompt tokens, {decode_tokens} decoded tokens each")
     engine = engine_factory(pages, n_req + 1)
-    run_workload(engine, lengths, portion, min(decode_tokens, 16), budget, raw["vocab_size"], seed=1)      # warm-up
-    runs = [run_workload(engine, lengths, portion, decode_tokens, budget, raw["vocab_size"], seed=2 + i)
+    run_workload(engine, lengths, portion, min(decode_tokens, 16), budget, raw["vocab_size"], seed=1, row_multiple=args.row_multiple)      # warm-up
+    runs = [run_workload(engine, lengths, portion, decode_tokens, budget, raw["vocab_size"], seed=2 + i, row_multiple=args.row_multiple)
             for i in range(max(1, args.steps if args.steps < 16 else 3))]
     elapsed, firsts, steps, prompts_done = min(runs, key=lambda r: r[0])
     p_tok, d_tok = sum(lengths), n_req * decode_tokens
@@ -318,7 +319,8 @@ def workload_main(args, raw, engine_factory) -> int:
         "data": "synthetic: random-init weights, uniform-random token ids, stop tokens ignored",
         "config": {"model": f"Qwen3-{args.shape} shape", "layers": args.layers, "requests": n_req,
                    "prompt_tokens": p_tok, "shortest_prompt": min(lengths), "longest_prompt": max(lengths),
-                   "portion": portion, "tokens_per_step": budget, "decode_tokens": decode_tokens, "kv_page_size": PAGE},
+                   "portion": portion, "tokens_per_step": budget, "decode_tokens": decode_tokens, "kv_page_size": PAGE,
+                   "row_multiple": args.row_multiple},
         "loop_steps": steps,
         "first_token_s": {"mean": round(sum(firsts) / len(firsts), 4), "max": round(max(firsts), 4)},
         # until the last request has its first token the steps are mostly prompt portions, after it only decode steps
@@ -355,6 +357,8 @@ def main() -> int:
     ap.add_argument("--no-extra-points", dest="extra_points", action="store_false",
                     help="only batch 1 and 64 and the prefill beside the headline (no further batches and contexts, "
                          "no per-kernel times, no 32-bit path)")
+    ap.add_argument("--row-multiple", type=int, default=256,
+                    help="workloads: cut prompt portions so that a step's tokens are a multiple of this (0: off)")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
     args = ap.parse_args()

@@ -208,6 +208,7 @@ struct PlanEntry { Req* req; int start, count; bool samples; };
 struct Sched {
     Cache* cache;
     int max_batch_size, max_tokens_per_step, prefill_chunk, max_seq_len;
+    int row_multiple = 0;                 // > 1: a portion that does not end its prompt is cut so that the step's tokens are a multiple of this
     std::unordered_set<int> stop_ids;
     std::unordered_map<int64_t, std::unique_ptr<Req>> reqs;
     std::deque<Req*> waiting;
@@ -249,6 +250,19 @@ struct Sched {
         for (size_t i = 0; i < plan.size();)
             if (plan[i].req == v) { budget += plan[i].count; plan.erase(plan.begin() + i); }
             else ++i;
+    }
+    // The tokens of a request that this step takes, given what it has left to feed and what the step's budget still
+    // allows.  The large products tile a step's rows (256 at a time in the vendor's GEMM: a step of 520 rows costs as
+    // much as one of 768), so a portion that is cut anyway is cut where the step's tokens so far make a whole
+    // multiple of `row_multiple`; a portion that ends its prompt is what it is.
+    int portion(int left, int budget) const {
+        int n = std::min(std::min(left, prefill_chunk), budget);
+        if (row_multiple > 1 && n < left) {
+            const int rows = max_tokens_per_step - budget + n;
+            const int over = rows % row_multiple;
+            if (over != 0 && rows - over >= row_multiple && n - over >= 1) n -= over;
+        }
+        return n;
     }
     void make_plan(bool fresh) {
         if (fresh) { plan.clear(); preempted.clear(); failed.clear(); broken = false; }
@@ -295,7 +309,7 @@ struct Sched {
             const int left = r->total() - r->computed;
             if (planned || left < 1) continue;
             if (left == 1 && r->n_output() > 0) continue;          // a decode that found no budget
-            const int n = std::min(std::min(left, prefill_chunk), budget);
+            const int n = portion(left, budget);
             if (cache->reserve(*cache->find(r->key), n) != 0) continue;   // waits for pages
             plan.push_back({r, r->computed, n, r->computed + n == r->total()});
             budget -= n;
@@ -310,7 +324,7 @@ struct Sched {
                 fail_request(r, buf, false);
                 continue;
             }
-            const int n = std::min(std::min(r->total() - r->computed, prefill_chunk), budget);
+            const int n = portion(r->total() - r->computed, budget);
             if (cache->add_sequence(r->key) < 0) {        // the key is in use outside this scheduler, or no slot is left
                 broken = true;
                 break;
@@ -659,6 +673,11 @@ void* iar_sched_create(void* cache, int max_batch_size, int max_tokens_per_step,
     return s;
 }
 void iar_sched_destroy(void* sched) { delete S(sched); }
+int iar_sched_set_row_multiple(void* sched, int row_multiple) {
+    if (row_multiple < 0) return fail(IAR_ERROR, "row_multiple must be >= 0");
+    S(sched)->row_multiple = row_multiple;
+    return 0;
+}
 
 int iar_sched_add(void* sched, int64_t key, const int* prompt, int n_prompt, int max_tokens, int bypass_stop,
                   const int* extra_stop, int n_extra) {

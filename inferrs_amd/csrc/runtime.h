@@ -72,6 +72,8 @@ long long iar_step_words(void* cache, int n_entries, const int64_t* keys, const 
 void* iar_sched_create(void* cache, int max_batch_size, int max_tokens_per_step, int prefill_chunk,
                        int max_seq_len, const int* stop_ids, int n_stop);
 void iar_sched_destroy(void* sched);
+// > 1: a prompt portion that does not end its prompt is cut so that the step's tokens are a multiple of this (0, 1: off)
+int iar_sched_set_row_multiple(void* sched, int row_multiple);
 int iar_sched_add(void* sched, int64_t key, const int* prompt, int n_prompt, int max_tokens, int bypass_stop,
                   const int* extra_stop, int n_extra);
 // A request that already has a cache entry (its first tokens were put there by other means) joins

@@ -26,11 +26,12 @@ class GenerationLoop:
     def __init__(self, engine: Engine, *, max_batch_size: int = 32, max_tokens_per_step: int = 2048,
                  prefill_chunk: Optional[int] = None, max_seq_len: Optional[int] = None,
                  stop_token_ids: Optional[Sequence[int]] = None, decode_run: int = 8,
-                 detokenize: Optional[Callable[[List[int]], str]] = None):
+                 detokenize: Optional[Callable[[List[int]], str]] = None, row_multiple: int = 256):
         """`decode_run`: when every running request decodes and nobody waits, up to this many decode
         steps are queued on the GPU at once (`Engine.decode_chain`; draws included, their random
         numbers and penalty windows kept on the device); 1 switches it off.
-        `detokenize`: output token ids -> text, for requests with stop strings."""
+        `detokenize`: output token ids -> text, for requests with stop strings.
+        `row_multiple`: see `Scheduler` (cut prompt portions so that a step's tokens are a multiple of it)."""
         self.engine = engine
         self.detokenize = detokenize
         self.decode_run = max(1, decode_run)
@@ -38,7 +39,7 @@ class GenerationLoop:
         self.scheduler = Scheduler(
             engine.cache, max_batch_size=min(max_batch_size, engine.cache.max_seqs),
             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk, max_seq_len=limit,
-            stop_token_ids=engine.stop_token_ids if stop_token_ids is None else stop_token_ids)
+            stop_token_ids=engine.stop_token_ids if stop_token_ids is None else stop_token_ids, row_multiple=row_multiple)
         self.sampler = Sampler(engine.device)
         self.steps = 0
         self._next_id = 0

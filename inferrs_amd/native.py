@@ -48,6 +48,7 @@ _SIGNATURES = {
                                c_longlong, _PI, _PI]),
     "iar_step_words": (c_longlong, [c_void_p, c_int, _PK, _PI, c_int, c_int, c_int]),
     "iar_sched_create": (c_void_p, [c_void_p, c_int, c_int, c_int, c_int, _PI, c_int]),
+    "iar_sched_set_row_multiple": (c_int, [c_void_p, c_int]),
     "iar_sched_destroy": (None, [c_void_p]),
     "iar_sched_add": (c_int, [c_void_p, c_int64, _PI, c_int, c_int, c_int, _PI, c_int]),
     "iar_sched_adopt": (c_int, [c_void_p, c_int64, _PI, c_int, c_int, c_int, c_int, _PI, c_int]),

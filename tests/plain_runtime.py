@@ -303,7 +303,7 @@ class Plan:
 class Scheduler:
     def __init__(self, cache: CacheManager, *, max_batch_size: int = 32, max_tokens_per_step: int = 2048,
                  prefill_chunk: Optional[int] = None, max_seq_len: int = 40960,
-                 stop_token_ids: Sequence[int] = ()):
+                 stop_token_ids: Sequence[int] = (), row_multiple: int = 256):
         """`max_batch_size`: most running requests (the reference's flag of that name, default 32,
         `inferrs/src/main.rs:137-138`); `max_tokens_per_step`: token budget of one step (default
         2048, `main.rs:141-142`); `prefill_chunk`: longest portion of one prompt in a step (None: the
@@ -319,12 +319,24 @@ class Scheduler:
         self.max_tokens_per_step = max_tokens_per_step
         self.prefill_chunk = prefill_chunk or max_tokens_per_step
         self.max_seq_len = max_seq_len
+        self.row_multiple = row_multiple
         self.stop_token_ids = frozenset(int(t) for t in stop_token_ids)
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []            # in order of admission
         self.finished: Dict[Hashable, Request] = {}
         self._arrivals = 0
         self._left_out: set = set()                 # decodes that found no budget in the last plan
+
+    def _portion(self, left: int, budget: int) -> int:
+        """Tokens of a request that this step takes: a portion that does not end its prompt is cut so that the step's
+        tokens so far are a whole multiple of `row_multiple`, when the step has that many."""
+        n = min(left, self.prefill_chunk, budget)
+        if self.row_multiple > 1 and n < left:
+            rows = self.max_tokens_per_step - budget + n
+            over = rows % self.row_multiple
+            if over and rows - over >= self.row_multiple and n - over >= 1:
+                n -= over
+        return n
 
     # ---- requests ---------------------------------------------------------------------------
     def add(self, request: Request) -> None:
@@ -388,7 +400,7 @@ class Scheduler:
                 continue
             if r.total - r.computed == 1 and r.output:
                 continue                                  # a decode that found no budget
-            n = min(r.total - r.computed, self.prefill_chunk, budget)
+            n = self._portion(r.total - r.computed, budget)
             if not self.cache.reserve(r.request_id, n):
                 continue                                  # waits for pages; decodes above free them as they finish
             plan.entries.append(PlannedEntry(r, r.tokens[r.computed:r.computed + n], r.computed + n == r.total))
@@ -403,7 +415,7 @@ class Scheduler:
                               f"pages, the pool has {self._pages_total()}", live=False)
                 plan.failed.append(r)
                 continue
-            n = min(r.total - r.computed, self.prefill_chunk, budget)
+            n = self._portion(r.total - r.computed, budget)
             self.cache.add_sequence(r.request_id)
             # admitted only when all it has so far, and one token more, would fit now: a request
             # that is let in on its first portion alone tends to be preempted later

@@ -236,7 +236,7 @@ def test_scheduler_takes_the_decisions_of_the_plain_one(seed):
     max_seqs = 6
     options = dict(max_batch_size=rng.randint(1, 6), max_tokens_per_step=rng.choice([4, 16, 64]),
                    prefill_chunk=rng.choice([None, 3, 16]), max_seq_len=rng.choice([24, 48, 4096]),
-                   stop_token_ids=[rng.randrange(3, 100), rng.randrange(3, 100)])
+                   stop_token_ids=[rng.randrange(3, 100), rng.randrange(3, 100)], row_multiple=rng.choice([0, 4, 8, 256]))
     needs = {0: FULL, 1: PagedKV(2, 16, window=rng.choice([6, 20]))} if seed % 2 else {0: FULL}
     ca = CacheManager(needs, page, num_pages, max_seqs)
     cb = plain.CacheManager(needs, page, num_pages, max_seqs)

@@ -267,3 +267,36 @@ def test_make_trace_program_and_modes(tmp_path):
     assert sorted(len(t) for t in info["requests"].values()) == [5, 37, 70] and info["max_tokens"] % 64 == 0
     assert sum(len(rows) for rows in info["rows"].values()) == 112 and len(lines) > 10
     assert all(0 <= t < 50 for line in lines for e in json.loads(line)["entries"] for t in e["tokens"])
+
+
+def test_cut_portions_make_the_steps_rows_a_whole_multiple():
+    """With `row_multiple` a portion that does not end its prompt is cut so that the step's tokens (decodes first, then
+    portions) are a whole multiple of it; a portion that ends its prompt is left alone, and so are steps with fewer
+    tokens than one multiple."""
+    cache = CacheManager({0: PagedKV(2, 16)}, 16, 400, 8)
+    sched = Scheduler(cache, max_batch_size=8, max_tokens_per_step=96, prefill_chunk=40, row_multiple=32)
+    long = Request("long", list(range(1, 131)), SamplingParams.greedy(max_tokens=4))
+    sched.add(long)
+    plan = sched.plan()
+    assert [len(e.tokens) for e in plan.entries] == [32]              # 40 would leave 8 over a multiple
+    sched.commit(plan, {})
+    short = Request("short", [5, 6, 7], SamplingParams.greedy(max_tokens=6))
+    sched.add(short)
+    plan = sched.plan()
+    # the running request's portion first (32 again), then the newcomer's whole prompt, which ends it: 35 tokens
+    assert [(e.request.request_id, len(e.tokens), e.samples) for e in plan.entries] == [("long", 32, False), ("short", 3, True)]
+    sched.commit(plan, {"short": 9})
+    plan = sched.plan()
+    # one decode, then a portion cut to 31 so that the step has 32 tokens
+    assert [(e.request.request_id, len(e.tokens)) for e in plan.entries] == [("short", 1), ("long", 31)]
+    sched.commit(plan, {"short": 9})
+    plan = sched.plan()
+    # 35 tokens are left of the long prompt: they end it and are taken whole
+    assert [(e.request.request_id, len(e.tokens), e.samples) for e in plan.entries] == [("short", 1, True), ("long", 35, True)]
+    # switched off, the portions are the chunk
+    off = Scheduler(CacheManager({0: PagedKV(2, 16)}, 16, 400, 8), max_batch_size=8, max_tokens_per_step=96, prefill_chunk=40,
+                    row_multiple=0)
+    off.add(Request("long", list(range(1, 131)), SamplingParams.greedy(max_tokens=4)))
+    assert [len(e.tokens) for e in off.plan().entries] == [40]
+    with pytest.raises(ValueError, match="row_multiple"):
+        Scheduler(cache, max_batch_size=8, row_multiple=-1)
