@@ -5,7 +5,9 @@ Paged groups: per layer a key array `[pages, n_kv_heads, page_size, head_dim]` a
 attention kernels multiply probabilities into them along the slots) in the model's precision,
 so one page of one head is `page_size * head_dim` contiguous elements.  Keys and values of one
 width share one allocation; a mixer whose values are wider or narrower than its keys
-(`PagedKV.v_head_dim`) gets two.  (The reference keeps `[pages * page_size, n_kv_heads, head_dim]` per layer,
+(`PagedKV.v_head_dim`) gets two.  A need may ask for its values as rows, `[pages, n_kv_heads,
+page_size, value_dim]` (`value_layout="rows"`), or for no value array at all (`values=False`:
+`LayerCache.v` is None).  (The reference keeps `[pages * page_size, n_kv_heads, head_dim]` per layer,
 `inferrs-models/src/kv_cache.rs:249-270`, and gathers it into a dense copy per pass; here the
 attention kernels read pages through the block table.)  Pages are not cleared on reuse:
 attention never reads beyond a request's length.
@@ -45,7 +47,11 @@ class CacheStorage:
         for g in manager.groups:
             need = g.need
             pages, ps = max(g.pool.num_pages, 1), manager.page_size
-            if need.value_dim == need.head_dim:
+            values = None
+            if not need.values:
+                keys = torch.zeros((len(g.layers), pages, need.n_kv_heads, ps, need.head_dim), dtype=dtype, device=device)
+                self.arrays.append(keys)
+            elif need.value_dim == need.head_dim:
                 arr = torch.zeros((len(g.layers), 2, pages, need.n_kv_heads, ps, need.head_dim), dtype=dtype, device=device)
                 self.arrays.append(arr)
                 keys, values = arr[:, 0], arr[:, 1]
@@ -54,8 +60,10 @@ class CacheStorage:
                 values = torch.zeros((len(g.layers), pages, need.n_kv_heads, ps, need.value_dim), dtype=dtype, device=device)
                 self.arrays += [keys, values]
             for i, layer in enumerate(g.layers):
-                self.layers[layer] = LayerCache(layer, g.index, keys[i],
-                                                values[i].view(pages, need.n_kv_heads, need.value_dim, ps))
+                v = None
+                if values is not None:
+                    v = values[i] if need.value_layout == "rows" else values[i].view(pages, need.n_kv_heads, need.value_dim, ps)
+                self.layers[layer] = LayerCache(layer, g.index, keys[i], v)
         for st in manager.states:
             arr = torch.zeros((manager.max_seqs, *st.need.shape), dtype=st.need.dtype, device=device)
             self.arrays.append(arr)

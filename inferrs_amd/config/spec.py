@@ -38,12 +38,16 @@ class PositionSpec:
     angle = position * theta**(-2i/rot_dim); pairing "half" pairs feature i
     with i + rot_dim/2, "interleaved" pairs 2i with 2i+1.
     kind "none": nothing is applied.
+    `scaling`: None, or a law that changes the angles' frequencies, as (name, factor): ("linear", f)
+    divides every frequency by f (positions are read as position / f).  A law that has no entry in
+    the position part is refused by name when the part is built.
     """
     kind: str = "rope"
     head_dim: int = 0
     rot_dim: int = 0
     theta: float = 10000.0
     pairing: str = "half"
+    scaling: Optional[Tuple[str, float]] = None
 
 
 @dataclass(frozen=True)

@@ -37,14 +37,26 @@ from ..weights.loader import TensorSpec
 @dataclass(frozen=True)
 class PagedKV:
     """Keys and values of every cached position, in pages; `window` keeps only the last ones.
-    `head_dim` is the width of a key; values have `v_head_dim` (None: the same)."""
+    `head_dim` is the width of a key; values have `v_head_dim` (None: the same).  `values=False`:
+    one array a layer, the keys' (a mixer that caches a single row a position, a latent one say, from
+    which it forms what it needs).  `value_layout`: how a page holds its values: "transposed"
+    `[head][dim][slot]`, what this package's attention kernels multiply probabilities into, or
+    "rows" `[head][slot][dim]`, as the keys lie."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
+    values: bool = True
+    value_layout: str = "transposed"
+
+    def __post_init__(self):
+        if self.value_layout not in ("transposed", "rows"):
+            raise ValueError(f"PagedKV: value_layout {self.value_layout!r} is neither 'transposed' nor 'rows'")
 
     @property
     def value_dim(self) -> int:
+        if not self.values:
+            return 0
         return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
     def page_elements(self, page_size: int) -> int:

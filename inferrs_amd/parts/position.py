@@ -23,6 +23,17 @@ def inverse_frequencies(theta: float, rot_dim: int) -> np.ndarray:
     return (np.float32(1.0) / power).astype(np.float32)
 
 
+def linear_scaling(inv_freq: np.ndarray, factor: float) -> np.ndarray:
+    """Positions read as position / factor: every frequency divided by it, in 32-bit."""
+    if not (factor > 0.0):
+        raise SpecError(f"rotary scaling 'linear' needs a positive factor, got {factor}")
+    return (inv_freq / np.float32(factor)).astype(np.float32)
+
+
+# name of a scaling law -> (inverse frequencies, factor) -> inverse frequencies; another law is another entry
+SCALING_LAWS = {"linear": linear_scaling}
+
+
 @register_position("rope")
 class Rotary(Position):
     graph_safe = True
@@ -35,7 +46,13 @@ class Rotary(Position):
         self.spec = spec
         self.rot_dim = spec.rot_dim
         self.interleaved = spec.pairing == "interleaved"
-        self.inv_freq = torch.from_numpy(inverse_frequencies(spec.theta, spec.rot_dim)).to(device)
+        inv_freq = inverse_frequencies(spec.theta, spec.rot_dim)
+        if spec.scaling is not None:
+            law, factor = spec.scaling
+            if law not in SCALING_LAWS:
+                raise SpecError(f"rotary scaling {law!r} has no entry (known: {sorted(SCALING_LAWS)})")
+            inv_freq = SCALING_LAWS[law](inv_freq, float(factor))
+        self.inv_freq = torch.from_numpy(inv_freq).to(device)
 
     def table(self, positions: torch.Tensor) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
         return ops.rope_table(positions, self.inv_freq)

@@ -131,3 +131,16 @@ def test_state_arrays_count_in_the_pool_sizing():
     manager = CacheManager({0: PagedKV(2, 16), 1: FixedState((1000,), torch.float32), 2: PagedKV(2, 16, None, 24)}, 8, 0, 5)
     assert CacheStorage.state_bytes(manager) == 5 * 1000 * 4
     assert CacheStorage.page_bytes(manager, torch.bfloat16) == (2 * 8 * 32 + 2 * 8 * 40) * 2
+
+
+def test_paged_needs_with_one_array_or_values_as_rows():
+    """What a paged need may ask of the storage beside keys and transposed values: no value array at all, or values as
+    rows; needs that differ in this do not share a group, and a page's bytes follow."""
+    keys_only = PagedKV(1, 24, values=False)
+    rows = PagedKV(2, 16, None, 8, value_layout="rows")
+    assert keys_only.value_dim == 0 and keys_only.page_elements(4) == 24 * 4
+    assert rows.page_elements(4) == 2 * 4 * (16 + 8)
+    manager = CacheManager({0: PagedKV(2, 16), 1: keys_only, 2: rows, 3: PagedKV(2, 16, None, 8)}, 4, 6, 2)
+    assert len(manager.groups) == 4
+    with pytest.raises(ValueError, match="value_layout"):
+        PagedKV(2, 16, value_layout="sideways")

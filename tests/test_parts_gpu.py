@@ -583,7 +583,7 @@ def test_steps_of_a_few_rows_with_and_without_the_products_taking_the_norms(tmp_
 
 @dataclass(frozen=True)
 class WideValueSpec:
-    """One-head causal attention without position encoding whose values (dv) are wider than its keys (dk)."""
+    """One-head causal attention without position encoding whose values (dv) are wider than its keys (dk), kept as rows."""
     hidden: int
     dk: int
     dv: int
@@ -625,7 +625,7 @@ def register_toy_ends():
 
         @classmethod
         def cache_need(cls, spec):
-            return PagedKV(1, spec.dk, None, v_head_dim=spec.dv)
+            return PagedKV(1, spec.dk, None, v_head_dim=spec.dv, value_layout="rows")
 
         def __init__(self, spec, tensors, dtype, device):
             self.spec = spec
@@ -636,17 +636,18 @@ def register_toy_ends():
             q, k, v = (ops.linear(h, self.w[n]) for n in "qkv")
             group = ctx.groups[cache.group]
             ps = group.page_size
-            assert tuple(cache.k.shape[1:]) == (1, ps, s.dk) and tuple(cache.v.shape[1:]) == (1, s.dv, ps)
+            # (this mixer asked for its values as rows, [page][head][slot][dim], not transposed as the package's own kernels want them)
+            assert tuple(cache.k.shape[1:]) == (1, ps, s.dk) and tuple(cache.v.shape[1:]) == (1, ps, s.dv)
             slots = group.slots.long()
             cache.k[slots // ps, 0, slots % ps] = k
-            cache.v[slots // ps, 0, :, slots % ps] = v
+            cache.v[slots // ps, 0, slots % ps] = v
             out = torch.empty((h.shape[0], s.dv), dtype=h.dtype, device=h.device)
             off = 0
             for row, (n, start) in enumerate(zip(ctx.q_lens, ctx.kv_starts)):      # a toy: one request at a time
                 total = start + n
                 pages = group.block_table[row, :-(-total // ps)].long()
                 keys = cache.k[pages, 0].reshape(-1, s.dk)[:total].float()
-                values = cache.v[pages, 0].permute(0, 2, 1).reshape(-1, s.dv)[:total].float()
+                values = cache.v[pages, 0].reshape(-1, s.dv)[:total].float()
                 scores = q[off:off + n].float() @ keys.T / s.dk ** 0.5
                 seen = torch.arange(total, device=h.device)[None, :] <= (start + torch.arange(n, device=h.device))[:, None]
                 out[off:off + n] = (torch.softmax(scores.masked_fill(~seen, float("-inf")), -1) @ values).to(h.dtype)
@@ -901,3 +902,152 @@ def test_an_activation_without_a_kernel_is_refused_by_name():
     spec = GatedMlpSpec(hidden=8, intermediate=8, activation="relu")
     with pytest.raises(SpecError, match="relu.*gelu_tanh.*silu"):
         part_class("ffn", spec)(spec, {}, torch.float32, DEV)
+
+
+# ---- a fifth toy architecture: a mixer that caches one latent row a position, in a paged array of its own ----------
+
+@dataclass(frozen=True)
+class LatentSpec:
+    """Causal attention over one cached row a position: c = W_c h is what the cache holds (no value array); a query
+    q = W_q h scores the rows, and the output is W_o . (softmax(q . c^T / sqrt(dl)) @ c)."""
+    hidden: int
+    latent: int
+    kind: str = "toy_latent"
+
+
+def register_toy_latent():
+    from inferrs_amd import ops
+    from inferrs_amd.config import GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, ScheduleEntry
+    from inferrs_amd.config.registry import register_architecture
+    from inferrs_amd.parts import Mixer, PagedKV, register_mixer
+    from inferrs_amd.weights import TensorSpec
+
+    @register_mixer("toy_latent")
+    class Latent(Mixer):
+        @classmethod
+        def tensors(cls, spec):
+            return {"c.weight": TensorSpec((spec.latent, spec.hidden)), "q.weight": TensorSpec((spec.latent, spec.hidden)),
+                    "o.weight": TensorSpec((spec.hidden, spec.latent))}
+
+        @classmethod
+        def cache_need(cls, spec):
+            return PagedKV(1, spec.latent, None, values=False)
+
+        def __init__(self, spec, tensors, dtype, device):
+            self.spec = spec
+            self.w = {n: tensors[n + ".weight"].to(device=device, dtype=dtype).contiguous() for n in "cqo"}
+
+        def forward(self, ctx, h, cache):
+            s = self.spec
+            assert cache.v is None                                   # one array a layer: the rows'
+            c, q = ops.linear(h, self.w["c"]), ops.linear(h, self.w["q"])
+            group = ctx.groups[cache.group]
+            ps = group.page_size
+            slots = group.slots.long()
+            cache.k[slots // ps, 0, slots % ps] = c
+            out = torch.empty_like(c)
+            off = 0
+            for row, (n, start) in enumerate(zip(ctx.q_lens, ctx.kv_starts)):      # a toy: one request at a time
+                total = start + n
+                pages = group.block_table[row, :-(-total // ps)].long()
+                rows = cache.k[pages, 0].reshape(-1, s.latent)[:total].float()
+                scores = q[off:off + n].float() @ rows.T / s.latent ** 0.5
+                seen = torch.arange(total, device=h.device)[None, :] <= (start + torch.arange(n, device=h.device))[:, None]
+                out[off:off + n] = (torch.softmax(scores.masked_fill(~seen, float("-inf")), -1) @ rows).to(h.dtype)
+                off += n
+            return ops.linear(out, self.w["o"])
+
+    class LatentConfig:
+        architecture = "ToyLatentForCausalLM"
+        model_type = "toy_latent"
+
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def to_dict(self):
+            return dict(self.raw, architectures=[self.architecture], model_type=self.model_type)
+
+        def to_spec(self):
+            r = self.raw
+            h = r["hidden_size"]
+            norm = NormSpec(size=h, eps=r["eps"])
+
+            def layer(i):
+                p = f"blocks.{i}."
+                return LayerSpec(mixer=LatentSpec(h, r["latent"]), ffn=GatedMlpSpec(hidden=h, intermediate=r["intermediate"]),
+                                 norms=(norm, norm), norm_names=(p + "norm1.weight", p + "norm2.weight"),
+                                 mixer_prefix=p + "mixer.", ffn_prefix=p + "ffn.")
+            return ModelSpec(architecture=self.architecture, vocab_size=r["vocab"], hidden=h,
+                             layers=tuple(layer(i) for i in range(r["layers"])),
+                             schedule=tuple(ScheduleEntry(i) for i in range(r["layers"])), final_norm=norm,
+                             final_norm_name="norm.weight", embed_name="embed.weight", head_name=None, max_position=512)
+
+    register_architecture(LatentConfig)
+    return LatentConfig
+
+
+def toy_latent_plain(p, raw, ids):
+    t = len(ids)
+    x = p["embed.weight"][torch.as_tensor(ids)]
+    causal = torch.arange(t)[None, :] > torch.arange(t)[:, None]
+    for i in range(raw["layers"]):
+        pre = f"blocks.{i}."
+        h = pm.rms_norm(x, p[pre + "norm1.weight"], raw["eps"])
+        c, q = pm.linear(h, p[pre + "mixer.c.weight"]), pm.linear(h, p[pre + "mixer.q.weight"])
+        s = (q @ c.T / raw["latent"] ** 0.5).masked_fill(causal, float("-inf"))
+        x = x + pm.linear(pm.softmax_last(s) @ c, p[pre + "mixer.o.weight"])
+        x = x + pm.mlp(pm.rms_norm(x, p[pre + "norm2.weight"], raw["eps"]), p[pre + "ffn.gate_proj.weight"],
+                       p[pre + "ffn.up_proj.weight"], p[pre + "ffn.down_proj.weight"])
+    return pm.linear(pm.rms_norm(x, p["norm.weight"], raw["eps"]), p["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype,page", [("float32", 4), ("bfloat16", 16)])
+def test_toy_mixer_with_one_cached_array(tmp_path, dtype, page):
+    """A mixer whose paged cache is one array a layer (no values): the storage gives it that and nothing else."""
+    from inferrs_amd.engine import Engine, run_trace
+    from inferrs_amd.weights import write_random_model
+    LatentConfig = register_toy_latent()
+    raw = dict(hidden_size=40, latent=24, intermediate=56, vocab=83, eps=1e-5, layers=2)
+    folder = write_random_model(str(tmp_path / "latent"), LatentConfig(raw), seed=7)
+    from safetensors.torch import load_file
+    p = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    reqs = {f"r{i}": random_tokens(n, 83, 40 + i) for i, n in enumerate([2, 33, 71])}
+    ref = {r: toy_latent_plain(p, raw, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for mode, trace in (("whole", tm.whole(reqs)), ("portions", tm.portions(reqs, [5, 2, 17])),
+                        ("mixed", tm.mixed(reqs, seed=2, max_live=3, decode_tail=6))):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-trace.max_tokens // page) + 2, max_seqs=4)
+        need = eng.cache.groups[0].need
+        assert not need.values and need.value_dim == 0 and len(eng.storage.arrays) == 1
+        assert eng.storage.arrays[0].shape[1:] == (eng.cache.groups[0].pool.num_pages, 1, page, 24)
+        per_page = 2 * 24 * page * (4 if dtype == "float32" else 2)                  # two layers, one row of 24 a slot
+        from inferrs_amd.cache import CacheStorage
+        assert CacheStorage.page_bytes(eng.cache, eng.model.dtype) == per_page
+        run_trace(eng, trace.lines, str(tmp_path / mode), io.StringIO())
+        got = trace.read(str(tmp_path / mode), 83)
+        err = max(float(np.abs(got[r][i] - ref[r][i]).max()) for r in reqs for i in range(len(reqs[r]))) / scale
+        assert err < (2e-5 if dtype == "float32" else 3e-2), f"{mode}: {err:.3e}"
+        eng.cache.check_invariants()
+
+
+def test_position_part_with_a_scaling_law():
+    """`PositionSpec.scaling`: ("linear", f) reads positions as position / f, so the angles at position f * p are
+    those of position p without it; a law without an entry is refused by name."""
+    from inferrs_amd.config import PositionSpec, SpecError
+    from inferrs_amd.parts import part_class
+    plain = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4)
+    scaled = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4, scaling=("linear", 4.0))
+    a = part_class("position", plain)(plain, {}, torch.float32, DEV)
+    b = part_class("position", scaled)(scaled, {}, torch.float32, DEV)
+    pos = torch.tensor([0, 1, 5, 300], dtype=torch.int32)
+    cos_a, sin_a = a.table(pos.to(DEV))
+    cos_b, sin_b = b.table((pos * 4).to(DEV))
+    assert float((cos_a - cos_b).abs().max()) < 1e-6 and float((sin_a - sin_b).abs().max()) < 1e-6
+    assert torch.equal(b.inv_freq.cpu(), a.inv_freq.cpu() / 4)
+    other = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4, scaling=("yarn", 4.0))
+    with pytest.raises(SpecError, match="yarn.*linear"):
+        part_class("position", other)(other, {}, torch.float32, DEV)
