@@ -88,21 +88,10 @@ int ia_gemm_mid_tune(int kc, int ns);
 int ia_gemm_mid_plan(int waves, int splits, int stages);
 int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                      hipStream_t stream);
-// the same for rows that are a norm's input times its weight, with their sums of squares sums_in [M][n_sums]: every sum
+// the same for up to 16 rows that are a norm's input times its weight, with their sums of squares sums_in [M][n_sums]: every sum
 // of the product is multiplied by the row's rsqrt(sum of sums_in / K + eps); out_mode 0 or 1
 int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                             const float* sums_in, int n_sums, float eps, hipStream_t stream);
-// The plain product of gemm_mid.hip that finishes itself: the block that stores its split of k last for a range of
-// features adds the splits up (in their order) and either stores the product (finish 1: out [M, N] bfloat16, the bits of
-// ia_sum_partials) or adds it to the residual stream in place (finish 2: resid [M, N]; the bits that ia_add_rmsnorm_partials
-// leaves there) and leaves the new rows' sums of squares, sums_out [M][ia_gemm_mid_blocks(N, K)], and the new rows times
-// next_w, scaled_out [M, N] (both may be null together).  parts: [ia_gemm_mid_splits(N, K)][M][N] floats of scratch;
-// counters: ia_gemm_mid_blocks(N, K) words that are zero before and after (calls that share them must not overlap);
-// sums_in as in ia_gemm_mid_bf16_scaled, for any number of rows.  N a multiple of 4.
-int ia_gemm_mid_blocks(int N, int K);
-int ia_gemm_mid_stream(float* parts, const void* x, const void* w, int M, int N, int K, int finish, void* out,
-                       void* resid, float* sums_out, void* scaled_out, const float* next_w, int add_one,
-                       const float* sums_in, int n_sums, float eps, int* counters, int n_counters, hipStream_t stream);
 int ia_sum_partials(void* out, const float* part, int splits, int M, int N, hipStream_t stream);
 // x += (sum of the splits, rounded to bfloat16) in place, out = rmsnorm(x) * w; bfloat16 rows of up to 8192 features.
 int ia_add_rmsnorm_partials(void* out, void* x, const float* part, int splits, const float* w, float eps,

@@ -118,141 +118,12 @@ __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* sw
     }
 }
 
-// ---- a split product that finishes itself -------------------------------------------------------------------------
-// A product whose k is split between blocks leaves sums that somebody has to add up, and a kernel of its own for that
-// (ia_sum_partials, ia_add_rmsnorm_partials) is 4.6 to 5 us of launch and latency in a decode step.  With `finish` the
-// block that stores its split last for a range of features, known by a counter in memory, adds the splits up itself, in
-// the order of the splits whoever comes last, and
-//   MID_FINISH_STORE   rounds the sums to bfloat16 into `out` [M, N]: the bits of ia_sum_partials;
-//   MID_FINISH_STREAM  adds the rounded product to the residual stream `resid` [M, N] in place, the sum formed in 32-bit
-//                      and rounded (the bits that ia_add_rmsnorm_partials leaves in the stream), and leaves the new rows'
-//                      sums of squares, block by block, in sums_out [M][blocks] and the new rows times next_w (1 + next_w
-//                      with add_one) in scaled_out [M, N] (may be null, with next_w): what the product after the norm
-//                      needs to finish that norm (sums_in).
-// A product that is not split does the same in every block, without the counter.
-// The hand-over: a block's sums are stored through to memory (device scope), every wave waits until the memory has
-// taken its own stores (s_waitcnt vmcnt(0): a wave's counter of memory operations counts a store down when it is
-// acknowledged), the block meets at a barrier, and only then one thread counts; the block that counts last reads the
-// sums past the caches (device scope), after a barrier behind the atomic's return.  The counters are zero between calls
-// (the last block puts its own back): calls that share them must not overlap.
-enum { MID_FINISH_NONE = 0, MID_FINISH_STORE = 1, MID_FINISH_STREAM = 2 };
-struct MidStream {
-    int finish;
-    int splits;
-    int* counters;              // [blocks], zero before and after
-    bf16_t* out;                // MID_FINISH_STORE
-    bf16_t* resid;              // MID_FINISH_STREAM
-    float* sums_out;
-    bf16_t* scaled_out;
-    const float* next_w;
-    int add_one;
-};
-
-__device__ __forceinline__ void put_across4(float* at, const gmid_f32x4& v) {
-    const uint64_t lo = (uint64_t)__float_as_uint(v[0]) | ((uint64_t)__float_as_uint(v[1]) << 32);
-    const uint64_t hi = (uint64_t)__float_as_uint(v[2]) | ((uint64_t)__float_as_uint(v[3]) << 32);
-    __hip_atomic_store((uint64_t*)at, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store((uint64_t*)at + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ gmid_f32x4 get_across4(const float* at) {
-    const uint64_t lo = __hip_atomic_load((const uint64_t*)at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint64_t hi = __hip_atomic_load((const uint64_t*)at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return (gmid_f32x4){__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)),
-                        __uint_as_float((uint32_t)hi), __uint_as_float((uint32_t)(hi >> 32))};
-}
-
-// Lane (r, g) of wave `tile` holds features n_first + 4 g + i of row 16 mt + r.  `parts` [splits][M][N]: the splits' sums
-// (not touched when the product is not split); `lds`: room for TILES * MT * 16 floats that nobody else uses any more.
-template <int MT, int TILES>
-__device__ __forceinline__ void mid_finish_stream(gmid_f32x4 (&acc)[MT], float* lds, int* s_last, float* parts, int M, int N,
-                                                  int r, int g, int tile, int n_first, int split, const MidStream& st) {
-    const int nb = n_first + 4 * g;
-    const bool cols = nb + 3 < N;                                         // (N is a multiple of 4: all four features or none)
-    if (st.splits > 1) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 16 + r;
-            if (m < M && cols) put_across4(parts + ((size_t)split * M + m) * N + nb, acc[mt]);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                  // the memory has this wave's sums ...
-        __syncthreads();                                                  // ... and every wave's, before the count
-        if (threadIdx.x == 0)
-            *s_last = __hip_atomic_fetch_add(st.counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == st.splits - 1 ? 1 : 0;
-        __syncthreads();
-        if (!*s_last) return;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 16 + r;
-            if (!(m < M && cols)) continue;
-            gmid_f32x4 total = get_across4(parts + (size_t)m * N + nb);
-            for (int s = 1; s < st.splits; ++s) {
-                const gmid_f32x4 o = get_across4(parts + ((size_t)s * M + m) * N + nb);
-                total[0] += o[0]; total[1] += o[1]; total[2] += o[2]; total[3] += o[3];
-            }
-            acc[mt] = total;
-        }
-    } else {
-        __syncthreads();                                                  // everybody is done with the stages (`lds`)
-    }
-    float sq[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + r;
-        sq[mt] = 0.f;
-        if (!(m < M && cols)) continue;
-        const size_t at = (size_t)m * N + nb;
-        if (st.finish == MID_FINISH_STORE) {
-            *(uint2*)(st.out + at) = make_uint2(pack_bf16x2(acc[mt][0], acc[mt][1]), pack_bf16x2(acc[mt][2], acc[mt][3]));
-            continue;
-        }
-        const uint2 old = *(const uint2*)(st.resid + at);
-        const uint16_t ob[4] = {(uint16_t)old.x, (uint16_t)(old.x >> 16), (uint16_t)old.y, (uint16_t)(old.y >> 16)};
-        uint16_t hb[4];
-        float h[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float product = bf16_bits_to_f32(f32_to_bf16_bits(acc[mt][i]));
-            hb[i] = f32_to_bf16_bits(product + bf16_bits_to_f32(ob[i]));
-            h[i] = bf16_bits_to_f32(hb[i]);
-            sq[mt] += h[i] * h[i];
-        }
-        *(uint2*)(st.resid + at) = make_uint2((uint32_t)hb[0] | ((uint32_t)hb[1] << 16), (uint32_t)hb[2] | ((uint32_t)hb[3] << 16));
-        if (st.scaled_out != nullptr) {
-            const float4 g4 = *(const float4*)(st.next_w + nb);
-            const float gw[4] = {g4.x, g4.y, g4.z, g4.w};
-            uint16_t sb[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) sb[i] = f32_to_bf16_bits(h[i] * (st.add_one ? 1.0f + gw[i] : gw[i]));
-            *(uint2*)(st.scaled_out + at) = make_uint2((uint32_t)sb[0] | ((uint32_t)sb[1] << 16), (uint32_t)sb[2] | ((uint32_t)sb[3] << 16));
-        }
-    }
-    if (st.finish == MID_FINISH_STREAM) {
-        // a row's sum of squares over the block's features: over the lanes that hold the row, then over the waves in their order
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            float s = sq[mt];
-            s += __shfl_xor(s, 16, IA_WAVE);
-            s += __shfl_xor(s, 32, IA_WAVE);
-            if (g == 0) lds[(tile * MT + mt) * 16 + r] = s;
-        }
-        __syncthreads();
-        for (int m = threadIdx.x; m < M; m += blockDim.x) {
-            float total = 0.f;
-            for (int wv = 0; wv < TILES; ++wv) total += lds[(wv * MT + (m >> 4)) * 16 + (m & 15)];
-            st.sums_out[(size_t)m * gridDim.x + blockIdx.x] = total;
-        }
-    }
-    if (st.splits > 1 && threadIdx.x == 0)
-        __hip_atomic_store(st.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // zero again for the next call
-}
-
 // KC: k steps of 32 in a chunk (a staged row is KC * 64 bytes); NS: stages, this chunk's and NS - 1 on their way; W: waves of
 // a block, a tile of 16 weight rows each (DUAL: W / 2 of gate rows, then W / 2 of up rows).
 template <int MT, bool DUAL, int KC, int NS, int W>
 __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-    int M, int N, int K, int k_per_block, const float* __restrict__ sums_in, int n_sums, float eps, int act,
-    const MidStream st) {
+    int M, int N, int K, int k_per_block, const float* __restrict__ sums_in, int n_sums, float eps, int act) {
     constexpr int CHUNK_K = KC * 32;
     constexpr int ROW_BYTES = KC * 64;
     constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;
@@ -314,22 +185,7 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
             }
         }
     }
-    __shared__ float mid_ss[MT * 16];
-    __shared__ int mid_last;
-    // more tiles of rows: a row a wave in turn, a lane one of the row's sums (rows of up to 64 sums; longer ones are added
-    // up at the end), asked for now as well
-    constexpr int SS_MANY = (MT * 16 + W - 1) / W;
-    float ss_many[MT == 1 ? 1 : SS_MANY];
-    const bool ss_short = MT > 1 && sums_in != nullptr && n_sums <= IA_WAVE;
-    if constexpr (MT > 1) {
-        if (ss_short) {
-#pragma unroll
-            for (int j = 0; j < SS_MANY; ++j) {
-                const int m = wave + j * W;
-                ss_many[j] = (m < M && lane < n_sums) ? sums_in[(size_t)m * n_sums + lane] : 0.f;
-            }
-        }
-    }
+    __shared__ float mid_ss[16];
 
     // ---- what this lane fetches of a stage: load i covers rows ROWS_PER_LOAD * (W i + wave) .. of the stage ----
     const char* src[LOADS];
@@ -452,33 +308,6 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
             acc[0][0] *= scale; acc[0][1] *= scale; acc[0][2] *= scale; acc[0][3] *= scale;
         }
     }
-    if constexpr (MT > 1) {
-        if (sums_in != nullptr) {
-#pragma unroll
-            for (int j = 0; j < SS_MANY; ++j) {
-                const int m = wave + j * W;
-                if (m >= M) continue;
-                float ss = 0.f;
-                if (ss_short) ss = ss_many[j];
-                else for (int b = lane; b < n_sums; b += IA_WAVE) ss += sums_in[(size_t)m * n_sums + b];
-                ss = wave_sum(ss);
-                if (lane == 0) mid_ss[m] = ss;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = mt * 16 + r;
-                const float scale = 1.0f / sqrtf(mid_ss[m < M ? m : 0] / (float)K + eps);
-                acc[mt][0] *= scale; acc[mt][1] *= scale; acc[mt][2] *= scale; acc[mt][3] *= scale;
-            }
-        }
-    }
-    if constexpr (!DUAL) {
-        if (st.finish != MID_FINISH_NONE) {
-            mid_finish_stream<MT, TILES>(acc, (float*)mid_s0, &mid_last, (float*)out, M, N, r, g, tile, n_first, split, st);
-            return;
-        }
-    }
     mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split, act);
 }
 
@@ -575,7 +404,7 @@ extern "C" int ia_gemm_mid_tune(int kc, int ns) {
 
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
-                      const float* sums_in, int n_sums, float eps, int act, const MidStream& st, hipStream_t stream) {
+                      const float* sums_in, int n_sums, float eps, int act, hipStream_t stream) {
     MidPlan plan = mid_plan(N, K, DUAL);
     if (out_mode != MID_OUT_PARTIAL && !DUAL && plan.splits != 1) {
         // a stored product cannot be split: four waves a block over all of k
@@ -591,7 +420,7 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
              K, splits, MID_CHUNK_MIN_K);
     IA_CHECK(plan.waves >= 2 && plan.waves <= MID_MAX_WAVES, "gemm_mid: a block of %d waves", plan.waves);
     const int k_block = K / splits;
-#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps, act, st)
+#define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps, act)
     if constexpr (MT > 4) {
         // more than 64 rows: chunks of 64 k, four stages deep, whatever the plan's depth
         switch (plan.waves) {
@@ -635,11 +464,11 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
 // ia_gemm_mid_splits(N, K), to be added up by the reader.  dual (an activation, IA_ACT_*): w = [gate; up] of N rows each, out = act(x . gate^T)
 // * (x . up^T) in bfloat16 (mode 0 only).  M in 1..128, K a multiple of 128.
 // sums_in [M][n_sums] (or null): the rows of x are a norm's input times its weight, and every sum of the product is multiplied by
-// the row's rsqrt(sum of its sums_in / K + eps); whole sums only (no split of k).
-static int mid_product(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
-                       const float* sums_in, int n_sums, float eps, const MidStream& st, hipStream_t stream) {
-    IA_CHECK(sums_in == nullptr || (n_sums > 0 && (out_mode != MID_OUT_PARTIAL || st.finish != MID_FINISH_NONE) && (((uintptr_t)sums_in) & 15) == 0),
-             "gemm_mid: rows with their sums of squares: whole sums, or a split product that finishes itself (n_sums=%d, mode %d)", n_sums, out_mode);
+// the row's rsqrt(sum of its sums_in / K + eps); up to 16 rows, whole sums only (no split of k).
+extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
+                                       const float* sums_in, int n_sums, float eps, hipStream_t stream) {
+    IA_CHECK(sums_in == nullptr || (M <= 16 && n_sums > 0 && out_mode != MID_OUT_PARTIAL && (((uintptr_t)sums_in) & 15) == 0),
+             "gemm_mid: rows with their sums of squares: up to 16 rows, whole sums (M=%d, n_sums=%d, mode %d)", M, n_sums, out_mode);
     IA_CHECK(M >= 1 && M <= 128 && N > 0 && K > 0, "gemm_mid: takes 1 to 128 rows, got M=%d N=%d K=%d", M, N, K);
     IA_CHECK(K % MID_CHUNK_MIN_K == 0, "gemm_mid: K=%d must be a multiple of %d (use another product)", K, MID_CHUNK_MIN_K);
     IA_CHECK(out_mode >= 0 && out_mode <= 2 && (!dual || out_mode == MID_OUT_BF16), "gemm_mid: output mode %d%s", out_mode,
@@ -647,82 +476,33 @@ static int mid_product(void* out, const void* x, const void* w, int M, int N, in
     IA_CHECK(dual >= 0 && dual <= IA_ACT_LAST, "gemm_mid: unknown activation %d", dual);
     IA_CHECK((((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0, "gemm_mid: operands must be 16-byte aligned");
     const int splits = out_mode == MID_OUT_PARTIAL && !dual ? mid_plan(N, K, false).splits : 1;
-    IA_CHECK(st.finish == MID_FINISH_NONE || st.splits == splits, "gemm_mid: the plan's %d splits against the caller's %d", splits, st.splits);
-    // (the sums of squares have a column for every block of the plan: a pipeline forced by ia_gemm_mid_tune has other blocks)
-    IA_CHECK(st.finish == MID_FINISH_NONE || g_mid_kc == 0, "gemm_mid: a product that finishes itself does not go with a pipeline "
-             "forced by ia_gemm_mid_tune");
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
     const int mt = (M + 15) / 16;
     int rc = 0;
-#define MID_ROWS(MTV, DUALV) launch_mid<MTV, DUALV>(out, out_mode, xb, wb, M, N, K, DUALV ? 1 : splits, sums_in, n_sums, eps, dual, st, stream)
     if (dual) {
-        if (mt == 1) rc = MID_ROWS(1, true);
-        else if (mt == 2) rc = MID_ROWS(2, true);
-        else if (mt == 3) rc = MID_ROWS(3, true);
-        else if (mt == 4) rc = MID_ROWS(4, true);
-        else if (mt <= 6) rc = MID_ROWS(6, true);
-        else rc = MID_ROWS(8, true);
+        if (mt == 1) rc = launch_mid<1, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 2) rc = launch_mid<2, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 3) rc = launch_mid<3, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 4) rc = launch_mid<4, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else if (mt <= 6) rc = launch_mid<6, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
+        else rc = launch_mid<8, true>(out, out_mode, xb, wb, M, N, K, 1, sums_in, n_sums, eps, dual, stream);
     } else {
-        if (mt == 1) rc = MID_ROWS(1, false);
-        else if (mt == 2) rc = MID_ROWS(2, false);
-        else if (mt == 3) rc = MID_ROWS(3, false);
-        else if (mt == 4) rc = MID_ROWS(4, false);
-        else if (mt <= 6) rc = MID_ROWS(6, false);
-        else rc = MID_ROWS(8, false);
+        if (mt == 1) rc = launch_mid<1, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 2) rc = launch_mid<2, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 3) rc = launch_mid<3, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt == 4) rc = launch_mid<4, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else if (mt <= 6) rc = launch_mid<6, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
+        else rc = launch_mid<8, false>(out, out_mode, xb, wb, M, N, K, splits, sums_in, n_sums, eps, dual, stream);
     }
-#undef MID_ROWS
     if (rc != 0) return rc;
     IA_LAUNCH_CHECK("gemm_mid");
     return 0;
 }
 
-static const MidStream MID_NO_STREAM = {MID_FINISH_NONE, 1, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
-
-extern "C" int ia_gemm_mid_bf16_scaled(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
-                                       const float* sums_in, int n_sums, float eps, hipStream_t stream) {
-    return mid_product(out, x, w, M, N, K, out_mode, dual, sums_in, n_sums, eps, MID_NO_STREAM, stream);
-}
-
 extern "C" int ia_gemm_mid_bf16(void* out, const void* x, const void* w, int M, int N, int K, int out_mode, int dual,
                                 hipStream_t stream) {
-    return mid_product(out, x, w, M, N, K, out_mode, dual, nullptr, 0, 0.f, MID_NO_STREAM, stream);
-}
-
-// Blocks along the features of the plain product with N output features and K inputs: the columns of its sums of squares.
-extern "C" int ia_gemm_mid_blocks(int N, int K) {
-    if (N <= 0 || K <= 0 || K % MID_CHUNK_MIN_K) return 0;
-    const int features = 16 * mid_plan(N, K, false).waves;
-    return (N + features - 1) / features;
-}
-
-// The plain product that finishes itself (see MidStream): x [M, K] . w [N, K]^T with k split ia_gemm_mid_splits(N, K) ways,
-// N a multiple of 4.
-//   parts    [splits][M][N] floats of scratch when the product is split (else unused, may be null)
-//   counters at least ia_gemm_mid_blocks(N, K) 32-bit words, zero before the call and zero again after it (calls that
-//            share them must not overlap)
-//   finish 1 out [M, N] bfloat16 receives the product
-//   finish 2 resid [M, N] += the product in place; sums_out [M][ia_gemm_mid_blocks(N, K)] the new rows' sums of squares;
-//            scaled_out [M, N] (or null, with next_w) the new rows times next_w [N] (1 + next_w with add_one)
-//   sums_in  [M][n_sums] (or null): as in ia_gemm_mid_bf16_scaled
-extern "C" int ia_gemm_mid_stream(float* parts, const void* x, const void* w, int M, int N, int K, int finish, void* out,
-                                  void* resid, float* sums_out, void* scaled_out, const float* next_w, int add_one,
-                                  const float* sums_in, int n_sums, float eps, int* counters, int n_counters,
-                                  hipStream_t stream) {
-    IA_CHECK(finish == MID_FINISH_STORE || finish == MID_FINISH_STREAM, "gemm_mid_stream: finish %d is neither 1 (store) nor 2 (stream)", finish);
-    IA_CHECK(N > 0 && K > 0 && K % MID_CHUNK_MIN_K == 0 && N % 4 == 0, "gemm_mid_stream: N=%d must be a multiple of 4 and K=%d of %d", N, K, MID_CHUNK_MIN_K);
-    const int splits = mid_plan(N, K, false).splits, blocks = ia_gemm_mid_blocks(N, K);
-    IA_CHECK(splits == 1 || (parts != nullptr && counters != nullptr && n_counters >= blocks),
-             "gemm_mid_stream: a product split %d ways needs scratch for its sums and %d counters (got %d)", splits, blocks, n_counters);
-    IA_CHECK(finish != MID_FINISH_STORE || out != nullptr, "gemm_mid_stream: no place for the product");
-    IA_CHECK(finish != MID_FINISH_STREAM || (resid != nullptr && sums_out != nullptr && (scaled_out == nullptr) == (next_w == nullptr)),
-             "gemm_mid_stream: the sum into a stream needs the stream, a place for the sums of squares, and the next norm's "
-             "weight together with a place for the scaled rows");
-    IA_CHECK((((uintptr_t)parts | (uintptr_t)out | (uintptr_t)resid | (uintptr_t)scaled_out | (uintptr_t)next_w) & 15) == 0,
-             "gemm_mid_stream: arrays must be 16-byte aligned");
-    const MidStream st = {finish, splits, counters, (bf16_t*)out, (bf16_t*)resid, sums_out, (bf16_t*)scaled_out, next_w, add_one};
-    // (the kernel's `out` is the scratch of the splits' sums; a product that is not split never writes it)
-    return mid_product(parts != nullptr ? (void*)parts : (void*)x, x, w, M, N, K, MID_OUT_PARTIAL, 0, sums_in, n_sums, eps, st, stream);
+    return ia_gemm_mid_bf16_scaled(out, x, w, M, N, K, out_mode, dual, nullptr, 0, 0.f, stream);
 }
 
 // ---- readers of the splits' sums ------------------------------------------------------------------------------

@@ -654,8 +654,7 @@ def widen(x: torch.Tensor) -> torch.Tensor:
 # norm's weight; the product after the norm (`linear` / `gated_silu_linear` given `NormedRows`) takes
 # those rows and multiplies its sums by the row's scale, rsqrt(mean of squares + eps).
 
-STREAM_MAX_ROWS = 128         # rows up to which the products take over the sums and norms of a step (up to 16 the skinny
-                              # products, from 17 on those of gemm_mid.hip, where they take the operands)
+STREAM_MAX_ROWS = 16          # rows up to which the products take over the sums and norms of a step
 
 
 class Added:
@@ -703,12 +702,6 @@ def _stream_product(x: torch.Tensor, w: torch.Tensor, n: int, out_dtype, dual: b
     return out
 
 
-def _mid_takes_normed_rows(x: NormedRows, w: torch.Tensor) -> bool:
-    """Whether the products of gemm_mid.hip finish the norm of these rows (17 rows and more)."""
-    return (SKINNY_MAX_ROWS < x.scaled.shape[0] <= MID_MAX_ROWS and _mid_finish_fits(x.scaled, w)
-            and x.sums.dtype == torch.float32 and x.sums.shape[0] == x.scaled.shape[0] and x.sums.is_contiguous())
-
-
 def _takes_normed_rows(x: NormedRows, w: torch.Tensor, n: int) -> bool:
     m, k = x.scaled.shape
     return (m <= SKINNY_MAX_ROWS and x.scaled.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] == k
@@ -725,15 +718,7 @@ def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=
     lets the norm add it)."""
     m, k = x.shape
     n = w.shape[0]
-    if m > SKINNY_MAX_ROWS:
-        if (m > STREAM_MAX_ROWS or bias is not None or not _mid_finish_fits(x, w) or resid.dtype != torch.bfloat16
-                or tuple(resid.shape) != (m, n) or not resid.is_contiguous()):
-            return None
-        next_w = getattr(next_norm, "weight", None)
-        if next_w is not None and (next_w.dtype != torch.float32 or next_w.numel() != n):
-            next_w = None
-        return gemm_mid_finish(x, w, resid=resid, next_w=next_w, add_one=bool(getattr(next_norm, "add_one", False)))
-    if (m == 0 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k
+    if (m > SKINNY_MAX_ROWS or m == 0 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k
             or not skinny_fits(x, w) or n >= 65536 or resid.dtype != torch.bfloat16 or tuple(resid.shape) != (m, n)
             or not resid.is_contiguous() or (bias is not None and bias.dtype != torch.bfloat16)):
         return None
@@ -818,82 +803,14 @@ def gemm_mid_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = tor
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     if sums_in is not None:
         _dev(sums_in); _f32(sums_in, "sums of squares")
-        if partial or sums_in.dim() != 2 or sums_in.shape[0] != m or not sums_in.is_contiguous():
-            raise KernelError(f"gemm_mid: sums of squares {tuple(sums_in.shape)} for {m} rows (whole sums only)")
+        if partial or m > 16 or sums_in.dim() != 2 or sums_in.shape[0] != m or not sums_in.is_contiguous():
+            raise KernelError(f"gemm_mid: sums of squares {tuple(sums_in.shape)} for {m} rows (up to 16, whole sums)")
         _check(lib.ia_gemm_mid_bf16_scaled(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
                                            act, _p(sums_in), sums_in.shape[1], ctypes.c_float(eps), _stream()))
         return out
     _check(lib.ia_gemm_mid_bf16(_p(out), _p(x), _p(w), m, n, k, 0 if out_dtype == torch.bfloat16 else 1,
                                 act, _stream()))
     return out
-
-
-# The counters of the products that finish themselves: zero between calls (the kernel puts them back).  One array a device:
-# calls that share it must follow each other (one stream, or a graph replayed on it), as an engine's steps do.
-_MID_COUNTERS: Dict[int, torch.Tensor] = {}
-_MID_COUNTERS_OUTGROWN: list = []                   # captured graphs may still hold their addresses: never freed
-MID_COUNTERS_MIN = 1 << 12
-
-
-def _mid_counters(device: torch.device, needed: int) -> torch.Tensor:
-    key = device.index if device.index is not None else torch.cuda.current_device()
-    have = _MID_COUNTERS.get(key)
-    if have is None or have.numel() < needed:
-        if torch.cuda.is_current_stream_capturing():
-            raise KernelError("gemm_mid_finish: the counters cannot be allocated under graph capture; run a product of this "
-                              "size once before capturing it")
-        if have is not None:
-            _MID_COUNTERS_OUTGROWN.append(have)
-        have = torch.zeros((max(MID_COUNTERS_MIN, 2 * needed),), dtype=torch.int32, device=device)
-        _MID_COUNTERS[key] = have
-    return have
-
-
-def _mid_finish_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
-    return isinstance(x, torch.Tensor) and mid_fits(x, w) and w.shape[0] % 4 == 0
-
-
-def gemm_mid_finish(x: torch.Tensor, w: torch.Tensor, *, resid: Optional[torch.Tensor] = None,
-                    next_w: Optional[torch.Tensor] = None, add_one: bool = False,
-                    sums_in: Optional[torch.Tensor] = None, eps: float = 0.0):
-    """x [m, k] . w [n, k]^T for 17 to 128 bfloat16 rows by the product of gemm_mid.hip that adds the splits of k up
-    itself (the block that stores its split last does it: no kernel of its own for the sum).  Without `resid` the result
-    [m, n] in bfloat16, the bits of the split product summed by `Partials.materialize`.  With `resid` [m, n]: the product
-    is added to it in place, as `add_rmsnorm_partials` adds it, and the result is (sums, scaled): the new rows' sums of
-    squares [m, blocks] and the new rows times `next_w` (None without one).  `sums_in` [m, blocks'] with `eps`: the rows of
-    x are a norm's input times its weight, and the product's sums are multiplied by the row's rsqrt(mean of squares + eps)."""
-    _dev(x, w, resid, next_w, sums_in)
-    m, k = x.shape
-    n = w.shape[0]
-    if not _mid_finish_fits(x, w) or not (1 <= m <= MID_MAX_ROWS):
-        raise KernelError(f"gemm_mid_finish: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype} "
-                          f"(1 to {MID_MAX_ROWS} bfloat16 rows, k a multiple of 128, n of 4)")
-    lib = library()
-    splits, blocks = lib.ia_gemm_mid_splits(n, k), lib.ia_gemm_mid_blocks(n, k)
-    parts = torch.empty((splits, m, n), dtype=torch.float32, device=x.device) if splits > 1 else None
-    counters = _mid_counters(x.device, blocks) if splits > 1 else None
-    if sums_in is not None:
-        _f32(sums_in, "sums of squares")
-        if sums_in.dim() != 2 or sums_in.shape[0] != m or not sums_in.is_contiguous():
-            raise KernelError(f"gemm_mid_finish: sums of squares {tuple(sums_in.shape)} for {m} rows")
-    n_sums = sums_in.shape[1] if sums_in is not None else 0
-    if resid is None:
-        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        _check(lib.ia_gemm_mid_stream(_p(parts), _p(x), _p(w), m, n, k, 1, _p(out), None, None, None, None, 0, _p(sums_in),
-                                      n_sums, ctypes.c_float(eps), _p(counters), counters.numel() if counters is not None else 0,
-                                      _stream()))
-        return out
-    if resid.dtype != torch.bfloat16 or tuple(resid.shape) != (m, n) or not resid.is_contiguous():
-        raise KernelError(f"gemm_mid_finish: the stream {tuple(resid.shape)} {resid.dtype} does not fit the product [{m}, {n}]")
-    _f32(next_w, "norm weight")
-    if next_w is not None and next_w.numel() != n:
-        raise KernelError(f"gemm_mid_finish: the next norm's weight has {next_w.numel()} entries, rows have {n}")
-    sums = torch.empty((m, blocks), dtype=torch.float32, device=x.device)
-    scaled = torch.empty_like(resid) if next_w is not None else None
-    _check(lib.ia_gemm_mid_stream(_p(parts), _p(x), _p(w), m, n, k, 2, None, _p(resid), _p(sums), _p(scaled), _p(next_w),
-                                  int(add_one), _p(sums_in), n_sums, ctypes.c_float(eps), _p(counters),
-                                  counters.numel() if counters is not None else 0, _stream()))
-    return sums, scaled
 
 
 def linear_partials(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None):
@@ -938,8 +855,6 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, mid: boo
         if _takes_normed_rows(x, w, w.shape[0]):
             _dev(x.scaled, w, x.sums)
             return _stream_product(x.scaled, w, w.shape[0], out_dtype, False, sums_in=x.sums, eps=x.eps, bias=bias)
-        if _mid_takes_normed_rows(x, w) and bias is None and out_dtype == torch.bfloat16:
-            return gemm_mid_finish(x.scaled, w, sums_in=x.sums, eps=x.eps)
         x = x.materialize()
     if x.dtype == torch.bfloat16 and skinny_fits(x, w) and x.shape[0] <= SKINNY_MAX_ROWS:
         return gemm_skinny_bf16(x, w, out_dtype, bias=bias)
@@ -960,8 +875,6 @@ def _linear_no_bias(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, mi
     if mid and mid_fits(x, w):
         if out_dtype == torch.float32:
             return gemm_mid_bf16(x, w, torch.float32)
-        if w.shape[0] % 4 == 0:
-            return gemm_mid_finish(x, w)                  # (a split product adds its splits up itself)
         y = gemm_mid_bf16(x, w, partial=True)
         return y.materialize() if isinstance(y, Partials) else y
     _dev(x, w)
@@ -1083,9 +996,6 @@ def gated_linear(x, w_gate_up: torch.Tensor, activation: str = "silu",
                 return gemm_mid_bf16(x.scaled, w_gate_up, dual=True, sums_in=x.sums, eps=x.eps, activation=activation)
             return _stream_product(x.scaled, w_gate_up, w_gate_up.shape[0] // 2, x.scaled.dtype, True,
                                    sums_in=x.sums, eps=x.eps, activation=activation, bias=bias)
-        if (even and bias is None and _mid_takes_normed_rows(x, w_gate_up)
-                and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES):
-            return gemm_mid_bf16(x.scaled, w_gate_up, dual=True, sums_in=x.sums, eps=x.eps, activation=activation)
         x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
         if bias is None and _mid_dual_fits(x, w_gate_up):

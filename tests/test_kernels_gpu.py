@@ -1040,94 +1040,3 @@ def test_a_product_with_a_bias_adds_itself_to_the_stream(m, n, k, add_one):
     new_rows = fused_stream.float().cpu().double()
     exact = new_rows / torch.sqrt(new_rows.pow(2).mean(-1, keepdim=True) + 1e-6) * (norm_w.double() + (1.0 if add_one else 0.0))
     close(ops.linear(rows, dev(w2), bias=dev(b2)), exact @ w2.double().t() + b2.double(), 2 ** -6, "norm's end and bias inside")
-
-
-@pytest.mark.parametrize("m", [17, 40, 64, 100, 128])
-@pytest.mark.parametrize("n,k,add_one", [(4096, 1024, False), (256, 1024, True), (6144, 512, False), (200, 896, False)])
-def test_mid_product_that_finishes_itself(m, n, k, add_one):
-    """The split product whose last block adds the splits up: stored, it has the bits of the splits summed by the kernel
-    of its own; added to a stream, the stream has the bits that the add-and-norm kernel on the splits leaves, the sums of
-    squares and the scaled rows are those of the new rows, and the product that reads them finishes the norm.  Twice in a
-    row on the same counters, with another product in between."""
-    from inferrs_amd import ops
-    lib = ops.library()
-    x = dev(randn(m, k, dtype=torch.bfloat16, seed=m))
-    w = dev(randn(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.05))
-    split = ops.gemm_mid_bf16(x, w, partial=True)
-    stored = split.materialize() if isinstance(split, ops.Partials) else split
-    assert isinstance(split, ops.Partials) == (lib.ia_gemm_mid_splits(n, k) > 1)
-    for _ in range(2):
-        assert torch.equal(ops.gemm_mid_finish(x, w), stored), "the stored product"
-    assert torch.equal(ops.linear(x, w), stored)
-    stream = randn(m, n, dtype=torch.bfloat16, seed=33)
-    norm_w = dev((0.0 if add_one else 1.0) + 0.1 * randn(n, dtype=torch.float32, seed=34))
-    plain_stream = dev(stream)
-    if isinstance(split, ops.Partials):
-        plain_rows = ops.add_rmsnorm_partials(plain_stream, split, norm_w, 1e-6, add_one)
-    else:
-        plain_rows = ops.add_rmsnorm(plain_stream, stored, norm_w, 1e-6, add_one)
-    blocks = lib.ia_gemm_mid_blocks(n, k)
-    for _ in range(2):
-        fused_stream = dev(stream)
-        sums, scaled = ops.linear_add(x, w, fused_stream, _Norm(norm_w, add_one))
-        assert tuple(sums.shape) == (m, blocks) and scaled.shape == fused_stream.shape
-        assert torch.equal(fused_stream, plain_stream), "the stream after the sum"
-        new_rows = fused_stream.float().cpu().double()
-        close(sums.sum(-1), new_rows.pow(2).sum(-1), 1e-5, "sums of squares")
-        per = -(-n // blocks)
-        per = -(-per // 16) * 16                                      # a block's features: whole tiles of 16
-        want_sums = torch.nn.functional.pad(new_rows.pow(2), (0, blocks * per - n)).view(m, blocks, per).sum(-1)
-        close(sums, want_sums, 1e-5, "sums of squares, block by block")
-        gain32 = norm_w.cpu() + 1.0 if add_one else norm_w.cpu()         # 32-bit arithmetic, as the kernel's
-        assert torch.equal(scaled.cpu(), (fused_stream.float().cpu() * gain32).to(torch.bfloat16)), "rows times the weight"
-        gain = gain32.double()
-    only = ops.linear_add(x, w, dev(stream))
-    assert only[1] is None and torch.equal(only[0], sums)
-    # the products that read such rows finish their norm
-    rows = ops.NormedRows(fused_stream, scaled, sums, norm_w, 1e-6, add_one)
-    # (the norm kernel on the stream and the one that adds the splits up add a row's squares in different orders)
-    close(rows.materialize(), plain_rows, 2 ** -7, "the rows' norm by the kernel of its own")
-    exact = new_rows / torch.sqrt(new_rows.pow(2).mean(-1, keepdim=True) + 1e-6) * gain
-    if n % 128 == 0:
-        n2 = 384
-        w2 = randn(n2, n, dtype=torch.bfloat16, seed=35, scale=0.03)
-        w3 = randn(2 * n2, n, dtype=torch.bfloat16, seed=36, scale=0.03)
-        from call_counter import CallCounter
-        with CallCounter("gemm_mid_finish", "gemm_mid_bf16", "rmsnorm") as counted:
-            got2 = ops.linear(rows, dev(w2))
-            got3 = ops.gated_linear(rows, dev(w3), "silu")
-        assert counted.calls == {"gemm_mid_finish": 1, "gemm_mid_bf16": 1, "rmsnorm": 0}, counted.calls
-        close(got2, exact @ w2.double().t(), 2 ** -6, "product with the norm's end inside")
-        g = (exact @ w3[:n2].double().t()).to(torch.bfloat16).double()
-        close(got3, g / (1 + torch.exp(-g)) * (exact @ w3[n2:].double().t()).to(torch.bfloat16).double(), 2 ** -6,
-              "gated product with the norm's end inside")
-        # a row's result does not depend on what stands beside it
-        if m >= 40:
-            some = ops.NormedRows(fused_stream[7:30].contiguous(), scaled[7:30].contiguous(), sums[7:30].contiguous(), norm_w, 1e-6, add_one)
-            assert torch.equal(ops.linear(some, dev(w2)), got2[7:30]) and torch.equal(ops.gated_linear(some, dev(w3)), got3[7:30])
-
-
-def test_mid_products_that_finish_themselves_with_every_shape_of_block():
-    """Forced shapes of block and splits of k: the counters, the splits' order and the sums of squares by block."""
-    from inferrs_amd import ops
-    lib = ops.library()
-    m, n, k = 70, 304, 2048
-    x = dev(randn(m, k, dtype=torch.bfloat16, seed=1))
-    w = dev(randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05))
-    stream = randn(m, n, dtype=torch.bfloat16, seed=3)
-    norm_w = dev(1.0 + 0.1 * randn(n, dtype=torch.float32, seed=4))
-    try:
-        for waves in (2, 3, 5, 8):
-            for splits in (1, 2, 8):
-                assert lib.ia_gemm_mid_plan(waves, splits, 3) == 0
-                y = ops.gemm_mid_bf16(x, w, partial=True)
-                stored = y.materialize() if isinstance(y, ops.Partials) else y
-                assert torch.equal(ops.gemm_mid_finish(x, w), stored), (waves, splits)
-                a, b = dev(stream), dev(stream)
-                want = ops.add_rmsnorm(a, stored, norm_w, 1e-6)
-                sums, scaled = ops.linear_add(x, w, b, _Norm(norm_w))
-                assert torch.equal(a, b) and sums.shape[1] == -(-n // (16 * waves)), (waves, splits)
-                close(sums.sum(-1), b.float().pow(2).sum(-1), 1e-5, "sums of squares")
-                assert torch.equal(ops.NormedRows(b, scaled, sums, norm_w, 1e-6, False).materialize(), want)
-    finally:
-        lib.ia_gemm_mid_plan(0, 0, 0)
