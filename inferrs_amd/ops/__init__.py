@@ -741,6 +741,22 @@ def linear_add(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, next_norm=
 # `Partials` stands for a product in that state.
 
 MID_MAX_ROWS = 128            # rows up to which the products of gemm_mid.hip take over from the vendor's GEMM
+# Rows from which a layer's products go to gemm_mid.hip, with kernels of their own for the sums of the splits and the norms,
+# instead of the skinny products that take over the stream's sums and norms: None = by the rule of `mid_from_rows`.
+MID_FROM_ROWS: Optional[int] = None
+MID_MIN_ROWS = 5              # fewest rows for which a split product is worth the kernel that adds it up
+
+
+def mid_from_rows(width: int) -> int:
+    """Rows of a step from which the products of a model of this width (the residual stream's) run on gemm_mid.hip.
+    Measured, decode steps at a context of 2,048 (ms a step, skinny products against gemm_mid.hip): width 4,096 (8B
+    shape) 6 rows 4.72 / 4.89, 8 rows 3.99 / 4.00, 9 rows 4.27 / 4.22, 12 rows 4.40 / 4.34, 16 rows 4.69 / 4.56; width
+    5,120, where the skinny product's blocks are no whole tiles and its waves' shares of k are uneven (14B shape): 4 rows
+    6.50 / 6.52, 6 rows 6.85 / 6.71, 8 rows 7.13 / 6.94, 12 rows 8.12 / 7.39, 16 rows 9.49 / 7.78 (32B shape: 8 rows 15.09 /
+    14.26, 16 rows 19.10 / 15.42)."""
+    if MID_FROM_ROWS is not None:
+        return MID_FROM_ROWS
+    return 9 if width & (width - 1) == 0 else MID_MIN_ROWS
 # [gate; up] weights beyond this many bytes go to the vendor's GEMM and the SiLU kernel also at 17 to 64 rows.  Measured at 32
 # rows (kernel after kernel, launch gaps included): 2 x 12,288 x 4,096 (201 MB) 49 us here against 49 + 5 us there,
 # 2 x 25,600 x 5,120 (524 MB) 125 us here against 96 + 5 us there; the plain products are faster here at every size
@@ -769,11 +785,12 @@ class Partials:
 
 
 def mid_fits(x: torch.Tensor, w: torch.Tensor, few_rows: bool = False) -> bool:
-    """Whether x . w^T goes to gemm_mid.hip: 17 to `MID_MAX_ROWS` rows (`few_rows`: from 1 row on)."""
+    """Whether x . w^T goes to gemm_mid.hip: from `mid_from_rows(k)` to `MID_MAX_ROWS` rows (`few_rows`: from 1 row on)."""
     if MID_PRODUCTS not in ("own", "library"):
         raise KernelError(f"INFERRS_AMD_MID_PRODUCTS / ops.MID_PRODUCTS: 'own' or 'library', not {MID_PRODUCTS!r}")
     return (MID_PRODUCTS == "own" and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-            and (0 if few_rows else SKINNY_MAX_ROWS) < x.shape[0] <= MID_MAX_ROWS and x.shape[1] % 128 == 0 and w.shape[1] == x.shape[1]
+            and (1 if few_rows else mid_from_rows(x.shape[1])) <= x.shape[0] <= MID_MAX_ROWS
+            and x.shape[1] % 128 == 0 and w.shape[1] == x.shape[1]
             and x.is_contiguous() and w.is_contiguous() and (x.data_ptr() | w.data_ptr()) % 16 == 0)
 
 
@@ -817,7 +834,9 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     """x . w^T for a reader that takes `Partials` (the norm that adds the product to the stream): split along k where the
     weight has few rows.  None when the product of 17 to 64 rows does not take these operands (a bias among them: the
     caller then forms the whole product, and `linear` adds the bias)."""
-    if bias is None and isinstance(x, torch.Tensor) and mid_fits(x, w):
+    # (whoever asks is in a step whose products go to gemm_mid.hip: the rule has been asked with the stream's width, and a
+    # product of another width follows it)
+    if bias is None and isinstance(x, torch.Tensor) and x.shape[0] >= MID_MIN_ROWS and mid_fits(x, w, few_rows=True):
         return gemm_mid_bf16(x, w, partial=True)
     return None
 
@@ -845,8 +864,8 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, mid: boo
     reference uses cuBLAS for all of them).  A 32-bit result of bfloat16 operands (logits) comes straight from
     the skinny kernel's accumulators for those few rows; beyond that it is the vendor's bfloat16
     result widened, which is what the reference does for every row (its logits are computed in
-    the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`).  `mid=False`: steps of 17 to 64 rows
-    go to the vendor's GEMM as well.  The skinny kernel adds a bias to its sums before it rounds them; behind every
+    the model's precision and cast for sampling, `inferrs/src/sampler.rs:182`).  From `mid_from_rows(k)` rows on (and up to
+    `MID_MAX_ROWS`) a bfloat16 result comes from gemm_mid.hip; `mid=False`: from the skinny product or the vendor's GEMM.  The skinny kernel adds a bias to its sums before it rounds them; behind every
     other product a kernel of its own adds it to the stored rows."""
     out_dtype = out_dtype or x.dtype
     if bias is not None and (bias.dtype != w.dtype or bias.numel() != w.shape[0]):
@@ -857,7 +876,9 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, mid: boo
             return _stream_product(x.scaled, w, w.shape[0], out_dtype, False, sums_in=x.sums, eps=x.eps, bias=bias)
         x = x.materialize()
     if x.dtype == torch.bfloat16 and skinny_fits(x, w) and x.shape[0] <= SKINNY_MAX_ROWS:
-        return gemm_skinny_bf16(x, w, out_dtype, bias=bias)
+        # (rows that both kernels take: a 32-bit result, the logits head's, stays with the skinny product)
+        if out_dtype != torch.bfloat16 or bias is not None or not mid or not mid_fits(x, w):
+            return gemm_skinny_bf16(x, w, out_dtype, bias=bias)
     y = _linear_no_bias(x, w, out_dtype if bias is None else x.dtype, mid)
     if bias is None:
         return y
@@ -998,7 +1019,8 @@ def gated_linear(x, w_gate_up: torch.Tensor, activation: str = "silu",
                                    sums_in=x.sums, eps=x.eps, activation=activation, bias=bias)
         x = x.materialize()
     if x.shape[0] <= SKINNY_MAX_ROWS and skinny_fits(x, w_gate_up):
-        if bias is None and _mid_dual_fits(x, w_gate_up):
+        if bias is None and (_mid_dual_fits(x, w_gate_up) or (
+                even and mid_fits(x, w_gate_up) and w_gate_up.numel() * w_gate_up.element_size() <= MID_DUAL_MAX_BYTES)):
             return gemm_mid_bf16(x, w_gate_up, dual=True, activation=activation)
         return gemm_skinny_bf16(x, w_gate_up, x.dtype, dual=True, activation=activation, bias=bias)
     if bias is None:

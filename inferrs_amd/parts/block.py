@@ -75,10 +75,11 @@ class Block(BlockBase):
         # times the weight of `ctx.stream_norm`, the norm that comes next: `next_norm` after this block),
         # and a part that says `takes_normed_rows` may get `ops.NormedRows` made of these, whose norm its
         # first product finishes.
-        few = x.dtype == torch.bfloat16 and 0 < x.shape[0] <= ops.STREAM_MAX_ROWS
-        # Steps of 17 to `ops.MID_MAX_ROWS` bfloat16 rows: a part's last product may stay split along k (`ops.Partials`); the norm
+        mid_from = ops.mid_from_rows(x.shape[1])
+        few = x.dtype == torch.bfloat16 and 0 < x.shape[0] <= min(ops.STREAM_MAX_ROWS, mid_from - 1)
+        # Steps of `ops.mid_from_rows(width)` to `ops.MID_MAX_ROWS` bfloat16 rows: a part's last product may stay split along k (`ops.Partials`); the norm
         # that adds it to the stream adds the splits up on the way (`normed` below, or whoever reads `pending`).
-        ctx.partial_sums = x.dtype == torch.bfloat16 and ops.SKINNY_MAX_ROWS < x.shape[0] <= ops.MID_MAX_ROWS
+        ctx.partial_sums = x.dtype == torch.bfloat16 and mid_from <= x.shape[0] <= ops.MID_MAX_ROWS
         h = normed(self.norm_mixer, x, pending, few and getattr(self.mixer, "takes_normed_rows", False))
         ctx.stream = x if few and getattr(self.mixer, "adds_to_stream", False) else None
         ctx.stream_norm = self.norm_ffn if getattr(self.ffn, "takes_normed_rows", False) else None

@@ -505,7 +505,7 @@ def test_products_around_a_residual_stream(m, n, k, n2, add_one):
     w3 = randn(2 * n2, n, dtype=torch.bfloat16, seed=36, scale=0.03)
     # the two-kernel way
     plain_stream = dev(stream)
-    plain_rows = ops.add_rmsnorm(plain_stream, ops.linear(dev(x), dev(w)), dev(norm_w), 1e-6, add_one)
+    plain_rows = ops.add_rmsnorm(plain_stream, ops.gemm_skinny_bf16(dev(x), dev(w)), dev(norm_w), 1e-6, add_one)
     # the products' way
     fused_stream = dev(stream)
     norm = _Norm(dev(norm_w), add_one)
@@ -1025,7 +1025,7 @@ def test_a_product_with_a_bias_adds_itself_to_the_stream(m, n, k, add_one):
     stream = randn(m, n, dtype=torch.bfloat16, seed=33)
     norm_w = (0.0 if add_one else 1.0) + 0.1 * randn(n, dtype=torch.float32, seed=34)
     plain_stream = dev(stream)
-    plain_rows = ops.add_rmsnorm(plain_stream, ops.linear(dev(x), dev(w), bias=dev(b)), dev(norm_w), 1e-6, add_one)
+    plain_rows = ops.add_rmsnorm(plain_stream, ops.gemm_skinny_bf16(dev(x), dev(w), bias=dev(b)), dev(norm_w), 1e-6, add_one)
     fused_stream = dev(stream)
     norm = _Norm(dev(norm_w), add_one)
     sums, scaled = ops.linear_add(dev(x), dev(w), fused_stream, norm, dev(b))
