@@ -54,6 +54,9 @@ long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int max_
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
                   int out_dtype, hipStream_t stream);
 // bias: bfloat16 [N] ([2 N] with dual), or null
+// (ia_gemm_tiled at up to 64 rows: the shape of its kernel for few rows, 100 * output features + staged rows a wave:
+// 816, 808, 416 or 1608; 0: the kernel's own rule)
+int ia_gemm_rows_tune(int shape);
 int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, const void* bias, int M, int N, int K,
                         int out_dtype, int dual, hipStream_t stream);
 // Large bfloat16 products in tiles of 256 x 256 (gemm_mfma.hip); K a multiple of 64; with `dual` w is [gate; up]

@@ -147,55 +147,62 @@ __global__ __launch_bounds__(256) void gemm_tiled128_kernel(TO* __restrict__ out
     }
 }
 
-// The same product for up to 16 rows (decode steps of the 32-bit path), bound by reading the weights: a wave owns 16
-// output features, so that a weight of 4,096 features still makes a block for every compute unit; lane (n, group of
-// four rows) adds up its four sums with k ascending, one chain of fused multiply-adds each, which gives the bits of the
-// tiled kernel.  Chunks of 256 k come into shared memory in whole rows, the next chunk on its way from memory while
-// this one is multiplied.  K a multiple of 4.
-#define GR_N 16
+// The same product for up to 16 rows (decode steps of the 32-bit path), bound by reading the weights.  A wave owns GN
+// output features and stages ROWS rows; lane (feature, group of ROWS * GN / 64 rows) adds up its rows' sums with k
+// ascending, one chain of fused multiply-adds each, which gives the bits of the tiled kernel whatever GN and ROWS are.
+// Chunks of 256 k come into shared memory in whole rows, the next chunk on its way from memory while this one is
+// multiplied.  A wave's time for a chunk is what its lanes multiply and what it stages of the rows, so fewer rows
+// and fewer features a wave (more waves) read the weights faster; the shapes that exist and the rule that picks one are
+// at the launch below.  K a multiple of 4.
 #define GR_K 256
 #define GR_PITCH (GR_K + 4)             // floats between staged rows: 16-byte aligned, no two of 16 lanes on a bank
-#define GR_ROWS 16
-#define GR_LOADS (GR_N * GR_K / 4 / IA_WAVE)     // loads of four elements a lane brings of each operand
+#define GR_ROWS 16                      // the most rows of one launch
 
-template <typename TI, typename TO>
+template <typename TI, typename TO, int GN, int ROWS>
 __global__ __launch_bounds__(IA_WAVE) void gemm_rows_kernel(TO* __restrict__ out, const TI* __restrict__ x,
                                                             const TI* __restrict__ w, int M, int N, int K) {
-    __shared__ __attribute__((aligned(16))) float ws[GR_N * GR_PITCH];
-    __shared__ __attribute__((aligned(16))) float xs[GR_ROWS * GR_PITCH];
+    constexpr int GROUPS = IA_WAVE / GN;                    // groups of rows
+    constexpr int RPL = ROWS / GROUPS;                      // rows a lane adds up
+    static_assert(GN * GROUPS == IA_WAVE && RPL * GROUPS == ROWS && RPL >= 1, "lane = (feature, group of rows)");
+    static_assert(GR_K / 4 == IA_WAVE, "a lane brings one piece of every staged row");
+    __shared__ __attribute__((aligned(16))) float ws[GN * GR_PITCH];
+    __shared__ __attribute__((aligned(16))) float xs[ROWS * GR_PITCH];
     const int lane = threadIdx.x;
-    const int nn = lane & 15, mg = lane >> 4;
-    const int n0 = blockIdx.x * GR_N;
-    // what this lane fetches: load i takes piece (lane % 64) of row i of the 16 (a row of a chunk is 64 pieces of four)
+    const int nn = lane % GN, mg = lane / GN;
+    const int n0 = blockIdx.x * GN;
+    // what this lane fetches: load i takes piece (lane % 64) of row i (a row of a chunk is 64 pieces of four)
     const int piece = lane * 4;
-    float4 wr[GR_LOADS], xr[GR_LOADS];
-    auto fetch = [&](int k0) {
+    float4 wr[GN], xr[ROWS];
+    auto fetch = [&](int k0, float4* wq, float4* xq) {
+        const int k = k0 + piece;
 #pragma unroll
-        for (int i = 0; i < GR_LOADS; ++i) {
-            const int k = k0 + piece;
+        for (int i = 0; i < GN; ++i) {
             const int n = n0 + i < N ? n0 + i : N - 1;         // (features beyond the matrix: never stored)
-            wr[i] = k < K ? gr_load4(w + (size_t)n * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-            xr[i] = (k < K && i < M) ? gr_load4(x + (size_t)i * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+            wq[i] = k < K ? gr_load4(w + (size_t)n * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+            xq[i] = (k < K && i < M) ? gr_load4(x + (size_t)i * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
     };
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    fetch(0);
-    for (int k0 = 0; k0 < K; k0 += GR_K) {
+    float acc[RPL];
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) acc[i] = 0.f;
+    // chunk k0 goes from its registers into shared memory, the next chunk takes the registers, and the sums go on
+    auto chunk = [&](int k0, float4* wq, float4* xq) {
         __syncthreads();                                        // everybody is done with the chunk before
 #pragma unroll
-        for (int i = 0; i < GR_LOADS; ++i) {
-            *(float4*)(ws + i * GR_PITCH + piece) = wr[i];
-            *(float4*)(xs + i * GR_PITCH + piece) = xr[i];
-        }
-        if (k0 + GR_K < K) fetch(k0 + GR_K);
+        for (int i = 0; i < GN; ++i) *(float4*)(ws + i * GR_PITCH + piece) = wq[i];
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) *(float4*)(xs + i * GR_PITCH + piece) = xq[i];
+        if (k0 + GR_K < K) fetch(k0 + GR_K, wq, xq);
         __syncthreads();
         const float* wmine = ws + nn * GR_PITCH;
-        const float* xmine = xs + mg * 4 * GR_PITCH;
+        const float* xmine = xs + mg * RPL * GR_PITCH;
 #pragma unroll 4
         for (int k4 = 0; k4 < GR_K / 4; ++k4) {
             const float4 wv = *(const float4*)(wmine + k4 * 4);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < RPL; ++i) {
                 const float4 xv = *(const float4*)(xmine + i * GR_PITCH + k4 * 4);
                 acc[i] = fmaf(xv.x, wv.x, acc[i]);
                 acc[i] = fmaf(xv.y, wv.y, acc[i]);
@@ -203,14 +210,47 @@ __global__ __launch_bounds__(IA_WAVE) void gemm_rows_kernel(TO* __restrict__ out
                 acc[i] = fmaf(xv.w, wv.w, acc[i]);
             }
         }
-    }
+    };
+    fetch(0, wr, xr);
+    for (int k0 = 0; k0 < K; k0 += GR_K) chunk(k0, wr, xr);
     const int n = n0 + nn;
     if (n < N)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (mg * 4 + i < M) st(out + (size_t)(mg * 4 + i) * N + n, acc[i]);
+        for (int i = 0; i < RPL; ++i)
+            if (mg * RPL + i < M) st(out + (size_t)(mg * RPL + i) * N + n, acc[i]);
 }
-static_assert(GR_LOADS == GR_N && GR_LOADS == GR_ROWS, "a lane brings one piece of every staged row");
+
+static int skinny_cus();
+static int g_rows_shape = 0;         // 0: by the rule below; else 100 * features + rows, forced (measurements and tests)
+extern "C" int ia_gemm_rows_tune(int shape) {
+    IA_CHECK(shape == 0 || shape == 816 || shape == 808 || shape == 416 || shape == 1608,
+             "gemm_rows_tune: no kernel of %d features and %d rows a wave", shape / 100, shape % 100);
+    g_rows_shape = shape;
+    return 0;
+}
+
+template <typename TI, typename TO, int GN, int ROWS>
+static void launch_rows_shape(void* o, const void* xi, const void* w, int rows, int N, int K, hipStream_t stream) {
+    gemm_rows_kernel<TI, TO, GN, ROWS><<<(unsigned)((N + GN - 1) / GN), IA_WAVE, 0, stream>>>((TO*)o, (const TI*)xi, (const TI*)w, rows, N, K);
+}
+
+// Up to 8 rows: 8 features a wave, 16 where that still makes eight waves for every compute unit's four schedulers;
+// 9 to 16 rows: 8 features, 4 while 8 would leave a scheduler without a wave.  (Measured at 8 rows and 4,096 k, this
+// rule against 16 features and 16 rows for every size: 6,144 features 77 -> 41 us, 4,096 72 -> 36, 24,576 162 -> 88,
+// 151,936 790 -> 483; at 16 rows 75 -> 50, 72 -> 44, 165 -> 144, 803 -> 796.)
+template <typename TI, typename TO>
+static void launch_rows(void* o, const void* xi, const void* w, int rows, int N, int K, hipStream_t stream) {
+    const int cus = skinny_cus();
+    int shape = g_rows_shape;
+    if (shape != 0 && shape % 100 < rows) shape = 816;            // a forced shape that does not hold the rows
+    if (shape == 0) shape = rows <= 8 ? (N >= 64 * cus ? 1608 : 808) : (N <= 32 * cus ? 416 : 816);
+    switch (shape) {
+    case 1608: launch_rows_shape<TI, TO, 16, 8>(o, xi, w, rows, N, K, stream); break;
+    case 808: launch_rows_shape<TI, TO, 8, 8>(o, xi, w, rows, N, K, stream); break;
+    case 416: launch_rows_shape<TI, TO, 4, 16>(o, xi, w, rows, N, K, stream); break;
+    default: launch_rows_shape<TI, TO, 8, 16>(o, xi, w, rows, N, K, stream); break;
+    }
+}
 
 // in_dtype: storage of x and w; out_dtype: storage of the result.
 extern "C" int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K,
@@ -221,20 +261,15 @@ extern "C" int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int
     // up to 64 rows, 16 at a time, where the tiles of 64 x 64 would be few (the weights are read once for every 16 rows:
     // at 32 rows of the 32-bit path a decode step of four layers at the sizes of an 8B model still takes a third of the time)
     if (M <= 4 * GR_ROWS && (M <= GR_ROWS || N <= 4096 * 4) && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) % (4 * elem)) == 0) {
-        const unsigned blocks = (unsigned)((N + GR_N - 1) / GR_N);
         const size_t out_elem = out_dtype == IA_F32 ? 4 : 2;
         for (int m0 = 0; m0 < M; m0 += GR_ROWS) {
             const int rows = M - m0 < GR_ROWS ? M - m0 : GR_ROWS;
             void* o = (char*)out + (size_t)m0 * N * out_elem;
             const void* xi = (const char*)x + (size_t)m0 * K * elem;
-            if (in_dtype == IA_F32 && out_dtype == IA_F32)
-                gemm_rows_kernel<float, float><<<blocks, IA_WAVE, 0, stream>>>((float*)o, (const float*)xi, (const float*)w, rows, N, K);
-            else if (in_dtype == IA_BF16 && out_dtype == IA_BF16)
-                gemm_rows_kernel<bf16_t, bf16_t><<<blocks, IA_WAVE, 0, stream>>>((bf16_t*)o, (const bf16_t*)xi, (const bf16_t*)w, rows, N, K);
-            else if (in_dtype == IA_BF16 && out_dtype == IA_F32)
-                gemm_rows_kernel<bf16_t, float><<<blocks, IA_WAVE, 0, stream>>>((float*)o, (const bf16_t*)xi, (const bf16_t*)w, rows, N, K);
-            else
-                IA_CHECK(false, "gemm_tiled: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+            if (in_dtype == IA_F32 && out_dtype == IA_F32) launch_rows<float, float>(o, xi, w, rows, N, K, stream);
+            else if (in_dtype == IA_BF16 && out_dtype == IA_BF16) launch_rows<bf16_t, bf16_t>(o, xi, w, rows, N, K, stream);
+            else if (in_dtype == IA_BF16 && out_dtype == IA_F32) launch_rows<bf16_t, float>(o, xi, w, rows, N, K, stream);
+            else IA_CHECK(false, "gemm_tiled: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
         }
         IA_LAUNCH_CHECK("gemm_rows");
         return 0;

@@ -1040,3 +1040,29 @@ def test_a_product_with_a_bias_adds_itself_to_the_stream(m, n, k, add_one):
     new_rows = fused_stream.float().cpu().double()
     exact = new_rows / torch.sqrt(new_rows.pow(2).mean(-1, keepdim=True) + 1e-6) * (norm_w.double() + (1.0 if add_one else 0.0))
     close(ops.linear(rows, dev(w2), bias=dev(b2)), exact @ w2.double().t() + b2.double(), 2 ** -6, "norm's end and bias inside")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_few_row_product_of_the_32_bit_path_with_every_block_shape(dtype):
+    """The product for up to 16 rows with 4, 8 or 16 output features and 8 or 16 staged rows a wave (100 * features +
+    rows names a shape; one that does not hold the rows gives way to one that does): one chain of fused multiply-adds
+    for every output in all of them, so the bits are the same, and those of the tiled kernel that takes more rows."""
+    from inferrs_amd import ops
+    lib = ops.library()
+    x = randn(80, 520, dtype=dtype, seed=1)
+    w = dev(randn(203, 520, dtype=dtype, seed=2, scale=0.05))
+    many = ops.gemm_tiled(dev(x), w).cpu()                      # 80 rows: tiles of 64 x 64
+    outs = {}
+    try:
+        for features in (816, 808, 416, 1608, 0):
+            assert lib.ia_gemm_rows_tune(features) == 0
+            outs[features] = [ops.gemm_tiled(dev(x[:m].contiguous()), w).cpu() for m in (1, 7, 8, 9, 16)]
+        assert lib.ia_gemm_rows_tune(1616) != 0 and "16 features and 16 rows" in lib.ia_last_error().decode()
+    finally:
+        lib.ia_gemm_rows_tune(0)
+    for features, got in outs.items():
+        for i, y in enumerate(got):
+            assert torch.equal(y, outs[816][i]), (features, i)
+            if dtype == torch.float32:
+                assert torch.equal(y, many[:y.shape[0]]), (features, y.shape)
+            close(y, x[:y.shape[0]].double() @ w.double().cpu().t(), tol(dtype, 2e-6), "few rows")
