@@ -40,7 +40,13 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_si
 # The larger dense models of the family differ in these sizes only.
 QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64)
-SHAPES = {"8B": QWEN3_8B, "14B": QWEN3_14B, "32B": QWEN3_32B}
+# The smallest shape is the one that the reference's defaults describe (`inferrs/src/config.rs:468-502`: width 1,024, 28 layers,
+# 16 query and 8 key/value heads, feed-forward 3,072, tied embeddings); two more small ones between it and the 8B shape.
+QWEN3_0_6B = dict(QWEN3_8B, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                  tie_word_embeddings=True)
+QWEN3_1_7B = dict(QWEN3_0_6B, hidden_size=2048, intermediate_size=6144)
+QWEN3_4B = dict(QWEN3_0_6B, hidden_size=2560, intermediate_size=9728, num_hidden_layers=36, num_attention_heads=32)
+SHAPES = {"0.6B": QWEN3_0_6B, "1.7B": QWEN3_1_7B, "4B": QWEN3_4B, "8B": QWEN3_8B, "14B": QWEN3_14B, "32B": QWEN3_32B}
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 PREFILL_TOKENS = 2048
