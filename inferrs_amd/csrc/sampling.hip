@@ -21,6 +21,8 @@
 // shorter way (sample_top_k): their first top_k tokens are picked out and sorted, and the
 // reference's steps run on that list as it runs them.  Rows without a top_k try that way with
 // the first 1,024 tokens of their list and take the long one when the list does not end there.
+// Probabilities, keys and each stretch's candidates for that list are the work of many blocks
+// a row (two kernels); one block a row then makes the choice.
 #include <mutex>
 
 #include "common.h"
@@ -376,30 +378,30 @@ __device__ Prefix shortest_prefix(const uint32_t* __restrict__ keys, const float
     return r;
 }
 
-// Index of the `rank`-th (1-based, ascending index) token whose key equals `key`.
+// Index of the `rank`-th (1-based, ascending index) token whose key equals `key` (-1: there are fewer).  A thread
+// counts a run of neighbouring tokens; the counts are scanned in the wave and over the waves, and the thread in
+// whose run the rank falls walks it.  `s_counts`: an entry a wave.
 __device__ int nth_with_key(const uint32_t* __restrict__ keys, int vocab, uint32_t key, int rank, int* s_counts) {
     const int per = (vocab + blockDim.x - 1) / blockDim.x;
     const int lo = threadIdx.x * per, hi = lo + per < vocab ? lo + per : vocab;
     int mine = 0;
     for (int c = lo; c < hi; ++c) mine += keys[c] == key;
-    __syncthreads();
-    s_counts[threadIdx.x] = mine;
-    __syncthreads();
-    __shared__ int s_found;
-    if (threadIdx.x == 0) {
-        s_found = -1;
-        int before = 0;
-        for (int t = 0; t < (int)blockDim.x; ++t) {
-            if (before + s_counts[t] >= rank) { s_found = t; s_counts[0] = before; break; }
-            before += s_counts[t];
-        }
+    const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+    int upto = mine;
+#pragma unroll
+    for (int o = 1; o < IA_WAVE; o <<= 1) {
+        const int other = __shfl_up(upto, o, IA_WAVE);
+        if (lane >= o) upto += other;
     }
-    __syncthreads();
     __shared__ int s_index;
+    __syncthreads();
+    if (lane == IA_WAVE - 1) s_counts[wave] = upto;
     if (threadIdx.x == 0) s_index = -1;
     __syncthreads();
-    if ((int)threadIdx.x == s_found) {
-        int seen = s_counts[0];
+    int before = upto - mine;
+    for (int w = 0; w < wave; ++w) before += s_counts[w];
+    if (before < rank && rank <= before + mine) {
+        int seen = before;
         for (int c = lo; c < hi; ++c)
             if (keys[c] == key && ++seen == rank) { s_index = c; break; }
     }
@@ -462,16 +464,13 @@ __device__ __forceinline__ void for_each_key(const uint32_t* __restrict__ keys, 
         }
     }
 }
-// `open`: the row has no top_k; k tokens are only the beginning of its list, whose weight is `total`.  The steps
-// then succeed if top_p or min_p end the list within these k, or else the walk ends there; if not, nothing is
-// written and false comes back (the caller goes the long way).
-__device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__ keys, const float* __restrict__ probs,
-                             int vocab, int rowi, int k, bool open, float total, float tp, float mp, float u, int want_top,
-                             float* __restrict__ lp_out, int* __restrict__ lp_ids, int* s_counts) {
+// The first k entries of the ordered list of `n` keys (keys descending, equal keys by ascending place): every
+// key above `kth`, and the keys equal to it up to place `last_tie`.  0 < k < n.  Three histograms over the
+// key's bits, 11 + 11 + 10 at a time, find the k-th largest key.
+struct Cut { uint32_t kth; int last_tie; };
+__device__ Cut top_k_cut(const uint32_t* __restrict__ keys, int n, int k, int* s_counts) {
     __shared__ int hist[2048];
-    __shared__ unsigned long long cand[SAMPLE_FAST_K];      // (key, ~index): larger is earlier in the list
-    __shared__ int s_bin, s_above, s_n, s_done;
-    // ---- the k-th largest key, 11 + 11 + 10 bits at a time
+    __shared__ int s_bin, s_above;
     uint32_t prefix = 0u;
     int prefix_bits = 0, need = k;
     for (int level = 0; level < 3; ++level) {
@@ -479,7 +478,7 @@ __device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
         const int shift = 32 - prefix_bits - bits;
         for (int i = threadIdx.x; i < 2048; i += blockDim.x) hist[i] = 0;
         __syncthreads();
-        for_each_key(keys, vocab, [&](int, uint32_t key) {
+        for_each_key(keys, n, [&](int, uint32_t key) {
             if (prefix_bits == 0 || (key >> (32 - prefix_bits)) == prefix)
                 atomicAdd(&hist[(key >> shift) & ((1u << bits) - 1u)], 1);
         });
@@ -516,14 +515,35 @@ __device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
         prefix_bits += bits;
         __syncthreads();
     }
-    const uint32_t kth = prefix;                            // `need` (>= 1) of the tokens with this key belong to the list
-    const int ties = hist[kth & 1023u];
+    Cut cut;
+    cut.kth = prefix;                                       // `need` (>= 1) of the tokens with this key belong to the list
+    const int ties = hist[cut.kth & 1023u];
     __syncthreads();
-    int last_tie = vocab;                                   // ties up to this index are taken
-    if (ties > need) last_tie = nth_with_key(keys, vocab, kth, need, s_counts);
+    cut.last_tie = n;                                       // ties up to this place are taken
+    if (ties > need) cut.last_tie = nth_with_key(keys, n, cut.kth, need, s_counts);
+    return cut;
+}
+
+// The reference's steps on the first k entries of a row's ordered list.  `keys` [n] holds the row's candidates in
+// the order of their tokens' indices (every stretch of the row has left its own first k there, so the row's first
+// k are among them), `token_of` [n] their tokens, `probs` the whole row's probabilities by token.
+// `open`: the row has no top_k; k tokens are only the beginning of its list, whose weight is `total`.  The steps
+// then succeed if top_p or min_p end the list within these k, or else the walk ends there; if not, nothing is
+// written and false comes back (the caller goes the long way).
+__device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__ keys, const int* __restrict__ token_of,
+                             const float* __restrict__ probs, int n_keys, int rowi, int k, bool open, float total,
+                             float tp, float mp, float u, int want_top, float* __restrict__ lp_out,
+                             int* __restrict__ lp_ids, int* s_counts) {
+    __shared__ unsigned long long cand[SAMPLE_FAST_K];      // (key, ~place): larger is earlier in the list
+    __shared__ int s_n, s_done;
+    Cut cut;
+    if (k < n_keys) cut = top_k_cut(keys, n_keys, k, s_counts);
+    else { cut.kth = 0u; cut.last_tie = n_keys; }
+    const uint32_t kth = cut.kth;
+    const int last_tie = cut.last_tie;
     if (threadIdx.x == 0) s_n = 0;
     __syncthreads();
-    for_each_key(keys, vocab, [&](int c, uint32_t key) {
+    for_each_key(keys, n_keys, [&](int c, uint32_t key) {
         if (key > kth || (key == kth && c <= last_tie)) {
             const int slot = atomicAdd(&s_n, 1);
             if (slot < SAMPLE_FAST_K) cand[slot] = ((unsigned long long)key << 32) | (uint32_t)~(uint32_t)c;
@@ -547,11 +567,11 @@ __device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
         }
     __syncthreads();
     __shared__ float cprob[SAMPLE_FAST_K];
-    for (int i = threadIdx.x; i < n; i += blockDim.x) cprob[i] = probs[(int)~(uint32_t)(cand[i] & 0xffffffffull)];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) cprob[i] = probs[token_of[(int)~(uint32_t)(cand[i] & 0xffffffffull)]];
     __syncthreads();
     if (threadIdx.x == 0) {
         // ---- the reference's steps 7 to 12 on its sorted list
-        auto index_of = [&](int i) { return (int)~(uint32_t)(cand[i] & 0xffffffffull); };
+        auto index_of = [&](int i) { return token_of[(int)~(uint32_t)(cand[i] & 0xffffffffull)]; };
         bool ended = !open, done = true;                    // ended: the list's end lies within these n tokens
         int len = n;
         if (tp < 1.0f) {
@@ -614,12 +634,228 @@ __device__ bool sample_top_k(int* __restrict__ out, const uint32_t* __restrict__
     return s_done != 0;
 }
 
-// workspace: [rows, 2, vocab] words: the keys, then the probabilities.
+// ---- a row's workspace and the two passes that fill it --------------------------------------
+// Temperature, softmax and the ordering keys of a row are the work of many blocks (a row of 152 k logits kept one
+// block busy for 150 us, whatever the batch): the row is cut into stretches of up to SAMPLE_STRETCH tokens, a block each
+// (a stretch's keys fit the block's shared memory).
+//   pass 1 (sample_partials_kernel): the stretch's maximum of z / temperature and its sum of exp(. - that maximum);
+//   pass 2 (sample_stretch_kernel): the row's maximum and sum from the stretches' (every block adds them up in the
+//     same order), probabilities and keys of the stretch, the sum of its probabilities, and the stretch's own
+//     first k entries of the ordered list (k: the row's top_k, or SAMPLE_FAST_K for a row without one), written
+//     in the order of their tokens at a place that follows from k and the stretches' lengths alone;
+//   then one block a row (sample_kernel) picks the row's first k among those candidates and walks them.
+// A row's words: keys [vocab], probabilities [vocab], the candidates' keys and tokens [stretches * SAMPLE_FAST_K]
+// each, and the stretches' maxima, sums and sums of probabilities [stretches] each.
+#define SAMPLE_STRETCH 4096
+#define SAMPLE_STAGED 8192              // candidates of a row that its last block keeps in shared memory
+#define SAMPLE_MAX_STRETCHES 1024       // the stretches' sums meet in a block's shared memory: 4 M tokens a row
+struct RowLayout {
+    int vocab, stretches, stretch;      // stretch: tokens a stretch (the last one may be shorter), a multiple of 4
+    long long words;                    // of a row
+    __host__ __device__ int length(int b) const { const int left = vocab - b * stretch; return left < stretch ? left : stretch; }
+    // candidates that the stretches before b leave when every stretch leaves its first k (or all it has)
+    __host__ __device__ int candidates_before(int b, int k) const {
+        const int each = k < stretch ? k : stretch;     // every stretch before the last is a whole one
+        return b * each;
+    }
+    __host__ __device__ int candidates(int k) const {
+        const int last = length(stretches - 1);
+        return candidates_before(stretches - 1, k) + (k < last ? k : last);
+    }
+    __device__ uint32_t* keys(uint32_t* ws, int row) const { return ws + (size_t)row * words; }
+    __device__ float* probs(uint32_t* ws, int row) const { return (float*)(keys(ws, row) + vocab); }
+    __device__ uint32_t* cand_keys(uint32_t* ws, int row) const { return keys(ws, row) + 2 * (size_t)vocab; }
+    __device__ int* cand_tokens(uint32_t* ws, int row) const { return (int*)(cand_keys(ws, row) + (size_t)stretches * SAMPLE_FAST_K); }
+    __device__ float* part_max(uint32_t* ws, int row) const { return (float*)(cand_tokens(ws, row) + (size_t)stretches * SAMPLE_FAST_K); }
+    __device__ float* part_sum(uint32_t* ws, int row) const { return part_max(ws, row) + stretches; }
+    __device__ float* part_total(uint32_t* ws, int row) const { return part_sum(ws, row) + stretches; }
+};
+
+static RowLayout row_layout(int vocab) {
+    RowLayout l;
+    l.vocab = vocab;
+    l.stretches = (vocab + SAMPLE_STRETCH - 1) / SAMPLE_STRETCH;
+    l.stretch = ((vocab + l.stretches - 1) / l.stretches + 3) & ~3;
+    const long long words = 2LL * vocab + 2LL * l.stretches * SAMPLE_FAST_K + 3LL * l.stretches;
+    l.words = (words + 3) & ~3LL;
+    return l;
+}
+
+// The temperature a row is sampled at; false: the row is a greedy one and has no use for probabilities.
+__device__ __forceinline__ bool row_temperature(const float* temperature, const int* n_top, int rowi, float& temp) {
+    temp = temperature[rowi];
+    if (temp < 1e-5f) {
+        if (n_top == nullptr || n_top[rowi] < 0) return false;
+        temp = 1e-5f;           // with log-probabilities the reference takes no shortcut (sampler.rs:176, :232-239)
+    }
+    return true;
+}
+
+// The row's maximum, the sum of exp(z / temperature - maximum) and (with `with_total`) the sum of the probabilities
+// from the stretches' (a stretch of nothing but -inf adds nothing to the sum); every block that asks gets the same bits.
+// `s_parts`: 3 * stretches floats of shared memory.  All threads of the block call it.
+struct RowSums { float mx, sum, total; };
+__device__ RowSums row_sums(const RowLayout& l, uint32_t* ws, int rowi, bool with_total, float* s_parts) {
+    const float* parts = l.part_max(ws, rowi);               // maxima, sums, totals: one after the other
+    const int n = (with_total ? 3 : 2) * l.stretches;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) s_parts[i] = parts[i];
+    __syncthreads();
+    RowSums r;
+    r.mx = -INFINITY;
+    for (int b = 0; b < l.stretches; ++b) r.mx = fmaxf(r.mx, s_parts[b]);
+    r.sum = 0.f;
+    for (int b = 0; b < l.stretches; ++b)
+        if (s_parts[b] > -INFINITY) r.sum += s_parts[l.stretches + b] * expf(s_parts[b] - r.mx);
+    r.total = 0.f;
+    if (with_total)
+        for (int b = 0; b < l.stretches; ++b) r.total += s_parts[2 * l.stretches + b];
+    __syncthreads();
+    return r;
+}
+
+__global__ __launch_bounds__(256) void sample_partials_kernel(const float* __restrict__ logits, uint32_t* __restrict__ workspace,
+                                                              const RowLayout l, const float* __restrict__ temperature,
+                                                              const int* __restrict__ n_top) {
+    __shared__ float scratch[32];
+    const int rowi = blockIdx.y, b = blockIdx.x;
+    float temp;
+    if (!row_temperature(temperature, n_top, rowi, temp)) return;
+    const float* row = logits + (size_t)rowi * l.vocab + (size_t)b * l.stretch;
+    const int n = l.length(b);
+    // temperature, and the softmax's two sums (sampler.rs:232-249); four loads under way
+    float mx = -INFINITY;
+    for (int c0 = threadIdx.x; c0 < n; c0 += 4 * blockDim.x) {
+        float z[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            z[j] = c < n ? row[c] : -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (c0 + j * (int)blockDim.x < n) mx = fmaxf(mx, z[j] / temp);
+    }
+    mx = wave_max(mx);
+    if ((threadIdx.x & (IA_WAVE - 1)) == 0) scratch[16 + threadIdx.x / IA_WAVE] = mx;
+    __syncthreads();
+    for (int w = 0; w < (int)(blockDim.x / IA_WAVE); ++w) mx = fmaxf(mx, scratch[16 + w]);
+    float sum = 0.f;
+    if (mx > -INFINITY)
+        for (int c0 = threadIdx.x; c0 < n; c0 += 4 * blockDim.x) {
+            float z[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = c0 + j * (int)blockDim.x;
+                z[j] = c < n ? row[c] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (c0 + j * (int)blockDim.x < n) sum += expf(z[j] / temp - mx);
+        }
+    sum = block_sum(sum, scratch);
+    if (threadIdx.x == 0) {
+        l.part_max(workspace, rowi)[b] = mx;
+        l.part_sum(workspace, rowi)[b] = sum;
+    }
+}
+
+// How many entries of a row's ordered list are picked out before the reference's steps run on them: the row's
+// top_k, SAMPLE_FAST_K for a row without one, 0 for a row that goes the long way (a top_k beyond SAMPLE_FAST_K, a
+// vocabulary within it, or the switch off).
+__device__ __forceinline__ int picked_out(int k, int vocab, int fast_top_k) {
+    if (!fast_top_k) return 0;
+    if (k > 0 && k < vocab) return k <= SAMPLE_FAST_K ? k : 0;
+    return vocab > SAMPLE_FAST_K ? SAMPLE_FAST_K : 0;
+}
+
+#define STRETCH_THREADS 256
+__global__ __launch_bounds__(STRETCH_THREADS) void sample_stretch_kernel(
+    const float* __restrict__ logits, uint32_t* __restrict__ workspace, const RowLayout l,
+    const float* __restrict__ temperature, const int* __restrict__ top_k, const int* __restrict__ n_top, int fast_top_k) {
+    __shared__ float scratch[32];
+    __shared__ int s_counts[STRETCH_THREADS];
+    __shared__ int s_waves[STRETCH_THREADS / IA_WAVE];
+    __shared__ uint32_t s_keys[SAMPLE_STRETCH];             // the stretch's keys: the choice below reads them several times
+    __shared__ float s_parts[2 * SAMPLE_MAX_STRETCHES];
+    const int rowi = blockIdx.y, b = blockIdx.x;
+    float temp;
+    if (!row_temperature(temperature, n_top, rowi, temp)) return;
+    const int lo = b * l.stretch, n = l.length(b);
+    const float* row = logits + (size_t)rowi * l.vocab + lo;
+    uint32_t* keys = l.keys(workspace, rowi) + lo;
+    float* probs = l.probs(workspace, rowi) + lo;
+    const RowSums rs = row_sums(l, workspace, rowi, false, s_parts);
+    // The list is ordered by the probabilities themselves, as the reference sorts them: logits whose
+    // probabilities round to the same number (or vanish together) are ties, taken in index order.
+    float t = 0.f;
+    for (int c0 = threadIdx.x; c0 < n; c0 += 4 * blockDim.x) {
+        float z[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            z[j] = c < n ? row[c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j * (int)blockDim.x;
+            if (c < n) {
+                const float e = expf(z[j] / temp - rs.mx);
+                const float pr = rs.sum > 0.f ? e / rs.sum : e;
+                const uint32_t key = order_key(pr);
+                probs[c] = pr;
+                keys[c] = key;
+                s_keys[c] = key;
+                t += pr;
+            }
+        }
+    }
+    t = block_sum(t, scratch);
+    if (threadIdx.x == 0) l.part_total(workspace, rowi)[b] = t;
+    const int k = picked_out(top_k[rowi], l.vocab, fast_top_k);
+    if (k == 0) return;
+    __syncthreads();
+    // ---- the stretch's own first k, in the order of their tokens
+    uint32_t* ck = l.cand_keys(workspace, rowi) + l.candidates_before(b, k);
+    int* ct = l.cand_tokens(workspace, rowi) + l.candidates_before(b, k);
+    if (k >= n) {
+        for (int c = threadIdx.x; c < n; c += blockDim.x) { ck[c] = s_keys[c]; ct[c] = lo + c; }
+        return;
+    }
+    const Cut cut = top_k_cut(s_keys, n, k, s_counts);
+    // a thread takes a run of neighbouring tokens, counts those of the list, and writes them behind what the
+    // threads before it have counted
+    const int per = (n + blockDim.x - 1) / blockDim.x;
+    const int first = threadIdx.x * per, last = first + per < n ? first + per : n;
+    int mine = 0;
+    for (int c = first; c < last; ++c) {
+        const uint32_t key = s_keys[c];
+        mine += (key > cut.kth || (key == cut.kth && c <= cut.last_tie)) ? 1 : 0;
+    }
+    int upto = mine;                                        // inclusive scan over the wave's lanes
+    const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
+#pragma unroll
+    for (int o = 1; o < IA_WAVE; o <<= 1) {
+        const int other = __shfl_up(upto, o, IA_WAVE);
+        if (lane >= o) upto += other;
+    }
+    if (lane == IA_WAVE - 1) s_waves[wave] = upto;
+    __syncthreads();
+    int at = upto - mine;
+    for (int w = 0; w < wave; ++w) at += s_waves[w];
+    for (int c = first; c < last; ++c) {
+        const uint32_t key = s_keys[c];
+        if (key > cut.kth || (key == cut.kth && c <= cut.last_tie)) {
+            if (at < k) { ck[at] = key; ct[at] = lo + c; }
+            ++at;
+        }
+    }
+}
+
 // n_top (may be null): per row -1 = no log-probabilities, else how many of the list's first entries are
 // reported besides the drawn token's (sampler.rs:285-352).  lp_out [rows, 1 + SAMPLE_MAX_TOP]: the drawn
 // token's log-probability within the kept list, then the entries'; lp_ids [rows, SAMPLE_MAX_TOP]: their ids (-1: none).
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
-    int* __restrict__ out, const float* __restrict__ logits, uint32_t* __restrict__ workspace, int vocab,
+    int* __restrict__ out, const float* __restrict__ logits, uint32_t* __restrict__ workspace, const RowLayout l,
     const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
     const float* __restrict__ min_p, const float* __restrict__ u, const int* __restrict__ n_top,
     float* __restrict__ lp_out, int* __restrict__ lp_ids, int fast_top_k) {
@@ -628,111 +864,41 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     __shared__ float sv[16];
     __shared__ int si[16];
     const int rowi = blockIdx.x;
+    const int vocab = l.vocab;
     const float* row = logits + (size_t)rowi * vocab;
-    float temp = temperature[rowi];
     const int want_top = n_top != nullptr ? n_top[rowi] : -1;
     if (want_top >= 0 && threadIdx.x < SAMPLE_MAX_TOP) {
         lp_ids[(size_t)rowi * SAMPLE_MAX_TOP + threadIdx.x] = -1;
         lp_out[(size_t)rowi * (1 + SAMPLE_MAX_TOP) + 1 + threadIdx.x] = -INFINITY;
     }
-    if (temp < 1e-5f) {
-        if (want_top < 0) {
-            argmax_row(row, vocab, sv, si, out + rowi);
-            return;
-        }
-        temp = 1e-5f;           // with log-probabilities the reference takes no shortcut (sampler.rs:176, :232-239)
-    }
-    uint32_t* keys = workspace + (size_t)rowi * 2 * vocab;
-    float* probs = (float*)(keys + vocab);
-
-    // temperature, softmax (sampler.rs:232-249)
-    // (the passes over the row keep four loads under way; a thread's sums run in the order of its indices)
-    float mx = -INFINITY;
-    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
-        float z[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + j * (int)blockDim.x;
-            z[j] = c < vocab ? row[c] : 0.f;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + j * (int)blockDim.x;
-            if (c < vocab) {
-                z[j] = z[j] / temp;
-                probs[c] = z[j];
-                mx = fmaxf(mx, z[j]);
-            }
-        }
-    }
-    mx = wave_max(mx);
-    __syncthreads();
-    if ((threadIdx.x & (IA_WAVE - 1)) == 0) scratch[threadIdx.x / IA_WAVE] = mx;
-    __syncthreads();
-    for (int w = 0; w < SAMPLE_THREADS / IA_WAVE; ++w) mx = fmaxf(mx, scratch[w]);
-    float sum = 0.f;
-    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
-        float z[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + j * (int)blockDim.x;
-            z[j] = c < vocab ? probs[c] : 0.f;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + j * (int)blockDim.x;
-            if (c < vocab) {
-                const float e = expf(z[j] - mx);
-                probs[c] = e;
-                sum += e;
-            }
-        }
-    }
-    sum = block_sum(sum, scratch);
-    // The list is ordered by the probabilities themselves, as the reference sorts them: logits whose
-    // probabilities round to the same number (or vanish together) are ties, taken in index order.
-    for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
-        float e[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + j * (int)blockDim.x;
-            e[j] = c < vocab ? probs[c] : 0.f;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + j * (int)blockDim.x;
-            if (c < vocab) {
-                const float pr = sum > 0.f ? e[j] / sum : e[j];
-                probs[c] = pr;
-                keys[c] = order_key(pr);
-            }
-        }
-    }
-    __syncthreads();
-
-    const int k = top_k[rowi];
-    if (fast_top_k && k > 0 && k < vocab && k <= SAMPLE_FAST_K) {
-        sample_top_k(out, keys, probs, vocab, rowi, k, false, 0.f, top_p[rowi], min_p[rowi], u[rowi], want_top, lp_out,
-                     lp_ids, s_counts);
+    float temp;
+    if (!row_temperature(temperature, n_top, rowi, temp)) {
+        argmax_row(row, vocab, sv, si, out + rowi);
         return;
     }
-    if (fast_top_k && (k <= 0 || k >= vocab) && vocab > SAMPLE_FAST_K) {
-        // without a top_k: the list's first 1,024 tokens, which hold the nucleus, the min_p cut or the walk's end
-        // for all but flat distributions; its weight is the sum the long way would use
-        float t = 0.f;
-        for (int c0 = threadIdx.x; c0 < vocab; c0 += 4 * blockDim.x) {
-            float pr[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int c = c0 + j * (int)blockDim.x;
-                pr[j] = c < vocab ? probs[c] : 0.f;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) t += pr[j];
+    const uint32_t* keys = l.keys(workspace, rowi);
+    const float* probs = l.probs(workspace, rowi);
+    __shared__ float s_parts[3 * SAMPLE_MAX_STRETCHES];
+    const RowSums rs = row_sums(l, workspace, rowi, true, s_parts);
+    const float sum = rs.sum, total = rs.total;             // total: the weight of the whole list
+
+    const int k = top_k[rowi];
+    const int picked = picked_out(k, vocab, fast_top_k);
+    if (picked > 0) {
+        // the list's first entries: the row's top_k, or, without one, 1,024 tokens, which hold the nucleus, the min_p
+        // cut or the walk's end for all but flat distributions
+        const bool open = !(k > 0 && k < vocab);
+        // (few candidates are read from shared memory: the choice among them reads them several times)
+        __shared__ uint32_t s_cand[SAMPLE_STAGED];
+        const int n_cand = l.candidates(picked);
+        const uint32_t* cand_keys = l.cand_keys(workspace, rowi);
+        if (n_cand <= SAMPLE_STAGED) {
+            for (int i = threadIdx.x; i < n_cand; i += blockDim.x) s_cand[i] = cand_keys[i];
+            __syncthreads();
+            cand_keys = s_cand;
         }
-        const float total = block_sum(t, scratch);
-        if (sample_top_k(out, keys, probs, vocab, rowi, SAMPLE_FAST_K, true, total, top_p[rowi], min_p[rowi], u[rowi],
-                         want_top, lp_out, lp_ids, s_counts))
+        if (sample_top_k(out, cand_keys, l.cand_tokens(workspace, rowi), probs, n_cand, rowi,
+                         picked, open, total, top_p[rowi], min_p[rowi], u[rowi], want_top, lp_out, lp_ids, s_counts))
             return;
     }
     // how long the kept prefix is (sampler.rs:256-283)
@@ -773,9 +939,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         filtered = wa + (float)kept.take * s_pk2;
     } else {
         kept.key = 0u; kept.above = 0; kept.ties = 0; kept.take = 0;
-        float t = 0.f;
-        for (int c = threadIdx.x; c < vocab; c += blockDim.x) t += probs[c];
-        filtered = block_sum(t, scratch);
+        filtered = total;
     }
 
     // the walk (sampler.rs:323-335): the first place where the running sum of p / filtered exceeds u
@@ -832,7 +996,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
 }
 
-extern "C" long long ia_sample_workspace(int rows, int vocab) { return (long long)rows * 2 * vocab; }
+// Words of workspace for `rows` rows (see the layout of a row above).
+extern "C" long long ia_sample_workspace(int rows, int vocab) {
+    return vocab > 0 && rows > 0 ? (long long)rows * row_layout(vocab).words : 0;
+}
 
 static int g_sample_fast = 1;
 // Measurement and test switch: 0 sends rows with a top_k through the bisections as well.
@@ -845,11 +1012,18 @@ extern "C" int ia_sample(int* out, const float* logits, void* workspace, int row
                          const float* temperature, const int* top_k, const float* top_p, const float* min_p,
                          const float* u, const int* n_top, float* lp_out, int* lp_ids, hipStream_t stream) {
     IA_CHECK(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
-    IA_CHECK(workspace != nullptr || rows == 0, "sample: needs a workspace of rows * 2 * vocab words");
+    IA_CHECK(workspace != nullptr || rows == 0, "sample: needs a workspace of ia_sample_workspace(rows, vocab) words");
     IA_CHECK((n_top == nullptr) == (lp_out == nullptr) && (n_top == nullptr) == (lp_ids == nullptr),
              "sample: the arrays of the log-probabilities come together");
+    IA_CHECK(rows <= 65535, "sample: at most 65535 rows a call, not %d", rows);
+    IA_CHECK(vocab <= SAMPLE_STRETCH * SAMPLE_MAX_STRETCHES, "sample: at most %d tokens a row, not %d", SAMPLE_STRETCH * SAMPLE_MAX_STRETCHES, vocab);
     if (rows == 0) return 0;
-    sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, (uint32_t*)workspace, vocab, temperature,
+    const RowLayout l = row_layout(vocab);
+    const dim3 grid((unsigned)l.stretches, (unsigned)rows);
+    sample_partials_kernel<<<grid, 256, 0, stream>>>(logits, (uint32_t*)workspace, l, temperature, n_top);
+    sample_stretch_kernel<<<grid, STRETCH_THREADS, 0, stream>>>(logits, (uint32_t*)workspace, l, temperature, top_k, n_top,
+                                                               g_sample_fast);
+    sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, (uint32_t*)workspace, l, temperature,
                                                        top_k, top_p, min_p, u, n_top, lp_out, lp_ids, g_sample_fast);
     IA_LAUNCH_CHECK("sample");
     return 0;

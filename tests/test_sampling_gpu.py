@@ -156,6 +156,32 @@ def test_equal_logits_are_taken_in_index_order():
 
 
 @pytest.mark.gpu
+def test_equal_favourites_across_the_stretches_of_a_row_are_taken_in_index_order():
+    """A row of 10,000 logits is the work of three blocks (stretches of 3,336 tokens), each of which leaves its own
+    first top_k behind: eleven equal favourites that straddle the first border, and a row of nothing but equal
+    logits, are still taken by ascending index over the whole row."""
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    z = torch.zeros(1, 10000)
+    z[0, 3330:3341] = 6.0
+    flat = torch.zeros(1, 10000)
+    seen, seen_flat = set(), set()
+    for step in range(60):
+        p = SamplingParams(temperature=1.0, top_p=1.0, top_k=8, repetition_penalty=1.0, seed=11)
+        prev = [0] * step
+        got = sampler.sample(z.to("cuda"), [p], [prev], [11])[0]
+        want = pm.sample(z[0], prev, temperature=1.0, top_p=1.0, top_k=8, repetition_penalty=1.0, seed=11)
+        assert got == want and 3330 <= got <= 3337, (step, got, want)
+        seen.add(got)
+        got = sampler.sample(flat.to("cuda"), [p], [prev], [11])[0]
+        assert got == pm.sample(flat[0], prev, temperature=1.0, top_p=1.0, top_k=8, repetition_penalty=1.0, seed=11)
+        assert 0 <= got <= 7
+        seen_flat.add(got)
+    assert max(seen) >= 3336 and min(seen) < 3336, seen          # tokens on both sides of the border were drawn
+    assert len(seen_flat) >= 5
+
+
+@pytest.mark.gpu
 def test_frequencies_follow_the_tempered_softmax():
     from inferrs_amd.sampling import Sampler
     sampler = Sampler("cuda:0")
