@@ -374,18 +374,26 @@ def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: i
 
 
 DECODE_WAVES = 1024            # the decode kernel holds a wave a SIMD: as many waves as the chip has SIMDs, no more
-DECODE_MIN_CHUNK = 128         # fewest keys a wave's share is worth (four steps of 32)
+DECODE_MIN_CHUNK = 64          # fewest keys a wave's share is worth (two steps of 32); 128 up to a context of 512
+DECODE_MANY_SPLITS = 32        # more splits than these only where a split would still hold more than 128 keys
 
 
 def decode_split(n_seqs: int, nkv: int, g: int, max_kv_len: int) -> Tuple[int, int]:
     """(splits, keys per split) for the decode kernel: the largest power of two that keeps the step's waves
-    (request x kv head x 16 query heads x split) within one round of the chip and a wave's share at 128 keys
-    or more.  Measured at head size 128, 32 query and 8 kv heads, context 8,192 (microseconds a layer): batch 1
+    (request x kv head x 16 query heads x split) within one round of the chip and a wave's share at 64 keys
+    or more; beyond 32 splits (eight blocks to merge) only where a share would exceed 128 keys.  Measured at head
+    size 128, 32 query and 8 kv heads, context 8,192 (microseconds a layer): batch 1
     18.0 with 64 splits against 20.0 with 128, batch 3 27.6 with 32 against 34.1 with 64, batch 8 52.4 with 16
-    against 55.5 with 32, batch 64 358 with 2 against 375 with 4."""
+    against 55.5 with 32, batch 64 358 with 2 against 375 with 4.  Shares of 64 keys against 128, the kernel called
+    back to back in a graph: batch 1 at a context of 1,024 11.3 against 13.0, of 2,048 12.4 against 13.7; batch 4
+    at 2,048 14.3 against 15.9; batch 8 at 1,024 13.3 against 14.6; at a context of 512 four splits are as good as
+    any (10.8), and 64 splits of 64 keys at 4,096 lose to 32 of 128 (batch 2: 17.0 against 16.0)."""
     items = n_seqs * nkv * -(-g // 16)
+    min_chunk = DECODE_MIN_CHUNK if max_kv_len > 512 else 128
     splits = 1
-    while items * splits * 2 <= DECODE_WAVES and max_kv_len >= 2 * splits * DECODE_MIN_CHUNK and splits < 128:
+    while items * splits * 2 <= DECODE_WAVES and max_kv_len >= 2 * splits * min_chunk and splits < 128:
+        if splits >= DECODE_MANY_SPLITS and max_kv_len <= splits * 128:
+            break
         splits *= 2
     chunk = -(-max_kv_len // splits)
     return splits, -(-chunk // 32) * 32
