@@ -98,16 +98,21 @@ def fill_context(engine, ids, context: int) -> None:
         engine.cache.commit(sid, context)
 
 
-def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decode_run: int = 8):
+def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decode_run: int = 8, sampled: bool = False):
     """(seconds for `steps` steps, mean context length during them).  The steps go through the
-    serving loop: scheduler, step function, greedy choice on the device."""
+    serving loop: scheduler, step function, greedy choice on the device; with `sampled` the choice is a draw
+    with the reference's default parameters (temperature 0.7, top_k 50, top_p 0.9, repetition penalty 1.1
+    over 64 tokens: `inferrs/src/main.rs:144-154`, `inferrs/src/sampler.rs:96-97`) and a fixed seed."""
     import torch
     from inferrs_amd.engine import GenerationLoop
     from inferrs_amd.engine.scheduler import Request
     from inferrs_amd.sampling import SamplingParams
     start_len = context - steps - warmup
     loop = GenerationLoop(engine, max_batch_size=batch, max_tokens_per_step=max(batch, 16), decode_run=decode_run)
-    params = SamplingParams.greedy(max_tokens=steps + warmup + 8, bypass_stop_tokens=True)
+    if sampled:
+        params = SamplingParams(max_tokens=steps + warmup + 8, bypass_stop_tokens=True, seed=7)
+    else:
+        params = SamplingParams.greedy(max_tokens=steps + warmup + 8, bypass_stop_tokens=True)
     ids = [f"d{i}" for i in range(batch)]
     # the requests enter as if their contexts had been run: random keys and values, and one generated token
     fill_context(engine, ids, start_len)
@@ -357,6 +362,8 @@ def main() -> int:
                     help="run fewer layers than the model has (recorded in the config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--sampled", action="store_true",
+                    help="the timed steps draw with the reference's default sampling parameters instead of the arg max (for profiles)")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="length of the prompt of the prefill")
     ap.add_argument("--runs", type=int, default=5, help="times the decode steps and the prefill are measured (mean and deviation)")
@@ -424,14 +431,14 @@ def main() -> int:
         print(json.dumps({"prefill": prefill_record(args.prefill_tokens, max(1, args.steps))}))
         return 0
     note(f"decode at batch {args.batch}, context {args.context}: {args.warmup} + {args.steps} steps, {args.runs} times")
-    elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run)
+    elapsed, mean_ctx = time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run, args.sampled)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
     nbytes = decode_bytes(raw, args.batch, mean_ctx, esize)
     achieved = nbytes / (elapsed / args.steps) / 1e9
     # the same K steps again, for the spread (the reference's bench: warm-up, then runs, mean and standard
     # deviation, inferrs/src/bench.rs:159-173,226-248); the headline stays the first K steps
-    repeats = [ms_per_step] + [time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run)[0]
+    repeats = [ms_per_step] + [time_decode(engine, args.batch, args.context, args.steps, args.warmup, args.decode_run, args.sampled)[0]
                                / args.steps * 1e3 for _ in range(max(0, args.runs - 1))]
     rep_mean, rep_std = mean_std(repeats)
 
@@ -462,10 +469,10 @@ def main() -> int:
         record["roofline"]["frac_of_measured"] = round(achieved / read_gbs, 4)
         points = {}
 
-        def decode_point(name: str, b: int, context: int):
+        def decode_point(name: str, b: int, context: int, sampled: bool = False):
             steps = max(8, args.steps // 2)
-            note(f"decode at batch {b}, context {context}: {steps} steps")
-            el, ctx_mean = time_decode(engine, b, context, steps, min(args.warmup, 4), args.decode_run)
+            note(f"decode at batch {b}, context {context}: {steps} steps" + (", default sampling parameters" if sampled else ""))
+            el, ctx_mean = time_decode(engine, b, context, steps, min(args.warmup, 4), args.decode_run, sampled)
             points[name] = round(b * steps / el, 2)
             fractions[name] = round(decode_bytes(raw, b, ctx_mean, esize) / (el / steps) / 1e9 / PEAK_HBM_GBS, 4)
 
@@ -504,6 +511,9 @@ def main() -> int:
                 if context < args.context:
                     for b in sorted(set([1, args.batch] + ([64] if 64 in points_batches else []))):
                         decode_point(f"decode_b{b}_ctx{context}", b, context)
+            # the same steps when every request draws with the reference's default parameters instead of the arg max
+            if 2048 < args.context:
+                decode_point(f"decode_b{args.batch}_ctx2048_sampled", args.batch, 2048, sampled=True)
             for tokens in (128, 512):
                 if tokens < args.prefill_tokens:
                     rec = prefill_record(tokens, 3)
