@@ -54,7 +54,7 @@ __device__ __forceinline__ float ag_merge_value(float big, float a, float part, 
 
 // VEC: the head size and the page size are multiples of four, so that four neighbouring dimensions of a key and
 // four neighbouring keys of a value's dimension are fetched with one load.  HEADS: query heads of a group (1 to 4).
-template <typename T, bool VEC, int HEADS>
+template <typename T, bool VEC, int HEADS, bool AHEAD>
 __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     T* __restrict__ out,                 // [n, nq, d]
     const T* __restrict__ q,             // [n, nq, d]
@@ -111,18 +111,161 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     const int tile_first = seg * AG_SEG_TILES > lo / AG_TILE ? seg * AG_SEG_TILES : lo / AG_TILE;
     const int tile_last = seg * AG_SEG_TILES + AG_SEG_TILES - 1 < pos / AG_TILE ? seg * AG_SEG_TILES + AG_SEG_TILES - 1 : pos / AG_TILE;
 
+    // ---- the pieces of a tile's work (the same arithmetic in the same order whoever stages the operands) -----------
+    float s[HEADS], alpha[HEADS];
+    // scores: lane j against key j, chunk c of the dimensions from the stage
+    auto scores = [&](int c) {
+        const float* mine = stage + lane * AG_PITCH;
+#pragma unroll 4
+        for (int e4 = 0; e4 < AG_CHUNK / 4; ++e4) {
+            const float4 kv = *(const float4*)(mine + e4 * 4);
+#pragma unroll
+            for (int h = 0; h < HEADS; ++h) {
+                const float4 qv = *(const float4*)(sq + h * dpad + c * AG_CHUNK + e4 * 4);
+                s[h] = fmaf(qv.x, kv.x, s[h]);
+                s[h] = fmaf(qv.y, kv.y, s[h]);
+                s[h] = fmaf(qv.z, kv.z, s[h]);
+                s[h] = fmaf(qv.w, kv.w, s[h]);
+            }
+        }
+    };
+    // running maximum and sum; the tile's probabilities go to shared memory
+    auto softmax = [&](bool valid) {
+#pragma unroll
+        for (int h = 0; h < HEADS; ++h) {
+            const float sc = valid ? s[h] * scale : -INFINITY;
+            const float m_new = fmaxf(m[h], wave_max(sc));
+            const float p = valid ? expf(sc - m_new) : 0.f;
+            alpha[h] = expf(m[h] - m_new);
+            l[h] = l[h] * alpha[h] + wave_sum(p);
+            sp[h][lane] = p;
+            m[h] = m_new;
+        }
+    };
+    // values: lane e adds up dimension c * 64 + e over the tile's keys from the stage
+    auto values = [&](int c) {
+        const float* mine = stage + lane * AG_PITCH;
+        float o[HEADS];
+#pragma unroll
+        for (int h = 0; h < HEADS; ++h) o[h] = so[h * dpad + c * AG_CHUNK + lane] * alpha[h];
+#pragma unroll 4
+        for (int k4 = 0; k4 < AG_TILE / 4; ++k4) {
+            const float4 vv = *(const float4*)(mine + k4 * 4);
+#pragma unroll
+            for (int h = 0; h < HEADS; ++h) {
+                const float4 pv = *(const float4*)(&sp[h][k4 * 4]);
+                o[h] = fmaf(pv.x, vv.x, o[h]);
+                o[h] = fmaf(pv.y, vv.y, o[h]);
+                o[h] = fmaf(pv.z, vv.z, o[h]);
+                o[h] = fmaf(pv.w, vv.w, o[h]);
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < HEADS; ++h) so[h * dpad + c * AG_CHUNK + lane] = o[h];
+    };
+    // key j's page of a tile, in lane j - j0: asked for once a tile, handed round
+    auto tile_pages = [&](int tile) {
+        const int j = tile * AG_TILE + lane;
+        return (j >= lo && j <= pos) ? bt[j / page_size] : 0;
+    };
+
+    if constexpr (VEC && AHEAD) {
+        // Steps of few tokens, a wave a segment.  A tile is 2 * chunks steps: the chunks of its keys, then the chunks of
+        // its values.  A step's operands are asked for while the step before it is multiplied (a wave is alone in its
+        // block and mostly alone on its SIMD: nobody else would hide the memory's latency), held in registers meanwhile
+        // and put on the stage when it is free: a decode step of 8 requests at a context of 8,192 in 32-bit 220 -> 150 us
+        // a layer.  (Steps of many tokens have waves enough on every SIMD, and the registers that hold a step's operands
+        // would cost them a tenth of their speed.)
+        constexpr int LOADS = AG_TILE / 4;
+        static_assert(AG_TILE == AG_CHUNK, "a step of either kind is as many loads");
+        const int steps = 2 * chunks;
+        float4 held[LOADS];
+        // keys: a load instruction takes four keys' rows of the chunk, 16 lanes a row, four dimensions a lane;
+        // values: four dimensions, 16 lanes a dimension, four neighbouring keys a lane (four keys never straddle a page)
+        auto ask = [&](int tile, int step, int pages) {
+            const int j0 = tile * AG_TILE;
+            if (step < chunks) {
+                const int e = step * AG_CHUNK + (lane & 15) * 4;
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i) {
+                    const int r = 4 * i + (lane >> 4);
+                    const int key = j0 + r;
+                    const int page = __shfl(pages, r);
+                    held[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (key >= lo && key <= pos && e < d)
+                        held[i] = ag_load4(k_cache + (((size_t)page * nkv + kvh) * page_size + key % page_size) * d + e);
+                }
+            } else {
+                const int c = step - chunks;
+                const int k4 = (lane & 15) * 4;
+                const int key = j0 + k4;
+                const int off = key % page_size;
+                const bool any = key + 3 >= lo && key <= pos;
+                // the page of the four keys, from a lane whose key is in the range (a page that a window has passed is
+                // not in the table any more; the keys of these four that are in the range share their page)
+                const int first_in = key >= lo ? k4 : (lo - j0 < AG_TILE ? lo - j0 : k4);
+                const int page = __shfl(pages, first_in);
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i) {
+                    const int e = c * AG_CHUNK + 4 * i + (lane >> 4);
+                    held[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (any && e < d) held[i] = ag_load4(v_cache + (((size_t)page * nkv + kvh) * d + e) * page_size + off);
+                }
+            }
+        };
+        // what was asked for goes on the stage; values of keys outside the token's range as zeros
+        auto put = [&](int tile, int step) {
+            if (step < chunks) {
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i)
+                    *(float4*)(stage + (4 * i + (lane >> 4)) * AG_PITCH + (lane & 15) * 4) = held[i];
+            } else {
+                const int k4 = (lane & 15) * 4;
+                const int key = tile * AG_TILE + k4;
+                const bool in0 = key >= lo && key <= pos, in1 = key + 1 >= lo && key + 1 <= pos;
+                const bool in2 = key + 2 >= lo && key + 2 <= pos, in3 = key + 3 >= lo && key + 3 <= pos;
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i) {
+                    float4 v = held[i];
+                    v.x = in0 ? v.x : 0.f;
+                    v.y = in1 ? v.y : 0.f;
+                    v.z = in2 ? v.z : 0.f;
+                    v.w = in3 ? v.w : 0.f;
+                    *(float4*)(stage + (4 * i + (lane >> 4)) * AG_PITCH + k4) = v;
+                }
+            }
+        };
+        int pages = tile_pages(tile_first);
+        if (tile_first <= tile_last) ask(tile_first, 0, pages);
+        for (int tile = tile_first; tile <= tile_last; ++tile) {
+            const int j = tile * AG_TILE + lane;
+            const bool valid = j >= lo && j <= pos;
+            const int pages_next = tile < tile_last ? tile_pages(tile + 1) : 0;
+#pragma unroll
+            for (int h = 0; h < HEADS; ++h) s[h] = 0.f;
+            for (int step = 0; step < steps; ++step) {
+                if (step == chunks) softmax(valid);
+                __syncthreads();                                      // the stage is free (and the probabilities are there)
+                put(tile, step);
+                if (step + 1 < steps) ask(tile, step + 1, pages);
+                else if (tile < tile_last) ask(tile + 1, 0, pages_next);
+                __syncthreads();
+                if (step < chunks) scores(step);
+                else values(step - chunks);
+            }
+            pages = pages_next;
+        }
+    } else {
     for (int tile = tile_first; tile <= tile_last; ++tile) {
         const int j0 = tile * AG_TILE;
         const int j = j0 + lane;
         const bool valid = j >= lo && j <= pos;
-        const int my_page = valid ? bt[j / page_size] : 0;            // key j's page: asked for once a tile, handed round
-        // ---- scores: lane j against key j ------------------------------------------------------------------
-        float s[HEADS];
+        const int my_page = tile_pages(tile);
 #pragma unroll
         for (int h = 0; h < HEADS; ++h) s[h] = 0.f;
         for (int c = 0; c < chunks; ++c) {
             __syncthreads();                                          // the stage is free
-            if (VEC) {
+            if constexpr (VEC) {
                 // a load instruction takes four keys' rows of this chunk: 16 lanes a row, four dimensions a lane
                 const int e = c * AG_CHUNK + (lane & 15) * 4;
                 float4 v[AG_TILE / 4];
@@ -149,36 +292,12 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
                 }
             }
             __syncthreads();
-            const float* mine = stage + lane * AG_PITCH;
-#pragma unroll 4
-            for (int e4 = 0; e4 < AG_CHUNK / 4; ++e4) {
-                const float4 kv = *(const float4*)(mine + e4 * 4);
-#pragma unroll
-                for (int h = 0; h < HEADS; ++h) {
-                    const float4 qv = *(const float4*)(sq + h * dpad + c * AG_CHUNK + e4 * 4);
-                    s[h] = fmaf(qv.x, kv.x, s[h]);
-                    s[h] = fmaf(qv.y, kv.y, s[h]);
-                    s[h] = fmaf(qv.z, kv.z, s[h]);
-                    s[h] = fmaf(qv.w, kv.w, s[h]);
-                }
-            }
+            scores(c);
         }
-        // ---- running maximum and sum --------------------------------------------------------------------------
-        float alpha[HEADS];
-#pragma unroll
-        for (int h = 0; h < HEADS; ++h) {
-            const float sc = valid ? s[h] * scale : -INFINITY;
-            const float m_new = fmaxf(m[h], wave_max(sc));
-            const float p = valid ? expf(sc - m_new) : 0.f;
-            alpha[h] = expf(m[h] - m_new);
-            l[h] = l[h] * alpha[h] + wave_sum(p);
-            sp[h][lane] = p;
-            m[h] = m_new;
-        }
-        // ---- values: lane e adds up dimension c * 64 + e over the tile's keys ------------------------------------
+        softmax(valid);
         for (int c = 0; c < chunks; ++c) {
             __syncthreads();                                          // the stage is free, the probabilities are there
-            if (VEC) {
+            if constexpr (VEC) {
                 // a load instruction takes four dimensions: 16 lanes a dimension, four neighbouring keys a lane
                 const int k4 = (lane & 15) * 4;
                 const int key = j0 + k4;
@@ -213,25 +332,9 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
                 }
             }
             __syncthreads();
-            const float* mine = stage + lane * AG_PITCH;
-            float o[HEADS];
-#pragma unroll
-            for (int h = 0; h < HEADS; ++h) o[h] = so[h * dpad + c * AG_CHUNK + lane] * alpha[h];
-#pragma unroll 4
-            for (int k4 = 0; k4 < AG_TILE / 4; ++k4) {
-                const float4 vv = *(const float4*)(mine + k4 * 4);
-#pragma unroll
-                for (int h = 0; h < HEADS; ++h) {
-                    const float4 pv = *(const float4*)(&sp[h][k4 * 4]);
-                    o[h] = fmaf(pv.x, vv.x, o[h]);
-                    o[h] = fmaf(pv.y, vv.y, o[h]);
-                    o[h] = fmaf(pv.z, vv.z, o[h]);
-                    o[h] = fmaf(pv.w, vv.w, o[h]);
-                }
-            }
-#pragma unroll
-            for (int h = 0; h < HEADS; ++h) so[h * dpad + c * AG_CHUNK + lane] = o[h];
+            values(c);
         }
+    }
     }
     // ---- the segment is done ---------------------------------------------------------------------------------------
     if (only_seg >= 0) {
@@ -338,9 +441,12 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     // loads of four elements: rows of the caches start at multiples of four elements, on aligned arrays
     const bool vec = d % 4 == 0 && page_size % 4 == 0 &&
                      (((uintptr_t)k_cache | (uintptr_t)v_cache) % (4 * elem)) == 0;
-#define AG_LAUNCH(T, V, H) attn_generic_kernel<T, V, H><<<grid, IA_WAVE, rows_bytes, stream>>>( \
-        (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, positions, token_seq, block_table, max_pages, nq, nkv, \
-        d, page_size, window, scale, workspace, segs)
+#define AG_ARGS(T) (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, positions, token_seq, block_table, max_pages, nq, nkv, \
+        d, page_size, window, scale, workspace, segs
+    // (a wave a segment, steps of few tokens: the operands are asked for a step ahead)
+#define AG_LAUNCH(T, V, H) do { \
+        if (V && workspace != nullptr) attn_generic_kernel<T, V, H, true><<<grid, IA_WAVE, rows_bytes, stream>>>(AG_ARGS(T)); \
+        else attn_generic_kernel<T, V, H, false><<<grid, IA_WAVE, rows_bytes, stream>>>(AG_ARGS(T)); } while (0)
 #define AG_HEADS_OF(T, V) do { \
         if (per_group == 1) AG_LAUNCH(T, V, 1); else if (per_group == 2) AG_LAUNCH(T, V, 2); \
         else if (per_group == 3) AG_LAUNCH(T, V, 3); else AG_LAUNCH(T, V, 4); } while (0)
@@ -349,6 +455,7 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     else IA_CHECK(false, "attention: unknown dtype %d", dtype);
 #undef AG_HEADS_OF
 #undef AG_LAUNCH
+#undef AG_ARGS
     IA_LAUNCH_CHECK("attention_generic");
     if (workspace != nullptr) {
         if (dtype == IA_F32)
