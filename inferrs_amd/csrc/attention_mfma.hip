@@ -963,11 +963,13 @@ __device__ __forceinline__ void lds_load16(const char* from, uint32_t lds_at) {
 // 8,192 tokens where two waves a SIMD run at 730, and the rescaling of accumulators that live in the matrix cores' own
 // registers cost as much again.)
 #define TILE_NBW 2
-template <bool ENABLED = (HD == 128)>
+// NBW_: column tiles of 16 a wave.  One instead of two halves a block's columns (64) and doubles the blocks: for steps
+// whose blocks of 128 columns would leave compute units without one (short prompts, few heads).
+template <bool ENABLED = (HD == 128), int NBW_ = TILE_NBW>
 __global__ __launch_bounds__(TILE_GROUPS * TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_tile_kernel(const AttnParams p) {
     if constexpr (ENABLED) {
-        constexpr int NBW = TILE_NBW;
+        constexpr int NBW = NBW_;
         constexpr int WAVE_COLS = 16 * NBW;
         constexpr int TILE_COLS = TILE_WAVES * WAVE_COLS;
         // Two stages for each group.  The loads that fill them are written as instructions of their own below
@@ -1247,6 +1249,20 @@ void attn_tile_kernel(const AttnParams p) {
             auto step = [&](auto edge_c, int u) {
                 const int k0 = kb + 32 * u;
                 uint4 vop[DB];
+                if constexpr (NBW == 1) {
+                    // one column tile: nothing of its own to lay beside the softmax (the SIMD's other wave is)
+                    f32x4 s0[2];
+                    uint4 pb0;
+                    float alpha0;
+                    scores(0, s0);
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HD * 2) + db * 512 + v_at);
+                    softmax(edge_c, 0, k0, s0, pb0, alpha0);
+                    if (u == 0) read_keys(1);
+                    rescale(0, alpha0);
+                    weighted(0, vop, pb0);
+                } else {
                 f32x4 s0[2], s1[2];
                 uint4 pb0, pb1;
                 float alpha0, alpha1;
@@ -1270,6 +1286,7 @@ void attn_tile_kernel(const AttnParams p) {
                 __builtin_amdgcn_sched_barrier(0);
                 rescale(1, alpha1);
                 weighted(1, vop, pb1);
+                }
             };
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
@@ -1365,8 +1382,21 @@ void attn_tile_kernel(const AttnParams p) {
 }
 
 static int g_tiles = 1;
-// Measurement switch: 0 keeps prompt portions on the kernel of single waves.
+// Measurement switch: 0 keeps prompt portions on the kernel of single waves; 2: blocks of 64 columns whatever the
+// step's size; 3: of 128.
 extern "C" void ia_attention_mfma_tiles(int on) { g_tiles = on; }
+
+// Compute units of the current device (asked for once a device).
+static int attn_cus() {
+    static int cus[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        cus[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
+    }
+    return cus[dev];
+}
 
 // Merges the partial results of the key splits of one (token, head): one block a row.  The
 // partial results were written by other compute units, so every read is a long way off: the
@@ -1589,12 +1619,24 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         return 0;
     } else if (HD == 128 && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
-        const int tile_cols = 16 * TILE_NBW * TILE_WAVES;
+        // Blocks of 128 columns; of 64 (twice as many, the same bits) where the keys are not split and the blocks of 128
+        // would be half a compute unit's worth or less, or, under a causal mask over most of the context, where the
+        // blocks' walks differ in length, one a compute unit or less.  Measured, 32 query and 8 key/value heads, whole
+        // prompts: 512 tokens 17.8 -> 15.1 us, 1,024 tokens (256 blocks) 28.2 -> 24.5, 2,048 tokens (512 blocks) 55.8 -> 69.7
+        // (not taken); 16 query heads: 1,024 tokens 25.8 -> 18.2, 2,048 tokens 44.4 -> 36.3; a portion of 512 tokens at a
+        // context of 2,048: 42.3 -> 29.7 (36.8 with the keys split in two), with 40 query heads (160 blocks) 43.0 -> 47.9 (not taken).
+        const long long tiles128 = (cols + 16 * TILE_NBW * TILE_WAVES - 1) / (16 * TILE_NBW * TILE_WAVES);
+        const long long blocks128 = tiles128 * nkv * n_seqs;
+        const bool causal_most = 2LL * max_q_len > max_kv_len;
+        const bool narrow = g_tiles == 2 || (g_tiles == 1 && splits == 1 &&
+                                             blocks128 <= (causal_most ? attn_cus() : attn_cus() / 2));
+        const int tile_cols = 16 * (narrow ? 1 : TILE_NBW) * TILE_WAVES;
         const long long tiles = (cols + tile_cols - 1) / tile_cols;
         IA_CHECK(tiles <= 65535, "attention_mfma: %lld tiles of columns in a request (at most 65535)", tiles);
         const dim3 tgrid((unsigned)(nkv * splits * n_seqs), (unsigned)tiles, 1);
         p.pair = 0;
-        attn_tile_kernel<><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
+        if (narrow) attn_tile_kernel<(HD == 128), 1><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
+        else attn_tile_kernel<><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
     } else if (nb == 1) {
         attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
     } else {

@@ -350,6 +350,7 @@ def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int) -> bool:
 ATTN_TILE_COLS = 128           # head size 128, prompt portions: columns a block of four waves
 ATTN_TILE_BLOCKS = 256         # blocks wanted (one a compute unit: eight waves) before the keys stop being split
 ATTN_TILE_MIN_CHUNK = 512      # fewest keys a block's share is worth (eight stages of 64)
+ATTN_TILE_WHOLE_UP_TO = 2048   # contexts up to this length are not split
 
 
 def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: int, d: int = 0) -> Tuple[int, int]:
@@ -357,11 +358,13 @@ def attention_split(n_seqs: int, nkv: int, g: int, max_q_len: int, max_kv_len: i
     when the batch alone has too few (request, kv head, column block) items to fill the chip."""
     cols = max_q_len * g
     if d == 128 and cols >= ATTN_TILE_COLS:
-        if 2 * max_q_len > max_kv_len:
+        if 2 * max_q_len > max_kv_len or max_kv_len <= ATTN_TILE_WHOLE_UP_TO:
             # whole prompts and portions that span most of their context: a block's walk ends at its own tokens, so
             # the later splits of the early blocks are empty and the partial sums of every row go through memory for
             # nothing (16 query and 8 key/value heads, 1,024 tokens, 128 blocks: 25.6 us whole against 28.2 in two
-            # splits; 2,048 tokens 44 against 63; 32 query heads, 512 tokens 18 against 26)
+            # splits; 2,048 tokens 44 against 63; 32 query heads, 512 tokens 18 against 26); short contexts likewise: the
+            # walks are short, and where the blocks are few the kernel halves them instead (a portion of 512 tokens at
+            # a context of 2,048, 32 query heads: 29.7 us whole in blocks of 64 columns against 36.8 in two splits)
             return 1, -(-max_kv_len // 64) * 64
         items = n_seqs * nkv * -(-cols // ATTN_TILE_COLS)
         splits = 1

@@ -368,6 +368,23 @@ def test_attention_mfma_prompt_portions_head_size_128(nq, nkv, page, window, len
         lib.ia_attention_mfma_tiles(1)
     close(single, want, 2 ** -7, "single waves")
     close(got, single.float().cpu(), 2 ** -7, "the two kernels")
+    # blocks of 64 columns and of 128 (the launch picks by the step's size; here each is forced): a column's keys are
+    # walked in the same order with the same arithmetic, so the bits are the same, with the keys split as well.  (Under a
+    # window a block's walk begins at the first stage that any of its columns sees, and which of the block's two
+    # groups of waves takes a stage follows from there: another width of block, another pairing, the same sums in
+    # another order.)
+    for splits in (1, 2, 3):
+        outs = []
+        for columns in (2, 3):
+            lib.ia_attention_mfma_tiles(columns)
+            try:
+                outs.append(ops.attention_mfma(*args, **dict(kw, splits=splits)))
+            finally:
+                lib.ia_attention_mfma_tiles(1)
+        if window is None:
+            assert torch.equal(outs[0], outs[1]), f"blocks of 64 and of 128 columns, splits={splits}"
+        close(outs[1], want, 2 ** -7, f"blocks of 128 columns, splits={splits}")
+        close(outs[0], want, 2 ** -7, f"blocks of 64 columns, splits={splits}")
 
 
 def test_attention_mfma_prompt_that_half_fills_the_chip():
