@@ -1,0 +1,112 @@
+"""The engine at the layer sizes of a real model (Qwen3-8B: width 4,096, 32 query and 8 key/value heads of 128,
+feed-forward 12,288; two layers and a vocabulary of 40,000 so that the plain implementation stays quick) against the
+plain implementation in 64-bit.  The tiny configurations reach every code path; this one runs the shapes that the
+size rules of the kernels pick at these widths (the skinny products with the stream inside up to 8 rows, the
+products of 9 to 128 rows with their split sums, the vendor's products beyond, [gate; up] on 256 blocks, the decode
+attention's splits, the tiled prompt attention, the 32-bit products' block shapes), whole steps of them together.
+
+Tolerances as in the replay tests: 32-bit 1e-5 of the largest logit; bfloat16 the bound measured on this model (the
+plain implementation in bfloat16 tensor arithmetic against itself in 64-bit)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+from tiny_configs import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+RAW = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=40000, hidden_size=4096,
+           intermediate_size=12288, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+           rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
+PROMPT, DECODED = 300, 24          # one long request: its prompt whole, then token by token
+CROWD, CROWD_PROMPT = 24, 30       # many short requests: their prompts in one step, then decoded together
+
+
+@pytest.fixture(scope="module")
+def real(tmp_path_factory):
+    """The model's folder (weights drawn on the GPU: the host's generator takes minutes at this size), the requests
+    and their 64-bit logits."""
+    from inferrs_amd.config import Qwen3Config
+    from inferrs_amd.parts import generated_tensors
+    from inferrs_amd.weights import random_tensors, write_safetensors
+    folder = str(tmp_path_factory.mktemp("real_sizes"))
+    config = Qwen3Config.from_dict(RAW)
+    tensors = random_tensors(generated_tensors(config.to_spec()), 3, torch.bfloat16, device="cuda:0")
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(config.to_dict(), f)
+    write_safetensors(os.path.join(folder, "model.safetensors"), {k: v.cpu() for k, v in tensors.items()})
+    del tensors
+    torch.cuda.empty_cache()
+    cfg, params = pm.read_model(folder, torch.float64)
+    reqs = {"long": random_tokens(PROMPT + DECODED, RAW["vocab_size"], 50)}
+    for i in range(CROWD):
+        reqs[f"c{i}"] = random_tokens(CROWD_PROMPT + 3 * i % 7 + 12, RAW["vocab_size"], 60 + i)
+    ref = {r: pm.forward(cfg, params, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    del params
+    cfg16, p16 = pm.read_model(folder, torch.bfloat16)
+    rounded = pm.forward(cfg16, p16, reqs["long"]).float().numpy()
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    bf16_bound = float(np.abs(rounded - ref["long"]).max()) / scale
+    return folder, reqs, ref, scale, bf16_bound
+
+
+def run(folder, reqs, dtype):
+    """{request: {position: logits}} of the long request (prompt whole, then single tokens) and of the crowd (prompts
+    in one step, then decode steps of 24, 12 and 8 requests), the next token always the request's own next one."""
+    from inferrs_amd.engine import Engine, Entry
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=CROWD + 2)
+    got = {r: {} for r in reqs}
+    toks = reqs["long"]
+    got["long"][PROMPT - 1] = eng.step([Entry("long", toks[:PROMPT], [PROMPT - 1])])[0].cpu().numpy()
+    for p in range(PROMPT, PROMPT + DECODED):
+        got["long"][p] = eng.step([Entry("long", [toks[p]], [0])])[0].cpu().numpy()
+    eng.end_request("long")
+    crowd = [r for r in reqs if r != "long"]
+    rows = eng.step([Entry(r, reqs[r][:CROWD_PROMPT], [CROWD_PROMPT - 1]) for r in crowd]).cpu().numpy()
+    for r, row in zip(crowd, rows):
+        got[r][CROWD_PROMPT - 1] = row
+    at = {r: CROWD_PROMPT for r in crowd}
+    live = list(crowd)
+    for step in range(12):
+        live = [r for r in live if at[r] < len(reqs[r])]
+        if step == 4:
+            for r in live[12:]:
+                eng.end_request(r)
+            live = live[:12]
+        if step == 8:
+            for r in live[8:]:
+                eng.end_request(r)
+            live = live[:8]
+        if not live:
+            break
+        rows = eng.step([Entry(r, [reqs[r][at[r]]], [0]) for r in live]).cpu().numpy()
+        for r, row in zip(live, rows):
+            got[r][at[r]] = row
+            at[r] += 1
+    return got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_layer_sizes_match_plain(real, dtype):
+    folder, reqs, ref, scale, bf16_bound = real
+    got = run(folder, reqs, dtype)
+    allowed = 1e-5 if dtype == "float32" else bf16_bound
+    assert sum(len(v) for v in got.values()) >= 1 + DECODED + CROWD + 4 * CROWD + 4 * 12 - 40
+    worst, where = 0.0, None
+    for r, rows in got.items():
+        for p, row in rows.items():
+            e = float(np.abs(row - ref[r][p]).max()) / scale
+            if not e <= worst:
+                worst, where = e, (r, p)
+    print(f"real layer sizes, {dtype}: worst difference {worst:.3e} of the largest logit ({scale:.2f}) at {where}, allowed {allowed:.3e}")
+    assert worst <= allowed, f"{dtype}: {worst:.3e} of the largest logit at {where} (allowed {allowed:.3e})"
+    # and the greedy choice agrees wherever the plain model's first two candidates are further apart than the bound
+    for r, rows in got.items():
+        for p, row in rows.items():
+            top2 = np.sort(ref[r][p])[-2:]
+            if top2[1] - top2[0] > 2 * allowed * scale:
+                assert int(np.argmax(row)) == int(np.argmax(ref[r][p])), (r, p)
