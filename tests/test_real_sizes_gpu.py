@@ -1,5 +1,6 @@
-"""The engine at the layer sizes of a real model (Qwen3-8B: width 4,096, 32 query and 8 key/value heads of 128,
-feed-forward 12,288; two layers and a vocabulary of 40,000 so that the plain implementation stays quick) against the
+"""The engine at the layer sizes of real models (Qwen3-8B: width 4,096, 32 query and 8 key/value heads of 128,
+feed-forward 12,288; Qwen3-14B: width 5,120, 40 query heads, feed-forward 17,408, a width that is no power of two;
+two layers each and a vocabulary of 40,000 so that the plain implementation stays quick) against the
 plain implementation in 64-bit.  The tiny configurations reach every code path; this one runs the shapes that the
 size rules of the kernels pick at these widths (the skinny products with the stream inside up to 8 rows, the
 products of 9 to 128 rows with their split sums, the vendor's products beyond, [gate; up] on 256 blocks, the decode
@@ -22,19 +23,20 @@ pytestmark = pytest.mark.gpu
 RAW = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=40000, hidden_size=4096,
            intermediate_size=12288, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
            rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
+SHAPES = {"8B": RAW, "14B": dict(RAW, hidden_size=5120, intermediate_size=17408, num_attention_heads=40)}
 PROMPT, DECODED = 300, 24          # one long request: its prompt whole, then token by token
 CROWD, CROWD_PROMPT = 24, 30       # many short requests: their prompts in one step, then decoded together
 
 
-@pytest.fixture(scope="module")
-def real(tmp_path_factory):
+@pytest.fixture(scope="module", params=sorted(SHAPES))
+def real(request, tmp_path_factory):
     """The model's folder (weights drawn on the GPU: the host's generator takes minutes at this size), the requests
     and their 64-bit logits."""
     from inferrs_amd.config import Qwen3Config
     from inferrs_amd.parts import generated_tensors
     from inferrs_amd.weights import random_tensors, write_safetensors
     folder = str(tmp_path_factory.mktemp("real_sizes"))
-    config = Qwen3Config.from_dict(RAW)
+    config = Qwen3Config.from_dict(SHAPES[request.param])
     tensors = random_tensors(generated_tensors(config.to_spec()), 3, torch.bfloat16, device="cuda:0")
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(config.to_dict(), f)
