@@ -1,7 +1,8 @@
 """The engine at the layer sizes of real models (Qwen3-8B: width 4,096, 32 query and 8 key/value heads of 128,
 feed-forward 12,288; Qwen3-14B: width 5,120, 40 query heads, feed-forward 17,408, a width that is no power of two;
 two layers each and a vocabulary of 40,000 so that the plain implementation stays quick) against the
-plain implementation in 64-bit.  The tiny configurations reach every code path; this one runs the shapes that the
+plain implementation in 64-bit: a prompt of 300 tokens whole and then token by token, 24 short requests decoded together,
+and (8B sizes) a prompt of 2,600 tokens in portions of 1,024 with tokens decoded behind it.  The tiny configurations reach every code path; this one runs the shapes that the
 size rules of the kernels pick at these widths (the skinny products with the stream inside up to 8 rows, the
 products of 9 to 128 rows with their split sums, the vendor's products beyond, [gate; up] on 256 blocks, the decode
 attention's splits, the tiled prompt attention, the 32-bit products' block shapes), whole steps of them together.
@@ -26,6 +27,7 @@ RAW = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=40
 SHAPES = {"8B": RAW, "14B": dict(RAW, hidden_size=5120, intermediate_size=17408, num_attention_heads=40)}
 PROMPT, DECODED = 300, 24          # one long request: its prompt whole, then token by token
 CROWD, CROWD_PROMPT = 24, 30       # many short requests: their prompts in one step, then decoded together
+FAR, FAR_PORTION, FAR_DECODED = 2600, 1024, 6     # a request with a context of thousands: its prompt in portions, then token by token
 
 
 @pytest.fixture(scope="module", params=sorted(SHAPES))
@@ -47,11 +49,22 @@ def real(request, tmp_path_factory):
     reqs = {"long": random_tokens(PROMPT + DECODED, RAW["vocab_size"], 50)}
     for i in range(CROWD):
         reqs[f"c{i}"] = random_tokens(CROWD_PROMPT + 3 * i % 7 + 12, RAW["vocab_size"], 60 + i)
-    ref = {r: pm.forward(cfg, params, t).numpy().astype(np.float32) for r, t in reqs.items()}
+    if request.param == "8B":
+        reqs["far"] = random_tokens(FAR + FAR_DECODED, RAW["vocab_size"], 51)
+    ref = {}
+    for r, t in reqs.items():
+        full = pm.forward(cfg, params, t)
+        if r == "far":            # (only the rows that the engine is asked for: the others would be 400 MB)
+            keep = sorted({lo for lo in range(0, FAR, FAR_PORTION)} | {min(FAR, lo + FAR_PORTION) - 1 for lo in range(0, FAR, FAR_PORTION)}
+                          | set(range(FAR, FAR + FAR_DECODED)))
+            ref[r] = {p: full[p].numpy().astype(np.float32) for p in keep}
+        else:
+            ref[r] = full.numpy().astype(np.float32)
+        del full
     del params
     cfg16, p16 = pm.read_model(folder, torch.bfloat16)
     rounded = pm.forward(cfg16, p16, reqs["long"]).float().numpy()
-    scale = max(float(np.abs(v).max()) for v in ref.values())
+    scale = max(float(np.abs(v).max()) for r, v in ref.items() if r != "far")
     bf16_bound = float(np.abs(rounded - ref["long"]).max()) / scale
     return folder, reqs, ref, scale, bf16_bound
 
@@ -60,14 +73,23 @@ def run(folder, reqs, dtype):
     """{request: {position: logits}} of the long request (prompt whole, then single tokens) and of the crowd (prompts
     in one step, then decode steps of 24, 12 and 8 requests), the next token always the request's own next one."""
     from inferrs_amd.engine import Engine, Entry
-    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=CROWD + 2)
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=200, max_seqs=CROWD + 2)
     got = {r: {} for r in reqs}
+    if "far" in reqs:
+        toks = reqs["far"]
+        for lo in range(0, FAR, FAR_PORTION):
+            hi = min(FAR, lo + FAR_PORTION)
+            rows = eng.step([Entry("far", toks[lo:hi], [0, hi - lo - 1])]).cpu().numpy()      # a portion's first and last token
+            got["far"][lo], got["far"][hi - 1] = rows[0], rows[1]
+        for p in range(FAR, FAR + FAR_DECODED):
+            got["far"][p] = eng.step([Entry("far", [toks[p]], [0])])[0].cpu().numpy()
+        eng.end_request("far")
     toks = reqs["long"]
     got["long"][PROMPT - 1] = eng.step([Entry("long", toks[:PROMPT], [PROMPT - 1])])[0].cpu().numpy()
     for p in range(PROMPT, PROMPT + DECODED):
         got["long"][p] = eng.step([Entry("long", [toks[p]], [0])])[0].cpu().numpy()
     eng.end_request("long")
-    crowd = [r for r in reqs if r != "long"]
+    crowd = [r for r in reqs if r.startswith("c")]
     rows = eng.step([Entry(r, reqs[r][:CROWD_PROMPT], [CROWD_PROMPT - 1]) for r in crowd]).cpu().numpy()
     for r, row in zip(crowd, rows):
         got[r][CROWD_PROMPT - 1] = row
