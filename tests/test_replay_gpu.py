@@ -180,6 +180,39 @@ def test_trace_run_program(models, tmp_path, dtype):
     assert err <= bound(folder, reqs, ref, dtype), f"{err:.3e} at {where}"
 
 
+def test_trace_run_reads_a_config_as_the_reference_does(models, tmp_path):
+    """The reference reads `attention_bias`, `use_sliding_window`, `hidden_act` and `rope_scaling` without acting on
+    them (inferrs-models/src/config.rs:291-292, 468-502).  The engine's entry points refuse such values; the replay
+    program, whose logits are compared with the reference's formulas, ignores them too, says so, and writes the logits
+    of the same folder without those keys."""
+    import json
+    import shutil
+    folder, raw, reqs, ref = pick(models, "A", False, "float32")
+    odd = str(tmp_path / "odd")
+    shutil.copytree(folder, odd)
+    with open(os.path.join(odd, "config.json")) as f:
+        config = json.load(f)
+    config.update(attention_bias=True, use_sliding_window=True, sliding_window=8, hidden_act="gelu",
+                  rope_scaling={"rope_type": "linear", "factor": 2.0})
+    with open(os.path.join(odd, "config.json"), "w") as f:
+        json.dump(config, f)
+    from inferrs_amd.config import ConfigError
+    from inferrs_amd.engine import Engine
+    with pytest.raises(ConfigError, match="use_sliding_window"):
+        Engine.from_folder(odd, dtype="float32", page_size=4, num_pages=8, max_seqs=1)
+    some = {k: reqs[k] for k in ("r3", "r4")}
+    trace = tm.whole(some)
+    out_dir = str(tmp_path / "out")
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", odd, "--dtype", "float32",
+         "--out", out_dir, "--max-tokens", str(trace.max_tokens)],
+        input=trace.text(), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "ignored here as well" in proc.stderr and "hidden_act = 'gelu'" in proc.stderr
+    err, where = worst(trace.read(out_dir, raw["vocab_size"]), ref, some)
+    assert err <= TOL_PLAIN_F32, f"{err:.3e} at {where}"
+
+
 def test_out_of_pages_is_an_error_and_takes_nothing(models):
     from inferrs_amd.cache import OutOfPages
     from inferrs_amd.engine import Engine, Entry
