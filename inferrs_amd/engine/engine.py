@@ -203,7 +203,8 @@ class Engine:
     def decode_chain(self, seq_ids: Sequence[Hashable], tokens: Sequence[int], steps: int,
                      pick=None) -> Optional[List[List[int]]]:
         """`steps` decode steps of the same requests, queued back to back: every step's choice
-        (the arg max, or `pick(logits, step, out)` writing int32 tokens into `out` on the device) is
+        (the arg max, or `pick(logits, step, out)` writing int32 tokens into `out` on the device; it may change `logits`, the
+        captured step's own buffer) is
         written on the device where the next step reads its token ids, so the host prepares and
         queues step i+1 while step i runs and waits once at the end.  The requests hold reserved
         pages for `steps` more tokens; nothing is committed here.  Returns the chosen tokens

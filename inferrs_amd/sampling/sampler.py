@@ -142,12 +142,13 @@ class ChainDraw:
                                 dtype=np.float32).reshape(steps, rows))
 
     def pick(self, logits: torch.Tensor, step: int, out: torch.Tensor) -> None:
-        """The tokens of the run's `step`-th step from its logits, into `out` (int32 [rows], on the device)."""
+        """The tokens of the run's `step`-th step from its logits, into `out` (int32 [rows], on the device).
+        The penalties are applied to `logits` in place: inside a run they are the captured step's own output buffer,
+        which the next step overwrites and nobody else reads."""
         if self.greedy:
             ops.argmax(logits, out=out)
             return
         if self.penalized:
-            logits = logits.clone()
             ops.penalize(logits, self.window, self.rep, self.freq, self.pres, self.bias_ids, self.bias_vals)
         out.copy_(ops.sample(logits, self.temperature, self.top_k, self.top_p, self.min_p, self.u[step]))
         if self.window is not None:
