@@ -2,7 +2,8 @@
 feed-forward 12,288; Qwen3-14B: width 5,120, 40 query heads, feed-forward 17,408, a width that is no power of two;
 two layers each and a vocabulary of 40,000 so that the plain implementation stays quick) against the
 plain implementation in 64-bit: a prompt of 300 tokens whole and then token by token, 24 short requests decoded together,
-and (8B sizes) a prompt of 2,600 tokens in portions of 1,024 with tokens decoded behind it.  The tiny configurations reach every code path; this one runs the shapes that the
+and (8B sizes) a prompt of 2,600 tokens in portions of 1,024 with tokens decoded behind it, and 40 tokens decoded from a
+context of 1,000 on.  The tiny configurations reach every code path; this one runs the shapes that the
 size rules of the kernels pick at these widths (the skinny products with the stream inside up to 8 rows, the
 products of 9 to 128 rows with their split sums, the vendor's products beyond, [gate; up] on 256 blocks, the decode
 attention's splits, the tiled prompt attention, the 32-bit products' block shapes), whole steps of them together.
@@ -28,6 +29,7 @@ SHAPES = {"8B": RAW, "14B": dict(RAW, hidden_size=5120, intermediate_size=17408,
 PROMPT, DECODED = 300, 24          # one long request: its prompt whole, then token by token
 CROWD, CROWD_PROMPT = 24, 30       # many short requests: their prompts in one step, then decoded together
 FAR, FAR_PORTION, FAR_DECODED = 2600, 1024, 6     # a request with a context of thousands: its prompt in portions, then token by token
+CROSS, CROSS_DECODED = 1000, 40    # a request whose decoded tokens pass a context of 1,024: another captured graph, another split of the keys
 
 
 @pytest.fixture(scope="module", params=sorted(SHAPES))
@@ -51,6 +53,7 @@ def real(request, tmp_path_factory):
         reqs[f"c{i}"] = random_tokens(CROWD_PROMPT + 3 * i % 7 + 12, RAW["vocab_size"], 60 + i)
     if request.param == "8B":
         reqs["far"] = random_tokens(FAR + FAR_DECODED, RAW["vocab_size"], 51)
+        reqs["cross"] = random_tokens(CROSS + CROSS_DECODED, RAW["vocab_size"], 52)
     ref = {}
     for r, t in reqs.items():
         full = pm.forward(cfg, params, t)
@@ -84,6 +87,11 @@ def run(folder, reqs, dtype):
         for p in range(FAR, FAR + FAR_DECODED):
             got["far"][p] = eng.step([Entry("far", [toks[p]], [0])])[0].cpu().numpy()
         eng.end_request("far")
+        toks = reqs["cross"]
+        got["cross"][CROSS - 1] = eng.step([Entry("cross", toks[:CROSS], [CROSS - 1])])[0].cpu().numpy()
+        for p in range(CROSS, CROSS + CROSS_DECODED):
+            got["cross"][p] = eng.step([Entry("cross", [toks[p]], [0])])[0].cpu().numpy()
+        eng.end_request("cross")
     toks = reqs["long"]
     got["long"][PROMPT - 1] = eng.step([Entry("long", toks[:PROMPT], [PROMPT - 1])])[0].cpu().numpy()
     for p in range(PROMPT, PROMPT + DECODED):
