@@ -59,6 +59,14 @@ int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, 
 int ia_gemm_rows_tune(int shape);
 int ia_gemm_skinny_bf16(void* out, const void* x, const void* w, const void* bias, int M, int N, int K,
                         int out_dtype, int dual, hipStream_t stream);
+// Large bfloat16 products through the vendor's library, hipBLASLt, called directly (vendor_gemm.hip).  ia_vendor_gemm_init
+// opens the library at `path` (the copy the process already holds) once; ia_vendor_gemm_bf16: out [M, N] = x [M, K] . w [N, K]^T,
+// contiguous, with `workspace_bytes` of device memory for kernels that want some.
+#define IA_VENDOR_NO_KERNEL 2     // ia_vendor_gemm_bf16: the library's search names no kernel for this shape
+int ia_vendor_gemm_init(const char* path);
+int ia_vendor_gemm_ready(void);
+int ia_vendor_gemm_bf16(void* out, const void* x, const void* w, int M, int N, int K, void* workspace,
+                        long long workspace_bytes, hipStream_t stream);
 // Large bfloat16 products in tiles of 256 x 256 (gemm_mfma.hip); K a multiple of 64; with `dual` w is [gate; up]
 // and out = act(x . gate^T) * (x . up^T).
 int ia_gemm_mfma_bf16(void* out, const void* x, const void* w, int M, int N, int K, int dual, hipStream_t stream);

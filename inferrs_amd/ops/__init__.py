@@ -106,6 +106,12 @@ def library(target: str = "core"):
     return lib if KernelTimer.active is None else _Timed(lib)
 
 
+def _raw_library(target: str = "core") -> ctypes.CDLL:
+    """The library without the timer around its entry points (for calls that a caller times under a name of its own)."""
+    library(target)
+    return _LIBS[target]
+
+
 def library_files() -> Dict[str, str]:
     """The libraries loaded so far: target -> file."""
     return dict(_LIB_PATHS)
@@ -124,7 +130,9 @@ def _check(code: int, target: str = "core") -> None:
 
 
 def _stream() -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # (the raw handle straight from the runtime: `torch.cuda.current_stream()` builds a Python object around it, 3 us
+    # a kernel call)
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
 
 
 def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
@@ -567,6 +575,75 @@ SKINNY_MAX_ROWS = 16
 LARGE_PRODUCTS = os.environ.get("INFERRS_AMD_LARGE_PRODUCTS", "library")
 
 
+# How the vendor's GEMM is called: "direct" (hipBLASLt through this package's own entry point, which keeps descriptors,
+# layouts and the library's choice of kernel for every shape: 7 us of host time a product) or "torch" (`F.linear`:
+# 18 us a product whatever its size, more than the GPU needs for the products of a small model).  "direct" falls back
+# to "torch", with a warning, where the library cannot be opened.
+VENDOR_GEMM = os.environ.get("INFERRS_AMD_VENDOR_GEMM", "direct")
+VENDOR_WORKSPACE_BYTES = 128 << 20
+_VENDOR_STATE: Dict[str, object] = {}
+
+
+def _vendor_library_path() -> Optional[str]:
+    """The hipBLASLt that this process has loaded (torch brings its own copy), else torch's, else the system's."""
+    try:
+        with open("/proc/self/maps") as f:
+            for line in f:
+                if "libhipblaslt.so" in line:
+                    return line.split(None, 5)[-1].strip()
+    except OSError:
+        pass
+    for path in (os.path.join(os.path.dirname(torch.__file__), "lib", "libhipblaslt.so"), "/opt/rocm/lib/libhipblaslt.so"):
+        if os.path.exists(path):
+            return path
+    return None
+
+
+def _vendor_direct() -> bool:
+    if VENDOR_GEMM not in ("direct", "torch"):
+        raise KernelError(f"INFERRS_AMD_VENDOR_GEMM / ops.VENDOR_GEMM: 'direct' or 'torch', not {VENDOR_GEMM!r}")
+    if VENDOR_GEMM == "torch":
+        return False
+    if "ready" not in _VENDOR_STATE:
+        path = _vendor_library_path()
+        lib = _raw_library()
+        ok = path is not None and lib.ia_vendor_gemm_init(path.encode()) == 0
+        if not ok:
+            import logging
+            logging.getLogger("inferrs_amd").warning(
+                "the vendor's GEMM library could not be opened directly (%s): its products go through torch",
+                lib.ia_last_error().decode() if path is not None else "libhipblaslt.so not found")
+        _VENDOR_STATE["ready"] = ok
+    return bool(_VENDOR_STATE["ready"])
+
+
+def vendor_gemm_bf16(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x [m, k] . w[n, k]^T in bfloat16 through the vendor's GEMM library."""
+    if not _vendor_direct() or x.shape[0] == 0:
+        return torch.nn.functional.linear(x, w)
+    _dev(x, w)
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"vendor_gemm: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)} {w.dtype}")
+    if not (x.is_contiguous() and w.is_contiguous()):
+        raise KernelError("vendor_gemm: operands must be contiguous")
+    key = ("workspace", x.device.index)
+    ws = _VENDOR_STATE.get(key)
+    if ws is None:
+        ws = _VENDOR_STATE[key] = torch.empty((VENDOR_WORKSPACE_BYTES,), dtype=torch.uint8, device=x.device)
+    refused = _VENDOR_STATE.setdefault("refused", set())
+    if (m, n, k) in refused:
+        return torch.nn.functional.linear(x, w)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    code = _raw_library().ia_vendor_gemm_bf16(_p(out), _p(x), _p(w), m, n, k, _p(ws), ws.numel(), _stream())
+    if code == 2:                                    # the library's search names no kernel for this shape (an odd k)
+        refused.add((m, n, k))
+        return torch.nn.functional.linear(x, w)
+    _check(code)
+    return out
+
+
 def _own_large(x: torch.Tensor, w: torch.Tensor) -> bool:
     if LARGE_PRODUCTS not in ("library", "own"):
         raise KernelError(f"INFERRS_AMD_LARGE_PRODUCTS / ops.LARGE_PRODUCTS: 'library' or 'own', not {LARGE_PRODUCTS!r}")
@@ -921,9 +998,9 @@ def _linear_no_bias(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, mi
     if _own_large(x, w):
         y = gemm_mfma_bf16(x, w)
     elif KernelTimer.active is not None:
-        y = KernelTimer.active.call("vendor_gemm", torch.nn.functional.linear, x, w)
+        y = KernelTimer.active.call("vendor_gemm", vendor_gemm_bf16, x, w)
     else:
-        y = torch.nn.functional.linear(x, w)
+        y = vendor_gemm_bf16(x, w)
     return widen(y) if out_dtype == torch.float32 else y
 
 

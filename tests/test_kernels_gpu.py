@@ -1083,3 +1083,20 @@ def test_few_row_product_of_the_32_bit_path_with_every_block_shape(dtype):
             if dtype == torch.float32:
                 assert torch.equal(y, many[:y.shape[0]]), (features, y.shape)
             close(y, x[:y.shape[0]].double() @ w.double().cpu().t(), tol(dtype, 2e-6), "few rows")
+
+
+@pytest.mark.parametrize("m,n,k", [(130, 72, 40), (512, 4096, 1024), (2048, 6144, 4096), (300, 1000, 136), (129, 64, 33), (1024, 1024, 3072)])
+def test_vendor_gemm_called_directly_is_the_product_that_torch_gets(m, n, k):
+    """The vendor's GEMM through this package's own entry point (descriptors and the library's choice of kernel kept
+    for every shape) against the exact product and against the same library through torch; a shape that the
+    library's search has no kernel for goes through torch and is remembered."""
+    from inferrs_amd import ops
+    x, w = randn(m, k, dtype=torch.bfloat16, seed=1), randn(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    assert ops.VENDOR_GEMM == "direct"
+    got = ops.vendor_gemm_bf16(dev(x), dev(w))
+    assert ops.library().ia_vendor_gemm_ready() == 1
+    again = ops.vendor_gemm_bf16(dev(x), dev(w))                    # the kept plan
+    assert torch.equal(got, again)
+    close(got, x.double() @ w.double().t(), 2 ** -7, "vendor's product")
+    through_torch = torch.nn.functional.linear(dev(x), dev(w))
+    close(got, through_torch.float().cpu(), 2 ** -7, "the two ways to the library")
