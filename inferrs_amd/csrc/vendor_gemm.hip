@@ -10,15 +10,23 @@
 // The library is the one that the process already holds (torch brings its own copy, with its kernels beside it):
 // it is opened by its path and its entry points are looked up by name, so nothing is linked against a second
 // copy.  Only the header's types are used at compile time.
+#include "common.h"
+#include "api.h"
+
+#if !__has_include(<hipblaslt/hipblaslt.h>)
+// (an installation without the library's header: its products go through torch, and the caller is told so)
+extern "C" int ia_vendor_gemm_init(const char*) { IA_CHECK(false, "vendor_gemm: built without the header of hipBLASLt"); }
+extern "C" int ia_vendor_gemm_ready(void) { return 0; }
+extern "C" int ia_vendor_gemm_bf16(void*, const void*, const void*, int, int, int, void*, long long, hipStream_t) {
+    IA_CHECK(false, "vendor_gemm: built without the header of hipBLASLt");
+}
+#else
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
 #include <cstdint>
 #include <mutex>
 #include <unordered_map>
-
-#include "common.h"
-#include "api.h"
 
 namespace {
 
@@ -140,3 +148,4 @@ extern "C" int ia_vendor_gemm_bf16(void* out, const void* x, const void* w, int 
     IA_CHECK(status == HIPBLAS_STATUS_SUCCESS, "vendor_gemm: hipblasLtMatmul failed for %d x %d x %d (status %d)", M, N, K, (int)status);
     return 0;
 }
+#endif
