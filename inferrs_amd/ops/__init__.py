@@ -82,6 +82,49 @@ class _Timed:
         return lambda *args: timer.call(name[3:], fn, *args)
 
 
+_C_TYPES = {"int": ctypes.c_int, "long long": ctypes.c_longlong, "unsigned long long": ctypes.c_ulonglong,
+            "float": ctypes.c_float, "double": ctypes.c_double, "hipStream_t": ctypes.c_void_p, "size_t": ctypes.c_size_t}
+_DECLARATIONS: Dict[str, Tuple[object, list]] = {}
+
+
+def _declarations() -> Dict[str, Tuple[object, list]]:
+    """Entry point -> (result type, argument types), read from the header that declares them (`csrc/api.h`): with the
+    types known, ctypes converts plain integers to pointers itself, and a call's arguments need no objects around them
+    (0.3 us each, a thousand a step)."""
+    if _DECLARATIONS:
+        return _DECLARATIONS
+    import re
+    with open(os.path.join(_build.CSRC, "api.h")) as f:
+        text = re.sub(r"//[^\n]*", "", f.read())
+
+    def ctype(decl: str):
+        decl = decl.strip()
+        if "*" in decl:
+            return ctypes.c_char_p if decl.replace("const", "").replace("*", "").split()[0] == "char" else ctypes.c_void_p
+        words = [w for w in decl.replace("const", "").split()]
+        for n in (3, 2, 1):                                 # the type's words, with or without a parameter's name behind them
+            for cut in (words[:n],):
+                if " ".join(cut) in _C_TYPES and len(words) - n <= 1:
+                    return _C_TYPES[" ".join(cut)]
+        raise KernelError(f"api.h: no ctypes type for {decl!r}")
+
+    for m in re.finditer(r"\b(int|long long|void|const char\s*\*)\s+(ia_\w+)\s*\(([^)]*)\)\s*;", text):
+        result, name, params = m.group(1), m.group(2), m.group(3).strip()
+        args = [] if params in ("", "void") else [ctype(a) for a in params.split(",")]
+        restype = None if result == "void" else (ctypes.c_char_p if "char" in result else _C_TYPES[result])
+        _DECLARATIONS[name] = (restype, args)
+    return _DECLARATIONS
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    for name, (restype, args) in _declarations().items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:                              # (an entry point of another library)
+            continue
+        fn.restype, fn.argtypes = restype, args
+
+
 def library(target: str = "core"):
     """A compiled kernel library; compiled on first use when no built one is found."""
     lib = _LIBS.get(target)
@@ -94,14 +137,7 @@ def library(target: str = "core"):
     lib.ia_last_error.restype = ctypes.c_char_p
     if lib.ia_abi_version() != 1:
         raise KernelError(f"{path}: unexpected ABI version {lib.ia_abi_version()}")
-    if target.startswith("attn_d"):
-        lib.ia_attention_mfma_workspace.restype = ctypes.c_longlong
-        lib.ia_attention_decode_workspace.restype = ctypes.c_longlong
-        lib.ia_attention_decode_counters.restype = ctypes.c_longlong
-    else:
-        lib.ia_sample_workspace.restype = ctypes.c_longlong
-        lib.ia_attention_generic_workspace.restype = ctypes.c_longlong
-        lib.ia_argmax_workspace.restype = ctypes.c_longlong
+    _declare(lib)
     _LIBS[target], _LIB_PATHS[target] = lib, path
     return lib if KernelTimer.active is None else _Timed(lib)
 
@@ -129,14 +165,15 @@ def _check(code: int, target: str = "core") -> None:
         raise KernelError(library(target).ia_last_error().decode("utf-8", "replace"))
 
 
-def _stream() -> ctypes.c_void_p:
+def _stream() -> int:
     # (the raw handle straight from the runtime: `torch.cuda.current_stream()` builds a Python object around it, 3 us
     # a kernel call)
-    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
-def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+def _p(t: Optional[torch.Tensor]) -> Optional[int]:
+    """A tensor's address as the entry points take it (their argument types are declared: see `_declarations`)."""
+    return None if t is None else t.data_ptr()
 
 
 def _dt(t: torch.Tensor) -> int:
