@@ -668,7 +668,15 @@ def vendor_gemm_bf16(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     key = ("workspace", x.device.index)
     ws = _VENDOR_STATE.get(key)
     if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            # (the library's handle and the workspace are made outside a capture: a product that is the first of its
+            # process and is being captured goes through torch)
+            return torch.nn.functional.linear(x, w)
         ws = _VENDOR_STATE[key] = torch.empty((VENDOR_WORKSPACE_BYTES,), dtype=torch.uint8, device=x.device)
+        warm = torch.zeros((16, 64), dtype=torch.bfloat16, device=x.device)
+        if _raw_library().ia_vendor_gemm_bf16(_p(torch.empty((16, 16), dtype=torch.bfloat16, device=x.device)), _p(warm),
+                                              _p(warm), 16, 16, 64, _p(ws), ws.numel(), _stream()) == 1:
+            _check(1)
     refused = _VENDOR_STATE.setdefault("refused", set())
     if (m, n, k) in refused:
         return torch.nn.functional.linear(x, w)

@@ -219,3 +219,24 @@ def test_preemption_in_bfloat16_stays_with_the_plain_model(tiny):
             toks.append(t)
     tight.cache.check_invariants()
     assert not tight.cache.sequences
+
+
+def test_captured_decode_steps_of_more_rows_than_the_own_products_take():
+    """160 requests decode together: their products go to the vendor's library, called directly, inside the captured
+    graph as in the eager step (every replay against the eager engine, bit for bit)."""
+    import torch
+    from inferrs_amd.config import Qwen3Config
+    from inferrs_amd.engine import Engine, Entry
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1000, hidden_size=256,
+               intermediate_size=512, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+               rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=512)
+    outs = {}
+    for graphs in (False, True):
+        eng = Engine.from_random(Qwen3Config.from_dict(raw), seed=1, dtype="bfloat16", page_size=16, num_pages=200,
+                                 max_seqs=170, use_graphs=graphs)
+        ids = [f"r{i}" for i in range(160)]
+        eng.step([Entry(r, [1 + i % 7, 2, 3, 4 + i % 5], [3]) for i, r in enumerate(ids)])
+        rows = [eng.step([Entry(r, [10 + step], [0]) for r in ids]).clone() for step in range(5)]
+        outs[graphs] = torch.stack(rows)
+        assert (eng.graph_replays >= 3) == graphs
+    assert torch.equal(outs[True], outs[False])
