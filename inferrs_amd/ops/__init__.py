@@ -113,6 +113,10 @@ def _declarations() -> Dict[str, Tuple[object, list]]:
         args = [] if params in ("", "void") else [ctype(a) for a in params.split(",")]
         restype = None if result == "void" else (ctypes.c_char_p if "char" in result else _C_TYPES[result])
         _DECLARATIONS[name] = (restype, args)
+    for must in ("ia_last_error", "ia_add_rmsnorm", "ia_gemm_skinny_bf16", "ia_attention_mfma", "ia_sample"):
+        if must not in _DECLARATIONS:
+            _DECLARATIONS.clear()
+            raise KernelError(f"api.h: the declaration of {must} was not found (the header's form has changed?)")
     return _DECLARATIONS
 
 
