@@ -172,7 +172,7 @@ def _check(code: int, target: str = "core") -> None:
 def _stream() -> int:
     # (the raw handle straight from the runtime: `torch.cuda.current_stream()` builds a Python object around it, 3 us
     # a kernel call)
-    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def _p(t: Optional[torch.Tensor]) -> Optional[int]:
