@@ -135,20 +135,23 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, decod
 
 
 def time_prefill(engine, n_tokens: int, runs: int, vocab: int):
-    """Seconds of each of `runs` prefills of one prompt of `n_tokens` tokens (after one that is not counted)."""
+    """Seconds of each of `runs` prefills of one prompt of `n_tokens` tokens, after three that are not counted: a shape's
+    first steps run eagerly and, where the host is their bound, the third is captured into a graph (prompts of up to
+    `Engine.GRAPH_MAX_TOKENS` tokens), so the counted runs are what a repeated shape settles at (the reference's own
+    bench counts five runs after one warm-up, `inferrs/src/bench.rs:27-33`)."""
     import torch
     from inferrs_amd.engine import Entry
     g = torch.Generator().manual_seed(2)
     prompt = torch.randint(0, vocab, (n_tokens,), generator=g).tolist()
     times = []
-    for r in range(runs + 1):
+    for r in range(runs + 3):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         engine.step([Entry("p", prompt, [n_tokens - 1])])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         engine.end_request("p")
-        if r > 0:
+        if r > 2:
             times.append(dt)
     return times
 

@@ -599,6 +599,7 @@ int iar_build_step(void* cache, int n_entries, const int64_t* keys, const int* q
         max_pages = pad_pages;
         max_kv = std::max(max_kv, pad_pages * ps);
         if (n_single) kv_single = std::max(kv_single, pad_pages * ps);
+        if (n_single < n_entries) kv_multi = std::max(kv_multi, pad_pages * ps);
     }
     const int n_want = want_off[n_entries];
     const long long total = 3LL * n + (n_entries + 1) + n_entries + n_want + (long long)n_groups * (n + (long long)n_entries * max_pages);

@@ -61,7 +61,8 @@ int iar_cache_check_invariants(void* cache);
 // the others after them; wanted rows keep the caller's order.  meta (16 ints): 0 total words,
 // 1 n tokens, 2 n requests, 3 n wanted, 4 max_pages, 5 max_q_len, 6 max_kv_len, 7 n_single,
 // 8 max_kv_single, 9 max_kv_multi, 10 n_groups.  order_out [s]: the caller's index of each request
-// in the new order.  pad_pages <= 0: as wide as needed.
+// in the new order.  pad_pages <= 0: as wide as needed; otherwise the tables are that wide and the bounds 6, 8 and 9
+// are at least the tokens that so many pages hold, so that they are the same for every step of that width.
 int iar_build_step(void* cache, int n_entries, const int64_t* keys, const int* q_lens, const int* tokens,
                    const int* want_counts, const int* want, int pad_pages, int advance, int32_t* out,
                    long long capacity, int* meta, int* order_out);

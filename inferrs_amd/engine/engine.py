@@ -11,6 +11,8 @@ everything earlier comes from the cache that previous steps left.
 from __future__ import annotations
 
 import logging
+import time
+from collections import OrderedDict
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import torch
@@ -39,8 +41,11 @@ class Entry:
 
 
 class Engine:
-    GRAPH_BUCKET_TOKENS = 1024      # a captured decode step serves context lengths up to a multiple of this
-    MAX_GRAPHS = 24
+    GRAPH_BUCKET_TOKENS = 1024      # a captured step serves context lengths up to a multiple of this
+    GRAPH_MAX_TOKENS = 1024         # steps of more tokens run eagerly: their kernels outlast the host, and a graph would hold their buffers
+    MAX_GRAPHS = 24                 # captured graphs kept (the one replayed longest ago goes first)
+    MAX_SHAPES_SEEN = 512           # shapes remembered as seen, with what was measured of them
+    GRAPH_HOST_SHARE = 0.8          # steps other than decode steps are captured where the host took this share of a step's time (0: always)
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: Optional[int] = None,
                  max_seqs: int = 32, cache_tokens: Optional[int] = None, memory_fraction: float = 0.9,
@@ -71,8 +76,8 @@ class Engine:
         self.cache = CacheManager(needs, page_size, num_pages, max_seqs)
         self.storage = CacheStorage(self.cache, model.dtype, self.device)
         self.builder = StepBuilder(self.cache, self.device)
-        # Decode steps (one token a request) are launch-bound: each distinct shape is captured
-        # into a HIP graph the second time it is seen and replayed from then on.
+        # Decode steps (one token a request) and steps of few tokens are bound by their launches: each distinct
+        # shape is captured into a HIP graph the second time it is seen and replayed from then on.
         self.use_graphs = use_graphs and model.graph_safe
         self.unused_tensors: List[str] = []
         self.stop_token_ids: Tuple[int, ...] = tuple(model.spec.eos_token_ids)
@@ -80,7 +85,8 @@ class Engine:
         self.load_notes: List[str] = model.load_notes(page_size)
         for note in self.load_notes:
             log.warning("%s", note)
-        self._graphs: Dict[Tuple[int, int, int], object] = {}
+        self._graphs: "OrderedDict[Tuple[int, ...], object]" = OrderedDict()      # shape -> (graph, its logits)
+        self._seen: "OrderedDict[Tuple[int, ...], object]" = OrderedDict()        # shapes that ran eagerly: "once", a measurement, or "eager" for good
         self._graphs_generation = self.builder.generation    # the staging buffer the graphs were captured over
         self.graph_replays = 0
 
@@ -146,9 +152,10 @@ class Engine:
         reserved for them are reserved here.  With `commit` the requests' cached lengths advance;
         a caller that passes False (the scheduler) does that itself.
 
-        The tensor that a decode step (one token a request) returns under `use_graphs` is the captured
-        graph's own output buffer: it holds this step's logits until the next step of the same shape
-        overwrites them.  Read or `.clone()` it before stepping again."""
+        The tensor that a step returns under `use_graphs` may be a captured graph's own output buffer (decode
+        steps and steps of up to `GRAPH_MAX_TOKENS` tokens whose shape has been seen before): it holds this
+        step's logits until the next step of the same shape overwrites them.  Read or `.clone()` it before
+        stepping again."""
         if not entries:
             raise StepError("a step needs at least one entry")
         vocab = self.spec.vocab_size
@@ -178,8 +185,9 @@ class Engine:
             raise
 
         triples = [(e.seq_id, e.tokens, e.want) for e in entries]
-        if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
-            logits = self._decode_step(triples)
+        n_tokens = sum(len(e.tokens) for e in entries)
+        if self.use_graphs and (n_tokens == len(entries) or n_tokens <= self.GRAPH_MAX_TOKENS):
+            logits = self._graphed_step(triples)
         else:
             logits = self.model.forward(self.builder.build(triples), self.storage)
         if commit:
@@ -197,8 +205,7 @@ class Engine:
             return False
         self._drop_stale_graphs()
         pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
-        entry = self._graphs.get((len(seq_ids), len(seq_ids), pad_pages))
-        return entry is not None and entry != "seen"
+        return self._decode_key(len(seq_ids), pad_pages) in self._graphs
 
     def decode_chain(self, seq_ids: Sequence[Hashable], tokens: Sequence[int], steps: int,
                      pick=None) -> Optional[List[List[int]]]:
@@ -213,7 +220,9 @@ class Engine:
         if not self.chain_ready(seq_ids, steps):
             return None
         pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
-        graph, logits = self._graphs[(len(seq_ids), len(seq_ids), pad_pages)]
+        key = self._decode_key(len(seq_ids), pad_pages)
+        graph, logits = self._graphs[key]
+        self._graphs.move_to_end(key)
         generation = self.builder.generation
         chosen = torch.empty((steps, len(seq_ids)), dtype=torch.int32, device=self.device)
         for i in range(steps):
@@ -230,33 +239,76 @@ class Engine:
             self.graph_replays += 1
         return chosen.cpu().tolist()
 
+    @staticmethod
+    def _decode_key(n_seqs: int, pad_pages: int) -> Tuple[int, ...]:
+        """The shape of a decode step of `n_seqs` requests that all want their logits."""
+        return (n_seqs, n_seqs, n_seqs, n_seqs, 1, pad_pages)
+
     def _drop_stale_graphs(self) -> None:
         """Captured graphs hold the address of the step builder's device buffer.  Any step, also one
-        that is not a decode step (a long prompt portion), may have made that buffer grow and move
+        that runs eagerly (a long prompt portion), may have made that buffer grow and move
         since: graphs captured over the old one are dropped before any of them is looked up."""
         if self._graphs_generation != self.builder.generation:
             self._graphs.clear()
+            self._seen.clear()
             self._graphs_generation = self.builder.generation
 
-    def _decode_step(self, triples) -> torch.Tensor:
-        """One token a request, through a captured graph when this shape has been seen before.
-        The block tables are padded to the bucket's width, so that every kernel argument is the
-        same for all context lengths of the bucket; lengths and pages are read from device memory.
-        The logits that are returned are the graph's own buffer: they hold until the next step."""
-        longest = self.cache.max_length([t[0] for t in triples]) + 1
+    def _graphed_step(self, triples) -> torch.Tensor:
+        """A step through a captured graph when its shape has been seen before.  The shape is what the launches
+        of a step depend on: the counts of requests, of tokens, of requests with a single token and of wanted
+        rows, the longest portion, and the width of the block tables.  The tables are padded to the bucket's
+        width and the bounds of the key lengths are the bucket's, so that every kernel argument is the same for
+        all context lengths of the bucket; lengths, positions and pages are read from device memory.  A shape's
+        eager steps run with the same arguments, so a step's logits do not depend on whether it was replayed.
+
+        Decode steps repeat by their nature and are captured the second time their shape is seen.  A capture
+        costs about one more step, which other steps only earn back where the host is their bound (small models,
+        few tokens): a shape's second step is timed, on the host and on the GPU, and its third is captured if
+        the host's share was `GRAPH_HOST_SHARE` or more; otherwise the shape stays eager.
+
+        The logits that a replayed step returns are the graph's own buffer: they hold until the next step of
+        the shape."""
+        singles = [t[0] for t in triples if len(t[1]) == 1]
+        longest = self.cache.max_length(singles) + 1 if singles else 0
+        for t in triples:
+            if len(t[1]) > 1:
+                longest = max(longest, self.cache.length(t[0]) + len(t[1]))
         pad_pages = self._bucket_pages(longest)
-        n_want = sum(len(t[2]) for t in triples)
         self._drop_stale_graphs()
         ctx = self.builder.build(triples, pad_pages=pad_pages)
         self._drop_stale_graphs()                       # (the buffer may have moved in this very build)
-        key = (len(triples), n_want, pad_pages)
+        key = (ctx.n_seqs, ctx.n_tokens, ctx.n_single, int(ctx.want_rows.shape[0]), ctx.max_q_len, pad_pages)
         entry = self._graphs.get(key)
-        if entry is None:
-            if len(self._graphs) >= self.MAX_GRAPHS:
-                self._graphs.pop(next(iter(self._graphs)))
-            self._graphs[key] = "seen"
-            return self.model.forward(ctx, self.storage)
-        if entry == "seen":
+        if entry is not None:
+            self._graphs.move_to_end(key)
+        else:
+            state = self._seen.get(key)
+            if state is None:
+                if len(self._seen) >= self.MAX_SHAPES_SEEN:
+                    self._seen.popitem(last=False)
+                self._seen[key] = "once"
+                return self.model.forward(ctx, self.storage)
+            if ctx.max_q_len > 1:
+                if state == "eager":
+                    return self.model.forward(ctx, self.storage)
+                if state == "once":
+                    # (the first step of a shape also pays for what is set up once; this one is the measure)
+                    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    begin.record()
+                    t0 = time.perf_counter()
+                    out = self.model.forward(ctx, self.storage)
+                    host_ms = (time.perf_counter() - t0) * 1e3
+                    end.record()
+                    self._seen[key] = (host_ms, begin, end)
+                    return out
+                host_ms, begin, end = state
+                # (a step that the GPU has not finished by now was not bound by the host either)
+                if self.GRAPH_HOST_SHARE > 0.0 and (not end.query() or host_ms < self.GRAPH_HOST_SHARE * begin.elapsed_time(end)):
+                    self._seen[key] = "eager"
+                    return self.model.forward(ctx, self.storage)
+            del self._seen[key]
+            while len(self._graphs) >= max(self.MAX_GRAPHS, 1):
+                self._graphs.popitem(last=False)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 out = self.model.forward(ctx, self.storage)

@@ -135,10 +135,11 @@ def plain_step(cache: plain.CacheManager, entries, pad_pages, advance):
         out += [np.asarray(slots, dtype=np.int32), table.reshape(-1)]
     kv = [st + n for st, n in zip(starts, q)]
     singles = [k for k, n in zip(kv, q) if n == 1]
+    multis = [k for k, n in zip(kv, q) if n != 1]
     meta = dict(n=sum(q), max_pages=max_pages, max_q=max(q), n_single=len(singles),
                 max_kv=max(kv + ([pad_pages * ps] if pad_pages else [])),
                 kv_single=max(singles + ([pad_pages * ps] if pad_pages and singles else []), default=0),
-                kv_multi=max([k for k, n in zip(kv, q) if n != 1], default=0))
+                kv_multi=max(multis + ([pad_pages * ps] if pad_pages and multis else []), default=0))
     return np.concatenate(out), meta, order
 
 

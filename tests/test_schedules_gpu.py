@@ -240,3 +240,100 @@ def test_captured_decode_steps_of_more_rows_than_the_own_products_take():
         outs[graphs] = torch.stack(rows)
         assert (eng.graph_replays >= 3) == graphs
     assert torch.equal(outs[True], outs[False])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_portions_of_a_prompt_across_a_bucket_boundary(tiny, dtype):
+    """Steps of few tokens are captured like decode steps where the host is their bound (forced here: the share of the
+    host that a capture asks for is set to nothing).  A prompt of 1,250 tokens in portions of 50 beside nothing else:
+    the shape repeats, so its first two steps run eagerly and the steps from the third on are replayed, until the
+    portion that passes 1,024 tokens starts another bucket.  The logits at every portion's first and last token are
+    those of an engine without graphs and of the plain model."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["D"]
+    vocab = TINY["D"]["vocab_size"]
+    total, portion = 1250, 50
+    toks = random_tokens(total, vocab, 77)
+    outs, replays = {}, []
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=total // 16 + 3, max_seqs=2, use_graphs=graphs)
+        eng.GRAPH_HOST_SHARE = 0.0
+        rows = []
+        for lo in range(0, total, portion):
+            rows.append(eng.step([Entry("p", toks[lo:lo + portion], [0, portion - 1])]).clone())
+            if graphs:
+                replays.append(eng.graph_replays)
+        eng.end_request("p")
+        eng.cache.check_invariants()
+        assert graphs or eng.graph_replays == 0
+        outs[graphs] = torch.cat(rows)
+    crossing = 1024 // portion                  # the portion that holds token 1,024
+    assert replays[1] == 0 and replays[crossing - 1] == crossing - 2           # eager, eager and timed, captured and replayed, replayed ...
+    assert replays[crossing + 1] == replays[crossing - 1]                      # another bucket: eager again
+    assert replays[-1] == replays[crossing - 1] + total // portion - crossing - 2
+    scale = float(outs[False].abs().max())
+    worst = float((outs[True] - outs[False]).abs().max()) / scale
+    assert worst <= (1e-6 if dtype == "float32" else 2e-2), worst
+    ref = pm.forward(cfg, params, toks)
+    at = [p for lo in range(0, total, portion) for p in (lo, lo + portion - 1)]
+    err = float((outs[True].cpu().double() - ref[at]).abs().max() / ref.abs().max())
+    assert err <= (1e-5 if dtype == "float32" else 3e-2), err
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_mixed_steps_equal_eager_ones(tiny, dtype):
+    """Two requests decode while others bring their prompts in portions of 24 tokens beside them: the mixed step's
+    shape repeats and is replayed from a graph from its third step on; between the rounds requests end and their pages go to the next.
+    Every step's logits are those of an engine without graphs, and the decoding requests' those of the plain model."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    rounds, portion, portions = 4, 24, 3
+    deco = {r: random_tokens(30 + rounds * portions + 2, vocab, 500 + i) for i, r in enumerate(("a", "b"))}
+    prompts = [random_tokens(portion * portions, vocab, 600 + i) for i in range(rounds)]
+    outs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=40, max_seqs=4, use_graphs=graphs)
+        eng.GRAPH_HOST_SHARE = 0.0                       # (captured whatever the host's share of the step)
+        eng.step([Entry(r, t[:30], []) for r, t in deco.items()])
+        at, rows = 30, []
+        for k, prompt in enumerate(prompts):
+            for j in range(portions):
+                entries = [Entry(f"p{k}", prompt[j * portion:(j + 1) * portion], [portion - 1])]
+                entries[1:1] = [Entry(r, [t[at]], [0]) for r, t in deco.items()]      # (the portion first, as a caller may give it)
+                rows.append(eng.step(entries).clone())
+                at += 1
+            eng.end_request(f"p{k}")
+        eng.cache.check_invariants()
+        if graphs:
+            assert eng.graph_replays >= rounds * portions - 2
+        outs[graphs] = rows
+    scale = max(float(r.abs().max()) for r in outs[False])
+    worst = max(float((g - e).abs().max()) for g, e in zip(outs[True], outs[False])) / scale
+    assert worst <= (1e-6 if dtype == "float32" else 2e-2), worst
+    for i, (r, t) in enumerate(deco.items()):
+        ref = pm.forward(cfg, params, t)
+        got = torch.stack([row[1 + i] for row in outs[True]]).cpu().double()
+        err = float((got - ref[30:30 + rounds * portions]).abs().max() / ref.abs().max())
+        assert err <= (1e-5 if dtype == "float32" else 3e-2), err
+    ref = pm.forward(cfg, params, prompts[-1])
+    got = torch.stack([row[0] for row in outs[True][-portions:]]).cpu().double()
+    err = float((got - ref[[portion - 1, 2 * portion - 1, 3 * portion - 1]]).abs().max() / ref.abs().max())
+    assert err <= (1e-5 if dtype == "float32" else 3e-2), err
+
+
+def test_a_shape_whose_step_the_gpu_bounds_stays_eager(tiny):
+    """The capture of a step other than a decode step is decided by a measurement: with a share that no host can
+    reach the shape is marked eager at its third step and never captured, and its logits are the same."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    prompt = random_tokens(40, vocab, 9)
+    eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=8, max_seqs=2)
+    eng.GRAPH_HOST_SHARE = 1e9
+    rows = []
+    for _ in range(5):
+        rows.append(eng.step([Entry("p", prompt, [39])]).clone())
+        eng.end_request("p")
+    assert eng.graph_replays == 0 and not eng._graphs and list(eng._seen.values()) == ["eager"]
+    assert all(torch.equal(rows[0], r) for r in rows[1:])
