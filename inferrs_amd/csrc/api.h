@@ -93,6 +93,9 @@ int ia_gemm_mid_fills(int N, int K, int dual);
 // (a fixed pipeline for measurements and tests: k steps of a chunk, 2 or 4, and stages, 2 to 4; (0, 0): the kernel's own
 // rule; no product depends on it bit for bit); anything else is an error and changes nothing
 int ia_gemm_mid_tune(int kc, int ns);
+// (how a block's waves share its products, for measurements and tests: 0 the kernel's own rule, 1 a tile of weight rows a
+// wave over all rows of the step, 2 two tiles a wave over half of the rows wherever the shape allows; the same bits)
+int ia_gemm_mid_blocking(int how);
 // (a fixed shape of the blocks for measurements and tests: waves a block, 2 to 8 (0: the kernel's own rule), ways k is split
 // and stages, 2 or 3 (2: four waves only); the caller's partial sums must have as many splits); a shape that has no
 // kernel is an error and changes nothing

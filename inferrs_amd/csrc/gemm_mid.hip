@@ -2,8 +2,10 @@
 // out[M, N] = x[M, K] . w[N, K]^T, bound by reading the weights once, like the skinny product, but with so
 // many rows that the activations can no longer be fetched by every wave for itself (at 64 rows they are as
 // large as a block's share of the weights).  65 to 128 rows (six or eight tiles of rows) walk k in chunks of 64, four
-// stages deep, so that the stages still fit a compute unit's shared memory; a wave then reads nine operands from
-// shared memory for eight matrix products, which is about what the memory delivers of weights meanwhile.  A [gate; up] whose blocks fill the chip evenly comes here with fewer rows
+// stages deep, so that the stages still fit a compute unit's shared memory.  From 49 rows on a wave takes two tiles of
+// weight rows over half of the step's rows where a block has an even number of waves (PAIRED below): at 128 rows six
+// operand reads from shared memory for eight matrix products instead of nine, in the same time that the memory takes to
+// deliver the weights.  A [gate; up] whose blocks fill the chip evenly comes here with fewer rows
 // too (ia_gemm_mid_bf16_scaled: rows of a residual stream whose norm the product finishes).
 //
 // The reference hands these products to cuBLAS like all others (`candle-core/src/cuda_backend/mod.rs:2260-2305`).
@@ -118,9 +120,68 @@ __device__ __forceinline__ void mid_finish(gmid_f32x4 (&acc)[MT], gmid_f32x4* sw
     }
 }
 
+// The end of the kernel for waves that hold two tiles of weight rows over MH tiles of rows from tile mt_first on
+// (PAIRED below).  DUAL: the two are the gate rows and the up rows of the same 16 features from n_first on, so nothing is
+// exchanged; otherwise the features n_first .. + 32.  The arithmetic is mid_finish's.
+template <int MH, bool DUAL>
+__device__ __forceinline__ void mid_finish_paired(gmid_f32x4 (&acc0)[MH], gmid_f32x4 (&acc1)[MH], void* out, int out_mode,
+                                                  int M, int N, int r, int g, int mt_first, int n_first, int split, int act) {
+#pragma unroll
+    for (int mt = 0; mt < MH; ++mt) {
+        const int m = (mt_first + mt) * 16 + r;
+        if (m >= M) continue;
+        if (DUAL) {
+            const int nb = n_first + 4 * g;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gate = bf16_bits_to_f32(f32_to_bf16_bits(acc0[mt][i]));
+                const float u = bf16_bits_to_f32(f32_to_bf16_bits(acc1[mt][i]));
+                v[i] = gate_act(gate, act) * u;
+            }
+            bf16_t* o = (bf16_t*)out + (size_t)m * N + nb;
+            if (nb + 3 < N && (N & 3) == 0) {
+                *(uint2*)o = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (nb + i < N) o[i].bits = f32_to_bf16_bits(v[i]);
+            }
+            continue;
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const gmid_f32x4 a = t == 0 ? acc0[mt] : acc1[mt];
+            const int nb = n_first + 16 * t + 4 * g;
+            if (out_mode == MID_OUT_BF16) {
+                bf16_t* o = (bf16_t*)out + (size_t)m * N + nb;
+                if (nb + 3 < N && (N & 3) == 0) {
+                    *(uint2*)o = make_uint2(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (nb + i < N) o[i].bits = f32_to_bf16_bits(a[i]);
+                }
+            } else {
+                float* o = (float*)out + ((size_t)(out_mode == MID_OUT_PARTIAL ? split : 0) * M + m) * N + nb;
+                if (nb + 3 < N && (N & 3) == 0) {
+                    *(gmid_f32x4*)o = a;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (nb + i < N) o[i] = a[i];
+                }
+            }
+        }
+    }
+}
+
 // KC: k steps of 32 in a chunk (a staged row is KC * 64 bytes); NS: stages, this chunk's and NS - 1 on their way; W: waves of
 // a block, a tile of 16 weight rows each (DUAL: W / 2 of gate rows, then W / 2 of up rows).
-template <int MT, bool DUAL, int KC, int NS, int W>
+// PAIRED: a wave multiplies two tiles of weight rows (DUAL: the gate rows and the up rows of the same features) with half of
+// the tiles of x, the block's first W / 2 waves with the first half and the others with the second: 2 + MT / 2 operand reads
+// from shared memory for MT matrix products instead of 1 + MT, and every sum in the same order.
+template <int MT, bool DUAL, int KC, int NS, int W, bool PAIRED = false>
 __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     void* __restrict__ out, int out_mode, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     int M, int N, int K, int k_per_block, const float* __restrict__ sums_in, int n_sums, float eps, int act) {
@@ -136,7 +197,10 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     constexpr int LOADS = (ROW_LOADS + W - 1) / W;          // load instructions a wave issues for a stage; where they do not
     constexpr int STAGE_BYTES = LOADS * W * 1024;           // divide, the last ones fetch a row of x again into a place nobody reads
     static_assert(!DUAL || W % 2 == 0, "gate and up rows: an even number of waves");
+    static_assert(!PAIRED || (W % 2 == 0 && MT % 2 == 0), "pairs of tiles over halves of the rows: even numbers of both");
     static_assert(NS >= 2 && NS <= 4 && (KC == 2 || KC == 4), "pipeline shape");
+    constexpr int MH = PAIRED ? MT / 2 : MT;                // tiles of rows a wave multiplies
+    constexpr int PAIRS = W / 2;
     __shared__ __attribute__((aligned(1024))) char mid_s0[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char mid_s1[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char mid_s2[NS > 2 ? STAGE_BYTES : 16];
@@ -159,6 +223,11 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
     constexpr int FEATURE_TILES = DUAL ? TILES / 2 : TILES;
     const int part = DUAL ? tile / FEATURE_TILES : 0;
     const int n_first = blockIdx.x * (16 * FEATURE_TILES) + 16 * (tile % FEATURE_TILES);
+    // PAIRED: the wave's two tiles of weight rows and the first of its tiles of x
+    const int pair = PAIRED ? wave % PAIRS : 0;
+    const int mt_first = PAIRED ? (wave / PAIRS) * MH : 0;
+    const int tile0 = PAIRED ? (DUAL ? pair : 2 * pair) : tile;
+    const int tile1 = PAIRED ? (DUAL ? FEATURE_TILES + pair : 2 * pair + 1) : tile;
     // rows 16 t + i of a stage's 256-byte (or 128-byte) rows collide on the same banks for every i: a row's pieces are
     // exchanged so that 16 rows at the same k fall on different places
     auto swizzle = [](int row) { return KC == 4 ? (row & 15) : ((row >> 1) & 7); };
@@ -204,15 +273,21 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
         }
         src[i] = (const char*)(base + k_begin) + piece * 16;
     }
-    uint32_t a_at[KC], b_at[KC];
+    uint32_t a_at[KC], a1_at[KC], b_at[KC];
 #pragma unroll
     for (int ks = 0; ks < KC; ++ks) {
-        b_at[ks] = (uint32_t)(r * ROW_BYTES + (((4 * ks + g) ^ swizzle(r)) * 16));
-        a_at[ks] = (uint32_t)((X_ROWS + 16 * tile) * ROW_BYTES) + b_at[ks];
+        const uint32_t in_tile = (uint32_t)(r * ROW_BYTES + (((4 * ks + g) ^ swizzle(r)) * 16));
+        b_at[ks] = (uint32_t)(mt_first * 16 * ROW_BYTES) + in_tile;
+        a_at[ks] = (uint32_t)((X_ROWS + 16 * tile0) * ROW_BYTES) + in_tile;
+        a1_at[ks] = (uint32_t)((X_ROWS + 16 * tile1) * ROW_BYTES) + in_tile;
     }
-    gmid_f32x4 acc[MT];
+    gmid_f32x4 acc[MH], acc1[PAIRED ? MH : 1];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MH; ++mt) acc[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
+    if constexpr (PAIRED) {
+#pragma unroll
+        for (int mt = 0; mt < MH; ++mt) acc1[mt] = (gmid_f32x4){0.f, 0.f, 0.f, 0.f};
+    }
     // Blocks start at different places of their range of k and wrap around: blocks that are started together and walk k in
     // step ask the same few memory channels at any moment (rows are a power of two apart).  The order of a sum depends
     // on the block, that is on the output feature, never on the step's rows.
@@ -234,11 +309,16 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
 #pragma unroll
         for (int ks = 0; ks < KC; ++ks) {
             const uint4 a = *(const uint4*)(stage + a_at[ks]);
+            uint4 a1 = a;
+            if constexpr (PAIRED) a1 = *(const uint4*)(stage + a1_at[ks]);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
+            for (int mt = 0; mt < MH; ++mt) {
                 const uint4 b = *(const uint4*)(stage + mt * (16 * ROW_BYTES) + b_at[ks]);
                 acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                     __builtin_bit_cast(gmid_bf16x8, a), __builtin_bit_cast(gmid_bf16x8, b), acc[mt], 0, 0, 0);
+                if constexpr (PAIRED)
+                    acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(gmid_bf16x8, a1), __builtin_bit_cast(gmid_bf16x8, b), acc1[mt], 0, 0, 0);
             }
         }
     };
@@ -308,7 +388,12 @@ __global__ __launch_bounds__(W * IA_WAVE) void gemm_mid_kernel(
             acc[0][0] *= scale; acc[0][1] *= scale; acc[0][2] *= scale; acc[0][3] *= scale;
         }
     }
-    mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split, act);
+    if constexpr (PAIRED) {
+        const int n_pair = blockIdx.x * (16 * FEATURE_TILES) + (DUAL ? 16 : 32) * pair;
+        mid_finish_paired<MH, DUAL>(acc, acc1, out, out_mode, M, N, r, g, mt_first, n_pair, split, act);
+    } else {
+        mid_finish<MT, DUAL, TILES>(acc, (gmid_f32x4*)mid_s1, out, out_mode, M, N, lane, r, g, tile, part, n_first, split, act);
+    }
 }
 
 // How a weight is shared out: a function of its shape and the chip alone, never of the rows of the step.
@@ -402,6 +487,16 @@ extern "C" int ia_gemm_mid_tune(int kc, int ns) {
     return 0;
 }
 
+// ia_gemm_mid_blocking(how): 0 the rule (two tiles of weight rows a wave over half of the rows where a step has more than
+// 48 rows and the block an even number of waves), 1 a tile a wave over all rows, always, 2 pairs wherever they can be.
+// For measurements and tests: both give the same bits.
+static int g_mid_blocking = 0;
+extern "C" int ia_gemm_mid_blocking(int how) {
+    IA_CHECK(how >= 0 && how <= 2, "gemm_mid_blocking: 0 (the rule), 1 (a tile a wave) or 2 (pairs), got %d", how);
+    g_mid_blocking = how;
+    return 0;
+}
+
 template <int MT, bool DUAL>
 static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w, int M, int N, int K, int splits,
                       const float* sums_in, int n_sums, float eps, int act, hipStream_t stream) {
@@ -421,8 +516,17 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
     IA_CHECK(plan.waves >= 2 && plan.waves <= MID_MAX_WAVES, "gemm_mid: a block of %d waves", plan.waves);
     const int k_block = K / splits;
 #define MID_SHAPE(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps, act)
+#define MID_PAIRED(KC, NS, W) gemm_mid_kernel<MT, DUAL, KC, NS, W, true><<<grid, W * IA_WAVE, 0, stream>>>(out, out_mode, x, w, M, N, K, k_block, sums_in, n_sums, eps, act)
     if constexpr (MT > 4) {
         // more than 64 rows: chunks of 64 k, four stages deep, whatever the plan's depth
+        if (g_mid_blocking != 1) {
+            switch (plan.waves) {
+                case 2: MID_PAIRED(2, 4, 2); return 0;
+                case 4: MID_PAIRED(2, 4, 4); return 0;
+                case 6: MID_PAIRED(2, 4, 6); return 0;
+                case 8: MID_PAIRED(2, 4, 8); return 0;
+            }
+        }
         switch (plan.waves) {
             case 2: MID_SHAPE(2, 4, 2); return 0;
             case 4: MID_SHAPE(2, 4, 4); return 0;
@@ -437,6 +541,16 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
             }
         }
     } else if (kc == 4 && plan.stages == 3) {
+        if constexpr (MT == 4 || MT == 2) {
+            if (MT == 4 ? g_mid_blocking != 1 : g_mid_blocking == 2) {
+                switch (plan.waves) {
+                    case 2: MID_PAIRED(4, 3, 2); return 0;
+                    case 4: MID_PAIRED(4, 3, 4); return 0;
+                    case 6: MID_PAIRED(4, 3, 6); return 0;
+                    case 8: MID_PAIRED(4, 3, 8); return 0;
+                }
+            }
+        }
         switch (plan.waves) {
             case 2: MID_SHAPE(4, 3, 2); return 0;
             case 4: MID_SHAPE(4, 3, 4); return 0;
@@ -456,6 +570,7 @@ static int launch_mid(void* out, int out_mode, const bf16_t* x, const bf16_t* w,
         if (kc == 2 && plan.stages == 4) { MID_SHAPE(2, 4, 4); return 0; }
     }
 #undef MID_SHAPE
+#undef MID_PAIRED
     IA_CHECK(false, "gemm_mid: no pipeline of %d waves, chunks of %d k steps, %d deep", plan.waves, kc, plan.stages);
     return 0;
 }

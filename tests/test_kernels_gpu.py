@@ -964,6 +964,42 @@ def test_mid_product_is_the_same_for_every_pipeline_shape():
         close(o[1], gate / (1 + torch.exp(-gate)) * up, 2 ** -7, "mid product with SiLU")
 
 
+@pytest.mark.parametrize("m", [20, 50, 64, 83, 96, 128])
+def test_mid_product_is_the_same_however_the_waves_share_a_block(m):
+    """A wave takes one tile of weight rows over all rows of the step, or two tiles (with the activation inside: the gate
+    rows and the up rows of the same features) over half of the rows: fewer operand reads, the same sums in the same
+    order.  Bit for bit, plain, split along k and with the activation inside, with features that fill no pair of tiles, for
+    every even number of waves."""
+    from inferrs_amd import ops
+    lib = ops.library()
+    n, k = 300, 1024
+    x = dev(randn(m, k, dtype=torch.bfloat16, seed=11))
+    w = dev(randn(n, k, dtype=torch.bfloat16, seed=12, scale=0.05))
+    wd = dev(randn(2 * n, k, dtype=torch.bfloat16, seed=13, scale=0.05))
+    try:
+        for waves in (0, 2, 4, 6, 8):
+            outs = []
+            for how in (1, 2):
+                assert lib.ia_gemm_mid_blocking(how) == 0
+                if waves:
+                    lib.ia_gemm_mid_plan(waves, 2, 3)
+                split = ops.gemm_mid_bf16(x, w, partial=True)
+                if waves:
+                    lib.ia_gemm_mid_plan(waves, 1, 3)
+                outs.append((split.parts.cpu() if isinstance(split, ops.Partials) else split.cpu(),
+                             ops.gemm_mid_bf16(x, w, torch.float32).cpu() if not waves else None,
+                             ops.gemm_mid_bf16(x, wd, dual=True).cpu()))
+            for a, b in zip(*outs):
+                assert a is None or torch.equal(a, b), (waves, m)
+        assert lib.ia_gemm_mid_blocking(3) != 0 and b"gemm_mid_blocking" in lib.ia_last_error()
+    finally:
+        lib.ia_gemm_mid_plan(0, 0, 0)
+        lib.ia_gemm_mid_blocking(0)
+    gate = (x.float().cpu() @ wd[:n].float().cpu().t()).bfloat16().float()
+    up = (x.float().cpu() @ wd[n:].float().cpu().t()).bfloat16().float()
+    close(outs[1][2], gate / (1 + torch.exp(-gate)) * up, 2 ** -7, "pairs of tiles with SiLU")
+
+
 def _gelu_tanh(x):
     return 0.5 * x * (1.0 + torch.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
 
