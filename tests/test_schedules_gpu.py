@@ -337,3 +337,27 @@ def test_a_shape_whose_step_the_gpu_bounds_stays_eager(tiny):
         eng.end_request("p")
     assert eng.graph_replays == 0 and not eng._graphs and list(eng._seen.values()) == ["eager"]
     assert all(torch.equal(rows[0], r) for r in rows[1:])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_portions_that_want_no_logits(tiny, dtype):
+    """Portions in the middle of a prompt ask for no logits: their shape (no wanted row) is captured and replayed like
+    any other, the cache they leave is the same, and the last portion's logits are those of an engine without graphs."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    toks = random_tokens(220, vocab, 5)
+    outs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=16, max_seqs=2, use_graphs=graphs)
+        eng.GRAPH_HOST_SHARE = 0.0
+        for lo in range(0, 200, 20):
+            empty = eng.step([Entry("p", toks[lo:lo + 20], [])])
+            assert tuple(empty.shape) == (0, vocab)
+        outs[graphs] = eng.step([Entry("p", toks[200:], [0, 19])]).clone()
+        assert eng.graph_replays == (8 if graphs else 0)
+    scale = float(outs[False].abs().max())
+    assert float((outs[True] - outs[False]).abs().max()) / scale <= (1e-6 if dtype == "float32" else 2e-2)
+    ref = pm.forward(cfg, params, toks)
+    err = float((outs[True].cpu().double() - ref[[200, 219]]).abs().max() / ref.abs().max())
+    assert err <= (1e-5 if dtype == "float32" else 3e-2), err
