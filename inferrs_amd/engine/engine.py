@@ -18,7 +18,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import torch
 
 from .. import ops
-from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..cache import CacheError, CacheManager, CacheStorage, OutOfPages
 from ..config.base import folder_stop_ids
 from ..config.registry import load_config
 from ..parts.assemble import generated_tensors, model_tensors
@@ -40,10 +40,14 @@ class Entry:
         self.seq_id, self.tokens, self.want = seq_id, list(tokens), list(want)
 
 
+# The hidden request whose rows fill a decode step up to the next of the batch sizes that graphs are captured for.
+_PAD = ("inferrs_amd", "rows that fill a decode step")
+
+
 class Engine:
     GRAPH_BUCKET_TOKENS = 1024      # a captured step serves context lengths up to a multiple of this
     GRAPH_MAX_TOKENS = 1024         # steps of more tokens run eagerly: their kernels outlast the host, and a graph would hold their buffers
-    MAX_GRAPHS = 24                 # captured graphs kept (the one replayed longest ago goes first)
+    MAX_GRAPHS = 48                 # captured graphs kept (the one replayed longest ago goes first)
     MAX_SHAPES_SEEN = 512           # shapes remembered as seen, with what was measured of them
     GRAPH_HOST_SHARE = 0.8          # steps other than decode steps are captured where the host took this share of a step's time (0: always)
 
@@ -73,7 +77,9 @@ class Engine:
             num_pages = max(1, budget // max(per_page, 1))
             # more than every request slot at the longest sequence is never used
             num_pages = min(num_pages, max_seqs * -(-model.spec.max_position // page_size))
-        self.cache = CacheManager(needs, page_size, num_pages, max_seqs)
+        # (one request slot more than asked for: the hidden request of the rows that fill a decode step takes none of the callers')
+        self.max_seqs = max_seqs
+        self.cache = CacheManager(needs, page_size, num_pages, max_seqs + 1)
         self.storage = CacheStorage(self.cache, model.dtype, self.device)
         self.builder = StepBuilder(self.cache, self.device)
         # Decode steps (one token a request) and steps of few tokens are bound by their launches: each distinct
@@ -194,6 +200,41 @@ class Engine:
             self.cache.commit_many([(e.seq_id, len(e.tokens)) for e in entries])
         return logits
 
+    @staticmethod
+    def padded_batch(n: int) -> int:
+        """The batch size whose graph a decode step of `n` requests runs on: every size up to 8 (where the products
+        change their kernels row by row), then in steps of 2 up to 16, of 4 up to 32, of 8 up to 64, of 16 up to
+        128 and of 32 beyond.  A batch that grows and shrinks request by request then walks through a few shapes
+        and not through one for every size."""
+        if n <= 8:
+            return n
+        step = 2 if n <= 16 else 4 if n <= 32 else 8 if n <= 64 else 16 if n <= 128 else 32
+        return -(-n // step) * step
+
+    def _pad_rows(self, n: int, tokens_ahead: int) -> int:
+        """Rows of the hidden request that a decode step of `n` requests gets on top, 0 when its size is one of
+        `padded_batch` or the rows cannot be had (no page free for them).  The hidden request has no cached token
+        and never gets one: each of its rows is token 0 at the first positions, written to its pages with the same
+        values by every row, and attends to itself alone; its logits are dropped.  It lives for the length of the
+        call that asked for it (`_drop_pad_rows` at that call's end): between steps nobody sees its pages missing,
+        and what its rows write reaches the pages before anything that a later step queues."""
+        extra = self.padded_batch(n) - n
+        if extra == 0:
+            return 0
+        try:
+            if not self.has_request(_PAD):
+                self.add_request(_PAD)
+            if not self.cache.ensure_reserved([(_PAD, tokens_ahead)]):
+                self._drop_pad_rows()
+                return 0
+        except CacheError:
+            return 0
+        return extra
+
+    def _drop_pad_rows(self) -> None:
+        if self.has_request(_PAD):
+            self.cache.free_sequence(_PAD)
+
     def _bucket_pages(self, longest: int) -> int:
         bucket_pages = max(1, self.GRAPH_BUCKET_TOKENS // self.page_size)
         return -(-(-(-longest // self.page_size)) // bucket_pages) * bucket_pages
@@ -205,7 +246,11 @@ class Engine:
             return False
         self._drop_stale_graphs()
         pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
-        return self._decode_key(len(seq_ids), pad_pages) in self._graphs
+        try:
+            n = len(seq_ids) + self._pad_rows(len(seq_ids), steps)
+        finally:
+            self._drop_pad_rows()
+        return self._decode_key(n, pad_pages) in self._graphs
 
     def decode_chain(self, seq_ids: Sequence[Hashable], tokens: Sequence[int], steps: int,
                      pick=None) -> Optional[List[List[int]]]:
@@ -220,24 +265,32 @@ class Engine:
         if not self.chain_ready(seq_ids, steps):
             return None
         pad_pages = self._bucket_pages(self.cache.max_length(seq_ids) + steps)
-        key = self._decode_key(len(seq_ids), pad_pages)
-        graph, logits = self._graphs[key]
-        self._graphs.move_to_end(key)
-        generation = self.builder.generation
-        chosen = torch.empty((steps, len(seq_ids)), dtype=torch.int32, device=self.device)
-        for i in range(steps):
-            triples = [(sid, [tok if i == 0 else 0], [0]) for sid, tok in zip(seq_ids, tokens)]
-            ctx = self.builder.build(triples, pad_pages=pad_pages, advance=i, skip_tokens=i > 0)
-            if self.builder.generation != generation:
-                raise RuntimeError("the staging buffer moved under a captured graph")
-            graph.replay()
-            if pick is None:
-                ops.argmax(logits, out=chosen[i])
-            else:
-                pick(logits, i, chosen[i])
-            ctx.token_ids.copy_(chosen[i])            # the next step's token ids, on the device
-            self.graph_replays += 1
-        return chosen.cpu().tolist()
+        n_real = len(seq_ids)
+        try:
+            extra = self._pad_rows(n_real, steps)     # (as in chain_ready: rows of the hidden request up to the graph's batch size)
+            key = self._decode_key(n_real + extra, pad_pages)
+            if key not in self._graphs:               # (the hidden request found pages a moment ago and finds none now)
+                return None
+            graph, logits = self._graphs[key]
+            self._graphs.move_to_end(key)
+            generation = self.builder.generation
+            # (zeros: the hidden request's rows take token 0 where `pick` chooses for the callers' rows only)
+            chosen = torch.zeros((steps, n_real + extra), dtype=torch.int32, device=self.device)
+            for i in range(steps):
+                triples = [(sid, [tok if i == 0 else 0], [0]) for sid, tok in zip(seq_ids, tokens)] + [(_PAD, [0], [0])] * extra
+                ctx = self.builder.build(triples, pad_pages=pad_pages, advance=i, skip_tokens=i > 0)
+                if self.builder.generation != generation:
+                    raise RuntimeError("the staging buffer moved under a captured graph")
+                graph.replay()
+                if pick is None:
+                    ops.argmax(logits, out=chosen[i])
+                else:
+                    pick(logits[:n_real], i, chosen[i, :n_real])
+                ctx.token_ids.copy_(chosen[i])            # the next step's token ids, on the device
+                self.graph_replays += 1
+        finally:
+            self._drop_pad_rows()
+        return chosen[:, :n_real].cpu().tolist()
 
     @staticmethod
     def _decode_key(n_seqs: int, pad_pages: int) -> Tuple[int, ...]:
@@ -254,6 +307,12 @@ class Engine:
             self._graphs_generation = self.builder.generation
 
     def _graphed_step(self, triples) -> torch.Tensor:
+        try:
+            return self._step_of_a_shape(triples)
+        finally:
+            self._drop_pad_rows()
+
+    def _step_of_a_shape(self, triples) -> torch.Tensor:
         """A step through a captured graph when its shape has been seen before.  The shape is what the launches
         of a step depend on: the counts of requests, of tokens, of requests with a single token and of wanted
         rows, the longest portion, and the width of the block tables.  The tables are padded to the bucket's
@@ -261,7 +320,9 @@ class Engine:
         all context lengths of the bucket; lengths, positions and pages are read from device memory.  A shape's
         eager steps run with the same arguments, so a step's logits do not depend on whether it was replayed.
 
-        Decode steps repeat by their nature and are captured the second time their shape is seen.  A capture
+        Decode steps repeat by their nature and are captured the second time their shape is seen; their batch is
+        filled up to the next size of `padded_batch` with rows of a hidden request, so that a batch which changes
+        request by request meets few shapes.  A capture
         costs about one more step, which other steps only earn back where the host is their bound (small models,
         few tokens): a shape's second step is timed, on the host and on the GPU, and its third is captured if
         the host's share was `GRAPH_HOST_SHARE` or more; otherwise the shape stays eager.
@@ -269,6 +330,10 @@ class Engine:
         The logits that a replayed step returns are the graph's own buffer: they hold until the next step of
         the shape."""
         singles = [t[0] for t in triples if len(t[1]) == 1]
+        n_want = sum(len(t[2]) for t in triples)
+        extra = self._pad_rows(len(triples), 1) if len(singles) == len(triples) else 0
+        if extra:
+            triples = list(triples) + [(_PAD, [0], [0])] * extra
         longest = self.cache.max_length(singles) + 1 if singles else 0
         for t in triples:
             if len(t[1]) > 1:
@@ -287,7 +352,7 @@ class Engine:
                 if len(self._seen) >= self.MAX_SHAPES_SEEN:
                     self._seen.popitem(last=False)
                 self._seen[key] = "once"
-                return self.model.forward(ctx, self.storage)
+                return self.model.forward(ctx, self.storage)[:n_want]
             if ctx.max_q_len > 1:
                 if state == "eager":
                     return self.model.forward(ctx, self.storage)
@@ -316,4 +381,4 @@ class Engine:
         graph, out = entry
         graph.replay()
         self.graph_replays += 1
-        return out
+        return out[:n_want] if extra else out

@@ -37,7 +37,7 @@ class GenerationLoop:
         self.decode_run = max(1, decode_run)
         limit = engine.spec.max_position if not max_seq_len else min(max_seq_len, engine.spec.max_position)
         self.scheduler = Scheduler(
-            engine.cache, max_batch_size=min(max_batch_size, engine.cache.max_seqs),
+            engine.cache, max_batch_size=min(max_batch_size, engine.max_seqs),
             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk, max_seq_len=limit,
             stop_token_ids=engine.stop_token_ids if stop_token_ids is None else stop_token_ids, row_multiple=row_multiple)
         self.sampler = Sampler(engine.device)

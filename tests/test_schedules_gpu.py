@@ -361,3 +361,87 @@ def test_captured_portions_that_want_no_logits(tiny, dtype):
     ref = pm.forward(cfg, params, toks)
     err = float((outs[True].cpu().double() - ref[[200, 219]]).abs().max() / ref.abs().max())
     assert err <= (1e-5 if dtype == "float32" else 3e-2), err
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_that_shrinks_request_by_request_meets_few_shapes(tiny, dtype):
+    """13 requests decode and one after the other ends: the steps of 13, 12, 11, 10 and 9 requests run on the graphs
+    of 14, 12 and 10 rows (the missing rows are a hidden request's, which lives inside a step only).  Every step's
+    logits are those of an engine without graphs, whose steps have no such rows; nothing of the hidden request is left."""
+    from inferrs_amd.engine import Engine, Entry
+    from inferrs_amd.engine.engine import _PAD
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    assert [Engine.padded_batch(n) for n in (1, 8, 9, 10, 13, 16, 17, 33, 100, 129)] == [1, 8, 10, 10, 14, 16, 20, 40, 112, 160]
+    seqs = {f"r{i:02d}": random_tokens(12 + 2 * i + 30, vocab, 70 + i) for i in range(13)}
+    outs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=13 * 9 + 2, max_seqs=13, use_graphs=graphs)
+        live = {r: 12 + 2 * i for i, r in enumerate(seqs)}
+        for r, n in live.items():
+            eng.step([Entry(r, seqs[r][:n], [])])
+        rows = []
+        for step in range(25):
+            if step and step % 5 == 0:
+                gone = sorted(live)[-1]
+                eng.end_request(gone)
+                del live[gone]
+            got = eng.step([Entry(r, [seqs[r][n]], [0]) for r, n in live.items()])
+            assert got.shape[0] == len(live)
+            rows.append(got.clone())
+            live = {r: n + 1 for r, n in live.items()}
+            assert not eng.has_request(_PAD)
+        eng.cache.check_invariants()
+        if graphs:
+            assert sorted(k[0] for k in eng._graphs if k[4] == 1) == [10, 12, 14] and eng.graph_replays >= 25 - 3
+        for r in live:
+            eng.end_request(r)
+        assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups) and not eng.cache.sequences
+        outs[graphs] = rows
+    scale = max(float(r.abs().max()) for r in outs[False])
+    worst = max(float((g - e).abs().max()) for g, e in zip(outs[True], outs[False])) / scale
+    assert worst <= (1e-6 if dtype == "float32" else 2e-2), worst
+    ref = pm.forward(cfg, params, seqs["r00"])
+    got = torch.stack([r[0] for r in outs[True]]).cpu().double()
+    err = float((got - ref[12:12 + 25]).abs().max() / ref.abs().max())
+    assert err <= (1e-5 if dtype == "float32" else 3e-2), err
+
+
+def test_a_pool_without_a_page_to_spare_runs_the_batch_as_it_is(tiny):
+    """The hidden request's rows need a page; where the callers' requests hold them all, the step runs with the rows
+    it has."""
+    from inferrs_amd.engine import Engine, Entry
+    folder, cfg, params = tiny["B"]
+    vocab = TINY["B"]["vocab_size"]
+    seqs = [random_tokens(7 + 6, vocab, 90 + i) for i in range(9)]
+    eng = Engine.from_folder(folder, dtype="bfloat16", page_size=8, num_pages=9 * 2, max_seqs=9)
+    for i, t in enumerate(seqs):
+        eng.step([Entry(i, t[:7], [])])
+    rows = []
+    for s in range(6):                                   # (from the second token on every request holds its two pages)
+        rows.append(eng.step([Entry(i, [t[7 + s]], [0]) for i, t in enumerate(seqs)]).clone())
+    assert [k[0] for k in eng._graphs if k[4] == 1] == [9] and eng.graph_replays >= 3      # (k[4]: the longest portion; 1 for decode steps)
+    ref = pm.forward(cfg, params, seqs[4])
+    got = torch.stack([r[4] for r in rows]).cpu().double()
+    assert float((got - ref[7:13]).abs().max() / ref.abs().max()) <= 3e-2
+
+
+def test_runs_of_decode_steps_with_rows_of_the_hidden_request(tiny):
+    """The generation loop queues runs of decode steps of 11 requests (graphs of 12 rows) that draw with seeds: the
+    tokens are those of single steps and of an engine without graphs' arithmetic, the hidden request's row is never seen."""
+    from inferrs_amd.engine import Engine, GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    prompts = [random_tokens(6 + i, vocab, 30 + i) for i in range(11)]
+    results = {}
+    for run in (1, 4):
+        eng = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=11 * 3 + 2, max_seqs=11)
+        loop = GenerationLoop(eng, decode_run=run, max_batch_size=11, stop_token_ids=[])
+        reqs = [loop.add(p, SamplingParams(temperature=0.9, top_k=20, seed=5 + i, max_tokens=18)) for i, p in enumerate(prompts)]
+        loop.run()
+        results[run] = [list(r.output) for r in reqs]
+        assert eng.graph_replays >= 10 and all(k[0] == 12 for k in eng._graphs if k[4] == 1 and k[0] > 8)
+        eng.cache.check_invariants()
+        assert not eng.cache.sequences
+    assert results[4] == results[1] and all(len(o) == 18 for o in results[1])
