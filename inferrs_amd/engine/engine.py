@@ -63,7 +63,7 @@ class Engine:
         self.device = model.device
         self.page_size = page_size
         needs = model.cache_needs()
-        probe = CacheManager(needs, page_size, 0, max_seqs)
+        probe = CacheManager(needs, page_size, 0, max_seqs + 1)
         if num_pages is None and cache_tokens is not None:
             num_pages = -(-cache_tokens // page_size)
         if num_pages is None:
