@@ -55,6 +55,18 @@ class SamplingParams:
         return self.repeat_last_n > 0 and (self.repetition_penalty != 1.0 or self.frequency_penalty != 0.0
                                            or self.presence_penalty != 0.0)
 
+    def draw_temperature(self, n_previous: int) -> float:
+        """The temperature that a token after `n_previous` others is drawn at (`sampler.rs:163-179`, `:232-236`):
+        the request's own; or 0 for the arg max, which a temperature under `SAMPLING_EPS` means only where nothing
+        changes the logits' order (no penalty over a window that holds a token, no bias) and no log-probability is
+        asked for; or else `SAMPLING_EPS`, at which the reference draws with the request's random number like at any
+        other temperature: among logits that are equal, or closer than a few times 1e-5, after the penalties, every
+        one can come."""
+        if self.temperature >= SAMPLING_EPS:
+            return self.temperature
+        untouched = not (self.has_penalty and n_previous > 0) and not self.logit_bias and not self.logprobs
+        return 0.0 if untouched else SAMPLING_EPS
+
     @property
     def is_plain_greedy(self) -> bool:
         """The reference's fast path: arg max of the untouched logits (`sampler.rs:171-179`)."""

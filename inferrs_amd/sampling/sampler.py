@@ -69,12 +69,12 @@ class Sampler:
             ops.penalize(logits, self._dev(window) if width else None, self._dev(rep), self._dev(freq),
                          self._dev(pres), bias_ids, bias_vals)
 
-        temperature = np.asarray([p.temperature for p in params], dtype=np.float32)
+        temperature = np.asarray([p.draw_temperature(len(prev)) for p, prev in zip(params, previous)], dtype=np.float32)
         top_k = np.asarray([p.top_k for p in params], dtype=np.int32)
         top_p = np.asarray([p.top_p for p in params], dtype=np.float32)
         min_p = np.asarray([p.min_p for p in params], dtype=np.float32)
         # the step of a draw is the number of tokens before it (`sampler.rs:323-325`)
-        u = np.asarray([rand_f32(seed, len(prev)) if p.temperature >= SAMPLING_EPS else 0.0
+        u = np.asarray([rand_f32(seed, len(prev)) if p.draw_temperature(len(prev)) >= SAMPLING_EPS else 0.0
                         for p, prev, seed in zip(params, previous, seeds)], dtype=np.float32)
         if not any(p.logprobs for p in params):
             out = ops.sample(logits, self._dev(temperature), self._dev(top_k), self._dev(top_p), self._dev(min_p),
@@ -132,12 +132,13 @@ class ChainDraw:
                     for j, (tid, b) in enumerate(sorted(p.logit_bias.items())):
                         ids[i, j], vals[i, j] = int(tid), float(b)
                 self.bias_ids, self.bias_vals = dev(ids), dev(vals)
-        self.temperature = dev(np.asarray([p.temperature for p in params], dtype=np.float32))
+        # (a window that holds a token at the run's start holds one at every step of it)
+        self.temperature = dev(np.asarray([p.draw_temperature(len(prev)) for p, prev in zip(params, previous)], dtype=np.float32))
         self.top_k = dev(np.asarray([p.top_k for p in params], dtype=np.int32))
         self.top_p = dev(np.asarray([p.top_p for p in params], dtype=np.float32))
         self.min_p = dev(np.asarray([p.min_p for p in params], dtype=np.float32))
         # the step of a draw is the number of tokens before it (`sampler.rs:323-325`)
-        self.u = dev(np.asarray([[rand_f32(seed, len(prev) + i) if p.temperature >= SAMPLING_EPS else 0.0
+        self.u = dev(np.asarray([[rand_f32(seed, len(prev) + i) if p.draw_temperature(len(prev)) >= SAMPLING_EPS else 0.0
                                   for p, prev, seed in zip(params, previous, seeds)] for i in range(steps)],
                                 dtype=np.float32).reshape(steps, rows))
 

@@ -222,6 +222,45 @@ def test_device_sampler_on_the_reference_cases(logits, history, kw, winner):
     assert got == [winner]
 
 
+def test_the_arg_max_is_taken_only_where_the_reference_takes_it():
+    """`sampler.rs:171-179`: a temperature under the threshold means the arg max of the untouched logits; with a penalty
+    over a window that holds a token, a bias or log-probabilities the reference goes on and draws at the threshold."""
+    eps = 1e-5
+    plain = SamplingParams(temperature=0.0, repetition_penalty=1.0)
+    assert plain.draw_temperature(0) == 0.0 and plain.draw_temperature(9) == 0.0
+    pen = SamplingParams(temperature=0.0, repetition_penalty=1.1)
+    assert pen.draw_temperature(0) == 0.0 and pen.draw_temperature(1) == eps          # an empty window changes nothing
+    assert SamplingParams(temperature=0.0, repetition_penalty=1.1, repeat_last_n=0).draw_temperature(5) == 0.0
+    assert SamplingParams(temperature=0.0, repetition_penalty=1.0, presence_penalty=0.5).draw_temperature(5) == eps
+    assert SamplingParams(temperature=0.0, repetition_penalty=1.0, logit_bias={3: 1.0}).draw_temperature(0) == eps
+    assert SamplingParams(temperature=0.0, repetition_penalty=1.0, logprobs=True).draw_temperature(0) == eps
+    assert SamplingParams(temperature=0.7).draw_temperature(5) == 0.7
+
+
+@pytest.mark.gpu
+def test_equal_favourites_under_a_penalty_at_temperature_zero_are_drawn():
+    """Two logits that are equal after a penalty touched the row, temperature 0: the reference does not take the arg max
+    there but draws at a temperature of 1e-5, so either favourite comes, by the request's random number; a third
+    that is 3e-5 below comes now and then too.  The device's draws are the plain transcription's, step by step, and
+    both favourites occur."""
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    z = torch.randn(1, 5000, generator=torch.Generator().manual_seed(1))
+    z[0, 1759] = z[0, 3155] = 7.0
+    z[0, 77] = 7.0 - 3e-5
+    kw = dict(temperature=0.0, top_p=1.0, top_k=1024, min_p=0.05, repetition_penalty=1.1, repeat_last_n=64,
+              frequency_penalty=0.3, presence_penalty=0.2)
+    seen = set()
+    for step in range(3, 43):
+        prev = [5, 6, 7] + [8] * (step - 3)
+        got = sampler.sample(z.to("cuda"), [SamplingParams(seed=11, **kw)], [prev], [11])[0]
+        assert got == pm.sample(z[0], prev, seed=11, **kw)
+        seen.add(got)
+    assert {1759, 3155} <= seen <= {1759, 3155, 77}
+    # without a token in the window nothing touches the row: the arg max, the first of the equal ones
+    assert sampler.sample(z.to("cuda"), [SamplingParams(seed=11, **kw)], [[]], [11]) == [1759]
+
+
 def test_sampling_params_defaults_are_the_reference_defaults():
     # inferrs/src/sampler.rs:90-112 and its test at :586-603
     p = SamplingParams()
