@@ -211,15 +211,18 @@ def rand_f32(seed: int, step: int) -> float:
 
 def sample(logits: torch.Tensor, previous: Sequence[int], *, temperature=0.7, top_p=0.9, top_k=50,
            min_p=0.0, repetition_penalty=1.1, repeat_last_n=64, frequency_penalty=0.0,
-           presence_penalty=0.0, seed: int = 0, logprobs: bool = False, top_logprobs: int = 0):
+           presence_penalty=0.0, seed: int = 0, logprobs: bool = False, top_logprobs: int = 0, logit_bias=None):
     """inferrs/src/sampler.rs:146-352, step by step, for a seeded request.  With `logprobs` the result is
     (token, its log-probability, [(id, log-probability)] of the kept list's first entries)."""
     z = logits.to(torch.float32).clone()
     vocab = z.numel()
     window = list(previous[-repeat_last_n:]) if repeat_last_n > 0 else []
     has_pen = (repetition_penalty != 1.0 or frequency_penalty != 0.0 or presence_penalty != 0.0) and window
-    if temperature < 1e-5 and not has_pen and not logprobs:                 # :176
+    if temperature < 1e-5 and not has_pen and not logit_bias and not logprobs:      # :175-179
         return int(torch.argmax(z))
+    for t, b in (logit_bias or {}).items():                                 # :185-190
+        if t < vocab:
+            z[t] = z[t] + torch.tensor(b, dtype=torch.float32)
     if repetition_penalty not in (1.0, 0.0) and window:                    # :196-209
         for t in dict.fromkeys(window):
             if t < vocab:

@@ -261,6 +261,35 @@ def test_equal_favourites_under_a_penalty_at_temperature_zero_are_drawn():
     assert sampler.sample(z.to("cuda"), [SamplingParams(seed=11, **kw)], [[]], [11]) == [1759]
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_a_bias_on_the_logits_against_the_plain_transcription(temperature):
+    """`sampler.rs:185-190`: the bias is added before the penalties; ids beyond the vocabulary are skipped; with a bias a
+    temperature of 0 is no arg max of the raw logits (a bias that lifts a token to the top wins, one that makes two equal
+    lets either come)."""
+    from inferrs_amd.sampling import Sampler
+    sampler = Sampler("cuda:0")
+    vocab = 3000
+    z = torch.randn(vocab, generator=torch.Generator().manual_seed(4)) * 2
+    top = int(torch.argmax(z))
+    second = int(torch.topk(z, 2).indices[1])
+    lift = {second: float(z[top] - z[second]) + 0.5, vocab + 7: 3.0}           # the second becomes the favourite
+    level = {17: 9.0 - float(z[17]), 2500: 9.0 - float(z[2500])}               # two tokens made equal, above all others
+    seen = set()
+    for bias in (lift, level):
+        for step in range(24):
+            prev = [1, 2] + [3] * step
+            kw = dict(temperature=temperature, top_p=0.95, top_k=40, repetition_penalty=1.2, repeat_last_n=16)
+            got = sampler.sample(z[None].to("cuda"), [SamplingParams(seed=9, logit_bias=bias, **kw)], [prev], [9])[0]
+            assert got == pm.sample(z, prev, seed=9, logit_bias=bias, **kw), (bias, step)
+            if bias is level:
+                seen.add(got)
+            elif temperature == 0.0:
+                assert got == second
+    if temperature == 0.0:
+        assert seen == {17, 2500}
+
+
 def test_sampling_params_defaults_are_the_reference_defaults():
     # inferrs/src/sampler.rs:90-112 and its test at :586-603
     p = SamplingParams()
