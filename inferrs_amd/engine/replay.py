@@ -36,7 +36,10 @@ def parse_step(line: str):
     for e in rec.get("entries") or []:
         if "id" not in e or "tokens" not in e:
             raise TraceError(f"step {rec['step']}: an entry needs 'id' and 'tokens'")
-        entries.append(Entry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want") or []]))
+        tokens, want = [int(t) for t in e["tokens"]], [int(w) for w in e.get("want") or []]
+        if not tokens and not want:
+            continue                                    # (an entry that brings nothing and asks for nothing)
+        entries.append(Entry(e["id"], tokens, want))
     return rec["step"], entries, list(rec.get("end") or [])
 
 

@@ -300,3 +300,19 @@ def test_cut_portions_make_the_steps_rows_a_whole_multiple():
     assert [len(e.tokens) for e in off.plan().entries] == [40]
     with pytest.raises(ValueError, match="row_multiple"):
         Scheduler(cache, max_batch_size=8, row_multiple=-1)
+
+
+def test_a_trace_line_is_read_as_it_is_written():
+    """The replay's reader: entries in their order with their wanted places in theirs, ids of any JSON kind, an entry that
+    brings nothing and asks for nothing left out, a step of nothing but ends, and errors that say what is missing."""
+    from inferrs_amd.engine.replay import TraceError, parse_step
+    step, entries, end = parse_step('{"step": 7, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [2, 0]}, '
+                                    '{"id": 4, "tokens": [9]}, {"id": "c", "tokens": [], "want": []}], "end": ["a"]}')
+    assert step == 7 and end == ["a"]
+    assert [(e.seq_id, e.tokens, e.want) for e in entries] == [("a", [5, 17, 3], [2, 0]), (4, [9], [])]
+    assert parse_step('{"step": 8, "end": ["b"]}') == (8, [], ["b"])
+    assert parse_step('{"step": 9, "entries": null, "end": null}') == (9, [], [])
+    for bad in ('{"entries": []}', 'not json', '[1, 2]', '{"step": 1, "entries": [{"tokens": [1]}]}',
+                '{"step": 1, "entries": [{"id": "a"}]}'):
+        with pytest.raises(TraceError):
+            parse_step(bad)
