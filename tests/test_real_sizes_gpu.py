@@ -1,5 +1,8 @@
 """The engine at the layer sizes of real models (Qwen3-8B: width 4,096, 32 query and 8 key/value heads of 128,
 feed-forward 12,288; Qwen3-14B: width 5,120, 40 query heads, feed-forward 17,408, a width that is no power of two;
+Qwen3-0.6B: width 1,024 under 16 heads of 128, so that the heads are twice as wide as the stream, the head tied to the
+table; Qwen3-4B: width 2,560, feed-forward 9,728; Qwen3-32B: 64 query heads, feed-forward 25,600, whose [gate; up] is past what
+the kernel with the activation inside takes at 17 to 64 rows;
 two layers each and a vocabulary of 40,000 so that the plain implementation stays quick) against the
 plain implementation in 64-bit: a prompt of 300 tokens whole and then token by token, 24 short requests decoded together,
 and (8B sizes) a prompt of 2,600 tokens in portions of 1,024 with tokens decoded behind it, and 40 tokens decoded from a
@@ -25,7 +28,10 @@ pytestmark = pytest.mark.gpu
 RAW = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=40000, hidden_size=4096,
            intermediate_size=12288, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
            rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
-SHAPES = {"8B": RAW, "14B": dict(RAW, hidden_size=5120, intermediate_size=17408, num_attention_heads=40)}
+SHAPES = {"8B": RAW, "14B": dict(RAW, hidden_size=5120, intermediate_size=17408, num_attention_heads=40),
+          "0.6B": dict(RAW, hidden_size=1024, intermediate_size=3072, num_attention_heads=16, tie_word_embeddings=True),
+          "4B": dict(RAW, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True),
+          "32B": dict(RAW, hidden_size=5120, intermediate_size=25600, num_attention_heads=64)}
 PROMPT, DECODED = 300, 24          # one long request: its prompt whole, then token by token
 CROWD, CROWD_PROMPT = 24, 30       # many short requests: their prompts in one step, then decoded together
 FAR, FAR_PORTION, FAR_DECODED = 2600, 1024, 6     # a request with a context of thousands: its prompt in portions, then token by token
