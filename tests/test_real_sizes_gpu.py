@@ -4,7 +4,7 @@ Qwen3-0.6B: width 1,024 under 16 heads of 128, so that the heads are twice as wi
 table; Qwen3-4B: width 2,560, feed-forward 9,728; Qwen3-32B: 64 query heads, feed-forward 25,600, whose [gate; up] is past what
 the kernel with the activation inside takes at 17 to 64 rows;
 two layers each and a vocabulary of 40,000 so that the plain implementation stays quick) against the
-plain implementation in 64-bit: a prompt of 300 tokens whole and then token by token, 24 short requests decoded together,
+plain implementation in 64-bit: a prompt of 300 tokens whole and then token by token, 24 short requests decoded together, the last of them beside the two portions of another request's prompt,
 and (8B sizes) a prompt of 2,600 tokens in portions of 1,024 with tokens decoded behind it, and 40 tokens decoded from a
 context of 1,000 on.  The tiny configurations reach every code path; this one runs the shapes that the
 size rules of the kernels pick at these widths (the skinny products with the stream inside up to 8 rows, the
@@ -36,6 +36,7 @@ PROMPT, DECODED = 300, 24          # one long request: its prompt whole, then to
 CROWD, CROWD_PROMPT = 24, 30       # many short requests: their prompts in one step, then decoded together
 FAR, FAR_PORTION, FAR_DECODED = 2600, 1024, 6     # a request with a context of thousands: its prompt in portions, then token by token
 CROSS, CROSS_DECODED = 1000, 40    # a request whose decoded tokens pass a context of 1,024: another captured graph, another split of the keys
+MIX, MIX_PORTION = 260, 150        # a request whose prompt comes in two portions beside the last eight decoding requests
 
 
 @pytest.fixture(scope="module", params=sorted(SHAPES))
@@ -57,6 +58,7 @@ def real(request, tmp_path_factory):
     reqs = {"long": random_tokens(PROMPT + DECODED, RAW["vocab_size"], 50)}
     for i in range(CROWD):
         reqs[f"c{i}"] = random_tokens(CROWD_PROMPT + 3 * i % 7 + 12, RAW["vocab_size"], 60 + i)
+    reqs["mix"] = random_tokens(MIX, RAW["vocab_size"], 53)
     if request.param == "8B":
         reqs["far"] = random_tokens(FAR + FAR_DECODED, RAW["vocab_size"], 51)
         reqs["cross"] = random_tokens(CROSS + CROSS_DECODED, RAW["vocab_size"], 52)
@@ -123,6 +125,14 @@ def run(folder, reqs, dtype):
             break
         rows = eng.step([Entry(r, [reqs[r][at[r]]], [0]) for r in live]).cpu().numpy()
         for r, row in zip(live, rows):
+            got[r][at[r]] = row
+            at[r] += 1
+    # two mixed steps: the decoding requests that are left beside a portion of another request's prompt
+    for lo, hi in ((0, MIX_PORTION), (MIX_PORTION, MIX)):
+        live = [r for r in live if at[r] < len(reqs[r])]
+        rows = eng.step([Entry("mix", reqs["mix"][lo:hi], [0, hi - lo - 1])] + [Entry(r, [reqs[r][at[r]]], [0]) for r in live]).cpu().numpy()
+        got["mix"][lo], got["mix"][hi - 1] = rows[0], rows[1]
+        for r, row in zip(live, rows[2:]):
             got[r][at[r]] = row
             at[r] += 1
     return got
