@@ -576,6 +576,23 @@ def main() -> int:
                 fractions[f"f32_prefill_{args.prefill_tokens}_layers{f32_layers}_fma"] = round(
                     prefill_flops(raw32, args.prefill_tokens) / min(times) / PEAK_FLOPS["fp32"], 4)
                 del eng32
+            # the smallest shape of the family, all its layers (the model that the reference's command line names as its
+            # example, inferrs/src/run.rs:35): steps so short that the kernels' fixed costs and, in eager steps, the host set the pace; prompts of
+            # a repeated length run from captured graphs there
+            if args.dtype == "bfloat16" and args.shape != "0.6B":
+                small = SHAPES["0.6B"]
+                note("the 0.6B shape: decode at batch 1 and 8 at a context of 2,048, prompts of 128 and 512 tokens")
+                eng_s = Engine.from_random(Qwen3Config.from_dict(small), seed=0, dtype="bfloat16", page_size=PAGE,
+                                           num_pages=8 * (2048 // PAGE + 2) + 8, max_seqs=9)
+                fill_storage(eng_s)
+                for b in (1, 8):
+                    el, ctx_mean = time_decode(eng_s, b, 2048, 16, 4, args.decode_run)
+                    points[f"shape0.6B_decode_b{b}_ctx2048"] = round(b * 16 / el, 2)
+                    fractions[f"shape0.6B_decode_b{b}_ctx2048"] = round(decode_bytes(small, b, ctx_mean, 2) / (el / 16) / 1e9 / PEAK_HBM_GBS, 4)
+                for tokens in (128, 512):
+                    times = time_prefill(eng_s, tokens, 3, small["vocab_size"])
+                    points[f"shape0.6B_prefill_{tokens}"] = round(tokens / (sum(times) / len(times)), 1)
+                del eng_s
     print(json.dumps(record))
     return 0
 
