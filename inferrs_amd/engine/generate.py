@@ -80,6 +80,10 @@ class GenerationLoop:
                                         [r.seed for r in running], k)
         tokens = self.engine.decode_chain(ids, [r.tokens[-1] for r in running], k,
                                           pick=None if draw.greedy else draw.pick)
+        if tokens is None:
+            # (the shape's graph wanted rows of the engine's hidden request, and the pages reserved above were the last:
+            # single steps then, which find their pages reserved)
+            return None
         done: List[Request] = []
         for i in range(k):
             done += sched.commit_decode(running, tokens[i])

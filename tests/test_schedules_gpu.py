@@ -445,3 +445,39 @@ def test_runs_of_decode_steps_with_rows_of_the_hidden_request(tiny):
         eng.cache.check_invariants()
         assert not eng.cache.sequences
     assert results[4] == results[1] and all(len(o) == 18 for o in results[1])
+
+
+def test_a_run_of_decode_steps_that_loses_its_hidden_rows_falls_back_to_single_steps(tiny):
+    """Nine requests decode on the graph of ten rows.  When the pages that a run of eight steps reserves for them are the
+    pool's last, the hidden request finds none, the run is not started (`decode_chain` says so) and the loop goes on
+    step by step: the tokens are those of a loop that never queues runs."""
+    from inferrs_amd.engine import Engine, Entry, GenerationLoop
+    from inferrs_amd.sampling import SamplingParams
+    folder, cfg, params = tiny["A"]
+    vocab = TINY["A"]["vocab_size"]
+    prompts = [random_tokens(13, vocab, 200 + i) for i in range(9)]
+    # the engine alone: the graph of ten rows is there, the pages go to the requests, the run is refused
+    eng = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=18, max_seqs=9)
+    for i, p in enumerate(prompts):
+        eng.step([Entry(i, p, [])])
+    for s in range(3):                                   # positions 13, 14, 15: a page each, nine to spare
+        eng.step([Entry(i, [1 + s], [0]) for i in range(9)])
+    assert [k[0] for k in eng._graphs if k[4] == 1] == [10]
+    ids = list(range(9))
+    assert eng.chain_ready(ids, 8)
+    for i in ids:
+        assert eng.cache.reserve(i, 8)
+    assert all(g.pool.num_free == 0 for g in eng.cache.groups)
+    assert eng.decode_chain(ids, [5] * 9, 8) is None
+    eng.cache.check_invariants()
+    # the loop: the same tokens with and without runs
+    results = {}
+    for run in (1, 8):
+        eng = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=18, max_seqs=9)
+        loop = GenerationLoop(eng, decode_run=run, max_batch_size=9, stop_token_ids=[])
+        reqs = [loop.add(p, SamplingParams.greedy(max_tokens=16)) for p in prompts]
+        loop.run()
+        results[run] = [list(r.output) for r in reqs]
+        eng.cache.check_invariants()
+        assert not eng.cache.sequences
+    assert results[8] == results[1] and all(len(o) == 16 for o in results[1])
