@@ -592,6 +592,8 @@ def main() -> int:
                 for tokens in (128, 512):
                     times = time_prefill(eng_s, tokens, 3, small["vocab_size"])
                     points[f"shape0.6B_prefill_{tokens}"] = round(tokens / (sum(times) / len(times)), 1)
+                    fractions[f"shape0.6B_prefill_{tokens}_mfma"] = round(
+                        prefill_flops(small, tokens) / (sum(times) / len(times)) / PEAK_FLOPS["bf16"], 4)
                 del eng_s
     print(json.dumps(record))
     return 0

@@ -42,7 +42,10 @@ def test_decode_record_has_the_agreed_keys():
     for step in rec["eager_steps"].values():
         assert step["wall_ms"] > 0 and step["graph_ms"] > 0 and step["kernel_calls"] > 0 and 0 <= step["host_frac"] < 1
     assert all(isinstance(v, (int, float)) and v > 0 for v in rec["points"].values())
-    assert set(rec["points"]) <= set(rec["points_hbm_frac"]) | {"prefill_8192", "prefill_128", "prefill_512", "f32_prefill_2048_layers2"}
+    # (every decode point has its share of the memory's peak under its own name, every prompt its share of the matrix peak)
+    assert set(rec["points"]) <= set(rec["points_hbm_frac"]) | {"prefill_8192", "prefill_128", "prefill_512", "f32_prefill_2048_layers2",
+                                                                  "shape0.6B_prefill_128", "shape0.6B_prefill_512"}
+    assert {"shape0.6B_decode_b1_ctx2048", "shape0.6B_decode_b8_ctx2048", "shape0.6B_prefill_128_mfma"} <= set(rec["points_hbm_frac"])
     assert rec["prefill"]["tokens"] == 2048 and rec["prefill"]["value"] > 0 and 0 < rec["prefill"]["frac"] < 1
     # mean and deviation over five repetitions, for decode and prefill
     assert rec["decode_runs"]["runs"] == 5 and rec["decode_runs"]["ms_per_step_mean"] > 0 and rec["decode_runs"]["ms_per_step_std"] >= 0
