@@ -144,8 +144,11 @@ class Part:
     kind = "?"
     # True when `forward` launches the same kernels with the same arguments for every step of
     # one shape, reading everything that changes (positions, pages, slots) from device memory:
-    # only then may a decode step that contains the part be captured into a graph and replayed.
+    # only then may a step that contains the part be captured into a graph and replayed.
     # A part that looks at the host-side lists of the step context must leave this False.
+    # A captured decode step may hold several rows of one hidden request (the engine fills a batch
+    # up to the size its graph was captured for): the same token at the same position with the same
+    # cache slot and state slot, so that every such row writes the same values to the same place.
     graph_safe = False
 
     @classmethod
